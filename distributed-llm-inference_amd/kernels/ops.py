@@ -1,0 +1,309 @@
+"""Typed wrappers around the library's ``extern "C"`` entry points.
+
+Every wrapper checks on the host that the operands have the device, type, layout and sizes that
+its kernel and launch grid assume, and raises :class:`KernelArgumentError` otherwise: a kernel is
+never launched on operands it was not written for. torch supplies device memory and the current
+stream; nothing here computes with torch.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+_c_int, _c_i64, _c_float, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+
+class KernelArgumentError(ValueError):
+    """Operands that a kernel does not take."""
+
+
+class KernelLaunchError(RuntimeError):
+    """The HIP runtime refused a launch."""
+
+
+_SIGNATURES = {
+    "dli_embedding": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_rms_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_add": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_gather_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_to_float": [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
+    "dli_copy_pages": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_i64, _c_int, _c_ptr],
+    "dli_fill": [_c_ptr, _c_float, _c_i64, _c_int, _c_ptr],
+    "dli_rope_kv_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                          _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_gemm_f32_nt": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int,
+                        _c_int, _c_int, _c_ptr],
+    "dli_attention_generic_tile_rows": [_c_int],
+    "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
+                              _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                              _c_int, _c_int, _c_ptr],
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def library() -> ctypes.CDLL:
+    """The loaded HIP library with argument types declared (compiled at the first call if absent)."""
+    global _lib
+    if _lib is None:
+        lib = build.load()
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(lib, name, None)
+            if fn is None:
+                raise build.KernelBuildError(f"{build.loaded_path()} lacks the entry point {name}")
+            fn.argtypes = argtypes
+            fn.restype = _c_int
+        _lib = lib
+    return _lib
+
+
+def _check(status: int, name: str) -> None:
+    if status == 0:
+        return
+    if status == -1:
+        raise KernelArgumentError(f"{name}: the kernel does not take these sizes")
+    raise KernelLaunchError(f"{name}: launch failed (status {status})")
+
+
+def _stream() -> _c_ptr:
+    return _c_ptr(torch.cuda.current_stream().cuda_stream)
+
+
+def _is_bf16(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return 1
+    if dtype == torch.float32:
+        return 0
+    raise KernelArgumentError(f"activation type {dtype} is neither float32 nor bfloat16")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> _c_ptr:
+    return _c_ptr(0 if t is None else t.data_ptr())
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelArgumentError(msg)
+
+
+def _dense(t: torch.Tensor, name: str, dtype: Optional[torch.dtype] = None, ndim: Optional[int] = None) -> None:
+    _require(t.is_cuda, f"{name} is not on the GPU")
+    _require(t.is_contiguous(), f"{name} is not contiguous")
+    if dtype is not None:
+        _require(t.dtype == dtype, f"{name} has type {t.dtype}, expected {dtype}")
+    if ndim is not None:
+        _require(t.dim() == ndim, f"{name} has {t.dim()} dimensions, expected {ndim}")
+
+
+def _rows(t: torch.Tensor, name: str, dtype: torch.dtype) -> None:
+    """A 2-D operand whose rows are contiguous (a row stride larger than the width is allowed)."""
+    _require(t.is_cuda, f"{name} is not on the GPU")
+    _require(t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= t.shape[1],
+             f"{name} is not a matrix with contiguous rows")
+    _require(t.dtype == dtype, f"{name} has type {t.dtype}, expected {dtype}")
+
+
+# ----------------------------------------------------------------------------- element-wise
+
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t] = table[ids[t]]``; ids int32 and already checked against the table's rows."""
+    _dense(table, "table", ndim=2)
+    _dense(ids, "ids", torch.int32, 1)
+    _dense(out, "out", table.dtype, 2)
+    _require(out.shape == (ids.shape[0], table.shape[1]), "out must be [len(ids), width]")
+    _check(library().dli_embedding(_ptr(table), _ptr(ids), _ptr(out), ids.shape[0], table.shape[1],
+                                   _is_bf16(table.dtype), _stream()), "embedding")
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+             delta: Optional[torch.Tensor] = None, sum_out: Optional[torch.Tensor] = None) -> None:
+    """``out = weight * cast(x * rsqrt(mean(x^2) + eps))``. With ``delta``: x is first replaced by
+    ``x + delta`` (written to ``sum_out``, which may be ``x`` itself)."""
+    _dense(x, "x", ndim=2)
+    _dense(weight, "weight", torch.float32, 1)
+    _dense(out, "out", x.dtype, 2)
+    _require(weight.shape[0] == x.shape[1], "weight length differs from the row width")
+    _require(out.shape == x.shape, "out differs from x in shape")
+    if delta is not None:
+        _dense(delta, "delta", x.dtype, 2)
+        _require(sum_out is not None, "delta needs sum_out")
+        _dense(sum_out, "sum_out", x.dtype, 2)
+        _require(delta.shape == x.shape and sum_out.shape == x.shape, "delta/sum_out differ from x in shape")
+    _check(library().dli_rms_norm(_ptr(x), _ptr(delta), _ptr(weight), _ptr(sum_out), _ptr(out), x.shape[0],
+                                  x.shape[1], float(eps), _is_bf16(x.dtype), _stream()), "rms_norm")
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = silu(gate_up[:, :I]) * gate_up[:, I:]``."""
+    _dense(gate_up, "gate_up", ndim=2)
+    _dense(out, "out", gate_up.dtype, 2)
+    _require(gate_up.shape[1] == 2 * out.shape[1] and gate_up.shape[0] == out.shape[0],
+             "gate_up must be [rows, 2*I] for out [rows, I]")
+    _check(library().dli_silu_mul(_ptr(gate_up), _ptr(out), out.shape[0], out.shape[1],
+                                  _is_bf16(out.dtype), _stream()), "silu_mul")
+
+
+def add(a: torch.Tensor, b: Optional[torch.Tensor], out: torch.Tensor,
+        bias: Optional[torch.Tensor] = None) -> None:
+    """``out = (a + bias) + b``; sums in 32-bit. ``out`` may alias ``a`` or ``b``."""
+    _dense(a, "a", ndim=2)
+    _dense(out, "out", a.dtype, 2)
+    _require(out.shape == a.shape, "out differs from a in shape")
+    if b is not None:
+        _dense(b, "b", a.dtype, 2)
+        _require(b.shape == a.shape, "b differs from a in shape")
+    if bias is not None:
+        _dense(bias, "bias", a.dtype, 1)
+        _require(bias.shape[0] == a.shape[1], "bias length differs from the row width")
+    _check(library().dli_add(_ptr(a), _ptr(b), _ptr(bias), _ptr(out), a.shape[0], a.shape[1],
+                             _is_bf16(a.dtype), _stream()), "add")
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[i] = x[rows[i]]``; rows int32, already checked against x's rows."""
+    _dense(x, "x", ndim=2)
+    _dense(rows, "rows", torch.int32, 1)
+    _dense(out, "out", x.dtype, 2)
+    _require(out.shape == (rows.shape[0], x.shape[1]), "out must be [len(rows), width]")
+    _check(library().dli_gather_rows(_ptr(x), _ptr(rows), _ptr(out), rows.shape[0], x.shape[1],
+                                     _is_bf16(x.dtype), _stream()), "gather_rows")
+
+
+def to_float(x: torch.Tensor, out: torch.Tensor) -> None:
+    _dense(x, "x")
+    _dense(out, "out", torch.float32)
+    _require(out.numel() == x.numel(), "out differs from x in size")
+    _check(library().dli_to_float(_ptr(x), _ptr(out), x.numel(), _is_bf16(x.dtype), _stream()), "to_float")
+
+
+def fill(x: torch.Tensor, value: float) -> None:
+    _dense(x, "x")
+    _check(library().dli_fill(_ptr(x), float(value), x.numel(), _is_bf16(x.dtype), _stream()), "fill")
+
+
+def copy_pages(pool: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Copy page ``src[i]`` onto page ``dst[i]`` in every layer, keys and values.
+
+    ``pool`` is ``[layers, 2, pages, ...]``; the page ids are int32 and already range-checked.
+    """
+    _dense(pool, "pool")
+    _require(pool.dim() >= 4 and pool.shape[1] == 2, "pool must be [layers, 2, pages, ...]")
+    _dense(src, "src", torch.int32, 1)
+    _dense(dst, "dst", torch.int32, 1)
+    _require(src.shape == dst.shape, "src and dst differ in length")
+    pages = pool.shape[2]
+    page_elems = pool[0, 0, 0].numel()
+    _check(library().dli_copy_pages(_ptr(pool), _ptr(src), _ptr(dst), src.shape[0], pool.shape[0] * 2, pages,
+                                    page_elems, _is_bf16(pool.dtype), _stream()), "copy_pages")
+
+
+# ----------------------------------------------------------------------------- position + cache write
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                  rotary_dim: int, slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                  v_pages: Optional[torch.Tensor], q_heads: int, kv_heads: int, head_dim: int) -> None:
+    """Rotate q (in place) and k, and write rotated k and raw v at each token's cache slot.
+
+    ``qkv`` is ``[tokens, (q_heads + 2*kv_heads) * head_dim]``; ``k_pages`` is
+    ``[pages, kv_heads, page_size, head_dim]`` and ``v_pages`` ``[pages, kv_heads, head_dim,
+    page_size]``; ``slots[t] = page * page_size + offset`` (negative: the token is not cached).
+    """
+    _rows(qkv, "qkv", qkv.dtype)
+    n = qkv.shape[0]
+    _require(qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim, "qkv width differs from (q+2kv)*head_dim")
+    _dense(positions, "positions", torch.int32, 1)
+    _require(positions.shape[0] == n, "positions differ from qkv in rows")
+    page_size = 1
+    if inv_freq is not None:
+        _dense(inv_freq, "inv_freq", torch.float32, 1)
+        _require(inv_freq.shape[0] * 2 == rotary_dim, "inv_freq must hold rotary_dim/2 frequencies")
+    if kv_heads > 0:
+        _require(slots is not None and k_pages is not None and v_pages is not None,
+                 "kv heads need slots and pages")
+        _dense(slots, "slots", torch.int32, 1)
+        _require(slots.shape[0] == n, "slots differ from qkv in rows")
+        _dense(k_pages, "k_pages", qkv.dtype, 4)
+        _dense(v_pages, "v_pages", qkv.dtype, 4)
+        page_size = k_pages.shape[2]
+        _require(k_pages.shape[1] == kv_heads and k_pages.shape[3] == head_dim,
+                 "k_pages must be [pages, kv_heads, page_size, head_dim]")
+        _require(v_pages.shape == (k_pages.shape[0], kv_heads, head_dim, page_size),
+                 "v_pages must be [pages, kv_heads, head_dim, page_size]")
+    _check(library().dli_rope_kv_write(
+        _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(inv_freq), rotary_dim, _ptr(slots), _ptr(k_pages),
+        _ptr(v_pages), n, q_heads, kv_heads, head_dim, page_size, _is_bf16(qkv.dtype), _stream()),
+        "rope_kv_write")
+
+
+# ----------------------------------------------------------------------------- matrix products
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             residual: Optional[torch.Tensor] = None) -> None:
+    """``out = a @ w.T (+ bias) (+ residual)`` in IEEE single precision; ``w`` is ``[n, k]``."""
+    _rows(a, "a", torch.float32)
+    _rows(w, "w", torch.float32)
+    _rows(out, "out", torch.float32)
+    m, k = a.shape
+    n = w.shape[0]
+    _require(w.shape[1] == k, "a and w differ in inner size")
+    _require(out.shape == (m, n), "out must be [rows of a, rows of w]")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == n, "bias length differs from rows of w")
+    ldr = 0
+    if residual is not None:
+        _rows(residual, "residual", torch.float32)
+        _require(residual.shape == (m, n), "residual differs from out in shape")
+        ldr = residual.stride(0)
+    _check(library().dli_gemm_f32_nt(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias), _ptr(residual),
+                                     ldr, _ptr(out), out.stride(0), m, n, k, _stream()), "gemm_f32")
+
+
+# ----------------------------------------------------------------------------- attention
+
+def attention_generic_tile_rows(head_dim: int) -> int:
+    rows = library().dli_attention_generic_tile_rows(head_dim)
+    if rows <= 0:
+        raise KernelArgumentError(
+            f"attention takes head_dim in steps of 16 up to 256, not {head_dim}")
+    return rows
+
+
+def attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                      q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
+                      tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
+                      window: int = 0) -> None:
+    """Paged causal attention for a batch of portions (vector units, 32-bit arithmetic).
+
+    ``q`` and ``out`` are ``[tokens, q_heads*head_dim]`` (rows contiguous, any row stride);
+    ``q_start [entries+1]``, ``kv_len [entries]``, ``block_tables [entries, width]`` describe the
+    requests; ``tile_entry/tile_q0`` list the query tiles of ``attention_generic_tile_rows`` rows.
+    """
+    _dense(k_pages, "k_pages", ndim=4)
+    dtype = k_pages.dtype
+    _rows(q, "q", dtype)
+    _rows(out, "out", dtype)
+    pages, kv_heads, page_size, head_dim = k_pages.shape
+    _dense(v_pages, "v_pages", dtype, 4)
+    _require(v_pages.shape == (pages, kv_heads, head_dim, page_size),
+             "v_pages must be [pages, kv_heads, head_dim, page_size]")
+    _require(q.shape[1] == q_heads * head_dim and out.shape == q.shape, "q/out must be [tokens, q_heads*head_dim]")
+    _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
+    for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
+        _dense(t, name, torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    entries = kv_len.shape[0]
+    _require(q_start.shape[0] == entries + 1 and block_tables.shape[0] >= entries,
+             "q_start/kv_len/block_tables disagree on the number of requests")
+    _require(tile_entry.shape == tile_q0.shape, "tile lists differ in length")
+    _check(library().dli_attention_generic(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start),
+        _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0),
+        tile_entry.shape[0], q_heads, kv_heads, head_dim, page_size, float(scale), int(window),
+        _is_bf16(dtype), _stream()), "attention_generic")

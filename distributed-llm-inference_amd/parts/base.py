@@ -1,0 +1,162 @@
+"""What a part of each family must provide.
+
+Every part is constructed as ``cls(runtime, **params)`` with its sizes and constants as keyword
+parameters (nothing is read from a model-wide configuration: a part does not know which model it
+is in), declares the tensors it binds (:meth:`Part.weight_specs`, names relative to its prefix) and
+receives them in :meth:`Part.load_weights`.
+
+Activations are ``[tokens, width]`` tensors of the runtime's activation type, rows of all requests
+of the step laid end to end; what belongs to which request is in the :class:`StepContext`.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Mapping, Optional
+
+import torch
+
+from .spec import WeightSpec
+
+
+@dataclass
+class Runtime:
+    """Where and in which type the model computes."""
+
+    device: torch.device
+    dtype: torch.dtype  # torch.float32 (true 32-bit path) or torch.bfloat16 (serving)
+
+    @property
+    def is_bf16(self) -> bool:
+        return self.dtype == torch.bfloat16
+
+    def empty(self, *shape: int, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return torch.empty(*shape, device=self.device, dtype=dtype or self.dtype)
+
+
+# ------------------------------------------------------------------------------ cache requirements
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """A mixer that keeps keys and values of ``kv_heads x head_dim`` per token in pages.
+
+    ``window`` > 0: only the last ``window`` keys are ever read, so pages that lie wholly before
+    the window may be given back while the request still runs. Layers with equal specs share one
+    group of pages and one block table.
+    """
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """A mixer that keeps a fixed-size state per request: ``shape`` elements of ``dtype`` in the
+    slot that the request holds from admission to its end. The slot is zeroed when a request
+    takes it."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    family: str = ""
+    kind: str = ""
+    prefix: str = ""
+
+    def __init__(self, runtime: Runtime) -> None:
+        self.rt = runtime
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        """Tensors of this part by local name (the checkpoint name is ``prefix + name``)."""
+        return {}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Receive the tensors of :meth:`weight_specs`, already on the device and typed by role."""
+
+    def sub_parts(self) -> dict[str, "Part"]:
+        """Parts owned by this one (their prefix is relative to the checkpoint root)."""
+        return {}
+
+
+class Embedding(Part):
+    """Token ids to rows: ``forward(ids int32 [n]) -> [n, hidden]``."""
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def table(self) -> torch.Tensor:
+        """The ``[vocab, hidden]`` table, for a head that is tied to it."""
+        raise NotImplementedError
+
+
+class Norm(Part):
+    """Row-wise normalisation: ``forward(x) -> y``; ``forward(x, delta)`` first replaces ``x`` by
+    ``x + delta`` in place (the residual sum, 32-bit arithmetic) and returns the norm of the sum."""
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How positions enter a mixer.
+
+    A rotary encoding exposes :meth:`rotary_table`: inverse frequencies ``[rotary_dim/2]``
+    (float32); the attention mixer then rotates inside its fused cache-write kernel. Any other
+    encoding returns ``None`` there and implements :meth:`apply`, which rewrites q and k
+    (``[tokens, heads, head_dim]`` views) before keys are cached.
+    """
+
+    def rotary_table(self) -> Optional[tuple[torch.Tensor, int]]:
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], positions: torch.Tensor) -> None:
+        """In-place change of q and k for the given absolute positions (default: nothing)."""
+
+
+class Mixer(Part):
+    """The part of a layer that mixes information between positions.
+
+    ``cache_spec()`` says what it keeps per request (pages of keys/values, a fixed-size state, or
+    nothing). ``forward(x, ctx, cache)`` gets the normalised rows, the step's context and the
+    :class:`dli_amd.cache.store.LayerCache` of its schedule entry (``None`` without cache), and
+    returns ``[tokens, hidden]``. With ``residual`` it returns ``residual + mixer(x)`` (it may fuse
+    the sum into its last kernel); the sum is made in 32-bit.
+    """
+
+    def cache_spec(self) -> Optional[PagedKVSpec | StateSpec]:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Position-wise part: ``forward(x, ctx, residual=None) -> [tokens, hidden]``."""
+
+    def forward(self, x: torch.Tensor, ctx: Any, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of a layer's parts: ``forward(x, ctx, cache, parts) -> x``.
+
+    ``parts`` maps the roles of the layer's :class:`LayerSpec` to built parts. The block owns the
+    residual stream's handling (where norms sit, where sums are made)."""
+
+    roles: tuple[str, ...] = ()
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, parts: Mapping[str, Part]) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Rows to logits: ``forward(x [k, hidden]) -> float32 [k, vocab]``. ``tie(table)`` gives a
+    tied head the embedding's table."""
+
+    def tie(self, table: torch.Tensor) -> None:
+        raise NotImplementedError
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError

@@ -1,0 +1,189 @@
+"""Each HIP kernel alone against a plain float64 reference, at sizes other than the engine's."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from kernel_refs import ref_paged_attention, ref_rms_norm, ref_rope
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 1.6e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dli_amd.kernels import ops as o
+
+    o.library()
+    return o
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_gather_rows(ops, dtype):
+    torch.manual_seed(0)
+    table = torch.randn(37, 50, device="cuda").to(dtype)
+    ids = torch.tensor([3, 36, 0, 3, 17], dtype=torch.int32, device="cuda")
+    out = torch.empty(5, 50, device="cuda", dtype=dtype)
+    ops.embedding(table, ids, out)
+    assert torch.equal(out.cpu(), table.cpu()[ids.cpu().long()])
+    out2 = torch.empty(5, 50, device="cuda", dtype=dtype)
+    ops.gather_rows(table, ids, out2)
+    assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width,eps", [(64, 1e-5), (192, 1e-6), (2050, 1e-5), (7, 1e-2)])
+def test_rms_norm(ops, dtype, width, eps):
+    torch.manual_seed(1)
+    x = (torch.randn(9, width, device="cuda") * 3).to(dtype)
+    x[2] = x[2] * 1e-3  # a small row: eps matters here
+    w = (1 + 0.1 * torch.randn(width, device="cuda")).float()
+    out = torch.empty_like(x)
+    ops.rms_norm(x, w, eps, out)
+    ref = ref_rms_norm(x.cpu(), w.cpu(), eps)
+    assert (out.cpu().double() - ref).abs().max() < tol(dtype) * 4
+    # fused residual: x + delta first
+    delta = torch.randn_like(x)
+    summed = torch.empty_like(x)
+    ops.rms_norm(x, w, eps, out, delta=delta, sum_out=summed)
+    s_ref = (x.float() + delta.float()).to(dtype)
+    assert torch.equal(summed, s_ref)
+    ref2 = ref_rms_norm(s_ref.cpu(), w.cpu(), eps)
+    assert (out.cpu().double() - ref2).abs().max() < tol(dtype) * 4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul_and_add(ops, dtype):
+    torch.manual_seed(2)
+    gu = (torch.randn(5, 2 * 23, device="cuda") * 4).to(dtype)
+    gu[0, 0] = 0.0
+    gu[0, 1] = 30.0
+    out = torch.empty(5, 23, device="cuda", dtype=dtype)
+    ops.silu_mul(gu, out)
+    g, u = gu.cpu().double()[:, :23], gu.cpu().double()[:, 23:]
+    ref = g * torch.sigmoid(g) * u
+    assert (out.cpu().double() - ref).abs().max() <= tol(dtype) * ref.abs().max()
+    assert out[0, 0].item() == 0.0
+    a, b = torch.randn(4, 10, device="cuda").to(dtype), torch.randn(4, 10, device="cuda").to(dtype)
+    bias = torch.randn(10, device="cuda").to(dtype)
+    o = torch.empty_like(a)
+    ops.add(a, b, o, bias=bias)
+    ref = a.cpu().double() + bias.cpu().double() + b.cpu().double()
+    assert (o.cpu().double() - ref).abs().max() < tol(dtype) * 4
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 5, 7), (3, 64, 64), (65, 130, 100), (200, 97, 258), (17, 384, 192)])
+def test_gemm_f32(ops, m, n, k):
+    torch.manual_seed(3)
+    a = torch.randn(m, k, device="cuda")
+    w = torch.randn(n, k, device="cuda")
+    bias = torch.randn(n, device="cuda")
+    res = torch.randn(m, n, device="cuda")
+    out = torch.empty(m, n, device="cuda")
+    ops.gemm_f32(a, w, out, bias=bias, residual=res)
+    ref = a.cpu().double() @ w.cpu().double().T + bias.cpu().double() + res.cpu().double()
+    assert (out.cpu().double() - ref).abs().max() < 1e-5 * math.sqrt(k) * 4
+    # a row's result does not depend on the other rows of the batch
+    out1 = torch.empty(1, n, device="cuda")
+    ops.gemm_f32(a[m - 1:m].contiguous(), w, out1, bias=bias, residual=res[m - 1:m].contiguous())
+    assert torch.equal(out1[0], out[m - 1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("qh,kvh,d,rd,bs", [(4, 4, 16, 16, 16), (6, 2, 32, 32, 8), (3, 1, 48, 32, 4), (2, 2, 80, 80, 16)])
+def test_rope_kv_write(ops, dtype, qh, kvh, d, rd, bs):
+    torch.manual_seed(4)
+    n, pages = 11, 9
+    qkv = torch.randn(n, (qh + 2 * kvh) * d, device="cuda").to(dtype)
+    orig = qkv.clone()
+    positions = torch.tensor([0, 1, 2, 3, 500, 4095, 7, 8, 9, 10, 11], dtype=torch.int32, device="cuda")
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rd, 2).float() / rd))).cuda()
+    perm = torch.randperm(pages * bs)[:n]
+    perm[5] = -1  # not cached
+    slots = perm.to(torch.int32).cuda()
+    k_pages = torch.full((pages, kvh, bs, d), 7.0, device="cuda").to(dtype)
+    v_pages = torch.full((pages, kvh, d, bs), 7.0, device="cuda").to(dtype)
+    ops.rope_kv_write(qkv, positions, inv_freq, rd, slots, k_pages, v_pages, qh, kvh, d)
+    o = orig.cpu().view(n, qh + 2 * kvh, d)
+    q_ref = ref_rope(o[:, :qh], positions.cpu(), inv_freq.cpu(), rd)
+    k_ref = ref_rope(o[:, qh:qh + kvh], positions.cpu(), inv_freq.cpu(), rd)
+    got = qkv.cpu().view(n, qh + 2 * kvh, d)
+    t = tol(dtype) * 4
+    assert (got[:, :qh].double() - q_ref).abs().max() < t
+    assert torch.equal(got[:, qh:], o[:, qh:])  # k and v columns of the input are left alone
+    kp, vp = k_pages.cpu(), v_pages.cpu()
+    written = torch.zeros(pages * bs, dtype=torch.bool)
+    for tkn in range(n):
+        s = int(perm[tkn])
+        if s < 0:
+            continue
+        written[s] = True
+        assert (kp[s // bs, :, s % bs, :].double() - k_ref[tkn]).abs().max() < t
+        assert torch.equal(vp[s // bs, :, :, s % bs], o[tkn, qh + kvh:])
+    for s in range(pages * bs):  # nothing else was touched
+        if not written[s]:
+            assert (kp[s // bs, :, s % bs, :] == 7.0).all() and (vp[s // bs, :, :, s % bs] == 7.0).all()
+    # position 0 is the identity
+    assert torch.equal(got[0, :qh], o[0, :qh])
+
+
+def _paged_case(dtype, qh, kvh, d, bs, lens, seed=0, poison=True):
+    """Random pools, scattered tables wider than needed whose spare entries name a poisoned page."""
+    g = torch.Generator().manual_seed(seed)
+    need = sum(-(-kv // bs) for _, kv in lens)
+    pages = need + 3
+    k_pages = torch.randn(pages, kvh, bs, d, generator=g)
+    v_pages = torch.randn(pages, kvh, d, bs, generator=g)
+    poison_page = pages - 1
+    if poison:
+        k_pages[poison_page] = float("nan")
+        v_pages[poison_page] = float("nan")
+    order = torch.randperm(pages - 1, generator=g).tolist()
+    width = max(-(-kv // bs) for _, kv in lens) + 2
+    tables, q_start, kv_len = [], [0], []
+    for q_len, kv in lens:
+        nb = -(-kv // bs)
+        row = [order.pop() for _ in range(nb)]
+        tables.append(row + [poison_page] * (width - nb))
+        q_start.append(q_start[-1] + q_len)
+        kv_len.append(kv)
+    q = torch.randn(q_start[-1], qh * d, generator=g)
+    return q.to(dtype), k_pages.to(dtype), v_pages.to(dtype), q_start, kv_len, tables
+
+
+def _tiles(q_start, bm):
+    te, tq = [], []
+    for e in range(len(q_start) - 1):
+        for q0 in range(0, q_start[e + 1] - q_start[e], bm):
+            te.append(e)
+            tq.append(q0)
+    return te, tq
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("qh,kvh,d,bs,window", [
+    (4, 4, 16, 16, 0), (6, 2, 32, 8, 0), (3, 3, 64, 4, 0), (8, 2, 128, 16, 0), (2, 1, 80, 16, 0),
+    (2, 2, 256, 32, 0), (5, 1, 48, 1, 0), (4, 2, 32, 8, 5), (4, 2, 64, 16, 37),
+])
+def test_attention_generic(ops, dtype, qh, kvh, d, bs, window):
+    # (query tokens now, keys after this step): decode rows, fresh prompts, portions on a prefix
+    lens = [(1, 1), (1, bs), (1, bs + 1), (1, 3 * bs - 1), (7, 7), (33, 33), (5, 40), (2, 131), (70, 70), (1, 300)]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(dtype, qh, kvh, d, bs, lens, seed=d + bs)
+    bm = ops.attention_generic_tile_rows(d)
+    te, tq = _tiles(q_start, bm)
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    out = torch.full(q.shape, 9.0, dtype=dtype, device="cuda")
+    scale = 1.0 / math.sqrt(d)
+    ops.attention_generic(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables),
+                          dev(te), dev(tq), qh, scale, window)
+    ref = ref_paged_attention(q, kp, vp, q_start, kv_len, tables, qh, scale, window)
+    err = (out.cpu().double() - ref).abs().max().item()
+    assert err < tol(dtype), err
