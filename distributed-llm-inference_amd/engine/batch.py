@@ -1,0 +1,93 @@
+"""One step's batch, as the step function gives it to the model.
+
+A step runs the next tokens of several requests at once: portions of prompts beside single decoded
+tokens, cut anywhere. :class:`StepEntry` is one request's share; :class:`StepContext` is the
+device-side description of the whole batch that every part reads. The rows of all entries are laid
+end to end: entries that bring exactly one token come first (they take the decode kernels), then the
+portions, each group in the order given.
+
+Reference: the runner's flattening of scheduled chunks (src/dli/engine/runner.py:53-183) and the
+metadata carriers of src/dli/model/kv_cache.py:94-210.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, Optional, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """``tokens`` continue request ``seq_id`` at absolute position ``start``; ``want`` lists the
+    offsets among these tokens whose logits are asked for (possibly none)."""
+
+    seq_id: Hashable
+    tokens: Sequence[int]
+    start: int
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupView:
+    """Addresses of one cache group for this step."""
+
+    slots: torch.Tensor          # int32 [tokens]: page * page_size + offset where each token's k,v go
+    block_tables: torch.Tensor   # int32 [entries, width]: pages of each request, in position order
+    table_width: int
+
+
+@dataclass
+class StepContext:
+    device: torch.device
+    page_size: int
+    num_tokens: int
+    num_entries: int
+    num_decode: int               # leading entries that bring exactly one token
+    token_ids: torch.Tensor       # int32 [tokens]
+    positions: torch.Tensor       # int32 [tokens], absolute
+    q_start: torch.Tensor         # int32 [entries + 1]: first row of each entry
+    kv_len: torch.Tensor          # int32 [entries]: keys of the request after this step
+    state_slots: torch.Tensor     # int32 [entries]
+    logit_rows: torch.Tensor      # int32 [k]: rows whose logits are wanted, in the caller's order
+    groups: list[GroupView]
+    # host copies (parts may need them to choose kernels and grids)
+    q_start_host: np.ndarray = field(default_factory=lambda: np.zeros(1, np.int32))
+    kv_len_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
+    state_slots_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
+    seq_ids: list = field(default_factory=list)
+    _tiles: dict = field(default_factory=dict)
+
+    @property
+    def max_kv_len(self) -> int:
+        return int(self.kv_len_host.max()) if self.num_entries else 0
+
+    def entry_rows(self, e: int) -> tuple[int, int]:
+        return int(self.q_start_host[e]), int(self.q_start_host[e + 1])
+
+    def is_fresh(self, e: int) -> bool:
+        """The entry starts its request at position 0 (per-request state must be reset)."""
+        q0, q1 = self.entry_rows(e)
+        return int(self.kv_len_host[e]) - (q1 - q0) == 0
+
+    def q_tiles(self, rows_per_tile: int, first_entry: int = 0,
+                last_entry: Optional[int] = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """Query tiles ``(entry, first query of the tile)`` of entries ``[first, last)``, as two
+        int32 device vectors; built once per step and tile height."""
+        last = self.num_entries if last_entry is None else last_entry
+        key = (rows_per_tile, first_entry, last)
+        hit = self._tiles.get(key)
+        if hit is None:
+            ent: list[int] = []
+            q0s: list[int] = []
+            for e in range(first_entry, last):
+                length = int(self.q_start_host[e + 1] - self.q_start_host[e])
+                for q0 in range(0, length, rows_per_tile):
+                    ent.append(e)
+                    q0s.append(q0)
+            both = torch.tensor([ent, q0s], dtype=torch.int32).to(self.device, non_blocking=False)
+            hit = (both[0].contiguous(), both[1].contiguous())
+            self._tiles[key] = hit
+        return hit

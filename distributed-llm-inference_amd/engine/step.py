@@ -1,0 +1,138 @@
+"""The step function: one batch of (request, its next tokens) in, logits at the wanted places out.
+
+It runs only the tokens it is given, as one batch, against the cache that earlier steps left:
+each entry's keys and values are written at the slots that the cache manager reserved for them,
+every row attends to its own request's pages, and afterwards the tokens are marked computed.
+The logits at a position do not depend on how the request's tokens were cut into steps, on what
+else is in the batch, or on which pages are used.
+
+Reference: ``ModelRunner.execute`` (src/dli/engine/runner.py:53-183): copy-on-write copies first,
+then the flattened batch with single-token rows before portions, one forward pass, logits in the
+caller's order, ``mark_computed`` for every chunk.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import RELEASED, CacheManager, CopyOp
+from ..cache.store import CacheStore
+from ..parts.model import Model
+from .batch import GroupView, StepContext, StepEntry
+
+
+class StepError(ValueError):
+    """A batch that the step function refuses (it would read or write outside a request's cache)."""
+
+
+class StepFunction:
+    def __init__(self, model: Model, manager: CacheManager, store: CacheStore) -> None:
+        if manager.page_size != store.page_size:
+            raise ValueError("cache manager and store disagree on the page size")
+        if manager.num_groups != max(1, len(store.groups)):
+            raise ValueError("cache manager and store disagree on the number of groups")
+        self.model, self.manager, self.store = model, manager, store
+        self.rt = model.rt
+        self.caches = model.bind_caches(store.layers)
+        self.vocab_size = model.spec.vocab_size
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ batch building
+
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Check the entries against the cache manager and lay the batch out on the device."""
+        mgr, ps = self.manager, self.manager.page_size
+        seen = set()
+        for e in entries:
+            if e.seq_id in seen:
+                raise StepError(f"request {e.seq_id!r} appears twice in one step")
+            seen.add(e.seq_id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.seq_id!r} brings no tokens")
+            if e.start != mgr.num_computed_tokens(e.seq_id):
+                raise StepError(
+                    f"request {e.seq_id!r}: portion starts at {e.start} but "
+                    f"{mgr.num_computed_tokens(e.seq_id)} tokens are computed")
+            if e.start + n > mgr.num_tokens(e.seq_id):
+                raise StepError(f"request {e.seq_id!r}: no cache slots reserved up to {e.start + n}")
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise StepError(f"request {e.seq_id!r}: token id {t} outside the vocabulary")
+            for wnt in e.want:
+                if not 0 <= int(wnt) < n:
+                    raise StepError(f"request {e.seq_id!r}: wanted place {wnt} outside its {n} tokens")
+
+        # single-token entries first, then portions; each kind in the given order
+        order = [i for i, e in enumerate(entries) if len(e.tokens) == 1] + \
+                [i for i, e in enumerate(entries) if len(e.tokens) != 1]
+        num_decode = sum(1 for e in entries if len(e.tokens) == 1)
+        q_start = np.zeros(len(entries) + 1, np.int32)
+        first_row = {}
+        for k, i in enumerate(order):
+            first_row[i] = int(q_start[k])
+            q_start[k + 1] = q_start[k] + len(entries[i].tokens)
+        total = int(q_start[-1])
+        token_ids = np.empty(total, np.int32)
+        positions = np.empty(total, np.int32)
+        kv_len = np.empty(len(entries), np.int32)
+        state_slots = np.empty(len(entries), np.int32)
+        n_groups = mgr.num_groups
+        slots = [np.empty(total, np.int32) for _ in range(n_groups)]
+        tables: list[list[tuple[int, ...]]] = [[] for _ in range(n_groups)]
+        for k, i in enumerate(order):
+            e = entries[i]
+            r0, n = int(q_start[k]), len(e.tokens)
+            token_ids[r0:r0 + n] = np.asarray(e.tokens, dtype=np.int32)
+            positions[r0:r0 + n] = np.arange(e.start, e.start + n, dtype=np.int32)
+            kv_len[k] = e.start + n
+            state_slots[k] = mgr.state_slot(e.seq_id)
+            for g in range(n_groups):
+                slots[g][r0:r0 + n] = mgr.slot_mapping(e.seq_id, e.start, e.start + n, g)
+                table = mgr.block_table(e.seq_id, g)
+                if len(table) * ps < e.start + n:
+                    raise StepError(f"request {e.seq_id!r}: block table shorter than its keys")
+                tables[g].append(table)
+        logit_rows = np.asarray(
+            [first_row[i] + int(w) for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
+
+        dev = self.rt.device
+        to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+        groups: list[GroupView] = []
+        for g in range(n_groups):
+            width = max((len(t) for t in tables[g]), default=1) or 1
+            host = np.zeros((max(len(entries), 1), width), np.int32)
+            limit = self.store.num_pages
+            for k, t in enumerate(tables[g]):
+                row = np.asarray(t, dtype=np.int64)
+                row = np.where(row == RELEASED, 0, row)  # pages that the window has passed: never read
+                if row.size and (row.min() < 0 or row.max() >= limit):
+                    raise StepError("a block table names a page outside the pool")
+                host[k, :len(t)] = row
+            if total and (slots[g].min() < 0 or slots[g].max() >= limit * ps):
+                raise StepError("a cache slot lies outside the pool")
+            groups.append(GroupView(to_dev(slots[g]), to_dev(host), width))
+        return StepContext(
+            device=dev, page_size=ps, num_tokens=total, num_entries=len(entries), num_decode=num_decode,
+            token_ids=to_dev(token_ids), positions=to_dev(positions), q_start=to_dev(q_start),
+            kv_len=to_dev(kv_len), state_slots=to_dev(state_slots), logit_rows=to_dev(logit_rows),
+            groups=groups, q_start_host=q_start, kv_len_host=kv_len, state_slots_host=state_slots,
+            seq_ids=[entries[i].seq_id for i in order])
+
+    # ------------------------------------------------------------------ the step
+
+    def run(self, entries: Sequence[StepEntry], copy_ops: Sequence[CopyOp] = ()) -> torch.Tensor:
+        """Run one step. Returns float32 logits ``[wanted places, vocab]`` on the device, in the
+        order of the entries and of each entry's ``want``."""
+        self.store.copy_pages(copy_ops)  # before any write of this step (runner.py:56)
+        if not entries:
+            return torch.empty(0, self.vocab_size, device=self.rt.device, dtype=torch.float32)
+        ctx = self.build_context(entries)
+        logits = self.model.forward(ctx, self.caches)
+        for e in entries:
+            self.manager.mark_computed(e.seq_id, e.start + len(e.tokens))
+        self.steps_run += 1
+        return logits

@@ -1,0 +1,99 @@
+"""Grouped-query self-attention over the paged cache, with position encoding and cache write.
+
+Order of work (reference: src/dli/model/llama.py:61-96,112-177): project q, k, v (one fused
+product: the three checkpoint matrices are stacked at load), rotate q and k and write rotated k and
+raw v at each token's cache slot (one kernel), attend to the request's pages (causal by absolute
+position, scale ``1/sqrt(head_dim)`` unless given, query head ``h`` reads kv head
+``h // (heads / kv_heads)``), project the result. Keys are cached after rotation: positions are
+absolute, so cached keys never change.
+
+Parameters only: the part knows its own sizes, not the model it sits in.
+``window`` > 0 restricts each query to the last ``window`` keys. ``shares_kv`` makes a mixer that
+has no k/v projections and reads the pages another schedule entry wrote.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .attention_kernels import paged_attention
+from .base import Mixer, PagedKVSpec, Part, Runtime
+from .linear import linear
+from .registry import build_part, register_part
+from .spec import PartSpec, WeightSpec
+
+
+@register_part("mixer", "gqa_attention")
+class GQAttention(Mixer):
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, num_kv_heads: int,
+                 head_dim: int, position: Optional[PartSpec] = None, qkv_bias: bool = False,
+                 o_bias: bool = False, window: int = 0, scale: Optional[float] = None,
+                 shares_kv: bool = False) -> None:
+        super().__init__(runtime)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads do not group onto {num_kv_heads} kv heads")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ops.KernelArgumentError(
+                f"attention takes head_dim in steps of 16 from 16 to 256, not {head_dim}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.window, self.shares_kv = head_dim, int(window), shares_kv
+        self.qkv_bias, self.o_bias = qkv_bias, o_bias
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.position = build_part("position", position or PartSpec("none"), runtime)
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    # -- weights
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        q, kv, h = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.hidden_size
+        names = {"q_proj": q} if self.shares_kv else {"q_proj": q, "k_proj": kv, "v_proj": kv}
+        specs = {f"{n}.weight": WeightSpec((rows, h)) for n, rows in names.items()}
+        if self.qkv_bias:
+            specs.update({f"{n}.bias": WeightSpec((rows,)) for n, rows in names.items()})
+        specs["o_proj.weight"] = WeightSpec((h, q))
+        if self.o_bias:
+            specs["o_proj.bias"] = WeightSpec((h,))
+        return specs
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        names = ["q_proj"] if self.shares_kv else ["q_proj", "k_proj", "v_proj"]
+        self.w_qkv = torch.cat([tensors[f"{n}.weight"] for n in names], dim=0).contiguous()
+        self.b_qkv = (torch.cat([tensors[f"{n}.bias"] for n in names], dim=0).contiguous()
+                      if self.qkv_bias else None)
+        self.w_o = tensors["o_proj.weight"]
+        self.b_o = tensors.get("o_proj.bias") if self.o_bias else None
+
+    def sub_parts(self) -> dict[str, Part]:
+        return {"position": self.position}
+
+    def cache_spec(self) -> Optional[PagedKVSpec]:
+        return None if self.shares_kv else PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    # -- step
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        if cache is None or cache.kind != "paged":
+            raise RuntimeError("gqa_attention needs a paged cache")
+        nh, d = self.num_heads, self.head_dim
+        nkv = 0 if self.shares_kv else self.num_kv_heads
+        if not self.shares_kv and not cache.writable:
+            raise RuntimeError("this attention writes its cache but was given a read-only one")
+        grp = ctx.groups[cache.group]
+        qkv = linear(self.rt, x, self.w_qkv, self.b_qkv)
+        table = self.position.rotary_table()
+        if table is None:
+            n = x.shape[0]
+            q_view = qkv[:, :nh * d].view(n, nh, d)
+            k_view = qkv[:, nh * d:(nh + nkv) * d].view(n, nkv, d) if nkv else None
+            self.position.apply(q_view, k_view, ctx.positions)
+            inv_freq, rotary_dim = None, 0
+        else:
+            inv_freq, rotary_dim = table
+        ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
+                          cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
+        q = qkv[:, :nh * d]
+        out = self.rt.empty(x.shape[0], nh * d)
+        paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        return linear(self.rt, out, self.w_o, self.b_o)

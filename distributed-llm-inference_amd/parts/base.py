@@ -79,6 +79,9 @@ class Part:
         """Parts owned by this one (their prefix is relative to the checkpoint root)."""
         return {}
 
+    def finalize(self) -> None:
+        """Called once after the weights are loaded: build device tables, fuse tensors."""
+
 
 class Embedding(Part):
     """Token ids to rows: ``forward(ids int32 [n]) -> [n, hidden]``."""
@@ -119,35 +122,38 @@ class Mixer(Part):
     """The part of a layer that mixes information between positions.
 
     ``cache_spec()`` says what it keeps per request (pages of keys/values, a fixed-size state, or
-    nothing). ``forward(x, ctx, cache)`` gets the normalised rows, the step's context and the
-    :class:`dli_amd.cache.store.LayerCache` of its schedule entry (``None`` without cache), and
-    returns ``[tokens, hidden]``. With ``residual`` it returns ``residual + mixer(x)`` (it may fuse
-    the sum into its last kernel); the sum is made in 32-bit.
+    nothing). ``forward(x, ctx, cache)`` gets the normalised rows, the step's context
+    (:class:`dli_amd.engine.batch.StepContext`) and the :class:`dli_amd.cache.store.LayerCache` of
+    its schedule entry (``None`` without cache), and returns ``[tokens, hidden]``. It must treat
+    each request's rows in order and must not let one request's rows influence another's.
     """
 
     def cache_spec(self) -> Optional[PagedKVSpec | StateSpec]:
         return None
 
-    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    """Position-wise part: ``forward(x, ctx, residual=None) -> [tokens, hidden]``."""
+    """Position-wise part: ``forward(x, ctx) -> [tokens, hidden]``."""
 
-    def forward(self, x: torch.Tensor, ctx: Any, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         raise NotImplementedError
 
 
 class Block(Part):
-    """Arrangement of a layer's parts: ``forward(x, ctx, cache, parts) -> x``.
+    """Arrangement of a layer's parts: where norms sit and where residual sums are made.
 
-    ``parts`` maps the roles of the layer's :class:`LayerSpec` to built parts. The block owns the
-    residual stream's handling (where norms sit, where sums are made)."""
+    ``forward(x, delta, ctx, cache, parts) -> (x, delta)``. The residual stream is ``x + delta``
+    (``delta`` may be ``None``): a block hands its last output back un-added so that the next norm
+    can make the sum and normalise in one kernel (``Norm.forward(x, delta)``). ``parts`` maps the
+    roles of the layer's :class:`LayerSpec` to built parts."""
 
     roles: tuple[str, ...] = ()
 
-    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, parts: Mapping[str, Part]) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
+                parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
         raise NotImplementedError
 
 

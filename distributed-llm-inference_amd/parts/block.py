@@ -1,0 +1,28 @@
+"""Pre-norm arrangement: ``x + mixer(norm(x))`` then ``x + feed_forward(norm(x))``
+(reference: src/dli/model/llama.py:194-213). The residual sums are made inside the norms that
+follow them (32-bit sum, rounded to the activation type, then normalised)."""
+
+from __future__ import annotations
+
+from typing import Any, Mapping, Optional
+
+import torch
+
+from .base import Block, Part, Runtime
+from .registry import register_part
+
+
+@register_part("block", "pre_norm")
+class PreNormBlock(Block):
+    roles = ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")
+
+    def __init__(self, runtime: Runtime) -> None:
+        super().__init__(runtime)
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
+                parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        h = parts["mixer_norm"].forward(x, delta)          # x <- x + delta
+        a = parts["mixer"].forward(h, ctx, cache)
+        h = parts["feed_forward_norm"].forward(x, a)       # x <- x + a
+        f = parts["feed_forward"].forward(h, ctx)
+        return x, f

@@ -1,0 +1,48 @@
+"""Gated feed-forward: ``down(act(gate(x)) * up(x))`` with ``act = silu`` (SwiGLU; reference:
+src/dli/model/llama.py:180-191). Gate and up matrices are stacked at load, so one product gives
+both halves; the activation kernel reads them side by side."""
+
+from __future__ import annotations
+
+from typing import Any, Mapping
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, Runtime
+from .linear import linear
+from .registry import register_part
+from .spec import WeightSpec
+
+
+@register_part("feed_forward", "gated_mlp")
+class GatedMLP(FeedForward):
+    def __init__(self, runtime: Runtime, *, hidden_size: int, intermediate_size: int,
+                 activation: str = "silu", bias: bool = False) -> None:
+        super().__init__(runtime)
+        if activation != "silu":
+            raise ValueError(f"gated_mlp has no kernel for activation {activation!r} (only 'silu')")
+        self.hidden_size, self.intermediate_size, self.bias = hidden_size, intermediate_size, bias
+        self.w_gate_up = self.b_gate_up = self.w_down = self.b_down = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        specs = {"gate_proj.weight": WeightSpec((i, h)), "up_proj.weight": WeightSpec((i, h)),
+                 "down_proj.weight": WeightSpec((h, i))}
+        if self.bias:
+            specs.update({"gate_proj.bias": WeightSpec((i,)), "up_proj.bias": WeightSpec((i,)),
+                          "down_proj.bias": WeightSpec((h,))})
+        return specs
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], 0).contiguous()
+        self.w_down = tensors["down_proj.weight"]
+        if self.bias:
+            self.b_gate_up = torch.cat([tensors["gate_proj.bias"], tensors["up_proj.bias"]], 0).contiguous()
+            self.b_down = tensors["down_proj.bias"]
+
+    def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
+        gate_up = linear(self.rt, x, self.w_gate_up, self.b_gate_up)
+        act = self.rt.empty(x.shape[0], self.intermediate_size)
+        ops.silu_mul(gate_up, act)
+        return linear(self.rt, act, self.w_down, self.b_down)

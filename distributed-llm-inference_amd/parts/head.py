@@ -1,0 +1,41 @@
+"""Output head: ``logits = x W^T`` with ``W`` the embedding table when tied, else its own matrix;
+no bias, no scaling (reference: src/dli/model/llama.py:237-240,304-305). Logits leave in float32."""
+
+from __future__ import annotations
+
+from typing import Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Head, Runtime
+from .linear import linear
+from .registry import register_part
+from .spec import WeightSpec
+
+
+@register_part("head", "linear_head")
+class LinearHead(Head):
+    def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, tied: bool) -> None:
+        super().__init__(runtime)
+        self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
+        self.weight: Optional[torch.Tensor] = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {} if self.tied else {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        if not self.tied:
+            self.weight = tensors["weight"]
+
+    def tie(self, table: torch.Tensor) -> None:
+        if self.tied:
+            self.weight = table
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        logits = linear(self.rt, x, self.weight)
+        if logits.dtype == torch.float32:
+            return logits
+        out = torch.empty(logits.shape, device=logits.device, dtype=torch.float32)
+        ops.to_float(logits, out)
+        return out

@@ -1,0 +1,35 @@
+"""``y = x W^T + b`` for both paths.
+
+On the 32-bit path the product is the engine's own IEEE single-precision kernel. On the bfloat16
+path it is the vendor library's matrix product through ``torch.mm`` (the reference's engine uses a
+library product there as well: ``F.linear``, src/dli/model/llama.py:72-74,95,190,305), bfloat16
+operands with 32-bit accumulation; the bias is added by the engine's own kernel.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Runtime
+
+
+def linear(rt: Runtime, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x [n, k] @ weight[m, k].T (+ bias [m]) -> [n, m]`` in the runtime's activation type."""
+    n, m = x.shape[0], weight.shape[0]
+    if out is None:
+        out = rt.empty(n, m)
+    if n == 0:
+        return out
+    if rt.dtype == torch.float32:
+        ops.gemm_f32(x, weight, out, bias=bias)
+        return out
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.shape[1] != weight.shape[1]:
+        raise ops.KernelArgumentError("linear: operands must be bfloat16 [n, k] and [m, k]")
+    torch.mm(x, weight.t(), out=out)
+    if bias is not None:
+        ops.add(out, None, out, bias=bias)
+    return out

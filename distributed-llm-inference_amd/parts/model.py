@@ -1,0 +1,131 @@
+"""A model put together from a :class:`ModelSpec`: embedding, scheduled layers, final norm, head.
+
+The model knows nothing of requests or pages: :meth:`Model.forward` takes a
+:class:`dli_amd.engine.batch.StepContext` and one :class:`dli_amd.cache.store.LayerCache` per
+schedule entry, runs the tokens of the step once through the schedule, and returns float32 logits
+of the wanted rows only (rows are selected before the final norm and the head, which are row-wise;
+reference: src/dli/model/llama.py:299-305).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Mapping, Optional, Sequence
+
+import torch
+
+from ..kernels import ops
+from .base import Part, Runtime
+from .registry import build_part
+from .spec import ModelSpec, WeightSpec
+
+# importing the modules registers the built-in parts
+from . import attention, block, embedding, feed_forward, head, norm, position  # noqa: F401,E402
+
+
+@dataclass
+class BuiltLayer:
+    block: Part
+    parts: dict[str, Part]
+
+
+def _walk(part: Part):
+    yield part
+    for sub in part.sub_parts().values():
+        yield from _walk(sub)
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, runtime: Runtime) -> None:
+        self.spec, self.rt = spec, runtime
+        self.embedding = build_part("embedding", spec.embedding, runtime)
+        self.layers: list[BuiltLayer] = []
+        for ls in spec.layers:
+            blk = build_part("block", ls.block, runtime)
+            missing = [r for r in blk.roles if r not in ls.parts]
+            if missing:
+                raise ValueError(f"block {ls.block.kind!r} needs the roles {missing}")
+            parts = {role: build_part(family, ps, runtime) for role, (family, ps) in ls.parts.items()}
+            self.layers.append(BuiltLayer(blk, parts))
+        self.final_norm = build_part("norm", spec.final_norm, runtime)
+        self.head = build_part("head", spec.head, runtime)
+
+    # ------------------------------------------------------------------ weights
+
+    def _all_parts(self) -> list[Part]:
+        tops: list[Part] = [self.embedding]
+        for layer in self.layers:
+            tops.append(layer.block)
+            tops.extend(layer.parts.values())
+        tops += [self.final_norm, self.head]
+        out: list[Part] = []
+        for t in tops:
+            out.extend(_walk(t))
+        return out
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        """Every tensor the model binds, by checkpoint name."""
+        out: dict[str, WeightSpec] = {}
+        for part in self._all_parts():
+            for local, ws in part.weight_specs().items():
+                name = part.prefix + local
+                if name in out and out[name] != ws:
+                    raise ValueError(f"two parts bind {name!r} with different specs")
+                out[name] = ws
+        return out
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Hand every part its tensors (by checkpoint name), tie the head, finalize."""
+        for part in self._all_parts():
+            local = {}
+            for name in part.weight_specs():
+                full = part.prefix + name
+                if full in tensors:
+                    local[name] = tensors[full]
+            part.load_weights(local)
+        self.head.tie(self.embedding.table())
+        for part in self._all_parts():
+            part.finalize()
+
+    # ------------------------------------------------------------------ cache needs
+
+    def cache_specs(self) -> list[Optional[Any]]:
+        """What each schedule entry keeps per request (``None``: nothing of its own)."""
+        out = []
+        for entry in self.spec.schedule:
+            mixer = self.layers[entry.layer].parts.get("mixer")
+            own = entry.cache_of is None and mixer is not None
+            out.append(mixer.cache_spec() if own else None)
+        return out
+
+    def bind_caches(self, layer_caches: Sequence[Any]) -> list[Any]:
+        """Per schedule entry, the cache it uses: its own, or a read-only view of another's."""
+        out = []
+        for i, entry in enumerate(self.spec.schedule):
+            if entry.cache_of is not None:
+                src = layer_caches[entry.cache_of]
+                out.append(src.reader() if src is not None else None)
+            else:
+                out.append(layer_caches[i])
+        return out
+
+    # ------------------------------------------------------------------ step
+
+    def forward(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
+        """Run the step's tokens through the schedule; float32 logits ``[wanted rows, vocab]``."""
+        x = self.embedding.forward(ctx.token_ids)
+        delta: Optional[torch.Tensor] = None
+        for entry, cache in zip(self.spec.schedule, caches):
+            layer = self.layers[entry.layer]
+            x, delta = layer.block.forward(x, delta, ctx, cache, layer.parts)
+        k = ctx.logit_rows.shape[0]
+        if k == 0:
+            return torch.empty(0, self.spec.vocab_size, device=self.rt.device, dtype=torch.float32)
+        xs = torch.empty(k, x.shape[1], device=x.device, dtype=x.dtype)
+        ops.gather_rows(x, ctx.logit_rows, xs)
+        ds = None
+        if delta is not None:
+            ds = torch.empty_like(xs)
+            ops.gather_rows(delta, ctx.logit_rows, ds)
+        h = self.final_norm.forward(xs, ds)
+        return self.head.forward(h)

@@ -26,3 +26,12 @@ def pytest_collection_modifyitems(config: pytest.Config, items: list[pytest.Item
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter, exitstatus, config) -> None:
+    mod = sys.modules.get("test_model_gpu")
+    worst = getattr(mod, "WORST", None)
+    if worst:
+        terminalreporter.write_line(
+            "largest logit error as a fraction of its bound: "
+            + ", ".join(f"{k} {v:.3f}" for k, v in sorted(worst.items())))

@@ -1,0 +1,59 @@
+"""Two tiny Llama configurations that differ in every size and option, and model folders for them."""
+
+from __future__ import annotations
+
+import tempfile
+from pathlib import Path
+
+# 2 layers, MHA, head_dim 16, default rope, tied head, eps 1e-5
+TINY_A = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 256, "hidden_size": 64,
+    "intermediate_size": 160, "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 4,
+    "head_dim": 16, "rms_norm_eps": 1e-5, "max_position_embeddings": 256, "rope_theta": 10000.0,
+    "tie_word_embeddings": True, "hidden_act": "silu",
+}
+# 3 layers, GQA 3:1, head_dim 32, llama3 rope, untied head, eps 1e-6, widths no power of two
+TINY_B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 384, "hidden_size": 192,
+    "intermediate_size": 512, "num_hidden_layers": 3, "num_attention_heads": 6, "num_key_value_heads": 2,
+    "head_dim": 32, "rms_norm_eps": 1e-6, "max_position_embeddings": 512, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64},
+    "tie_word_embeddings": False, "hidden_act": "silu",
+}
+# odd sizes everywhere: 5 heads of 48 on a width of 200 (head_dim given, not hidden/heads),
+# biases, linear rope, vocabulary 301
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 301, "hidden_size": 200,
+    "intermediate_size": 136, "num_hidden_layers": 2, "num_attention_heads": 5, "num_key_value_heads": 1,
+    "head_dim": 48, "rms_norm_eps": 1e-5, "max_position_embeddings": 1024, "rope_theta": 10000.0,
+    "rope_scaling": {"type": "linear", "factor": 2.0}, "attention_bias": True, "mlp_bias": True,
+    "tie_word_embeddings": False, "hidden_act": "silu",
+}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+_made: dict = {}
+_tmp = None
+
+
+# Weights are drawn with std = 1.2 / sqrt(hidden) instead of the usual 0.02: attention scores then
+# have a spread of about one, so attention is far from uniform (a key in the wrong place, a wrong
+# rotation or a wrong mask changes the logits) without being so sharp that bfloat16's rounding of a
+# score is blown up into a different distribution.
+STD = {"A": 0.15, "B": 0.085, "C": 0.085}
+
+
+def model_folder(name: str, seed: int = 11, std: float | None = None, norm_jitter: float = 0.1) -> Path:
+    """A temporary folder with config.json and model.safetensors of configuration ``name``."""
+    from dli_amd.weights import write_random_model
+
+    global _tmp
+    std = STD[name] if std is None else std
+    key = (name, seed, std, norm_jitter)
+    if key not in _made:
+        if _tmp is None:
+            _tmp = tempfile.TemporaryDirectory(prefix="dli_amd_tiny_")
+        out = Path(_tmp.name) / f"{name}_{seed}_{std}_{norm_jitter}"
+        write_random_model(out, CONFIGS[name], seed=seed, std=std, norm_jitter=norm_jitter)
+        _made[key] = out
+    return _made[key]
