@@ -1,0 +1,180 @@
+"""Measures decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+The default run is the Llama-3.2-1B shape with random weights in bfloat16: 8 requests decode
+greedily at a context of about 4096 tokens through the engine's own step loop (schedule, one
+batched step, sampling), W untimed steps and then exactly K timed ones between device
+synchronisations. One JSON line reports decoded tokens a second, the time of a 2,048-token prefill
+step, the decode step's memory roofline, and decode throughput at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+# MI355X published peaks
+HBM_GBPS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LLAMA_3_2_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 128256, "hidden_size": 2048,
+    "intermediate_size": 8192, "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 64, "rms_norm_eps": 1e-5, "max_position_embeddings": 131072, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": True, "hidden_act": "silu",
+}
+
+
+def make_engine(raw, dtype, batch, context, block_size, budget):
+    import torch
+
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.parts.base import Runtime
+    from dli_amd.weights.loader import build_model, parse_dtype
+    from dli_amd.weights.random_init import fill_random_on_device
+
+    rt = Runtime(torch.device("cuda:0"), parse_dtype(dtype))
+    model, cfg = build_model(raw, rt)
+    model.config = cfg
+    fill_random_on_device(model, seed=0, std=0.02)
+    pages = batch * (-(-context // block_size) + 1) + 8
+    engine = LLMEngine.for_model(
+        model, num_blocks=pages, block_size=block_size, enable_prefix_caching=False,
+        config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget))
+    return engine, cfg
+
+
+def decode_run(engine, cfg, batch, context, steps, warmup):
+    """Tokens a second and milliseconds a step of ``steps`` decode steps at about ``context``."""
+    import torch
+
+    from dli_amd.sampling import SamplingParams
+
+    gen = torch.Generator().manual_seed(batch)
+    prompt_len = context - steps - warmup - 1
+    total = steps + warmup + 1
+    for i in range(batch):
+        prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).tolist()
+        engine.add_request(f"b{batch}-{i}", prompt, SamplingParams(max_tokens=total, ignore_eos=True))
+    while any(r.num_computed_tokens < prompt_len for r in engine.scheduler.running) or engine.scheduler.waiting:
+        engine.step()  # prefill, in portions under the token budget
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = engine.step()
+        assert len(out) == batch
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    while engine.has_unfinished():
+        engine.step()
+    return batch * steps / dt, dt / steps * 1e3
+
+
+def prefill_run(engine, cfg, tokens, repeats=3):
+    import torch
+
+    from dli_amd.sampling import SamplingParams
+
+    gen = torch.Generator().manual_seed(99)
+    best = float("inf")
+    for r in range(repeats + 1):
+        prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
+        engine.add_request(f"p{r}", prompt, SamplingParams(max_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()  # the whole prompt is one portion: budget >= tokens
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert not engine.has_unfinished()
+        if r > 0:
+            best = min(best, dt)
+    return best
+
+
+def prefill_flops(cfg, tokens):
+    h, d = cfg.hidden_size, cfg.head_dim
+    q, kv = cfg.num_heads * d, cfg.num_kv_heads * d
+    linear = cfg.num_layers * (h * (q + 2 * kv) + q * h + 3 * h * cfg.intermediate_size)
+    attention = cfg.num_layers * 2 * cfg.num_heads * d * tokens * (tokens + 1)  # QK^T and PV, causal
+    return 2.0 * linear * tokens + attention + 2.0 * cfg.vocab_size * h  # + the head for one row
+
+
+def decode_bytes(cfg, batch, context, itemsize):
+    weights = (cfg.num_parameters()) * itemsize
+    kv_per_token = 2 * cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * itemsize
+    return weights + batch * context * kv_per_token
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
+        return 2
+
+    import torch
+
+    raw = dict(LLAMA_3_2_1B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    itemsize = 2 if short == "bf16" else 4
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=2048)
+
+    tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup)
+    achieved = decode_bytes(cfg, args.batch, args.context, itemsize) / (ms * 1e-3) / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8, Llama-3.2-1B shape",
+        "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
+        "config": {
+            "model": "Llama-3.2-1B shape", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single GPU", "layers": cfg.num_layers, "layers_of_config": full_layers,
+            "hidden": cfg.hidden_size, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
+            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+            "rms_norm_eps": cfg.rms_norm_eps, "rope": f"{cfg.rope.rope_type} theta {cfg.rope.theta:g} factor {cfg.rope.factor:g}",
+            "tied_head": cfg.tie_word_embeddings, "kv_block_size": args.block_size, "prefill_tokens": 2048,
+            "sampling": "greedy",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+    }
+    if not args.no_points:
+        t = prefill_run(engine, cfg, 2048)
+        line["prefill"] = {"value": round(2048 / t, 1), "tokens": 2048, "ms": round(t * 1e3, 3),
+                           "frac": round(prefill_flops(cfg, 2048) / t / PEAK_FLOPS[short], 4)}
+        points = {}
+        for b in (1, 64):
+            steps = min(args.steps, 32)
+            points[f"decode_b{b}"] = round(decode_run(engine, cfg, b, args.context, steps, min(args.warmup, 4))[0], 1)
+        line["points"] = points
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,216 @@
+"""The engine's step loop and Python entry point.
+
+One ``step()``: schedule, run the scheduled tokens as one batch through the step function, sample
+a token for every request whose chunk reached its last known token, append it, finish what is done
+(reference: src/dli/engine/engine.py:183-246). Each phase is timed (``StepStats``).
+"""
+
+from __future__ import annotations
+
+import itertools
+import random
+import time
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Any, Callable, Collection, Iterable, Optional, Protocol, Sequence
+
+from ..cache.manager import CacheManager
+from ..sampling.params import SamplingParams
+from .request import FinishReason, Priority, Request
+from .scheduler import Scheduler, SchedulerConfig, SchedulerOutput
+
+
+class Runner(Protocol):
+    """Runs a scheduler decision. Afterwards every scheduled chunk's keys are written and marked
+    computed in the cache manager. Returns logits, one row per chunk with ``needs_logits``, in
+    schedule order (reference: src/dli/engine/runner.py:18-25)."""
+
+    def execute(self, sched: SchedulerOutput) -> Any: ...
+
+
+TokenSampler = Callable[[Any, Sequence[SamplingParams], Sequence[Optional[int]], Sequence[int]], list[int]]
+
+
+class ModelRunner:
+    """The runner for a real model: turns chunks into step entries for the step function."""
+
+    def __init__(self, core: Any) -> None:
+        self.core = core
+
+    def execute(self, sched: SchedulerOutput) -> Any:
+        from .batch import StepEntry
+
+        entries = []
+        for ch in sched.chunks:
+            req = ch.request
+            n_prompt = len(req.prompt_ids)
+            lo, hi = ch.start, ch.start + ch.num_tokens
+            if hi <= n_prompt:
+                tokens = req.prompt_ids[lo:hi]
+            else:
+                tokens = (req.prompt_ids[lo:] if lo < n_prompt else []) + req.output_ids[max(0, lo - n_prompt):hi - n_prompt]
+            entries.append(StepEntry(req.request_id, tokens, ch.start,
+                                     (ch.num_tokens - 1,) if ch.needs_logits else ()))
+        return self.core.step.run(entries, sched.copy_ops)
+
+
+@dataclass(frozen=True)
+class RequestOutput:
+    request_id: str
+    new_token_ids: list[int]
+    finished: bool
+    finish_reason: Optional[FinishReason]
+
+
+@dataclass(frozen=True)
+class StepStats:
+    """Shape and timing (seconds) of one step (reference: src/dli/engine/engine.py:39-54)."""
+
+    num_seqs: int
+    num_batched_tokens: int
+    num_prefill_tokens: int
+    num_decode_tokens: int
+    num_preempted: int
+    schedule_s: float
+    forward_s: float
+    postprocess_s: float
+
+    @property
+    def total_s(self) -> float:
+        return self.schedule_s + self.forward_s + self.postprocess_s
+
+
+@dataclass
+class EngineStats:
+    steps: list[StepStats] = field(default_factory=list)
+
+
+class LLMEngine:
+    """Continuous-batching engine over the paged cache; single-threaded.
+
+    Build with :meth:`for_model`. Tests may inject any :class:`Runner` and token sampler together
+    with the cache manager they work on.
+    """
+
+    def __init__(self, runner: Runner, manager: CacheManager, config: Optional[SchedulerConfig] = None, *,
+                 eos_token_ids: Collection[int] = (), seed: int = 0,
+                 sampler: Optional[TokenSampler] = None) -> None:
+        self.runner = runner
+        self.manager = manager
+        self.scheduler = Scheduler(config or SchedulerConfig(), manager)
+        self.eos = frozenset(eos_token_ids)
+        self._rng = random.Random(seed)
+        self._arrivals = itertools.count()
+        self._step_no = 0
+        if sampler is None:
+            from ..sampling.sampler import sample as sampler  # the GPU sampler
+        self._sample = sampler
+        self.stats = EngineStats()
+
+    @classmethod
+    def for_model(cls, model: Any, *, num_blocks: Optional[int] = None, kv_cache_gb: Optional[float] = None,
+                  block_size: int = 16, config: Optional[SchedulerConfig] = None,
+                  eviction_policy: str = "lru", enable_prefix_caching: bool = True,
+                  eos_token_ids: Collection[int] = (), seed: int = 0, dtype: str = "bfloat16",
+                  device: str = "cuda") -> "LLMEngine":
+        """Engine for a loaded model or a model folder.
+
+        ``num_blocks`` pages of ``block_size`` tokens, or as many as ``kv_cache_gb`` GiB hold
+        (default 1 GiB), as the reference's server takes them (src/dli/server/__main__.py:150-156).
+        """
+        from ..weights.loader import load_model
+        from .core import build_core, pages_for_budget
+
+        if num_blocks is not None and kv_cache_gb is not None:
+            raise ValueError("give num_blocks or kv_cache_gb, not both")
+        if isinstance(model, (str, Path)):
+            model = load_model(model, dtype=dtype, device=device)
+        if num_blocks is None:
+            gib = 1.0 if kv_cache_gb is None else kv_cache_gb
+            num_blocks = pages_for_budget(model, block_size, int(gib * 2 ** 30))
+        config = config or SchedulerConfig()
+        core = build_core(model, num_pages=num_blocks, page_size=block_size, max_seqs=config.max_num_seqs,
+                          enable_prefix_caching=enable_prefix_caching, eviction_policy=eviction_policy)
+        engine = cls(ModelRunner(core), core.manager, config, eos_token_ids=eos_token_ids, seed=seed)
+        engine.core = core
+        return engine
+
+    # ------------------------------------------------------------------ API
+
+    def add_request(self, request_id: str, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None, *,
+                    priority: Priority = Priority.INTERACTIVE, tenant: str = "default") -> Request:
+        """Queue a request. One that can never fit finishes at once with CAPACITY."""
+        if not prompt_ids:
+            raise ValueError("prompt must be non-empty")
+        params = params or SamplingParams()
+        seed = params.seed if params.seed is not None else self._rng.getrandbits(63)
+        req = Request(request_id=request_id, prompt_ids=[int(t) for t in prompt_ids], params=params,
+                      arrival_seq=next(self._arrivals), priority=priority, tenant=tenant,
+                      seed=None if params.greedy else seed, arrival_step=self._step_no)
+        self.scheduler.add(req)
+        return req
+
+    def abort(self, request_id: str) -> bool:
+        return self.scheduler.abort(request_id) is not None
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_unfinished
+
+    def step(self) -> list[RequestOutput]:
+        t0 = time.perf_counter()
+        sched = self.scheduler.schedule()
+        t1 = time.perf_counter()
+        outputs: list[RequestOutput] = []
+        if sched.chunks:
+            logits = self.runner.execute(sched)
+            t2 = time.perf_counter()
+            sampling = [c for c in sched.chunks if c.needs_logits]
+            for ch in sched.chunks:
+                ch.request.num_computed_tokens += ch.num_tokens
+            tokens = self._sample(
+                logits, [c.request.params for c in sampling], [c.request.seed for c in sampling],
+                [len(c.request.output_ids) for c in sampling])
+            if len(tokens) != len(sampling):
+                raise RuntimeError("the sampler returned a wrong number of tokens")
+            for ch, tok in zip(sampling, tokens):
+                outputs.append(self._append_token(ch.request, int(tok)))
+        else:
+            t2 = t1
+        t3 = time.perf_counter()
+        prefill = sum(c.num_tokens for c in sched.chunks if c.num_tokens > 1 or not c.needs_logits)
+        total = sched.num_batched_tokens
+        self.stats.steps.append(StepStats(
+            num_seqs=len(sched.chunks), num_batched_tokens=total, num_prefill_tokens=prefill,
+            num_decode_tokens=total - prefill, num_preempted=len(sched.preempted),
+            schedule_s=t1 - t0, forward_s=t2 - t1, postprocess_s=t3 - t2))
+        self._step_no += 1
+        return outputs
+
+    def generate(self, prompts: Iterable[Sequence[int]],
+                 params: SamplingParams | Sequence[SamplingParams] | None = None) -> list[list[int]]:
+        """Run prompts (token ids) to completion; generated ids in input order."""
+        prompts = list(prompts)
+        if params is None or isinstance(params, SamplingParams):
+            per = [params or SamplingParams()] * len(prompts)
+        else:
+            per = list(params)
+            if len(per) != len(prompts):
+                raise ValueError("one SamplingParams per prompt, or one for all")
+        tag = next(self._arrivals)
+        reqs = [self.add_request(f"gen-{tag}-{i}", p, per[i]) for i, p in enumerate(prompts)]
+        while self.has_unfinished():
+            self.step()
+        return [r.output_ids for r in reqs]
+
+    # ------------------------------------------------------------------ internals
+
+    def _append_token(self, req: Request, tok: int) -> RequestOutput:
+        req.output_ids.append(tok)
+        reason: Optional[FinishReason] = None
+        if tok in req.params.stop_token_ids or (not req.params.ignore_eos and tok in self.eos):
+            reason = FinishReason.STOP
+        elif len(req.output_ids) >= req.params.max_tokens:
+            reason = FinishReason.LENGTH
+        if reason is not None:
+            self.scheduler.finish(req, reason)
+        return RequestOutput(req.request_id, [tok], reason is not None, reason)

@@ -39,6 +39,7 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_f32_nt": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int,
                         _c_int, _c_int, _c_ptr],
+    "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
@@ -307,3 +308,27 @@ def attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
         _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0),
         tile_entry.shape[0], q_heads, kv_heads, head_dim, page_size, float(scale), int(window),
         _is_bf16(dtype), _stream()), "attention_generic")
+
+
+# ----------------------------------------------------------------------------- sampling
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           seeds: torch.Tensor, counters: torch.Tensor, out: torch.Tensor) -> None:
+    """One token per row of float32 ``logits [rows, vocab]``.
+
+    Rows with ``temperature == 0`` or ``top_k == 1`` take the argmax (lowest id on ties); the others
+    apply temperature, top-k (``<= 0``: off), top-p and draw with Philox(seed, counter).
+    """
+    _rows(logits, "logits", torch.float32)
+    rows, vocab = logits.shape
+    _dense(temperature, "temperature", torch.float32, 1)
+    _dense(top_k, "top_k", torch.int32, 1)
+    _dense(top_p, "top_p", torch.float32, 1)
+    _dense(seeds, "seeds", torch.int64, 1)
+    _dense(counters, "counters", torch.int64, 1)
+    _dense(out, "out", torch.int32, 1)
+    for name, t in (("temperature", temperature), ("top_k", top_k), ("top_p", top_p), ("seeds", seeds),
+                    ("counters", counters), ("out", out)):
+        _require(t.shape[0] == rows, f"{name} must have one value per row")
+    _check(library().dli_sample(_ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k),
+                                _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(out), _stream()), "sample")

@@ -1,0 +1,369 @@
+"""The cache manager without a model: no page or slot lost, held twice or freed twice.
+
+Vectors from the reference's tests/unit/kv/test_block_manager.py (page size 4, 16 pages,
+watermark 0) and tests/unit/kv/test_hashing_and_policies.py.
+"""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+
+from dli_amd.cache import (
+    RELEASED, CacheManager, CopyOp, CostAwarePolicy, GroupSpec, LRUPolicy, NoFreePagesError, NoFreeSlotError,
+    ROOT_PARENT, SequenceError, StateSlots, chain_hashes, page_hash,
+)
+
+
+def mk(num_pages=16, page_size=4, **kw):
+    kw.setdefault("watermark", 0.0)
+    return CacheManager(num_pages=num_pages, page_size=page_size, **kw)
+
+
+# ------------------------------------------------------------------ allocation and addressing
+
+def test_prompt_takes_ceil_pages_and_slots_follow_the_table():
+    m = mk()
+    a = m.allocate("a", list(range(9)))
+    assert len(a.block_table) == 3 and m.num_available_pages == 13 and a.num_cached_tokens == 0
+    t = a.block_table
+    assert m.slot_mapping("a", 2, 8) == [t[0] * 4 + 2, t[0] * 4 + 3, t[1] * 4, t[1] * 4 + 1, t[1] * 4 + 2, t[1] * 4 + 3]
+    with pytest.raises(ValueError):
+        m.slot_mapping("a", 0, 10)
+    m.check_invariants()
+
+
+def test_appends_take_a_page_at_boundaries_only():
+    m = mk()
+    m.allocate("a", [1, 2, 3])
+    assert len(m.block_table("a")) == 1
+    m.append_slots("a", [4])
+    assert len(m.block_table("a")) == 1
+    m.append_slots("a", [5])
+    assert len(m.block_table("a")) == 2
+    m.append_slots("a", [6, 7, 8, 9])
+    assert len(m.block_table("a")) == 3 and m.num_tokens("a") == 9
+    m.check_invariants()
+
+
+def test_errors_leave_the_state_unchanged():
+    m = mk(num_pages=4)
+    m.allocate("a", list(range(10)))
+    with pytest.raises(NoFreePagesError):
+        m.allocate("b", list(range(8)))
+    with pytest.raises(SequenceError):
+        m.allocate("a", [1])
+    with pytest.raises(ValueError):
+        m.allocate("c", [])
+    m.append_slots("a", [0, 0])  # fills page 3
+    m.append_slots("a", [0, 0, 0, 0])  # takes the last page
+    with pytest.raises(NoFreePagesError):
+        m.append_slots("a", [0])
+    assert m.num_tokens("a") == 16 and not m.has_sequence("b")
+    with pytest.raises(SequenceError):
+        m.free("zzz")
+    m.free("a")
+    with pytest.raises(SequenceError):
+        m.free("a")  # freed twice
+    m.check_invariants()
+    assert m.stats().free_pages == 4
+
+
+def test_watermark_holds_pages_back_at_admission_only():
+    m = CacheManager(num_pages=10, page_size=4, watermark=0.2)
+    assert not m.can_allocate(list(range(36)))  # 9 pages would leave 1 < 2
+    assert m.can_allocate(list(range(32)))
+    m.allocate("a", list(range(32)))
+    m.append_slots("a", list(range(8)))  # appends may use the reserve
+    assert m.num_available_pages == 0
+    m.check_invariants()
+
+
+# ------------------------------------------------------------------ content reuse
+
+def test_pages_are_reusable_only_after_they_are_computed():
+    m = mk()
+    p = list(range(10))
+    m.allocate("a", p)
+    assert m.allocate("b", p).num_cached_tokens == 0  # allocated, not computed: no hit
+    m.mark_computed("a", 10)
+    assert m.allocate("c", p).num_cached_tokens == 8
+    m.check_invariants()
+
+
+def test_last_token_page_is_never_served_from_the_index():
+    m = mk()
+    p = list(range(8))  # exactly two pages
+    m.allocate("a", p)
+    m.mark_computed("a", 8)
+    assert m.allocate("b", p).num_cached_tokens == 4
+    q = p[:5] + [99] + p[6:] + [1, 2]
+    assert m.allocate("c", q).num_cached_tokens == 4  # differs inside page 2
+    m.check_invariants()
+
+
+def test_namespaces_do_not_share():
+    m = mk()
+    p = list(range(9))
+    m.allocate("a", p, namespace=b"x")
+    m.mark_computed("a", 9)
+    assert m.allocate("b", p, namespace=b"y").num_cached_tokens == 0
+    assert m.allocate("c", p, namespace=b"x").num_cached_tokens == 8
+
+
+def test_decoded_tokens_complete_pages_that_become_reusable():
+    m = mk()
+    m.allocate("a", [1, 2, 3])
+    m.mark_computed("a", 3)
+    for t in range(4, 10):
+        m.append_slots("a", [t])
+        m.mark_computed("a", m.num_tokens("a"))
+    assert m.allocate("b", list(range(1, 10)) + [0]).num_cached_tokens == 8
+    m.check_invariants()
+
+
+def test_duplicate_prompts_admitted_together_keep_private_pages():
+    m = mk()
+    p = list(range(9))
+    m.allocate("a", p)
+    m.allocate("b", p)
+    m.mark_computed("a", 9)
+    m.mark_computed("b", 9)
+    assert m.stats().duplicate_registrations == 2
+    m.free("a")
+    m.free("b")
+    m.check_invariants()
+    assert m.num_available_pages == 16
+
+
+def test_leaves_are_reclaimed_first_and_revived_pages_are_safe():
+    m = mk(num_pages=4)
+    p = list(range(13))  # 4 pages, 3 of them full
+    m.allocate("a", p)
+    m.mark_computed("a", 13)
+    m.free("a")
+    assert m.stats().cached_idle_pages == 3 and m.stats().free_pages == 1
+    m.allocate("b", [50, 51, 52, 53, 54])  # 2 pages: the free one and the deepest cached leaf
+    assert m.stats().evictions == 1
+    m.free("b")
+    assert m.allocate("c", p[:9]).num_cached_tokens == 8  # the two-page prefix survived
+    m.check_invariants()
+    with pytest.raises(NoFreePagesError):  # the revived pages cannot be reclaimed for someone else
+        m.allocate("d", [7] * 9)
+    m.free("c")
+    m.reset_prefix_cache()
+    m.check_invariants()
+    assert m.stats().free_pages == 4
+
+
+def test_fork_shares_pages_and_copies_on_write():
+    m = mk()
+    m.allocate("a", list(range(6)))
+    m.mark_computed("a", 6)
+    m.fork("a", "b")
+    shared = m.block_table("a")[-1]
+    ops = m.append_slots("b", [7])
+    assert ops == [CopyOp(src=shared, dst=m.block_table("b")[-1], group=0)]
+    assert m.block_table("a")[-1] == shared and m.block_table("b")[0] == m.block_table("a")[0]
+    assert m.append_slots("a", [8]) == []  # a is the only holder now
+    assert m.stats().cow_copies == 1
+    m.check_invariants()
+    m2 = mk()
+    m2.allocate("a", list(range(8)))
+    m2.fork("a", "b")
+    assert m2.append_slots("b", [1]) == []  # fork at a page boundary: nothing to copy
+    m2.check_invariants()
+
+
+def test_without_content_reuse_nothing_is_kept():
+    m = mk(enable_prefix_caching=False)
+    p = list(range(9))
+    m.allocate("a", p)
+    m.mark_computed("a", 9)
+    m.free("a")
+    assert m.stats().cached_idle_pages == 0 and m.allocate("b", p).num_cached_tokens == 0
+
+
+# ------------------------------------------------------------------ identities and policies
+
+def test_page_identities():
+    a, b = chain_hashes(b"m", [1, 2, 3, 4, 5, 6], 3), chain_hashes(b"m", [9, 9, 9, 4, 5, 6], 3)
+    assert len(a) == len(b) == 2 and a[1] != b[1]
+    assert len(chain_hashes(b"m", list(range(7)), 3)) == 2  # the partial tail has no identity
+    assert page_hash(b"ab", ROOT_PARENT, [1, 2, 3]) != page_hash(b"a", ROOT_PARENT, [1, 2, 3])
+    assert page_hash(b"", ROOT_PARENT, [2 ** 40]) != page_hash(b"", ROOT_PARENT, [0])
+    import hashlib
+    import struct
+    want = hashlib.sha256(struct.pack("<I", 1) + b"m" + bytes(32) + struct.pack("<3q", 1, 2, 3)).digest()
+    assert a[0] == want
+
+
+def test_reclaim_policies():
+    p = LRUPolicy()
+    for page in (1, 2, 3):
+        p.add_candidate(page)
+    p.remove_candidate(1)
+    p.add_candidate(1)
+    assert [p.pop_victim() for _ in range(3)] == [2, 3, 1]
+    with pytest.raises(LookupError):
+        p.pop_victim()
+    c = CostAwarePolicy(depth_weight=0.0)
+    c.on_cached(1, 0)
+    for _ in range(5):
+        c.on_hit(1)
+    c.add_candidate(1)
+    c.on_cached(2, 0)
+    c.add_candidate(2)
+    assert c.pop_victim() == 2  # a page hit often outlives a recent one-off
+    d = CostAwarePolicy(depth_weight=1.0)
+    d.on_cached(1, 10)
+    d.on_cached(2, 0)
+    d.add_candidate(1)
+    d.add_candidate(2)
+    assert d.pop_victim() == 2
+    e = CostAwarePolicy()
+    e.on_cached(7, 0)
+    for _ in range(10000):
+        e.add_candidate(7)
+        e.remove_candidate(7)
+    assert e.heap_size() < 200
+
+
+# ------------------------------------------------------------------ groups, windows, state slots
+
+def test_window_group_gives_pages_back_while_the_request_runs():
+    m = CacheManager([GroupSpec(), GroupSpec("window", 6)], num_pages=[32, 8], page_size=4, watermark=0.0)
+    assert not m.prefix_caching  # content reuse needs a single full group
+    m.allocate("a", list(range(10)))
+    assert len(m.block_table("a", 0)) == 3 and len(m.block_table("a", 1)) == 3
+    m.mark_computed("a", 10)
+    # next query at position 10 sees keys 5..10: page 0 (keys 0..3) is passed
+    assert m.block_table("a", 1)[0] == RELEASED and m.block_table("a", 1)[1] != RELEASED
+    assert m.block_table("a", 0)[0] != RELEASED
+    used_before = m.pools[1].num_pages - m.pools[1].num_available
+    for t in range(40):  # far more tokens than the 8 window pages could hold
+        m.append_slots("a", [t])
+        m.mark_computed("a", m.num_tokens("a"))
+        m.check_invariants()
+    assert m.pools[1].num_pages - m.pools[1].num_available <= used_before + 1
+    assert m.stats().window_pages_released >= 10
+    with pytest.raises(ValueError):
+        m.slot_mapping("a", 0, 1, group=1)
+    m.free("a")
+    m.check_invariants()
+    assert all(p.num_available == p.num_pages for p in m.pools)
+
+
+def test_state_slots_are_taken_and_given_back():
+    m = mk(max_seqs=2)
+    a = m.allocate("a", [1]).state_slot
+    b = m.allocate("b", [1]).state_slot
+    assert {a, b} == {0, 1} and not m.can_allocate([1])
+    with pytest.raises(NoFreeSlotError):
+        m.allocate("c", [1])
+    m.free("a")
+    assert m.allocate("c", [1]).state_slot == a
+    m.check_invariants()
+    s = StateSlots(1)
+    slot = s.take()
+    s.give_back(slot)
+    with pytest.raises(AssertionError):
+        s.give_back(slot)
+
+
+# ------------------------------------------------------------------ random orders
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("policy", ["lru", "cost"])
+def test_random_orders_of_requests_keep_every_invariant(seed, policy):
+    rng = random.Random(seed)
+    page_size = rng.choice([1, 2, 4, 8])
+    groups = [GroupSpec()] if seed % 2 == 0 else [GroupSpec(), GroupSpec("window", rng.choice([3, 8, 17]))]
+    m = CacheManager(groups, num_pages=rng.randrange(6, 40), page_size=page_size, max_seqs=5,
+                     eviction_policy=policy, watermark=rng.choice([0.0, 0.1]))
+    shadow: dict = {}   # request -> tokens, as the manager should know them
+    stems = [[rng.randrange(5) for _ in range(rng.randrange(1, 30))] for _ in range(4)]
+    n_id = 0
+    for _ in range(600):
+        op = rng.random()
+        try:
+            if op < 0.3:
+                toks = list(rng.choice(stems)) + [rng.randrange(5) for _ in range(rng.randrange(0, 6))]
+                alloc = m.allocate(n_id, toks)
+                assert alloc.num_cached_tokens % page_size == 0 and alloc.num_cached_tokens < len(toks)
+                shadow[n_id] = toks
+                n_id += 1
+            elif op < 0.55 and shadow:
+                rid = rng.choice(list(shadow))
+                new = [rng.randrange(5) for _ in range(rng.randrange(1, 5))]
+                m.append_slots(rid, new)
+                shadow[rid] = shadow[rid] + new
+            elif op < 0.8 and shadow:
+                rid = rng.choice(list(shadow))
+                lo = m.num_computed_tokens(rid)
+                m.mark_computed(rid, rng.randrange(lo, len(shadow[rid]) + 1))
+            elif op < 0.88 and shadow:
+                rid = rng.choice(list(shadow))
+                m.fork(rid, n_id)
+                shadow[n_id] = list(shadow[rid])
+                n_id += 1
+            elif shadow:
+                rid = rng.choice(list(shadow))
+                m.free(rid)
+                del shadow[rid]
+        except (NoFreePagesError, NoFreeSlotError):
+            pass  # refused: the state must be unchanged, which the invariants below check
+        m.check_invariants()
+        for rid, toks in shadow.items():
+            assert m.num_tokens(rid) == len(toks)
+        st = m.stats()
+        assert st.free_pages + st.cached_idle_pages + st.used_pages == st.num_pages
+    for rid in list(shadow):
+        m.free(rid)
+    m.reset_prefix_cache()
+    m.check_invariants()
+    assert m.stats().free_pages == m.stats().num_pages, "pages were lost"
+    assert m.slots.num_free == 5, "state slots were lost"
+
+
+def test_shadow_cache_never_serves_wrong_or_unwritten_content():
+    """A shadow of the device memory: slot -> (token prefix that was written there). A hit must
+    point at pages whose shadow equals the new prompt's prefix, and a write must never land in a
+    page that another request holds."""
+    rng = random.Random(7)
+    ps = 4
+    m = mk(num_pages=24, page_size=ps)
+    written: dict[int, tuple] = {}
+    live: dict = {}
+    for step in range(800):
+        if rng.random() < 0.4 or not live:
+            toks = [rng.randrange(3) for _ in range(rng.randrange(1, 25))]
+            try:
+                alloc = m.allocate(step, toks)
+            except (NoFreePagesError, NoFreeSlotError):
+                if live:
+                    rid = rng.choice(list(live))
+                    m.free(rid)
+                    del live[rid]
+                continue
+            for p in range(alloc.num_cached_tokens):
+                slot = m.slot_mapping(step, p, p + 1)[0]
+                assert written.get(slot) == tuple(toks[:p + 1]), "a hit serves wrong or unwritten content"
+            live[step] = toks
+        else:
+            rid = rng.choice(list(live))
+            toks = live[rid]
+            lo = m.num_computed_tokens(rid)
+            hi = rng.randrange(lo, len(toks) + 1)
+            for p in range(lo, hi):  # the step function writes these slots
+                slot = m.slot_mapping(rid, p, p + 1)[0]
+                page = slot // ps
+                holders = sum(1 for other in live if page in m.block_table(other))
+                assert holders == 1, "a write lands in a page that another request holds"
+                written[slot] = tuple(toks[:p + 1])
+            m.mark_computed(rid, hi)
+            if hi == len(toks) and rng.random() < 0.5:
+                m.free(rid)
+                del live[rid]
+        m.check_invariants()
