@@ -25,6 +25,8 @@ if str(ROOT) not in sys.path:
 HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
+SLACK = 96  # decode steps that early requests may run before the timed ones
+
 LLAMA_3_2_1B = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 128256, "hidden_size": 2048,
     "intermediate_size": 8192, "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8,
@@ -47,7 +49,7 @@ def make_engine(raw, dtype, batch, context, block_size, budget):
     model, cfg = build_model(raw, rt)
     model.config = cfg
     fill_random_on_device(model, seed=0, std=0.02)
-    pages = batch * (-(-context // block_size) + 1) + 8
+    pages = batch * (-(-(context + SLACK) // block_size) + 1) + 8
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=False,
         config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget))
@@ -62,23 +64,28 @@ def decode_run(engine, cfg, batch, context, steps, warmup):
 
     gen = torch.Generator().manual_seed(batch)
     prompt_len = context - steps - warmup - 1
-    total = steps + warmup + 1
+    ids = []
     for i in range(batch):
         prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).tolist()
-        engine.add_request(f"b{batch}-{i}", prompt, SamplingParams(max_tokens=total, ignore_eos=True))
-    while any(r.num_computed_tokens < prompt_len for r in engine.scheduler.running) or engine.scheduler.waiting:
+        ids.append(f"b{batch}-{i}")
+        # requests that were admitted first decode a few tokens while the others still prefill
+        engine.add_request(ids[-1], prompt, SamplingParams(max_tokens=steps + warmup + 1 + SLACK, ignore_eos=True))
+    guard = 0
+    while engine.scheduler.waiting or any(r.num_computed_tokens < prompt_len for r in engine.scheduler.running):
         engine.step()  # prefill, in portions under the token budget
+        guard += 1
+        assert guard < SLACK, "prefill took more steps than the pool has slack for"
     for _ in range(warmup):
         engine.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         out = engine.step()
-        assert len(out) == batch
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    while engine.has_unfinished():
-        engine.step()
+    assert len(out) == batch and len(engine.scheduler.running) == batch
+    for rid in ids:
+        engine.abort(rid)
     return batch * steps / dt, dt / steps * 1e3
 
 
@@ -142,7 +149,7 @@ def main() -> int:
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
     max_batch = max(args.batch, 1 if args.no_points else 64)
-    engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=2048)
+    engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=8192)
 
     tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup)
     achieved = decode_bytes(cfg, args.batch, args.context, itemsize) / (ms * 1e-3) / 1e9
