@@ -1,0 +1,407 @@
+// Paged attention on the matrix cores (bfloat16 operands, 32-bit accumulation), for decode
+// (one query per request, keys split over workgroups, partial results merged) and for portions of
+// prompts (tiles of queries, causal by absolute position).
+//
+// Both kernels compute the transposed products, so that every per-query statistic of the online
+// softmax lives in the lane that owns the query's column and no operand is ever transposed:
+//
+//   S^T [16 keys x 16 columns]   = K [16 keys x d]   * Q^T [d x 16 columns]
+//   O^T [16 dims x 16 columns]  += V^T [16 dims x 16 keys] * P^T [16 keys x 16 columns]
+//
+// with v_mfma_f32_16x16x16_bf16: operand A gives lane l row l%16 and the four k-indices
+// 4*(l/16)..+3; operand B gives lane l column l%16 and the same k-indices; the result gives lane l
+// column l%16 and rows 4*(l/16)..+3. So S^T comes out exactly in the layout that P^T needs as
+// operand B of the second product. A "column" is a query head of the group in the decode kernel
+// and a query position in the prefill kernel.
+//
+// K pages are [kv_heads][page_size][head_dim] and V pages [kv_heads][head_dim][page_size]: operand
+// A of the first product reads head_dim-contiguous keys, operand A of the second reads
+// key-contiguous dims. The d index of the first product is permuted (lane group g takes the
+// contiguous range [g*d/4, (g+1)*d/4)), identically for K and Q, which leaves the dot product
+// unchanged and makes each lane's K load one contiguous run.
+//
+// Needs page_size % 16 == 0 and head_dim = 16*DCH with DCH <= 8; other shapes take the generic
+// kernel. Scores are scaled by `scale`; exp is taken as exp2 with log2(e) folded into the scale.
+// P is rounded to bfloat16 for the second product while the running sum keeps the unrounded
+// values (as the reference's kernel does: src/dli/model/paged_attention.py:128-168).
+#include "common.h"
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4v mfma16(short4v a, short4v b, float4v c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ short bf16_bits(float x) {
+  bf16_t b = (bf16_t)x;
+  return *reinterpret_cast<short*>(&b);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Online-softmax state of one column tile (16 columns; this lane owns column lane%16).
+template <int DCH>
+struct ColumnTile {
+  float m, l;
+  float4v o[DCH];
+  __device__ __forceinline__ void init() {
+    m = -INFINITY;
+    l = 0.f;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) o[c] = float4v{0.f, 0.f, 0.f, 0.f};
+  }
+};
+
+// One tile of 16 keys starting at logical key `t` (page-aligned by 16) against one column tile.
+// `limit[i]` for i in 0..3: the largest visible key for this lane's column (causal / request end),
+// `lowest`: the smallest visible key (window); keys outside become -inf.
+template <int DCH>
+__device__ __forceinline__ void attend_tile(ColumnTile<DCH>& st, const short4v (&kreg)[DCH],
+                                            const short4v (&qreg)[DCH], const short4v (&vreg)[DCH],
+                                            int t, int grp, int last_visible, int first_visible,
+                                            float scale_log2e, bool need_mask) {
+  float4v s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) s = mfma16(kreg[c], qreg[c], s);
+  float sv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) sv[i] = s[i] * scale_log2e;
+  if (need_mask) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = t + 4 * grp + i;
+      if (key > last_visible || key < first_visible) sv[i] = -INFINITY;
+    }
+  }
+  float tile_max = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, DLI_WAVE));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, DLI_WAVE));
+  const float m_new = fmaxf(st.m, tile_max);
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = fast_exp2(st.m - m_safe);
+  float p[4];
+  float tile_sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    p[i] = fast_exp2(sv[i] - m_safe);
+    tile_sum += p[i];
+  }
+  tile_sum += __shfl_xor(tile_sum, 16, DLI_WAVE);
+  tile_sum += __shfl_xor(tile_sum, 32, DLI_WAVE);
+  st.l = st.l * alpha + tile_sum;
+  st.m = m_new;
+  const short4v pb = {bf16_bits(p[0]), bf16_bits(p[1]), bf16_bits(p[2]), bf16_bits(p[3])};
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) {
+    st.o[c] *= alpha;
+    st.o[c] = mfma16(vreg[c], pb, st.o[c]);
+  }
+}
+
+template <int DCH>
+__device__ __forceinline__ void load_k(short4v (&kreg)[DCH], const bf16_t* __restrict__ k_pages,
+                                       int64_t page, int kv_heads, int kvh, int page_size, int off,
+                                       int col, int grp) {
+  constexpr int D = DCH * 16;
+  const bf16_t* p = k_pages + ((page * kv_heads + kvh) * page_size + off + col) * D + grp * (D / 4);
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) kreg[c] = *reinterpret_cast<const short4v*>(p + c * 4);
+}
+
+// Keys at or beyond `end_key` are replaced by zero so that a zero probability never multiplies
+// whatever a not yet written slot holds.
+template <int DCH>
+__device__ __forceinline__ void load_v(short4v (&vreg)[DCH], const bf16_t* __restrict__ v_pages,
+                                       int64_t page, int kv_heads, int kvh, int page_size, int off,
+                                       int col, int grp, int t, int end_key) {
+  constexpr int D = DCH * 16;
+  const bf16_t* p = v_pages + ((page * kv_heads + kvh) * D + col) * page_size + off + 4 * grp;
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) vreg[c] = *reinterpret_cast<const short4v*>(p + (int64_t)c * 16 * page_size);
+  if (t + 16 > end_key) {
+#pragma unroll
+    for (int c = 0; c < DCH; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (t + 4 * grp + i >= end_key) vreg[c][i] = 0;
+  }
+}
+
+// ------------------------------------------------------------------------------------ decode
+// grid (splits, kv_heads * head_tiles, requests); 256 threads. Request e's single query is row e.
+template <int DCH>
+__global__ __launch_bounds__(256) void attention_decode_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
+    float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ kv_len,
+    const int* __restrict__ block_tables, int table_stride, int q_heads, int kv_heads, int page_size,
+    float scale_log2e, int window, int splits) {
+  constexpr int D = DCH * 16;
+  __shared__ float sm_o[3][D][16];
+  __shared__ float sm_m[3][16], sm_l[3][16];
+
+  const int split = blockIdx.x, e = blockIdx.z;
+  const int group = q_heads / kv_heads;
+  const int head_tiles = (group + 15) / 16;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y % head_tiles;
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int col = lane % 16, grp = lane / 16;
+  const int head_in_group = ht * 16 + col;
+  const bool valid = head_in_group < group;
+  const int head = kvh * group + head_in_group;
+
+  const int n_keys = kv_len[e];
+  const int first_visible = window > 0 ? max(0, n_keys - window) : 0;
+  const int begin = first_visible / 16 * 16;
+  const int chunk = (((n_keys - begin + splits - 1) / splits) + 15) / 16 * 16;
+  const int k0 = begin + split * chunk;
+  const int k1 = min(n_keys, k0 + chunk);
+  const int* table = block_tables + (int64_t)e * table_stride;
+
+  short4v qreg[DCH];
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) qreg[c] = short4v{0, 0, 0, 0};
+  if (valid) {
+    const bf16_t* qp = q + (int64_t)e * q_stride + (int64_t)head * D + grp * (D / 4);
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) qreg[c] = *reinterpret_cast<const short4v*>(qp + c * 4);
+  }
+
+  ColumnTile<DCH> st;
+  st.init();
+  for (int t = k0 + wave * 16; t < k1; t += 64) {
+    const int64_t page = table[t / page_size];
+    const int off = t % page_size;
+    short4v kreg[DCH], vreg[DCH];
+    load_k<DCH>(kreg, k_pages, page, kv_heads, kvh, page_size, off, col, grp);
+    load_v<DCH>(vreg, v_pages, page, kv_heads, kvh, page_size, off, col, grp, t, k1);
+    const bool need_mask = t + 16 > k1 || t < first_visible;
+    attend_tile<DCH>(st, kreg, qreg, vreg, t, grp, k1 - 1, first_visible, scale_log2e, need_mask);
+  }
+
+  // merge the four waves' states in wave 0
+  if (wave > 0) {
+    if (grp == 0) {
+      sm_m[wave - 1][col] = st.m;
+      sm_l[wave - 1][col] = st.l;
+    }
+#pragma unroll
+    for (int c = 0; c < DCH; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sm_o[wave - 1][c * 16 + 4 * grp + i][col] = st.o[c][i];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float m_all = st.m;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, sm_m[w][col]);
+  const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+  float scale_own = fast_exp2(st.m - m_safe);
+  float l_all = st.l * scale_own;
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) st.o[c] *= scale_own;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const float sw = fast_exp2(sm_m[w][col] - m_safe);
+    l_all += sm_l[w][col] * sw;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st.o[c][i] += sm_o[w][c * 16 + 4 * grp + i][col] * sw;
+  }
+  if (!valid) return;
+  if (splits == 1) {
+    const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+    bf16_t* op = out + (int64_t)e * out_stride + (int64_t)head * D + 4 * grp;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) {
+      const short4v packed = {bf16_bits(st.o[c][0] * inv), bf16_bits(st.o[c][1] * inv),
+                              bf16_bits(st.o[c][2] * inv), bf16_bits(st.o[c][3] * inv)};
+      *reinterpret_cast<short4v*>(op + c * 16) = packed;
+    }
+  } else {
+    const int64_t slot = ((int64_t)e * q_heads + head) * splits + split;
+    float* po = part_o + slot * D + 4 * grp;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) *reinterpret_cast<float4v*>(po + c * 16) = st.o[c];
+    if (grp == 0) {
+      part_ml[slot * 2] = m_all;
+      part_ml[slot * 2 + 1] = l_all;
+    }
+  }
+}
+
+// grid (q_heads, requests), 64 threads: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                             const float* __restrict__ part_ml,
+                                                             bf16_t* __restrict__ out,
+                                                             int64_t out_stride, int q_heads,
+                                                             int head_dim, int splits) {
+  const int head = blockIdx.x, e = blockIdx.y;
+  const int64_t base = ((int64_t)e * q_heads + head) * splits;
+  float m_all = -INFINITY;
+  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
+  const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+  float l_all = 0.f;
+  for (int s = 0; s < splits; ++s)
+    l_all += part_ml[(base + s) * 2 + 1] * fast_exp2(part_ml[(base + s) * 2] - m_safe);
+  const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+  for (int d = threadIdx.x; d < head_dim; d += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s)
+      acc += part_o[(base + s) * head_dim + d] * fast_exp2(part_ml[(base + s) * 2] - m_safe);
+    out[(int64_t)e * out_stride + (int64_t)head * head_dim + d] = (bf16_t)(acc * inv);
+  }
+}
+
+// ------------------------------------------------------------------------------------ prefill
+// grid (query tiles of 128, q_heads); 256 threads; each wave owns 32 consecutive queries
+// (two column tiles) of one request and walks that request's keys up to its last query.
+#define PF_TILE_ROWS 128
+template <int DCH>
+__global__ __launch_bounds__(256) void attention_prefill_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
+    const int* __restrict__ q_start, const int* __restrict__ kv_len,
+    const int* __restrict__ block_tables, int table_stride, const int* __restrict__ tile_entry,
+    const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
+    int window) {
+  constexpr int D = DCH * 16;
+  const int e = tile_entry[blockIdx.x];
+  const int head = blockIdx.y;
+  const int kvh = head / (q_heads / kv_heads);
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int col = lane % 16, grp = lane / 16;
+  const int tok0 = q_start[e];
+  const int q_len = q_start[e + 1] - tok0;
+  const int n_keys = kv_len[e];
+  const int first_pos = n_keys - q_len;
+  const int q0 = tile_q0[blockIdx.x] + wave * 32;  // this wave's first query
+  if (q0 >= q_len) return;
+  const int* table = block_tables + (int64_t)e * table_stride;
+
+  short4v qreg[2][DCH];
+  ColumnTile<DCH> st[2];
+  int pos[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    st[j].init();
+    const int qi = q0 + j * 16 + col;
+    pos[j] = qi < q_len ? first_pos + qi : -1;  // -1: no query in this column, nothing is visible
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) qreg[j][c] = short4v{0, 0, 0, 0};
+    if (qi < q_len) {
+      const bf16_t* qp = q + (int64_t)(tok0 + qi) * q_stride + (int64_t)head * D + grp * (D / 4);
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) qreg[j][c] = *reinterpret_cast<const short4v*>(qp + c * 4);
+    }
+  }
+  const int wave_rows = min(32, q_len - q0);
+  const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + wave_rows - 1;
+  const int begin = window > 0 ? max(0, pos_lo - window + 1) / 16 * 16 : 0;
+  const int end = pos_hi + 1;  // keys [begin, end) may be visible to some query of this wave
+  const bool second = wave_rows > 16;
+
+  for (int t = begin; t < end; t += 16) {
+    const int64_t page = table[t / page_size];
+    const int off = t % page_size;
+    short4v kreg[DCH], vreg[DCH];
+    load_k<DCH>(kreg, k_pages, page, kv_heads, kvh, page_size, off, col, grp);
+    load_v<DCH>(vreg, v_pages, page, kv_heads, kvh, page_size, off, col, grp, t, end);
+    // a tile needs masking if it reaches beyond the first query's position or before the window
+    const bool need_mask = t + 15 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
+    const int low0 = window > 0 ? pos[0] - window + 1 : 0;
+    attend_tile<DCH>(st[0], kreg, qreg[0], vreg, t, grp, pos[0], low0, scale_log2e, need_mask);
+    if (second) {
+      const int low1 = window > 0 ? pos[1] - window + 1 : 0;
+      attend_tile<DCH>(st[1], kreg, qreg[1], vreg, t, grp, pos[1], low1, scale_log2e, need_mask);
+    }
+  }
+
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int qi = q0 + j * 16 + col;
+    if (qi >= q_len) continue;
+    const float inv = st[j].l > 0.f ? 1.f / st[j].l : 0.f;
+    bf16_t* op = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * D + 4 * grp;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) {
+      const short4v packed = {bf16_bits(st[j].o[c][0] * inv), bf16_bits(st[j].o[c][1] * inv),
+                              bf16_bits(st[j].o[c][2] * inv), bf16_bits(st[j].o[c][3] * inv)};
+      *reinterpret_cast<short4v*>(op + c * 16) = packed;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------ host side
+#define LOG2E 1.4426950408889634f
+
+extern "C" int dli_attention_mfma_supports(int head_dim, int page_size) {
+  return head_dim > 0 && head_dim % 16 == 0 && head_dim <= 128 && page_size > 0 && page_size % 16 == 0;
+}
+
+extern "C" int dli_attention_prefill_tile_rows() { return PF_TILE_ROWS; }
+
+extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pages,
+                                         const void* v_pages, void* out, int64_t out_stride,
+                                         float* part_o, float* part_ml, const int* kv_len,
+                                         const int* block_tables, int table_stride, int requests,
+                                         int q_heads, int kv_heads, int head_dim, int page_size,
+                                         float scale, int window, int splits, hipStream_t stream) {
+  if (requests <= 0) return DLI_OK;
+  if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
+      q_heads % kv_heads != 0 || splits < 1 || splits > 65535 || requests > 65535 ||
+      (splits > 1 && (part_o == nullptr || part_ml == nullptr)) || q_stride % 4 != 0 ||
+      out_stride % 4 != 0)
+    return DLI_ERR_ARGUMENT;
+  const int head_tiles = (q_heads / kv_heads + 15) / 16;
+  const dim3 grid(splits, kv_heads * head_tiles, requests);
+#define DECODE_CASE(N)                                                                            \
+  case N:                                                                                         \
+    attention_decode_kernel<N><<<grid, 256, 0, stream>>>(                                         \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
+        out_stride, part_o, part_ml, kv_len, block_tables, table_stride, q_heads, kv_heads,       \
+        page_size, scale * LOG2E, window, splits);                                                \
+    break;
+  switch (head_dim / 16) {
+    DECODE_CASE(1) DECODE_CASE(2) DECODE_CASE(3) DECODE_CASE(4)
+    DECODE_CASE(5) DECODE_CASE(6) DECODE_CASE(7) DECODE_CASE(8)
+    default: return DLI_ERR_ARGUMENT;
+  }
+#undef DECODE_CASE
+  if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
+  if (splits > 1) {
+    attention_merge_kernel<<<dim3(q_heads, requests), 64, 0, stream>>>(
+        part_o, part_ml, (bf16_t*)out, out_stride, q_heads, head_dim, splits);
+  }
+  return dli_launch_status();
+}
+
+extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages,
+                                          const void* v_pages, void* out, int64_t out_stride,
+                                          const int* q_start, const int* kv_len,
+                                          const int* block_tables, int table_stride,
+                                          const int* tile_entry, const int* tile_q0, int tiles,
+                                          int q_heads, int kv_heads, int head_dim, int page_size,
+                                          float scale, int window, hipStream_t stream) {
+  if (tiles <= 0) return DLI_OK;
+  if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
+      q_heads % kv_heads != 0 || q_heads > 65535 || q_stride % 4 != 0 || out_stride % 4 != 0)
+    return DLI_ERR_ARGUMENT;
+  const dim3 grid(tiles, q_heads);
+#define PREFILL_CASE(N)                                                                           \
+  case N:                                                                                         \
+    attention_prefill_kernel<N><<<grid, 256, 0, stream>>>(                                        \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
+        out_stride, q_start, kv_len, block_tables, table_stride, tile_entry, tile_q0, q_heads,    \
+        kv_heads, page_size, scale * LOG2E, window);                                              \
+    break;
+  switch (head_dim / 16) {
+    PREFILL_CASE(1) PREFILL_CASE(2) PREFILL_CASE(3) PREFILL_CASE(4)
+    PREFILL_CASE(5) PREFILL_CASE(6) PREFILL_CASE(7) PREFILL_CASE(8)
+    default: return DLI_ERR_ARGUMENT;
+  }
+#undef PREFILL_CASE
+  return dli_launch_status();
+}

@@ -64,6 +64,10 @@ class StepContext:
     def max_kv_len(self) -> int:
         return int(self.kv_len_host.max()) if self.num_entries else 0
 
+    @property
+    def max_decode_kv_len(self) -> int:
+        return int(self.kv_len_host[:self.num_decode].max()) if self.num_decode else 0
+
     def entry_rows(self, e: int) -> tuple[int, int]:
         return int(self.q_start_host[e]), int(self.q_start_host[e + 1])
 

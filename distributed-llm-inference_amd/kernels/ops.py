@@ -41,6 +41,12 @@ _SIGNATURES = {
                         _c_int, _c_int, _c_ptr],
     "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
+    "dli_attention_mfma_supports": [_c_int, _c_int],
+    "dli_attention_prefill_tile_rows": [],
+    "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                                   _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                               _c_int, _c_int, _c_ptr],
@@ -309,6 +315,81 @@ def attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
         tile_entry.shape[0], q_heads, kv_heads, head_dim, page_size, float(scale), int(window),
         _is_bf16(dtype), _stream()), "attention_generic")
 
+
+
+def attention_mfma_supports(head_dim: int, page_size: int, dtype: torch.dtype) -> bool:
+    """Whether the matrix-core attention kernels take this shape (else: the generic kernel)."""
+    return dtype == torch.bfloat16 and bool(library().dli_attention_mfma_supports(head_dim, page_size))
+
+
+def attention_prefill_tile_rows() -> int:
+    return int(library().dli_attention_prefill_tile_rows())
+
+
+def _check_paged(q, k_pages, v_pages, out, q_heads):
+    _dense(k_pages, "k_pages", torch.bfloat16, 4)
+    _rows(q, "q", torch.bfloat16)
+    _rows(out, "out", torch.bfloat16)
+    pages, kv_heads, page_size, head_dim = k_pages.shape
+    _dense(v_pages, "v_pages", torch.bfloat16, 4)
+    _require(v_pages.shape == (pages, kv_heads, head_dim, page_size),
+             "v_pages must be [pages, kv_heads, head_dim, page_size]")
+    _require(q.shape[1] == q_heads * head_dim and out.shape == q.shape, "q/out must be [rows, q_heads*head_dim]")
+    _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
+    _require(q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and q.data_ptr() % 8 == 0 and out.data_ptr() % 8 == 0,
+             "q/out rows must be 8-byte aligned")
+    _require(bool(library().dli_attention_mfma_supports(head_dim, page_size)),
+             f"the matrix-core attention takes head_dim 16..128 in steps of 16 and pages of a multiple of 16, "
+             f"not head_dim {head_dim}, page size {page_size}")
+    return kv_heads, page_size, head_dim
+
+
+def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                     kv_len: torch.Tensor, block_tables: torch.Tensor, q_heads: int, scale: float,
+                     window: int = 0, splits: int = 1, part_o: Optional[torch.Tensor] = None,
+                     part_ml: Optional[torch.Tensor] = None) -> None:
+    """Decode attention: row ``e`` of ``q`` is request ``e``'s single query over its ``kv_len[e]`` keys.
+
+    With ``splits > 1`` each request's keys are cut into that many runs whose partial results go
+    through ``part_o [rows, q_heads, splits, head_dim]`` and ``part_ml [rows, q_heads, splits, 2]``
+    (float32) and are merged by a second kernel.
+    """
+    kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
+    rows = q.shape[0]
+    _dense(kv_len, "kv_len", torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    _require(kv_len.shape[0] >= rows and block_tables.shape[0] >= rows, "one kv_len and table row per request")
+    _require(1 <= splits <= 65535 and rows <= 65535, "splits and requests must fit the grid")
+    if splits > 1:
+        _require(part_o is not None and part_ml is not None, "splits > 1 needs the partial-result buffers")
+        _dense(part_o, "part_o", torch.float32)
+        _dense(part_ml, "part_ml", torch.float32)
+        _require(part_o.numel() >= rows * q_heads * splits * head_dim and part_ml.numel() >= rows * q_heads * splits * 2,
+                 "partial-result buffers are too small")
+    _check(library().dli_attention_decode_bf16(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml),
+        _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size,
+        float(scale), int(window), int(splits), _stream()), "attention_decode")
+
+
+def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                      q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
+                      tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
+                      window: int = 0) -> None:
+    """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
+    :func:`attention_prefill_tile_rows` queries."""
+    kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
+    for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
+        _dense(t, name, torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    entries = kv_len.shape[0]
+    _require(q_start.shape[0] == entries + 1 and block_tables.shape[0] >= entries,
+             "q_start/kv_len/block_tables disagree on the number of requests")
+    _require(tile_entry.shape == tile_q0.shape, "tile lists differ in length")
+    _check(library().dli_attention_prefill_bf16(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
+        _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tile_entry.shape[0], q_heads,
+        kv_heads, head_dim, page_size, float(scale), int(window), _stream()), "attention_prefill")
 
 # ----------------------------------------------------------------------------- sampling
 

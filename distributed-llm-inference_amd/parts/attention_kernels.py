@@ -2,7 +2,7 @@
 
 The true 32-bit path, and shapes that the matrix-core kernels do not take, run the vector-unit
 kernel over all entries. The bfloat16 path sends entries that bring one token to the split-key
-decode kernel and portions to the tiled prefill kernel when their shapes allow it.
+decode kernel and portions to the tiled prefill kernel.
 """
 
 from __future__ import annotations
@@ -13,14 +13,45 @@ import torch
 
 from ..kernels import ops
 
+NUM_CUS = 256            # MI355X
+WORKGROUPS_WANTED = 4 * NUM_CUS
+MIN_KEYS_PER_SPLIT = 128
+MAX_SPLITS = 64
+
+
+def choose_splits(requests: int, kv_head_tiles: int, max_keys: int) -> int:
+    """How many runs to cut each request's keys into for the decode kernel: enough workgroups
+    to fill the GPU about four times over, never runs under 128 keys (reference's rule of the
+    same kind: src/dli/model/paged_attention.py:63-74)."""
+    programs = max(1, requests * kv_head_tiles)
+    want = -(-WORKGROUPS_WANTED // programs)
+    most = max(1, max_keys // MIN_KEYS_PER_SPLIT)
+    return max(1, min(want, most, MAX_SPLITS))
+
 
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                     ctx: Any, grp: Any, q_heads: int, scale: float, window: int = 0) -> None:
     """Attention of every row of the step over its request's pages, into ``out``."""
     if ctx.num_tokens == 0:
         return
-    head_dim = k_pages.shape[3]
-    rows = ops.attention_generic_tile_rows(head_dim)
-    tile_entry, tile_q0 = ctx.q_tiles(rows)
-    ops.attention_generic(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
-                          tile_entry, tile_q0, q_heads, scale, window)
+    _, kv_heads, page_size, head_dim = k_pages.shape
+    if not ops.attention_mfma_supports(head_dim, page_size, k_pages.dtype):
+        rows = ops.attention_generic_tile_rows(head_dim)
+        tile_entry, tile_q0 = ctx.q_tiles(rows)
+        ops.attention_generic(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                              tile_entry, tile_q0, q_heads, scale, window)
+        return
+    nd = ctx.num_decode
+    if nd > 0:
+        group = q_heads // kv_heads
+        splits = choose_splits(nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty(nd * q_heads * splits * head_dim, device=q.device, dtype=torch.float32)
+            part_ml = torch.empty(nd * q_heads * splits * 2, device=q.device, dtype=torch.float32)
+        ops.attention_decode(q[:nd], k_pages, v_pages, out[:nd], ctx.kv_len, grp.block_tables, q_heads,
+                             scale, window, splits, part_o, part_ml)
+    if ctx.num_entries > nd:
+        tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(), first_entry=nd)
+        ops.attention_prefill(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                              tile_entry, tile_q0, q_heads, scale, window)

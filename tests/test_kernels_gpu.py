@@ -187,3 +187,78 @@ def test_attention_generic(ops, dtype, qh, kvh, d, bs, window):
     ref = ref_paged_attention(q, kp, vp, q_start, kv_len, tables, qh, scale, window)
     err = (out.cpu().double() - ref).abs().max().item()
     assert err < tol(dtype), err
+
+
+MFMA_SHAPES = [(4, 4, 16, 16), (6, 2, 32, 16), (32, 8, 64, 16), (14, 2, 64, 32), (8, 8, 128, 16), (5, 1, 80, 16),
+               (3, 3, 48, 64), (40, 2, 64, 16), (7, 7, 112, 16)]
+
+
+@pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
+@pytest.mark.parametrize("splits", [1, 4, 16])
+@pytest.mark.parametrize("window", [0, 45])
+def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
+    """One query per request against scattered, over-wide tables whose spare entries name a
+    poisoned page; lengths at the page's edges; every split factor gives the same result."""
+    rng = torch.Generator().manual_seed(d * 7 + bs)
+    rand = [int(x) for x in torch.randint(1, 40 * bs, (6,), generator=rng)]
+    lens = [(1, n) for n in [1, bs, bs + 1, 3 * bs - 1, 15, 16, 17] + rand]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + bs + splits)
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
+    scale = 1.0 / math.sqrt(d)
+    n = len(lens)
+    part_o = torch.full((n * qh * splits * d,), float("nan"), device="cuda")
+    part_ml = torch.full((n * qh * splits * 2,), float("nan"), device="cuda")
+    ops.attention_decode(q.cuda(), kp.cuda(), vp.cuda(), out, dev(kv_len), dev(tables), qh, scale, window, splits,
+                         part_o, part_ml)
+    ref = ref_paged_attention(q, kp, vp, q_start, kv_len, tables, qh, scale, window)
+    err = (out.cpu().double() - ref).abs().max().item()
+    assert err < tol(torch.bfloat16), err
+
+
+@pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window):
+    lens = [(2, 2), (7, 7), (33, 33), (5, 40), (2, 131), (129, 129), (16, 16), (31, 300), (140, 333), (1, 50)]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + bs)
+    te, tq = _tiles(q_start, ops.attention_prefill_tile_rows())
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
+    scale = 1.0 / math.sqrt(d)
+    ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables),
+                          dev(te), dev(tq), qh, scale, window)
+    ref = ref_paged_attention(q, kp, vp, q_start, kv_len, tables, qh, scale, window)
+    err = (out.cpu().double() - ref).abs().max().item()
+    assert err < tol(torch.bfloat16), err
+
+
+def test_attention_finds_one_far_key_among_hundreds(ops):
+    """One key far back is made to dominate (its q.k is scaled up); the output must be its value.
+    A kernel that drops, misplaces or mis-masks a page cannot pass."""
+    qh, kvh, d, bs = 8, 2, 64, 16
+    lens = [(1, 700), (3, 700)]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=3, poison=False)
+    kp, vp, q = kp.float(), vp.float(), q.float() * 0.05
+    far = 37
+    for e in range(2):
+        page, off = tables[e][far // bs], far % bs
+        kp[page, :, off, :] = 1.0
+        for row in range(q_start[e], q_start[e + 1]):
+            q[row] = q[row] + 4.0  # q.k of that key: 4*64 = 256 before scaling, 32 after
+    q, kp, vp = q.bfloat16(), kp.bfloat16(), vp.bfloat16()
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    scale = 1.0 / math.sqrt(d)
+    out = torch.zeros(q.shape, dtype=torch.bfloat16, device="cuda")
+    ops.attention_decode(q[:1].cuda(), kp.cuda(), vp.cuda(), out[:1], dev(kv_len), dev(tables), qh, scale, 0, 4,
+                         torch.empty(qh * 4 * d, device="cuda"), torch.empty(qh * 4 * 2, device="cuda"))
+    te, tq = _tiles(q_start, ops.attention_prefill_tile_rows())
+    te, tq = [t for t in te if t == 1], [q0 for t, q0 in zip(te, tq) if t == 1]
+    ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables),
+                          dev(te), dev(tq), qh, scale, 0)
+    for e in range(2):
+        page, off = tables[e][far // bs], far % bs
+        for row in range(q_start[e], q_start[e + 1]):
+            got = out[row].float().cpu().view(qh, d)
+            for h in range(qh):
+                want = vp[page, h // (qh // kvh), :, off].float()
+                assert (got[h] - want).abs().max() < 0.05, (e, row, h)
