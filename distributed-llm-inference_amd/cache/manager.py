@@ -189,6 +189,10 @@ class CacheManager:
         """Page ids of the request in ``group``; :data:`RELEASED` where a window has passed."""
         return tuple(self._seq(seq_id).tables[group])
 
+    def table_ref(self, seq_id: SeqId, group: int = 0) -> list[int]:
+        """The request's live page list in ``group`` (read only: it changes as the request grows)."""
+        return self._seq(seq_id).tables[group]
+
     def state_slot(self, seq_id: SeqId) -> int:
         return self._seq(seq_id).state_slot
 

@@ -29,6 +29,8 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--no-prefix-caching", action="store_true",
                    help="no reuse of cached pages across requests")
+    p.add_argument("--cuda-graphs", action=argparse.BooleanOptionalAction, default=True,
+                   help="replay decode steps through HIP graphs (steps that fit no captured shape run eagerly)")
     p.add_argument("--max-num-seqs", type=int, default=64)
     p.add_argument("--max-num-batched-tokens", type=int, default=512)
 
@@ -62,7 +64,7 @@ def cmd_generate(args: argparse.Namespace) -> int:
         kv_cache_gb=args.kv_cache_gb, block_size=args.block_size, max_num_seqs=args.max_num_seqs,
         max_num_batched_tokens=args.max_num_batched_tokens,
         enable_prefix_caching=not args.no_prefix_caching, eos_token_ids=tuple(args.eos_token_ids or ()),
-        seed=args.engine_seed)
+        seed=args.engine_seed, cuda_graphs=args.cuda_graphs, device=args.device)
     for ids in out:
         print(json.dumps(ids))
     return 0

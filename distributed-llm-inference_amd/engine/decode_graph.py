@@ -1,0 +1,188 @@
+"""HIP-graph replay of decode steps.
+
+A step in which every request brings exactly one token always launches the same kernels with the
+same grids; only the contents of a few small integer arrays change (token ids, positions, cache
+slots, lengths, block tables). Such steps are captured once per (batch bucket, key-split factor)
+into a HIP graph whose kernels read those arrays from fixed device addresses; a later step copies
+its arrays there with one host-to-device copy and replays the graph. That removes the per-kernel
+launch cost, which would otherwise exceed the step's memory time at small batches.
+
+A batch smaller than its bucket is padded with rows that have no keys and no cache slot: they
+write nothing and their logits are dropped. Capture uses the same model code as eager steps.
+No memset node is recorded: buffers that must start at zero are cleared by fill kernels.
+
+The reference replays CUDA graphs of batched decode in fixed buckets the same way
+(src/dli/engine/cuda_graph.py:19-21,137-144), padding rows into a scratch block.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import RELEASED
+from ..kernels import ops
+from ..parts.attention_kernels import choose_splits
+from .batch import GroupView, StepContext, StepEntry
+
+
+def _bucket(n: int) -> int:
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+@dataclass
+class _Captured:
+    graph: torch.cuda.CUDAGraph
+    ctx: StepContext
+    host: torch.Tensor      # pinned int32 staging, same layout as dev
+    dev: torch.Tensor
+    logits: torch.Tensor
+    views: dict             # name -> numpy view into host
+    width: int              # block-table entries per row
+    rows: list              # per row: (request, pages already written into its table row)
+
+
+class DecodeGraphs:
+    def __init__(self, step_fn, *, max_batch: int, max_blocks_per_seq: int) -> None:
+        self.step_fn = step_fn
+        self.rt = step_fn.rt
+        self.max_batch = max_batch
+        self.max_width = max(1, max_blocks_per_seq)
+        self.n_groups = step_fn.manager.num_groups
+        self.captured: dict[tuple[int, int, int], _Captured] = {}
+        self.replays = 0
+        self.enabled = self._supported()
+
+    def _supported(self) -> bool:
+        """Only the matrix-core decode path is captured: every paged layer must take it."""
+        if self.rt.dtype != torch.bfloat16 or self.step_fn.store.stateful:
+            return False
+        ps = self.step_fn.store.page_size
+        for cache in self.step_fn.store.layers:
+            if cache is None or cache.kind != "paged":
+                return False
+            if not ops.attention_mfma_supports(cache.k_pages.shape[3], ps, cache.k_pages.dtype):
+                return False
+        return True
+
+    def can_run(self, entries: Sequence[StepEntry]) -> bool:
+        if not self.enabled or not entries or len(entries) > self.max_batch:
+            return False
+        ps = self.step_fn.manager.page_size
+        return all(len(e.tokens) == 1 and e.start + 1 <= self.max_width * ps for e in entries)
+
+    # ------------------------------------------------------------------ capture
+
+    def _layout(self, b: int, width: int) -> tuple[dict, int]:
+        fields = [("token_ids", b), ("positions", b), ("q_start", b + 1), ("kv_len", b), ("state_slots", b),
+                  ("logit_rows", b)]
+        for g in range(self.n_groups):
+            fields += [(f"slots{g}", b), (f"tables{g}", b * width)]
+        offsets, at = {}, 0
+        for name, n in fields:
+            offsets[name] = (at, n)
+            at += -(-n // 4) * 4  # 16-byte aligned starts
+        return offsets, at
+
+    def _capture(self, b: int, splits: int, width: int) -> _Captured:
+        dev_name = self.rt.device
+        offsets, total = self._layout(b, width)
+        host = torch.zeros(total, dtype=torch.int32).pin_memory()
+        dev = torch.zeros(total, dtype=torch.int32, device=dev_name)
+        hv = host.numpy()
+        views = {name: hv[o:o + n] for name, (o, n) in offsets.items()}
+        dv = {name: dev[o:o + n] for name, (o, n) in offsets.items()}
+        # a batch of padding rows: no keys, no slot
+        views["q_start"][:] = np.arange(b + 1)
+        views["logit_rows"][:] = np.arange(b)
+        for g in range(self.n_groups):
+            views[f"slots{g}"][:] = -1
+        dev.copy_(host)
+        groups = [GroupView(dv[f"slots{g}"], dv[f"tables{g}"].view(b, width), width)
+                  for g in range(self.n_groups)]
+        ctx = StepContext(
+            device=dev_name, page_size=self.step_fn.manager.page_size, num_tokens=b, num_entries=b,
+            num_decode=b, token_ids=dv["token_ids"], positions=dv["positions"], q_start=dv["q_start"],
+            kv_len=dv["kv_len"], state_slots=dv["state_slots"], logit_rows=dv["logit_rows"], groups=groups,
+            q_start_host=np.arange(b + 1, dtype=np.int32), kv_len_host=np.zeros(b, np.int32),
+            state_slots_host=np.zeros(b, np.int32), seq_ids=[None] * b)
+        ctx.forced_splits = splits
+        model, caches = self.step_fn.model, self.step_fn.caches
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):  # warm up libraries and the allocator outside the capture
+                model.forward(ctx, caches)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = model.forward(ctx, caches)
+        return _Captured(graph, ctx, host, dev, logits, views, width, [None] * b)
+
+    # ------------------------------------------------------------------ replay
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Logits ``[wanted, vocab]`` of a decode-only step (a view of the graph's output: use it
+        before the next step)."""
+        mgr = self.step_fn.manager
+        ps, n = mgr.page_size, len(entries)
+        b = _bucket(n)
+        max_kv = max(e.start + 1 for e in entries)
+        width = max(16, _bucket(-(-max_kv // ps)))
+        splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv))
+        key = (b, splits, width)
+        cap = self.captured.get(key)
+        if cap is None:
+            cap = self.captured[key] = self._capture(b, splits, width)
+        v = cap.views
+        limit = self.step_fn.store.num_pages
+        token_ids, positions, kv_len, state_slots = v["token_ids"], v["positions"], v["kv_len"], v["state_slots"]
+        kv_len[n:] = 0
+        token_ids[n:] = 0
+        positions[n:] = 0
+        rows = []
+        for i, e in enumerate(entries):
+            tok = int(e.tokens[0])
+            if not 0 <= tok < self.step_fn.vocab_size:
+                raise ValueError(f"request {e.seq_id!r}: token id {tok} outside the vocabulary")
+            token_ids[i] = tok
+            positions[i] = e.start
+            kv_len[i] = e.start + 1
+            state_slots[i] = mgr.state_slot(e.seq_id)
+            known = cap.rows[i]
+            for g in range(self.n_groups):
+                table = mgr.table_ref(e.seq_id, g)
+                page = table[e.start // ps]
+                if not 0 <= page < limit:
+                    raise ValueError("a block table names a page outside the pool")
+                v[f"slots{g}"][i] = page * ps + e.start % ps
+                row = v[f"tables{g}"][i * width:(i + 1) * width]
+                full = mgr.groups[g].kind == "full"
+                # a request that keeps its row only appends pages (the last one may have been
+                # swapped by a copy-on-write): rewrite from the last page known
+                lo = max(0, known[1][g] - 1) if (known is not None and known[0] == e.seq_id and full) else 0
+                row[lo:len(table)] = table[lo:]
+                if not full:
+                    np.maximum(row, 0, out=row)  # pages that the window has passed are never read
+            cap.rows[i] = (e.seq_id, [len(mgr.table_ref(e.seq_id, g)) for g in range(self.n_groups)])
+            if e.want:
+                rows.extend(i for _ in e.want)
+        for g in range(self.n_groups):
+            v[f"slots{g}"][n:] = -1
+        for i in range(n, b):
+            cap.rows[i] = None
+        cap.dev.copy_(cap.host, non_blocking=True)
+        cap.graph.replay()
+        self.replays += 1
+        if rows == list(range(n)):
+            return cap.logits[:n]
+        if not rows:
+            return cap.logits[:0]
+        return cap.logits[torch.tensor(rows, device=cap.logits.device)]

@@ -112,11 +112,15 @@ class LLMEngine:
                   block_size: int = 16, config: Optional[SchedulerConfig] = None,
                   eviction_policy: str = "lru", enable_prefix_caching: bool = True,
                   eos_token_ids: Collection[int] = (), seed: int = 0, dtype: str = "bfloat16",
-                  device: str = "cuda") -> "LLMEngine":
+                  device: str = "cuda", cuda_graphs: bool = True,
+                  max_model_len: Optional[int] = None) -> "LLMEngine":
         """Engine for a loaded model or a model folder.
 
         ``num_blocks`` pages of ``block_size`` tokens, or as many as ``kv_cache_gb`` GiB hold
         (default 1 GiB), as the reference's server takes them (src/dli/server/__main__.py:150-156).
+        ``cuda_graphs``: replay decode-only steps through HIP graphs (the reference's option of
+        this name replays CUDA graphs; here it is on by default and falls back to eager steps for
+        shapes whose decode path is not captured).
         """
         from ..weights.loader import load_model
         from .core import build_core, pages_for_budget
@@ -131,6 +135,9 @@ class LLMEngine:
         config = config or SchedulerConfig()
         core = build_core(model, num_pages=num_blocks, page_size=block_size, max_seqs=config.max_num_seqs,
                           enable_prefix_caching=enable_prefix_caching, eviction_policy=eviction_policy)
+        if cuda_graphs:
+            longest = num_blocks * block_size
+            core.step.enable_decode_graphs(config.max_num_seqs, min(max_model_len or longest, longest))
         engine = cls(ModelRunner(core), core.manager, config, eos_token_ids=eos_token_ids, seed=seed)
         engine.core = core
         return engine

@@ -17,7 +17,7 @@ from .scheduler import SchedulerConfig
 
 def greedy_generate(model: Any, prompt_ids: Sequence[int], max_new_tokens: int, *,
                     eos_token_ids: Collection[int] = (), block_size: int = 16,
-                    dtype: str = "bfloat16") -> list[int]:
+                    dtype: str = "bfloat16", cuda_graphs: bool = True) -> list[int]:
     """Generate up to ``max_new_tokens`` tokens by taking the argmax each step."""
     if not prompt_ids:
         raise ValueError("prompt_ids must be non-empty")
@@ -27,7 +27,7 @@ def greedy_generate(model: Any, prompt_ids: Sequence[int], max_new_tokens: int, 
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, eos_token_ids=eos_token_ids, dtype=dtype,
         config=SchedulerConfig(max_num_seqs=1, max_num_batched_tokens=max(512, len(prompt_ids))),
-        enable_prefix_caching=False)
+        enable_prefix_caching=False, cuda_graphs=cuda_graphs)
     return engine.generate([prompt_ids], SamplingParams(max_tokens=max_new_tokens))[0]
 
 
@@ -35,10 +35,12 @@ def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
              params: SamplingParams | Sequence[SamplingParams] | None = None, *,
              dtype: str = "bfloat16", num_blocks: Optional[int] = None, kv_cache_gb: Optional[float] = None,
              block_size: int = 16, max_num_seqs: int = 64, max_num_batched_tokens: int = 512,
-             enable_prefix_caching: bool = True, eos_token_ids: Collection[int] = (), seed: int = 0) -> list[list[int]]:
+             enable_prefix_caching: bool = True, eos_token_ids: Collection[int] = (), seed: int = 0,
+             cuda_graphs: bool = True, device: str = "cuda") -> list[list[int]]:
     """Load ``model`` (a folder or a loaded model), run ``prompts`` to completion, return token ids."""
     engine = LLMEngine.for_model(
         model, num_blocks=num_blocks, kv_cache_gb=kv_cache_gb, block_size=block_size, dtype=dtype,
         config=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=max_num_batched_tokens),
-        enable_prefix_caching=enable_prefix_caching, eos_token_ids=eos_token_ids, seed=seed)
+        enable_prefix_caching=enable_prefix_caching, eos_token_ids=eos_token_ids, seed=seed,
+        cuda_graphs=cuda_graphs, device=device)
     return engine.generate(prompts, params)

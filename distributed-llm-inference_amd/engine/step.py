@@ -39,6 +39,25 @@ class StepFunction:
         self.caches = model.bind_caches(store.layers)
         self.vocab_size = model.spec.vocab_size
         self.steps_run = 0
+        self.graphs = None  # DecodeGraphs, when the engine enables graph replay of decode steps
+        tiles = [1]
+        for i, cache in enumerate(store.layers):
+            if cache is not None and cache.kind == "paged":
+                mixer = self.model.layers[self.model.spec.schedule[i].layer].parts.get("mixer")
+                kv_heads = cache.k_pages.shape[1]
+                q_heads = int(getattr(mixer, "num_heads", kv_heads))
+                tiles.append(kv_heads * -(-(q_heads // kv_heads) // 16))
+        self.decode_head_tiles = max(tiles)  # workgroups per request and key split in decode attention
+
+    def enable_decode_graphs(self, max_batch: int, max_model_len: int) -> None:
+        """Replay decode-only steps through HIP graphs (bfloat16 with the matrix-core decode path
+        only; other steps run eagerly)."""
+        from .decode_graph import DecodeGraphs
+
+        self.graphs = DecodeGraphs(self, max_batch=max_batch,
+                                   max_blocks_per_seq=-(-max_model_len // self.manager.page_size))
+        if not self.graphs.enabled:
+            self.graphs = None
 
     # ------------------------------------------------------------------ batch building
 
@@ -130,8 +149,21 @@ class StepFunction:
         self.store.copy_pages(copy_ops)  # before any write of this step (runner.py:56)
         if not entries:
             return torch.empty(0, self.vocab_size, device=self.rt.device, dtype=torch.float32)
-        ctx = self.build_context(entries)
-        logits = self.model.forward(ctx, self.caches)
+        if self.graphs is not None and not copy_ops and self.graphs.can_run(entries):
+            for e in entries:  # the same checks as build_context makes
+                if e.start != self.manager.num_computed_tokens(e.seq_id):
+                    raise StepError(f"request {e.seq_id!r}: portion starts at {e.start} but "
+                                    f"{self.manager.num_computed_tokens(e.seq_id)} tokens are computed")
+                if e.start + 1 > self.manager.num_tokens(e.seq_id):
+                    raise StepError(f"request {e.seq_id!r}: no cache slot reserved at {e.start}")
+                if any(int(w) != 0 for w in e.want):
+                    raise StepError(f"request {e.seq_id!r}: wanted place outside its one token")
+            if len({e.seq_id for e in entries}) != len(entries):
+                raise StepError("a request appears twice in one step")
+            logits = self.graphs.run(entries)
+        else:
+            ctx = self.build_context(entries)
+            logits = self.model.forward(ctx, self.caches)
         for e in entries:
             self.manager.mark_computed(e.seq_id, e.start + len(e.tokens))
         self.steps_run += 1

@@ -44,7 +44,8 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
     nd = ctx.num_decode
     if nd > 0:
         group = q_heads // kv_heads
-        splits = choose_splits(nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len)
+        splits = getattr(ctx, "forced_splits", None) or choose_splits(
+            nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len)
         part_o = part_ml = None
         if splits > 1:
             part_o = torch.empty(nd * q_heads * splits * head_dim, device=q.device, dtype=torch.float32)

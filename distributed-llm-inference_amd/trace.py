@@ -83,6 +83,7 @@ class TraceRunner:
         # No content reuse here: a step must run exactly the tokens it brings.
         core = build_core(model_dir, num_pages=num_pages, page_size=page_size, max_seqs=max_live,
                           dtype=dtype, enable_prefix_caching=False, watermark=0.0)
+        core.step.enable_decode_graphs(max_live, num_pages * page_size)  # as serving does
         self.session = TraceSession(core)
 
     def run_step(self, record: dict) -> Optional[Path]:
