@@ -1,0 +1,380 @@
+// Matrix product for a few rows of activations (decode): y[m][n] = sum_k xhat[m][k] * w[n][k],
+// m < 64, with the work that surrounds it in a decoder layer fused in, so that a layer needs few
+// launches and the weights stream from HBM exactly once.
+//
+// One workgroup owns 16 output features (rows n of w) for all activation rows; its waves split k
+// among themselves and add up through LDS in a fixed order. Products run on the matrix cores as
+//   acc[16 n x 16 m] += W[16 n x 32 k] * xhat^T[32 k x 16 m]      (v_mfma_f32_16x16x32_bf16)
+// where lane l supplies row/column l%16 and eight k values. Inside a block of 128 k the lane
+// group g = l/16 takes the contiguous run [32g, 32g+32) and the four products of the block use its
+// four runs of eight: the same permutation of k for both operands, so the sum is unchanged and a
+// lane reads 64 contiguous bytes of its weight row.
+//
+// Fused in (template switches):
+//   NORM     xhat = cast(norm_w[k] * cast(x[m][k] * rs[m])), rs[m] = rsqrt(sum_k x^2 / K + eps),
+//            the row sums of squares being handed over in parts by the kernel that wrote x
+//            (RMSNorm: src/dli/model/llama.py:40-44); otherwise xhat = x.
+//   EPI_STORE     y (+ bias) stored as bf16
+//   EPI_SWIGLU    two products per workgroup, rows n (gate) and n + up_offset (up) of w:
+//                 stores cast(silu(gate)) * up (src/dli/model/llama.py:190)
+//   EPI_RESIDUAL  stream[m][n] = cast(stream[m][n] + cast(y + bias)) in place (the residual sum, in
+//                 32-bit), and this tile's part of sum_n stream[m][n]^2 for the norm that follows
+//   EPI_F32       y stored as float32 (logits)
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2, EPI_F32 = 3 };
+
+__device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// Activation fragment of eight k values: the raw loads, and the norm applied afterwards (so the
+// loads can be issued a block ahead of their use).
+template <bool NORM>
+struct XFrag {
+  bf16x8 v;
+  float4v w0, w1;
+};
+template <>
+struct XFrag<false> {
+  bf16x8 v;
+};
+
+template <bool NORM>
+__device__ __forceinline__ XFrag<NORM> fetch_x(const bf16_t* __restrict__ xrow,
+                                               const float* __restrict__ norm_w, int k, bool live) {
+  XFrag<NORM> f;
+  f.v = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  if (live) f.v = *reinterpret_cast<const bf16x8*>(xrow + k);
+  if constexpr (NORM) {
+    f.w0 = *reinterpret_cast<const float4v*>(norm_w + k);
+    f.w1 = *reinterpret_cast<const float4v*>(norm_w + k + 4);
+  }
+  return f;
+}
+
+template <bool NORM>
+__device__ __forceinline__ bf16x8 finish_x(const XFrag<NORM>& f, float rs) {
+  if constexpr (!NORM) {
+    return f.v;
+  } else {
+    bf16x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float normed = (float)(bf16_t)((float)f.v[i] * rs);
+      v[i] = (bf16_t)((i < 4 ? f.w0[i] : f.w1[i - 4]) * normed);
+    }
+    return v;
+  }
+}
+
+// KS waves split k, NS groups of waves split the workgroup's tiles, each wave owns NT tiles:
+// a workgroup computes NS*NT tiles of 16 features with KS*NS waves. The activation fragments are
+// loaded once per block of k and reused for the wave's NT tiles.
+template <int KS, int NS, int NT, int MT, int EPI, bool NORM>
+__global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
+    const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
+    const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
+    const bf16_t* __restrict__ bias, void* __restrict__ out, int64_t ldo,
+    bf16_t* __restrict__ stream, int64_t lds_, float* __restrict__ ssq_out, int M, int N, int K,
+    int up_offset) {
+  constexpr int NA = EPI == EPI_SWIGLU ? 2 : 1;  // weight row sets per tile (gate and up)
+  constexpr int KR = KS > 1 ? KS - 1 : 1;
+  __shared__ float red[KR][NS][NT][NA][MT][4][64];  // k-split waves 1.. hand their tiles to wave 0
+
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int ks = wave % KS, ns = wave / KS;
+  const int col = lane % 16, grp = lane / 16;
+  const int tile0 = (blockIdx.x * NS + ns) * NT;  // first of this wave's tiles
+
+  // weight rows of this lane (clamped at the matrix's end: such rows are computed and dropped)
+  const bf16_t* wrow[NT][NA];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+      const int n = min((tile0 + j) * 16 + col, N - 1) + a * up_offset;
+      wrow[j][a] = w + (int64_t)n * K;
+    }
+
+  const bf16_t* xrow[MT];
+  bool live[MT];
+  float rs[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + col;
+    live[t] = m < M;
+    xrow[t] = x + (int64_t)min(m, M - 1) * ldx;
+    rs[t] = 1.f;
+  }
+  if constexpr (NORM) {
+    // rs[m] from the parts of sum x^2 that the producer of x left. Every wave computes the rows of
+    // its own lanes: lane group g adds the parts p = g, g+4, ... of row m = 16t + col, the four
+    // groups are added in a fixed order.
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = min(t * 16 + col, M - 1);
+      float sum = 0.f;
+#pragma unroll 8
+      for (int p = grp; p < ssq_parts; p += 4) sum += ssq_in[(int64_t)p * M + m];
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      rs[t] = rsqrtf(sum / (float)K + eps);
+    }
+  }
+
+  float4v acc[NT][NA][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[j][a][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // this wave's share of the k steps of 32
+  const int steps = K / 32;
+  const int s_begin = (int)((int64_t)steps * ks / KS), s_end = (int)((int64_t)steps * (ks + 1) / KS);
+  int s = s_begin;
+  // blocks of 128: lane group g reads k in [32g, 32g + 32). The weights of the next block are
+  // requested before the products of the current one, so two blocks are in flight per wave.
+  bf16x8 af[NT][NA][4];
+  XFrag<NORM> xf[MT][4];
+  if (s + 4 <= s_end) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          af[j][a][q] = *reinterpret_cast<const bf16x8*>(wrow[j][a] + s * 32 + grp * 32 + q * 8);
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xf[t][q] = fetch_x<NORM>(xrow[t], norm_w, s * 32 + grp * 32 + q * 8, live[t]);
+  }
+  for (; s + 4 <= s_end; s += 4) {
+    const int kb = s * 32 + grp * 32;
+    bf16x8 nf[NT][NA][4];
+    XFrag<NORM> nx[MT][4];
+    const bool more = s + 8 <= s_end;
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            nf[j][a][q] = *reinterpret_cast<const bf16x8*>(wrow[j][a] + kb + 128 + q * 8);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) nx[t][q] = fetch_x<NORM>(xrow[t], norm_w, kb + 128 + q * 8, live[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bf16x8 bf = finish_x<NORM>(xf[t][q], rs[t]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int a = 0; a < NA; ++a) acc[j][a][t] = mfma32(af[j][a][q], bf, acc[j][a][t]);
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) af[j][a][q] = nf[j][a][q];
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xf[t][q] = nx[t][q];
+    }
+  }
+  for (; s < s_end; ++s) {  // single steps: lane group g reads k in [8g, 8g + 8)
+    const int kb = s * 32 + grp * 8;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const bf16x8 bf = finish_x<NORM>(fetch_x<NORM>(xrow[t], norm_w, kb, live[t]), rs[t]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+          acc[j][a][t] = mfma32(*reinterpret_cast<const bf16x8*>(wrow[j][a] + kb), bf, acc[j][a][t]);
+    }
+  }
+
+  // k-split wave 0 of each group adds the other waves' partial tiles to its own, in wave order
+  if (KS > 1) {
+    if (ks != 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[ks - 1][ns][j][a][t][i][lane] = acc[j][a][t][i];
+    }
+    __syncthreads();
+    if (ks == 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float v = acc[j][a][t][i];
+              for (int wv = 0; wv < KS - 1; ++wv) v += red[wv][ns][j][a][t][i][lane];
+              acc[j][a][t][i] = v;
+            }
+    }
+  }
+
+  // lane holds y[m = 16t + col][n = 16*tile + 4*grp + i]
+  if (ks == 0) {
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int tile = tile0 + j;
+    const int nb = tile * 16 + 4 * grp;
+    if (tile * 16 >= N) continue;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + col;
+      float y[NA][4];
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          y[a][i] = acc[j][a][t][i];
+          if (bias != nullptr && nb + i < N) y[a][i] += (float)bias[nb + i + a * up_offset];
+        }
+      float sq = 0.f;
+      if (m < M) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = nb + i;
+          if (n >= N) continue;
+          if (EPI == EPI_STORE) {
+            reinterpret_cast<bf16_t*>(out)[(int64_t)m * ldo + n] = (bf16_t)y[0][i];
+          } else if (EPI == EPI_F32) {
+            reinterpret_cast<float*>(out)[(int64_t)m * ldo + n] = y[0][i];
+          } else if (EPI == EPI_SWIGLU) {
+            const float g = (float)(bf16_t)y[0][i], u = (float)(bf16_t)y[NA - 1][i];
+            const float sg = (float)(bf16_t)(g / (1.f + expf(-g)));
+            reinterpret_cast<bf16_t*>(out)[(int64_t)m * ldo + n] = (bf16_t)(sg * u);
+          } else {  // EPI_RESIDUAL
+            bf16_t* sp = stream + (int64_t)m * lds_ + n;
+            const bf16_t summed = (bf16_t)((float)*sp + (float)(bf16_t)y[0][i]);
+            *sp = summed;
+            sq += (float)summed * (float)summed;
+          }
+        }
+      }
+      if (EPI == EPI_RESIDUAL) {
+        sq += __shfl_xor(sq, 16, 64);
+        sq += __shfl_xor(sq, 32, 64);
+        if (grp == 0 && m < M) ssq_out[(int64_t)tile * M + m] = sq;
+      }
+    }
+  }
+  }
+}
+
+// Embedding rows with the sum of squares of each (one part), for the first layer's norm.
+__global__ void embedding_ssq_kernel(const bf16_t* __restrict__ table, const int* __restrict__ ids,
+                                     bf16_t* __restrict__ out, float* __restrict__ ssq, int width) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const bf16_t* src = table + (int64_t)ids[row] * width;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const bf16_t v = src[i];
+    out[row * width + i] = v;
+    s += (float)v * (float)v;
+  }
+  const float total = block_sum(s, scratch);
+  if (threadIdx.x == 0) ssq[row] = total;
+}
+
+#define SK_PARAMS                                                                                 \
+  const void *x, int64_t ldx, const float *ssq_in, int ssq_parts, const float *norm_w, float eps,   \
+      const void *w, const void *bias, void *out, int64_t ldo, void *stream_buf, int64_t lds_,      \
+      float *ssq_out, int M, int N, int K, int up_offset, hipStream_t stream
+#define SK_ARGS \
+  x, ldx, ssq_in, ssq_parts, norm_w, eps, w, bias, out, ldo, stream_buf, lds_, ssq_out, M, N, K, up_offset, stream
+
+template <int KS, int NS, int NT, int MT, int EPI, bool NORM>
+static void launch_skinny(SK_PARAMS) {
+  const int tiles = (N + 15) / 16;
+  const int groups = (tiles + NS * NT - 1) / (NS * NT);
+  skinny_gemm_kernel<KS, NS, NT, MT, EPI, NORM><<<groups, KS * NS * 64, 0, stream>>>(
+      (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
+      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
+}
+
+// shapes of the workgroup: 0: 4 k-waves x 1 tile (few tiles, short k); 1: 8 k-waves x 1 tile (few
+// tiles, long k); 2: 4 n-waves x 2 tiles, no k split (many tiles: the activations are read once
+// per 8 tiles); 3: 2 k-waves x 2 n-waves x 2 tiles
+template <int MT, int EPI, bool NORM>
+static void dispatch_shape(int shape, SK_PARAMS) {
+  switch (shape) {
+    case 0: launch_skinny<4, 1, 1, MT, EPI, NORM>(SK_ARGS); break;
+    case 1: launch_skinny<8, 1, 1, MT, EPI, NORM>(SK_ARGS); break;
+    case 2: launch_skinny<1, 4, 2, MT, EPI, NORM>(SK_ARGS); break;
+    default: launch_skinny<2, 2, 2, MT, EPI, NORM>(SK_ARGS); break;
+  }
+}
+
+template <int EPI, bool NORM>
+static int dispatch_skinny(int shape, int mt, SK_PARAMS) {
+  if (mt == 1) dispatch_shape<1, EPI, NORM>(shape, SK_ARGS);
+  else if (mt == 2) dispatch_shape<2, EPI, NORM>(shape, SK_ARGS);
+  else dispatch_shape<4, EPI, NORM>(shape, SK_ARGS);
+  return dli_launch_status();
+}
+
+extern "C" int dli_skinny_gemm_max_rows() { return 64; }
+
+// epilogue: 0 store bf16, 1 swiglu (N = features of one half, up rows at +up_offset), 2 residual,
+// 3 store float32. norm_w == nullptr: no norm. shape: the workgroup shape, see dispatch_shape.
+extern "C" int dli_skinny_gemm(const void* x, int64_t ldx, const float* ssq_in, int ssq_parts,
+                               const float* norm_w, float eps, const void* w, const void* bias,
+                               void* out, int64_t ldo, void* stream_buf, int64_t lds_,
+                               float* ssq_out, int M, int N, int K, int up_offset, int epilogue,
+                               int shape, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return DLI_OK;
+  if (M > 64 || K <= 0 || K % 32 != 0 || ldx % 8 != 0 || shape < 0 || shape > 3 || epilogue < 0 ||
+      epilogue > 3 || (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)) ||
+      (epilogue == EPI_RESIDUAL && (stream_buf == nullptr || ssq_out == nullptr || norm_w != nullptr)) ||
+      (epilogue != EPI_RESIDUAL && out == nullptr))
+    return DLI_ERR_ARGUMENT;
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const bool norm = norm_w != nullptr;
+  switch (epilogue) {
+    case EPI_STORE:
+      return norm ? dispatch_skinny<EPI_STORE, true>(shape, mt, SK_ARGS) : dispatch_skinny<EPI_STORE, false>(shape, mt, SK_ARGS);
+    case EPI_SWIGLU:
+      return norm ? dispatch_skinny<EPI_SWIGLU, true>(shape, mt, SK_ARGS) : dispatch_skinny<EPI_SWIGLU, false>(shape, mt, SK_ARGS);
+    case EPI_RESIDUAL:
+      return dispatch_skinny<EPI_RESIDUAL, false>(shape, mt, SK_ARGS);
+    default:
+      return norm ? dispatch_skinny<EPI_F32, true>(shape, mt, SK_ARGS) : dispatch_skinny<EPI_F32, false>(shape, mt, SK_ARGS);
+  }
+}
+
+extern "C" int dli_embedding_ssq(const void* table, const int* ids, void* out, float* ssq, int rows,
+                                 int width, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0) return DLI_ERR_ARGUMENT;
+  embedding_ssq_kernel<<<rows, 256, 0, stream>>>((const bf16_t*)table, ids, (bf16_t*)out, ssq, width);
+  return dli_launch_status();
+}

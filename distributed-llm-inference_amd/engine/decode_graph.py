@@ -113,6 +113,7 @@ class DecodeGraphs:
             q_start_host=np.arange(b + 1, dtype=np.int32), kv_len_host=np.zeros(b, np.int32),
             state_slots_host=np.zeros(b, np.int32), seq_ids=[None] * b)
         ctx.forced_splits = splits
+        ctx.all_rows_wanted = True  # logit_rows is the identity here
         model, caches = self.step_fn.model, self.step_fn.caches
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())

@@ -40,6 +40,10 @@ _SIGNATURES = {
     "dli_gemm_f32_nt": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int,
                         _c_int, _c_int, _c_ptr],
     "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "dli_skinny_gemm_max_rows": [],
+    "dli_skinny_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
+                        _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
     "dli_attention_prefill_tile_rows": [],
@@ -271,6 +275,92 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional
     _check(library().dli_gemm_f32_nt(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(bias), _ptr(residual),
                                      ldr, _ptr(out), out.stride(0), m, n, k, _stream()), "gemm_f32")
 
+
+SKINNY_STORE, SKINNY_SWIGLU, SKINNY_RESIDUAL, SKINNY_F32 = 0, 1, 2, 3
+
+
+def skinny_gemm_supports(rows: int, k: int, dtype: torch.dtype) -> bool:
+    """Whether the decode product kernel takes ``rows`` activation rows of width ``k``."""
+    return dtype == torch.bfloat16 and 0 < rows <= 64 and k > 0 and k % 32 == 0
+
+
+def skinny_gemm_shape(n: int, k: int) -> int:
+    """Workgroup shape for ``n`` output features of depth ``k``: with few tiles of 16 features the
+    waves of a workgroup split k (8 ways when k is long), with many they split the tiles so that
+    the activations are read once per 8 tiles."""
+    tiles = -(-n // 16)
+    if tiles >= 2048:
+        return 2
+    if tiles >= 768:
+        return 3
+    return 1 if k >= 4096 else 0
+
+
+def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optional[torch.Tensor] = None,
+                bias: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
+                ssq_in: Optional[torch.Tensor] = None, stream: Optional[torch.Tensor] = None,
+                ssq_out: Optional[torch.Tensor] = None, shape: Optional[int] = None) -> None:
+    """``y = xhat @ w.T`` for at most 64 rows of bfloat16 ``x``, with fused surroundings.
+
+    ``norm_w``/``eps``/``ssq_in [parts, rows]``: xhat is the RMSNorm of x, the row sums of squares
+    being given in parts. Epilogues: ``SKINNY_STORE`` (``out`` bfloat16 ``[rows, n]``),
+    ``SKINNY_SWIGLU`` (``w`` is ``[2n, k]``: gate rows then up rows; ``out [rows, n]`` gets
+    ``silu(gate) * up``), ``SKINNY_RESIDUAL`` (``stream [rows, n]`` becomes ``stream + y`` in place
+    and ``ssq_out [ceil(n/16), rows]`` receives the parts of its row sums of squares),
+    ``SKINNY_F32`` (``out`` float32).
+    """
+    _rows(x, "x", torch.bfloat16)
+    _dense(w, "w", torch.bfloat16, 2)
+    m, k = x.shape
+    _require(w.shape[1] == k, "x and w differ in inner size")
+    _require(skinny_gemm_supports(m, k, x.dtype), f"the decode product takes 1..64 rows and k % 32 == 0, not {m} x {k}")
+    _require(x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+    n = w.shape[0] // 2 if epilogue == SKINNY_SWIGLU else w.shape[0]
+    up_offset = n if epilogue == SKINNY_SWIGLU else 0
+    if epilogue == SKINNY_SWIGLU:
+        _require(w.shape[0] == 2 * n, "swiglu needs gate rows and up rows")
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == w.shape[0], "bias length differs from rows of w")
+    parts = 0
+    if norm_w is not None:
+        _require(epilogue != SKINNY_RESIDUAL, "the residual epilogue takes no fused norm")
+        _dense(norm_w, "norm_w", torch.float32, 1)
+        _require(norm_w.shape[0] == k and norm_w.data_ptr() % 16 == 0, "norm weight must have k aligned values")
+        _require(ssq_in is not None, "a fused norm needs the sums of squares")
+        _dense(ssq_in, "ssq_in", torch.float32, 2)
+        _require(ssq_in.shape[1] == m and ssq_in.shape[0] >= 1, "ssq_in must be [parts, rows]")
+        parts = ssq_in.shape[0]
+    ldo = lds = 0
+    if epilogue == SKINNY_RESIDUAL:
+        _require(stream is not None and ssq_out is not None, "the residual epilogue needs stream and ssq_out")
+        _rows(stream, "stream", torch.bfloat16)
+        _dense(ssq_out, "ssq_out", torch.float32, 2)
+        _require(stream.shape == (m, n) and ssq_out.shape == (-(-n // 16), m), "stream [rows, n], ssq_out [ceil(n/16), rows]")
+        lds = stream.stride(0)
+    else:
+        _require(out is not None, "this epilogue needs out")
+        _rows(out, "out", torch.float32 if epilogue == SKINNY_F32 else torch.bfloat16)
+        _require(out.shape == (m, n), "out must be [rows, n]")
+        ldo = out.stride(0)
+    if shape is None:
+        shape = skinny_gemm_shape(n, k)
+    _require(shape in (0, 1, 2, 3), "shape must be 0..3")
+    _check(library().dli_skinny_gemm(
+        _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
+        _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, shape, _stream()), "skinny_gemm")
+
+
+def embedding_ssq(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, ssq: torch.Tensor) -> None:
+    """``out[t] = table[ids[t]]`` and ``ssq[0, t] = sum(out[t]^2)`` (bfloat16 table)."""
+    _dense(table, "table", torch.bfloat16, 2)
+    _dense(ids, "ids", torch.int32, 1)
+    _dense(out, "out", torch.bfloat16, 2)
+    _dense(ssq, "ssq", torch.float32, 2)
+    _require(out.shape == (ids.shape[0], table.shape[1]) and ssq.shape == (1, ids.shape[0]),
+             "out [len(ids), width], ssq [1, len(ids)]")
+    _check(library().dli_embedding_ssq(_ptr(table), _ptr(ids), _ptr(out), _ptr(ssq), ids.shape[0], table.shape[1],
+                                       _stream()), "embedding_ssq")
 
 # ----------------------------------------------------------------------------- attention
 

@@ -21,7 +21,7 @@ import torch
 
 from ..kernels import ops
 from .attention_kernels import paged_attention
-from .base import Mixer, PagedKVSpec, Part, Runtime
+from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
 from .linear import linear
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
@@ -97,3 +97,39 @@ class GQAttention(Mixer):
         out = self.rt.empty(x.shape[0], nh * d)
         paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         return linear(self.rt, out, self.w_o, self.b_o)
+
+    # -- decode steps with few rows: the norm before and the residual sum after are fused into
+    #    the two projections' kernels
+    def streams(self, ctx: Any) -> bool:
+        nh, d = self.num_heads, self.head_dim
+        return (self.rt.is_bf16 and ctx.num_decode == ctx.num_entries and self.hidden_size % 8 == 0
+                and ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype)
+                and ops.skinny_gemm_supports(ctx.num_tokens, nh * d, self.rt.dtype)
+                and ops.attention_mfma_supports(d, ctx.page_size, self.rt.dtype))
+
+    def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any, cache: Any) -> None:
+        """``stream.x += attention(norm(stream.x))``, the norm inside the first product's kernel and
+        the sum inside the last one's."""
+        nh, d = self.num_heads, self.head_dim
+        nkv = 0 if self.shares_kv else self.num_kv_heads
+        grp = ctx.groups[cache.group]
+        n = stream.x.shape[0]
+        norm_w, eps = norm.fused_params()
+        qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
+        ops.skinny_gemm(stream.x, self.w_qkv, epilogue=ops.SKINNY_STORE, out=qkv, bias=self.b_qkv,
+                        norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        table = self.position.rotary_table()
+        if table is None:
+            q_view = qkv[:, :nh * d].view(n, nh, d)
+            k_view = qkv[:, nh * d:(nh + nkv) * d].view(n, nkv, d) if nkv else None
+            self.position.apply(q_view, k_view, ctx.positions)
+            inv_freq, rotary_dim = None, 0
+        else:
+            inv_freq, rotary_dim = table
+        ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
+                          cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
+        out = self.rt.empty(n, nh * d)
+        paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        ssq = torch.empty(-(-self.hidden_size // 16), n, device=self.rt.device, dtype=torch.float32)
+        ops.skinny_gemm(out, self.w_o, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, ssq_out=ssq, bias=self.b_o)
+        stream.ssq = ssq

@@ -60,6 +60,17 @@ class StateSpec:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass
+class DecodeStream:
+    """The residual stream of a step with few rows, in the form the fused decode kernels pass on:
+    ``x [rows, hidden]`` already holds every residual sum, and ``ssq [parts, rows]`` holds each
+    row's sum of squares in parts, as the kernel that last wrote ``x`` left them (the next
+    RMSNorm is computed from them inside the product kernel that consumes ``x``)."""
+
+    x: torch.Tensor
+    ssq: torch.Tensor
+
+
 class Part:
     family: str = ""
     kind: str = ""
@@ -81,6 +92,12 @@ class Part:
 
     def finalize(self) -> None:
         """Called once after the weights are loaded: build device tables, fuse tensors."""
+
+    def streams(self, ctx: Any) -> bool:
+        """Whether this part can run ``ctx``'s step on a :class:`DecodeStream` (its
+        ``forward_stream``). Parts that do not implement the fused form return False, and the
+        model then runs the step through the plain ``forward`` methods."""
+        return False
 
 
 class Embedding(Part):

@@ -8,7 +8,7 @@ from typing import Any, Mapping, Optional
 
 import torch
 
-from .base import Block, Part, Runtime
+from .base import Block, DecodeStream, Part, Runtime
 from .registry import register_part
 
 
@@ -26,3 +26,11 @@ class PreNormBlock(Block):
         h = parts["feed_forward_norm"].forward(x, a)       # x <- x + a
         f = parts["feed_forward"].forward(h, ctx)
         return x, f
+
+    def streams(self, ctx: Any, parts: Mapping[str, Part]) -> bool:
+        fused_norms = all(hasattr(parts[r], "fused_params") for r in ("mixer_norm", "feed_forward_norm"))
+        return fused_norms and parts["mixer"].streams(ctx) and parts["feed_forward"].streams(ctx)
+
+    def forward_stream(self, stream: DecodeStream, ctx: Any, cache: Any, parts: Mapping[str, Part]) -> None:
+        parts["mixer"].forward_stream(stream, parts["mixer_norm"], ctx, cache)
+        parts["feed_forward"].forward_stream(stream, parts["feed_forward_norm"], ctx)

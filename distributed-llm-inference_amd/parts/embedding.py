@@ -7,7 +7,7 @@ from typing import Mapping
 import torch
 
 from ..kernels import ops
-from .base import Embedding, Runtime
+from .base import DecodeStream, Embedding, Runtime
 from .registry import register_part
 from .spec import WeightSpec
 
@@ -33,3 +33,13 @@ class TokenEmbedding(Embedding):
         out = self.rt.empty(ids.shape[0], self.hidden_size)
         ops.embedding(self.table(), ids, out)
         return out
+
+    def streams(self, ctx) -> bool:
+        return self.rt.is_bf16
+
+    def forward_stream(self, ids: torch.Tensor) -> DecodeStream:
+        n = ids.shape[0]
+        out = self.rt.empty(n, self.hidden_size)
+        ssq = torch.empty(1, n, device=self.rt.device, dtype=torch.float32)
+        ops.embedding_ssq(self.table(), ids, out, ssq)
+        return DecodeStream(out, ssq)

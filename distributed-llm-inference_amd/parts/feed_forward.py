@@ -9,7 +9,7 @@ from typing import Any, Mapping
 import torch
 
 from ..kernels import ops
-from .base import FeedForward, Runtime
+from .base import DecodeStream, FeedForward, Norm, Runtime
 from .linear import linear
 from .registry import register_part
 from .spec import WeightSpec
@@ -46,3 +46,20 @@ class GatedMLP(FeedForward):
         act = self.rt.empty(x.shape[0], self.intermediate_size)
         ops.silu_mul(gate_up, act)
         return linear(self.rt, act, self.w_down, self.b_down)
+
+    def streams(self, ctx: Any) -> bool:
+        n = ctx.num_tokens
+        return (self.rt.is_bf16 and self.hidden_size % 8 == 0
+                and ops.skinny_gemm_supports(n, self.hidden_size, self.rt.dtype)
+                and ops.skinny_gemm_supports(n, self.intermediate_size, self.rt.dtype))
+
+    def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any) -> None:
+        """``stream.x += mlp(norm(stream.x))``, norm and sum inside the two products' kernels."""
+        n = stream.x.shape[0]
+        norm_w, eps = norm.fused_params()
+        act = self.rt.empty(n, self.intermediate_size)
+        ops.skinny_gemm(stream.x, self.w_gate_up, epilogue=ops.SKINNY_SWIGLU, out=act, bias=self.b_gate_up,
+                        norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        ssq = torch.empty(-(-self.hidden_size // 16), n, device=self.rt.device, dtype=torch.float32)
+        ops.skinny_gemm(act, self.w_down, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, ssq_out=ssq, bias=self.b_down)
+        stream.ssq = ssq

@@ -8,7 +8,7 @@ from typing import Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .base import Head, Runtime
+from .base import DecodeStream, Head, Norm, Runtime
 from .linear import linear
 from .registry import register_part
 from .spec import WeightSpec
@@ -38,4 +38,15 @@ class LinearHead(Head):
             return logits
         out = torch.empty(logits.shape, device=logits.device, dtype=torch.float32)
         ops.to_float(logits, out)
+        return out
+
+    def streams(self, ctx) -> bool:
+        return self.rt.is_bf16 and ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype)
+
+    def forward_stream(self, stream: DecodeStream, norm: Norm) -> torch.Tensor:
+        """Logits of every row of the stream, the final norm computed inside the product."""
+        norm_w, eps = norm.fused_params()
+        out = torch.empty(stream.x.shape[0], self.vocab_size, device=self.rt.device, dtype=torch.float32)
+        ops.skinny_gemm(stream.x, self.weight, epilogue=ops.SKINNY_F32, out=out, norm_w=norm_w, eps=eps,
+                        ssq_in=stream.ssq)
         return out

@@ -111,8 +111,33 @@ class Model:
 
     # ------------------------------------------------------------------ step
 
+    STREAM_ROWS = 16  # steps with at most this many rows, all decoding, take the fused kernels
+
+    def _streams(self, ctx: Any) -> bool:
+        if not 0 < ctx.num_tokens <= self.STREAM_ROWS or ctx.num_decode != ctx.num_entries:
+            return False
+        if not (self.embedding.streams(ctx) and self.head.streams(ctx) and hasattr(self.final_norm, "fused_params")):
+            return False
+        return all(hasattr(l.block, "forward_stream") and l.block.streams(ctx, l.parts) for l in self.layers)
+
+    def _forward_stream(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
+        stream = self.embedding.forward_stream(ctx.token_ids)
+        for entry, cache in zip(self.spec.schedule, caches):
+            layer = self.layers[entry.layer]
+            layer.block.forward_stream(stream, ctx, cache, layer.parts)
+        logits = self.head.forward_stream(stream, self.final_norm)
+        k = ctx.logit_rows.shape[0]
+        if getattr(ctx, "all_rows_wanted", False):
+            return logits
+        out = torch.empty(k, logits.shape[1], device=logits.device, dtype=torch.float32)
+        if k:
+            ops.gather_rows(logits, ctx.logit_rows, out)
+        return out
+
     def forward(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
         """Run the step's tokens through the schedule; float32 logits ``[wanted rows, vocab]``."""
+        if self._streams(ctx):
+            return self._forward_stream(ctx, caches)
         x = self.embedding.forward(ctx.token_ids)
         delta: Optional[torch.Tensor] = None
         for entry, cache in zip(self.spec.schedule, caches):

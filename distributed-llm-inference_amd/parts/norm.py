@@ -26,6 +26,10 @@ class RMSNorm(Norm):
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors["weight"]
 
+    def fused_params(self) -> tuple[torch.Tensor, float]:
+        """Weight and eps, for a consumer that computes this norm inside its own kernel."""
+        return self.weight, self.eps
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         out = torch.empty_like(x)
         if delta is None:

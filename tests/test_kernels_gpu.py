@@ -262,3 +262,73 @@ def test_attention_finds_one_far_key_among_hundreds(ops):
             for h in range(qh):
                 want = vp[page, h // (qh // kvh), :, off].float()
                 assert (got[h] - want).abs().max() < 0.05, (e, row, h)
+
+
+def _ref_norm_bf16(x, w, eps):
+    """RMSNorm with the engine's rounding: cast(w * cast(x * r))."""
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (w * (xf * r).bfloat16().float()).bfloat16()
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("n,k,shape", [(48, 64, 0), (100, 192, 2), (301, 160, 1), (512, 2048, 1), (64, 416, 3),
+                                       (1000, 96, 2), (2048, 8192, 1)])
+def test_skinny_gemm_epilogues(ops, m, n, k, shape):
+    torch.manual_seed(m * 1000 + n)
+    x = torch.randn(m, k, device="cuda").bfloat16()
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    bias = torch.randn(n, device="cuda").bfloat16()
+    ref = x.cpu().double() @ w.cpu().double().T + bias.cpu().double()
+    out = torch.full((m, n), 7.0, device="cuda", dtype=torch.bfloat16)
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_STORE, out=out, bias=bias, shape=shape)
+    assert (out.cpu().double() - ref).abs().max() < 3e-2
+    out32 = torch.empty(m, n, device="cuda")
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_F32, out=out32, shape=shape)
+    assert (out32.cpu().double() - (ref - bias.cpu().double())).abs().max() < 1e-4 * math.sqrt(k)
+    # a row's result does not depend on the other rows
+    one = torch.empty(1, n, device="cuda")
+    ops.skinny_gemm(x[m - 1:m].contiguous(), w, epilogue=ops.SKINNY_F32, out=one, shape=shape)
+    assert torch.equal(one[0], out32[m - 1])
+    # residual: stream += y, with the parts of its row sums of squares
+    stream = torch.randn(m, n, device="cuda").bfloat16()
+    before = stream.clone()
+    ssq = torch.full((-(-n // 16), m), float("nan"), device="cuda")
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_RESIDUAL, stream=stream, ssq_out=ssq, bias=bias, shape=shape)
+    want = (before.float() + out.float()).bfloat16()
+    assert torch.equal(stream, want)
+    assert torch.allclose(ssq.sum(0), stream.float().pow(2).sum(-1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("m", [1, 8, 33])
+@pytest.mark.parametrize("shape", [0, 2, 3])
+@pytest.mark.parametrize("inter,k,parts", [(160, 64, 1), (512, 192, 5), (8192, 2048, 128)])
+def test_skinny_gemm_norm_and_swiglu(ops, m, inter, k, shape, parts):
+    torch.manual_seed(m + inter)
+    x = (torch.randn(m, k, device="cuda") * 2).bfloat16()
+    nw = (1 + 0.1 * torch.randn(k, device="cuda")).float()
+    w = (torch.randn(2 * inter, k, device="cuda") / math.sqrt(k)).bfloat16()
+    xs = x.float().pow(2)
+    cut = torch.linspace(0, k, parts + 1).long().tolist()
+    ssq = torch.stack([xs[:, a:b].sum(-1) for a, b in zip(cut[:-1], cut[1:])]).contiguous()
+    eps = 1e-5
+    xhat = _ref_norm_bf16(x, nw, eps)
+    gu = (xhat.cpu().double() @ w.cpu().double().T)
+    g, u = gu[:, :inter].bfloat16().double(), gu[:, inter:].bfloat16().double()
+    ref = (g * torch.sigmoid(g)).bfloat16().double() * u
+    out = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_SWIGLU, out=out, norm_w=nw, eps=eps, ssq_in=ssq, shape=shape)
+    assert (out.cpu().double() - ref).abs().max() < 2e-2 * max(1.0, ref.abs().max().item())
+    y = torch.empty(m, 2 * inter, device="cuda", dtype=torch.bfloat16)
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_STORE, out=y, norm_w=nw, eps=eps, ssq_in=ssq, shape=shape)
+    assert (y.cpu().double() - gu).abs().max() < 3e-2 * max(1.0, gu.abs().max().item())
+
+
+def test_embedding_with_sum_of_squares(ops):
+    table = torch.randn(50, 96, device="cuda").bfloat16()
+    ids = torch.tensor([4, 49, 0, 4], dtype=torch.int32, device="cuda")
+    out = torch.empty(4, 96, device="cuda", dtype=torch.bfloat16)
+    ssq = torch.empty(1, 4, device="cuda")
+    ops.embedding_ssq(table, ids, out, ssq)
+    assert torch.equal(out, table[ids.long()])
+    assert torch.allclose(ssq[0], out.float().pow(2).sum(-1), rtol=1e-5)
