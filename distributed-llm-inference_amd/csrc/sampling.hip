@@ -63,11 +63,43 @@ __device__ int block_sum_i(int v, int* scratch) {
   return total;
 }
 
+// Stage one of the argmax: each workgroup scans one chunk of one row and leaves its best
+// (value, lowest index). grid (chunks, rows).
+#define ARGMAX_CHUNKS 64
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits,
+                                                             int64_t row_stride, int vocab,
+                                                             float* __restrict__ part_val,
+                                                             int* __restrict__ part_idx) {
+  __shared__ ArgBest best[4];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int per = (vocab + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+  const int lo = chunk * per, hi = min(vocab, lo + per);
+  const float* x = logits + (int64_t)row * row_stride;
+  ArgBest mine = {-INFINITY, 0x7fffffff};
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) mine = better(mine, ArgBest{x[i], i});
+#pragma unroll
+  for (int m = DLI_WAVE / 2; m > 0; m >>= 1) {
+    ArgBest o;
+    o.v = __shfl_xor(mine.v, m, DLI_WAVE);
+    o.i = __shfl_xor(mine.i, m, DLI_WAVE);
+    mine = better(mine, o);
+  }
+  if (threadIdx.x % DLI_WAVE == 0) best[threadIdx.x / DLI_WAVE] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    ArgBest top = best[0];
+    for (int w = 1; w < (int)(blockDim.x / DLI_WAVE); ++w) top = better(top, best[w]);
+    part_val[row * ARGMAX_CHUNKS + chunk] = top.v;
+    part_idx[row * ARGMAX_CHUNKS + chunk] = top.i;
+  }
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int64_t row_stride, int vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint64_t* __restrict__ seeds,
-    const uint64_t* __restrict__ counters, int* __restrict__ out) {
+    const uint64_t* __restrict__ counters, const float* __restrict__ part_val,
+    const int* __restrict__ part_idx, int* __restrict__ out) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
   __shared__ ArgBest best[16];
@@ -80,9 +112,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int k = top_k[row];
   const bool greedy = temp == 0.f || k == 1;
 
-  // maximum (and its lowest index)
+  // maximum (and its lowest index), from the chunks' results of stage one
   ArgBest mine = {-INFINITY, 0x7fffffff};
-  for (int i = tid; i < vocab; i += blockDim.x) mine = better(mine, ArgBest{x[i], i});
+  if (tid < ARGMAX_CHUNKS)
+    mine = ArgBest{part_val[row * ARGMAX_CHUNKS + tid], part_idx[row * ARGMAX_CHUNKS + tid]};
 #pragma unroll
   for (int m = DLI_WAVE / 2; m > 0; m >>= 1) {
     ArgBest o;
@@ -186,13 +219,20 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (chosen < 0 && tid == 0) out[row] = top.i;  // no mass at all (cannot happen: the maximum is kept)
 }
 
+// Floats and ints of scratch that dli_sample needs per row.
+extern "C" int dli_sample_scratch_per_row() { return ARGMAX_CHUNKS; }
+
 extern "C" int dli_sample(const float* logits, int64_t row_stride, int rows, int vocab,
                           const float* temperature, const int* top_k, const float* top_p,
-                          const uint64_t* seeds, const uint64_t* counters, int* out,
-                          hipStream_t stream) {
+                          const uint64_t* seeds, const uint64_t* counters, float* part_val,
+                          int* part_idx, int* out, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
-  if (vocab <= 0 || row_stride < vocab) return DLI_ERR_ARGUMENT;
+  if (vocab <= 0 || row_stride < vocab || rows > 65535 || part_val == nullptr || part_idx == nullptr)
+    return DLI_ERR_ARGUMENT;
+  argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, rows), 256, 0, stream>>>(logits, row_stride, vocab,
+                                                                       part_val, part_idx);
+  if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab, temperature, top_k,
-                                                     top_p, seeds, counters, out);
+                                                     top_p, seeds, counters, part_val, part_idx, out);
   return dli_launch_status();
 }

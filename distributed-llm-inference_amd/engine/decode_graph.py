@@ -46,6 +46,7 @@ class _Captured:
     views: dict             # name -> numpy view into host
     width: int              # block-table entries per row
     rows: list              # per row: (request, pages already written into its table row)
+    tokens_host: Optional[torch.Tensor] = None  # pinned int32 [b]: sampled tokens (sampling graphs)
 
 
 class DecodeGraphs:
@@ -55,7 +56,7 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self.max_width = max(1, max_blocks_per_seq)
         self.n_groups = step_fn.manager.num_groups
-        self.captured: dict[tuple[int, int, int], _Captured] = {}
+        self.captured: dict[tuple[int, int, int, bool], _Captured] = {}
         self.replays = 0
         self.enabled = self._supported()
 
@@ -82,6 +83,7 @@ class DecodeGraphs:
     def _layout(self, b: int, width: int) -> tuple[dict, int]:
         fields = [("token_ids", b), ("positions", b), ("q_start", b + 1), ("kv_len", b), ("state_slots", b),
                   ("logit_rows", b)]
+        fields += [("temperature", b), ("top_p", b), ("top_k", b), ("seeds", 2 * b), ("counters", 2 * b)]
         for g in range(self.n_groups):
             fields += [(f"slots{g}", b), (f"tables{g}", b * width)]
         offsets, at = {}, 0
@@ -90,7 +92,7 @@ class DecodeGraphs:
             at += -(-n // 4) * 4  # 16-byte aligned starts
         return offsets, at
 
-    def _capture(self, b: int, splits: int, width: int) -> _Captured:
+    def _capture(self, b: int, splits: int, width: int, sampled: bool) -> _Captured:
         dev_name = self.rt.device
         offsets, total = self._layout(b, width)
         host = torch.zeros(total, dtype=torch.int32).pin_memory()
@@ -122,26 +124,52 @@ class DecodeGraphs:
                 model.forward(ctx, caches)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        views["temperature"].view(np.float32)[:] = 0.0  # padding rows are greedy
+        views["top_p"].view(np.float32)[:] = 1.0
+        views["top_k"][:] = -1
+        tokens_host = tokens_dev = scratch = None
+        if sampled:
+            tokens_host = torch.zeros(b, dtype=torch.int32).pin_memory()
+            tokens_dev = torch.zeros(b, dtype=torch.int32, device=dev_name)
+            scratch = ops.sample_scratch(b, dev_name)
+
+        def body():
+            logits = model.forward(ctx, caches)
+            if sampled:
+                ops.sample(logits, dv["temperature"].view(torch.float32), dv["top_k"],
+                           dv["top_p"].view(torch.float32), dv["seeds"].view(torch.int64),
+                           dv["counters"].view(torch.int64), tokens_dev, scratch)
+                tokens_host.copy_(tokens_dev, non_blocking=True)
+            return logits
+
+        dev.copy_(host)
+        with torch.cuda.stream(side):
+            body()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            logits = model.forward(ctx, caches)
-        return _Captured(graph, ctx, host, dev, logits, views, width, [None] * b)
+            logits = body()
+        return _Captured(graph, ctx, host, dev, logits, views, width, [None] * b, tokens_host)
 
     # ------------------------------------------------------------------ replay
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Logits ``[wanted, vocab]`` of a decode-only step (a view of the graph's output: use it
-        before the next step)."""
+    def run(self, entries: Sequence[StepEntry], sampling: Optional[Sequence[tuple]] = None):
+        """A decode-only step. Without ``sampling``: logits ``[wanted, vocab]`` (a view of the
+        graph's output: use it before the next step). With ``sampling``, one
+        ``(temperature, top_k, top_p, seed, draw index)`` per entry: the graph samples too and the
+        chosen token ids come back as a list."""
         mgr = self.step_fn.manager
         ps, n = mgr.page_size, len(entries)
         b = _bucket(n)
         max_kv = max(e.start + 1 for e in entries)
         width = max(16, _bucket(-(-max_kv // ps)))
         splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv))
-        key = (b, splits, width)
+        sampled = sampling is not None
+        key = (b, splits, width, sampled)
         cap = self.captured.get(key)
         if cap is None:
-            cap = self.captured[key] = self._capture(b, splits, width)
+            cap = self.captured[key] = self._capture(b, splits, width, sampled)
         v = cap.views
         limit = self.step_fn.store.num_pages
         token_ids, positions, kv_len, state_slots = v["token_ids"], v["positions"], v["kv_len"], v["state_slots"]
@@ -179,9 +207,18 @@ class DecodeGraphs:
             v[f"slots{g}"][n:] = -1
         for i in range(n, b):
             cap.rows[i] = None
+        if sampled:
+            temp, top_p = v["temperature"].view(np.float32), v["top_p"].view(np.float32)
+            seeds, counters = v["seeds"].view(np.int64), v["counters"].view(np.int64)
+            temp[n:] = 0.0
+            for i, (t, k, p, seed, draw) in enumerate(sampling):
+                temp[i], v["top_k"][i], top_p[i], seeds[i], counters[i] = t, k, p, seed, draw
         cap.dev.copy_(cap.host, non_blocking=True)
         cap.graph.replay()
         self.replays += 1
+        if sampled:
+            torch.cuda.current_stream().synchronize()
+            return cap.tokens_host[:n].tolist()
         if rows == list(range(n)):
             return cap.logits[:n]
         if not rows:

@@ -38,6 +38,18 @@ class ModelRunner:
         self.core = core
 
     def execute(self, sched: SchedulerOutput) -> Any:
+        return self.core.step.run(self._entries(sched), sched.copy_ops)
+
+    def execute_and_sample(self, sched: SchedulerOutput) -> list[int]:
+        """Run the step and choose a token for every chunk that needs one, on the GPU (inside
+        the replayed graph for decode steps); token ids in schedule order."""
+        from ..sampling.sampler import sampling_tuple
+
+        sampling = [sampling_tuple(c.request.params, c.request.seed, len(c.request.output_ids))
+                    for c in sched.chunks if c.needs_logits]
+        return self.core.step.run(self._entries(sched), sched.copy_ops, sampling=sampling)
+
+    def _entries(self, sched: SchedulerOutput) -> list:
         from .batch import StepEntry
 
         entries = []
@@ -51,7 +63,7 @@ class ModelRunner:
                 tokens = (req.prompt_ids[lo:] if lo < n_prompt else []) + req.output_ids[max(0, lo - n_prompt):hi - n_prompt]
             entries.append(StepEntry(req.request_id, tokens, ch.start,
                                      (ch.num_tokens - 1,) if ch.needs_logits else ()))
-        return self.core.step.run(entries, sched.copy_ops)
+        return entries
 
 
 @dataclass(frozen=True)
@@ -102,6 +114,7 @@ class LLMEngine:
         self._rng = random.Random(seed)
         self._arrivals = itertools.count()
         self._step_no = 0
+        self._sample_is_default = sampler is None
         if sampler is None:
             from ..sampling.sampler import sample as sampler  # the GPU sampler
         self._sample = sampler
@@ -169,14 +182,19 @@ class LLMEngine:
         t1 = time.perf_counter()
         outputs: list[RequestOutput] = []
         if sched.chunks:
-            logits = self.runner.execute(sched)
-            t2 = time.perf_counter()
             sampling = [c for c in sched.chunks if c.needs_logits]
+            fused = getattr(self.runner, "execute_and_sample", None) if self._sample_is_default else None
+            if fused is not None:
+                tokens = fused(sched)
+            else:
+                logits = self.runner.execute(sched)
+            t2 = time.perf_counter()
             for ch in sched.chunks:
                 ch.request.num_computed_tokens += ch.num_tokens
-            tokens = self._sample(
-                logits, [c.request.params for c in sampling], [c.request.seed for c in sampling],
-                [len(c.request.output_ids) for c in sampling])
+            if fused is None:
+                tokens = self._sample(
+                    logits, [c.request.params for c in sampling], [c.request.seed for c in sampling],
+                    [len(c.request.output_ids) for c in sampling])
             if len(tokens) != len(sampling):
                 raise RuntimeError("the sampler returned a wrong number of tokens")
             for ch, tok in zip(sampling, tokens):

@@ -143,9 +143,14 @@ class StepFunction:
 
     # ------------------------------------------------------------------ the step
 
-    def run(self, entries: Sequence[StepEntry], copy_ops: Sequence[CopyOp] = ()) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], copy_ops: Sequence[CopyOp] = (),
+            sampling: Optional[Sequence[tuple]] = None):
         """Run one step. Returns float32 logits ``[wanted places, vocab]`` on the device, in the
-        order of the entries and of each entry's ``want``."""
+        order of the entries and of each entry's ``want``.
+
+        With ``sampling`` (one ``(temperature, top_k, top_p, seed, draw index)`` for each wanted
+        place, temperature 0 meaning greedy) a token is chosen at every wanted place and the list
+        of token ids is returned instead."""
         self.store.copy_pages(copy_ops)  # before any write of this step (runner.py:56)
         if not entries:
             return torch.empty(0, self.vocab_size, device=self.rt.device, dtype=torch.float32)
@@ -160,11 +165,34 @@ class StepFunction:
                     raise StepError(f"request {e.seq_id!r}: wanted place outside its one token")
             if len({e.seq_id for e in entries}) != len(entries):
                 raise StepError("a request appears twice in one step")
-            logits = self.graphs.run(entries)
+            use_graph_sampler = sampling is not None and all(len(e.want) == 1 for e in entries)
+            logits = self.graphs.run(entries, sampling if use_graph_sampler else None)
+            if use_graph_sampler:
+                tokens, logits = logits, None
         else:
             ctx = self.build_context(entries)
             logits = self.model.forward(ctx, self.caches)
         for e in entries:
             self.manager.mark_computed(e.seq_id, e.start + len(e.tokens))
         self.steps_run += 1
-        return logits
+        if sampling is None:
+            return logits
+        if logits is None:
+            return tokens
+        return self._sample(logits, sampling)
+
+    def _sample(self, logits: torch.Tensor, sampling: Sequence[tuple]) -> list[int]:
+        from ..kernels import ops
+
+        rows = logits.shape[0]
+        if rows != len(sampling):
+            raise StepError("one sampling tuple is needed for each wanted place")
+        if rows == 0:
+            return []
+        dev = logits.device
+        floats = torch.tensor([[s[0] for s in sampling], [s[2] for s in sampling]], dtype=torch.float32).to(dev)
+        top_k = torch.tensor([s[1] for s in sampling], dtype=torch.int32).to(dev)
+        longs = torch.tensor([[s[3] for s in sampling], [s[4] for s in sampling]], dtype=torch.int64).to(dev)
+        out = torch.empty(rows, dtype=torch.int32, device=dev)
+        ops.sample(logits, floats[0], top_k, floats[1], longs[0], longs[1], out)
+        return out.cpu().tolist()

@@ -39,7 +39,9 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_f32_nt": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int,
                         _c_int, _c_int, _c_ptr],
-    "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                   _c_ptr],
+    "dli_sample_scratch_per_row": [],
     "dli_skinny_gemm_max_rows": [],
     "dli_skinny_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
                         _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -483,8 +485,17 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
 
 # ----------------------------------------------------------------------------- sampling
 
+def sample_scratch(rows: int, device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
+    """Scratch that :func:`sample` needs for ``rows`` rows (values and indices of the argmax's
+    first stage)."""
+    per = int(library().dli_sample_scratch_per_row())
+    return (torch.empty(rows * per, device=device, dtype=torch.float32),
+            torch.empty(rows * per, device=device, dtype=torch.int32))
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           seeds: torch.Tensor, counters: torch.Tensor, out: torch.Tensor) -> None:
+           seeds: torch.Tensor, counters: torch.Tensor, out: torch.Tensor,
+           scratch: Optional[tuple[torch.Tensor, torch.Tensor]] = None) -> None:
     """One token per row of float32 ``logits [rows, vocab]``.
 
     Rows with ``temperature == 0`` or ``top_k == 1`` take the argmax (lowest id on ties); the others
@@ -501,5 +512,12 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     for name, t in (("temperature", temperature), ("top_k", top_k), ("top_p", top_p), ("seeds", seeds),
                     ("counters", counters), ("out", out)):
         _require(t.shape[0] == rows, f"{name} must have one value per row")
+    if scratch is None:
+        scratch = sample_scratch(rows, logits.device)
+    per = int(library().dli_sample_scratch_per_row())
+    _dense(scratch[0], "scratch values", torch.float32)
+    _dense(scratch[1], "scratch indices", torch.int32)
+    _require(scratch[0].numel() >= rows * per and scratch[1].numel() >= rows * per, "sampling scratch is too small")
     _check(library().dli_sample(_ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k),
-                                _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(out), _stream()), "sample")
+                                _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(scratch[0]), _ptr(scratch[1]),
+                                _ptr(out), _stream()), "sample")

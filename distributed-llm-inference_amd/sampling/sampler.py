@@ -19,6 +19,15 @@ from .params import SamplingParams
 _MASK63 = (1 << 63) - 1
 
 
+def sampling_tuple(params: SamplingParams, seed: Optional[int], draw_index: int) -> tuple:
+    """``(temperature, top_k, top_p, seed, draw index)`` as the sampling kernel takes them;
+    temperature 0 stands for every greedy request."""
+    if not params.greedy and seed is None:
+        raise ValueError("a request that samples stochastically has no seed for its generator")
+    return (0.0 if params.greedy else float(params.temperature), int(params.top_k), float(params.top_p),
+            int(seed or 0) & _MASK63, int(draw_index))
+
+
 def sample(logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[Optional[int]],
            draw_indices: Sequence[int]) -> list[int]:
     """One token id per row of float32 ``logits [rows, vocab]`` (device tensor).
@@ -34,12 +43,11 @@ def sample(logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequen
     for i, (p, s) in enumerate(zip(params, seeds)):
         if not p.greedy and s is None:
             raise ValueError(f"row {i} samples stochastically but has no seed for its generator")
+    tuples = [sampling_tuple(p, s, d) for p, s, d in zip(params, seeds, draw_indices)]
     dev = logits.device
-    host = torch.tensor(
-        [[0.0 if p.greedy else p.temperature for p in params], [p.top_p for p in params]], dtype=torch.float32)
-    ints = torch.tensor([p.top_k for p in params], dtype=torch.int32)
-    longs = torch.tensor([[(s or 0) & _MASK63 for s in seeds], [int(d) for d in draw_indices]], dtype=torch.int64)
-    fdev, idev, ldev = host.to(dev), ints.to(dev), longs.to(dev)
+    floats = torch.tensor([[t[0] for t in tuples], [t[2] for t in tuples]], dtype=torch.float32).to(dev)
+    top_k = torch.tensor([t[1] for t in tuples], dtype=torch.int32).to(dev)
+    longs = torch.tensor([[t[3] for t in tuples], [t[4] for t in tuples]], dtype=torch.int64).to(dev)
     out = torch.empty(rows, dtype=torch.int32, device=dev)
-    ops.sample(logits, fdev[0], idev, fdev[1], ldev[0], ldev[1], out)
+    ops.sample(logits, floats[0], top_k, floats[1], longs[0], longs[1], out)
     return out.cpu().tolist()
