@@ -11,3 +11,6 @@ __all__ = [
     "Part", "PartSpec", "PositionEncoding", "Runtime", "ScheduleEntry", "StateSpec", "WeightSpec",
     "build_part", "part_class", "register_part", "registered_parts", "unregister_part",
 ]
+
+# importing the modules registers the parts that ship with the engine
+from . import attention, block, embedding, feed_forward, head, norm, position  # noqa: E402,F401

@@ -129,3 +129,95 @@ def test_graph_replay_equals_eager_steps(name, block):
     for i, (a, b) in enumerate(zip(eager, graphed)):
         assert a.shape == b.shape
         assert torch.equal(a, b), f"step {i}: graph replay differs from the eager step by {(a - b).abs().max()}"
+
+
+def test_shared_prefix_sampling_preemption_config_b():
+    """Six prompts that share a 40-token prefix, sampled at temperature 0.8 with per-request seeds
+    in a pool so small that requests are preempted: with and without content reuse of cache pages,
+    and each request alone, the tokens are the same (32-bit path)."""
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    name = "B"
+    rng = random.Random(31)
+    vocab = 384
+    prefix = [rng.randrange(vocab) for _ in range(40)]
+    ps = [prefix + [rng.randrange(vocab) for _ in range(n)] for n in (5, 22, 90, 37, 61, 12)]
+    params = [SamplingParams(max_tokens=32, temperature=0.8, seed=1000 + i) for i in range(len(ps))]
+
+    def run(prompts, pars, **kw):
+        eng = LLMEngine.for_model(str(model_folder(name)), dtype="float32", block_size=8, **kw)
+        outs = eng.generate(prompts, pars)
+        eng.manager.check_invariants()
+        return outs, eng
+
+    alone = [run([p], [q], num_blocks=64, config=SchedulerConfig(max_num_seqs=2, max_num_batched_tokens=256))[0][0]
+             for p, q in zip(ps, params)]
+    tight = dict(num_blocks=44, config=SchedulerConfig(max_num_seqs=6, max_num_batched_tokens=48))
+    with_reuse, eng = run(ps, params, enable_prefix_caching=True, **tight)
+    assert sum(s.num_preempted for s in eng.stats.steps) > 0
+    assert eng.manager.stats().prompt_tokens_hit > 0
+    without, _ = run(ps, params, enable_prefix_caching=False, **tight)
+    assert with_reuse == alone and without == alone
+    assert all(len(o) == 32 for o in alone) and len({tuple(o) for o in alone}) > 1
+
+
+def test_seeded_request_is_the_same_alone_and_in_a_busy_batch_bf16():
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    name = "A"
+    ps = prompts(name, [9, 30, 14, 21, 6], seed=33)
+    sp = SamplingParams(max_tokens=20, temperature=0.9, top_k=40, top_p=0.95, seed=7)
+
+    def run(which):
+        eng = LLMEngine.for_model(str(model_folder(name)), dtype="float32", num_blocks=64, block_size=16,
+                                  config=SchedulerConfig(max_num_seqs=8, max_num_batched_tokens=64))
+        pars = [sp if i == 2 else SamplingParams(max_tokens=25, temperature=1.0, seed=50 + i) for i in which]
+        return eng.generate([ps[i] for i in which], pars)[which.index(2)]
+
+    assert run([2]) == run([0, 1, 2, 3, 4]) == run([2, 4])
+
+
+def test_trace_run_program(tmp_path):
+    """bin/trace_run as a user runs it: steps on standard input, `done` lines, <step>.f32 files."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parent.parent
+    name = "A"
+    cfg, w = P.load_folder(model_folder(name))
+    a, b = prompts(name, [70, 19], seed=41)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:37], "want": [0, 36]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[37:39], "want": []}, {"id": "b", "tokens": b[:17], "want": [16]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[17:18], "want": [0]}], "end": []},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[39:70], "want": [30]}, {"id": "b", "tokens": b[18:19], "want": [0]}], "end": ["b"]},
+        {"step": 7, "entries": [{"id": "c", "tokens": b, "want": [18]}], "end": ["a", "c"]},
+    ]
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / dtype
+        proc = subprocess.run(
+            [sys.executable, str(root / "bin" / "trace_run"), "--model", str(model_folder(name)), "--dtype", dtype,
+             "--out", str(out), "--max-tokens", "192"],
+            input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        ref_a, ref_b = P.forward_logits(w, cfg, a), P.forward_logits(w, cfg, b)
+        want = {0: ref_a[[0, 36]], 1: ref_b[[16]], 2: ref_b[[17]], 3: torch.stack([ref_a[69], ref_b[18]]), 7: ref_b[[18]]}
+        assert sorted(p.name for p in out.iterdir()) == sorted(f"{k}.f32" for k in want)
+        for k, ref in want.items():
+            got = np.fromfile(out / f"{k}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])
+            err = np.abs(got - ref.numpy()).max()
+            assert err < (1e-4 if dtype == "float32" else 0.08 * float(ref.abs().max())), (dtype, k, err)
+    # a trace that asks for more than the pool holds fails with one clear line
+    proc = subprocess.run(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model", str(model_folder(name)), "--dtype", "float32",
+         "--out", str(tmp_path / "x"), "--max-tokens", "64"],
+        input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": a, "want": [0]}], "end": []}) + "\n",
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode != 0 and "NoFreePagesError" in proc.stderr

@@ -1,0 +1,255 @@
+"""Each part alone against the plain implementation's function for it, the cache store's page
+copies, and the proof that another mixer plugs in: a toy mixer with state of its own is
+registered, built and stepped here without a change to the framework's files."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+from tiny_configs import TINY_A, TINY_B, model_folder
+
+pytestmark = pytest.mark.gpu
+
+
+def rt(dtype=torch.float32):
+    from dli_amd.parts import Runtime
+
+    return Runtime(torch.device("cuda"), dtype)
+
+
+def test_norm_part_alone():
+    from dli_amd.parts import PartSpec, build_part
+
+    norm = build_part("norm", PartSpec("rms_norm", dict(width=192, eps=1e-6)), rt())
+    w = (1 + 0.1 * torch.randn(192)).cuda()
+    norm.load_weights({"weight": w})
+    x = torch.randn(7, 192, device="cuda") * 3
+    ref = P.rms_norm(x.cpu().double(), w.cpu().double(), 1e-6)
+    assert (norm.forward(x.clone()).cpu().double() - ref).abs().max() < 1e-5
+    delta = torch.randn_like(x)
+    stream = x.clone()
+    out = norm.forward(stream, delta)
+    assert torch.allclose(stream, x + delta)  # the residual sum is made in place
+    ref2 = P.rms_norm((x + delta).cpu().double(), w.cpu().double(), 1e-6)
+    assert (out.cpu().double() - ref2).abs().max() < 1e-5
+    assert norm.weight_specs()["weight"].role == "float32"
+
+
+@pytest.mark.parametrize("raw", [TINY_A, TINY_B])
+def test_rotary_part_alone(raw):
+    from dli_amd.architectures.llama import build_llama_spec
+    from dli_amd.config import LlamaConfig
+    from dli_amd.parts import build_part
+
+    cfg = LlamaConfig.from_hf_dict(raw)
+    spec = build_llama_spec(cfg).layers[0].parts["mixer"][1].params["position"]
+    part = build_part("position", spec, rt())
+    table, dim = part.rotary_table()
+    assert dim == cfg.head_dim
+    ref = P.inverse_frequencies(P.rope_settings(raw), cfg.head_dim)
+    assert torch.allclose(table.cpu(), ref, rtol=2e-7, atol=0)
+
+
+def test_feed_forward_part_alone():
+    from dli_amd.parts import PartSpec, build_part
+
+    for dtype, tol in ((torch.float32, 1e-4), (torch.bfloat16, 5e-2)):
+        ff = build_part("feed_forward", PartSpec("gated_mlp", dict(hidden_size=64, intermediate_size=160, bias=True)), rt(dtype))
+        w = {k: (torch.randn(*s.shape) / math.sqrt(s.shape[-1])).to(dtype) for k, s in ff.weight_specs().items()}
+        ff.load_weights({k: v.cuda() for k, v in w.items()})
+        x = torch.randn(5, 64).to(dtype)
+        ref = P.swiglu_mlp(x.double(), {k: v.double() for k, v in w.items()}, "")
+        got = ff.forward(x.cuda(), None)
+        assert (got.cpu().double() - ref).abs().max() < tol * max(1.0, ref.abs().max().item())
+
+
+def test_embedding_and_head_parts_alone():
+    from dli_amd.parts import PartSpec, build_part
+
+    emb = build_part("embedding", PartSpec("token_embedding", dict(vocab_size=301, hidden_size=72)), rt())
+    table = torch.randn(301, 72).cuda()
+    emb.load_weights({"weight": table})
+    ids = torch.tensor([0, 300, 17], dtype=torch.int32, device="cuda")
+    assert torch.equal(emb.forward(ids), table[ids.long()])
+    for tied in (True, False):
+        head = build_part("head", PartSpec("linear_head", dict(vocab_size=301, hidden_size=72, tied=tied)), rt())
+        own = torch.randn(301, 72).cuda()
+        head.load_weights({} if tied else {"weight": own})
+        head.tie(table)
+        x = torch.randn(4, 72, device="cuda")
+        ref = x.cpu().double() @ (table if tied else own).cpu().double().T
+        assert (head.forward(x).cpu().double() - ref).abs().max() < 1e-4
+        assert bool(head.weight_specs()) == (not tied)
+
+
+@pytest.mark.parametrize("name,dtype,page", [("A", "float32", 16), ("B", "float32", 8), ("B", "bfloat16", 16)])
+def test_attention_part_alone(name, dtype, page):
+    """The mixer of layer 0 with the model's own weights, fed rows directly: a fresh prompt, then
+    a portion on top of it, against plain attention over the whole sequence."""
+    from dli_amd.engine.batch import StepEntry
+    from dli_amd.engine.core import build_core
+
+    core = build_core(model_folder(name), num_pages=16, page_size=page, max_seqs=2, dtype=dtype,
+                      enable_prefix_caching=False, watermark=0.0)
+    cfg, w = P.load_folder(model_folder(name))
+    sizes = P.model_sizes(cfg)
+    mixer = core.model.layers[0].parts["mixer"]
+    n = 23
+    torch.manual_seed(1)
+    x = torch.randn(n, cfg["hidden_size"]).to(core.model.rt.dtype)
+    cos, sin = P.rope_cos_sin(P.inverse_frequencies(P.rope_settings(cfg), sizes["head_dim"]), torch.arange(n), torch.float64)
+    ref = P.attention_block(x.double(), {k: v.double() for k, v in w.items()}, "model.layers.0.self_attn.", sizes, cos, sin)
+    core.manager.allocate("r", list(range(n)), respect_watermark=False)
+    outs = []
+    for lo, hi in ((0, 14), (14, 23)):
+        ctx = core.step.build_context([StepEntry("r", list(range(lo, hi)), lo, ())])
+        outs.append(mixer.forward(x[lo:hi].cuda().contiguous(), ctx, core.step.caches[0]))
+        core.manager.mark_computed("r", hi)
+    got = torch.cat(outs).cpu().double()
+    tol = 1e-4 if dtype == "float32" else 4e-2
+    assert (got - ref).abs().max() < tol * max(1.0, ref.abs().max().item())
+
+
+def test_page_copies_cover_every_layer():
+    from dli_amd.cache.manager import CopyOp
+    from dli_amd.engine.core import build_core
+
+    core = build_core(model_folder("A"), num_pages=8, page_size=16, max_seqs=2, dtype="bfloat16")
+    pool = core.store.pools[0]
+    pool.copy_(torch.randn(pool.shape, device="cuda").to(pool.dtype))
+    before = pool.clone()
+    core.store.copy_pages([CopyOp(src=2, dst=5), CopyOp(src=7, dst=0)])
+    assert torch.equal(pool[:, :, 5], before[:, :, 2]) and torch.equal(pool[:, :, 0], before[:, :, 7])
+    keep = [1, 2, 3, 4, 6, 7]
+    assert torch.equal(pool[:, :, keep], before[:, :, keep])
+    with pytest.raises(ValueError):
+        core.store.copy_pages([CopyOp(src=1, dst=8)])
+
+
+# ------------------------------------------------------------------ a toy mixer with state of its own
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
+    """An exponential moving average over a request's rows: y_t = s_t W, s_t = a*s_{t-1} + x_t.
+    Its state lives in the request's state slot. The model below alternates it with attention
+    layers and runs one layer twice; stepping it in portions and mixed batches must equal running
+    each request whole."""
+    from typing import Any, Mapping
+
+    from dli_amd.cache.manager import CacheManager
+    from dli_amd.cache.store import CacheStore, group_specs
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import EngineCore
+    from dli_amd.engine.step import StepFunction
+    from dli_amd.parts import (LayerSpec, Mixer, ModelSpec, PartSpec, ScheduleEntry, StateSpec, WeightSpec,
+                               register_part, unregister_part)
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    @register_part("mixer", "toy_ema")
+    class ToyEMA(Mixer):
+        def __init__(self, runtime, *, hidden_size: int, decay: float) -> None:
+            super().__init__(runtime)
+            self.hidden_size, self.decay = hidden_size, decay
+            self.w = None
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.hidden_size, self.hidden_size))}
+
+        def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+            self.w = tensors["mix.weight"]
+
+        def cache_spec(self):
+            return StateSpec((self.hidden_size,), torch.float32)
+
+        def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+            out = torch.empty_like(x)
+            for e in range(ctx.num_entries):  # a toy: plain torch, one request after the other
+                r0, r1 = ctx.entry_rows(e)
+                slot = int(ctx.state_slots_host[e])
+                state = torch.zeros_like(cache.state[slot]) if ctx.is_fresh(e) else cache.state[slot].clone()
+                for r in range(r0, r1):
+                    state = self.decay * state + x[r].float()
+                    out[r] = (state @ self.w.float().T).to(x.dtype)
+                cache.state[slot] = state
+            return out
+
+    def parse(raw):
+        return dict(raw)
+
+    def build(cfg):
+        h = cfg["hidden_size"]
+        norm = dict(width=h, eps=cfg["eps"])
+        pos = PartSpec("rotary", dict(dim=16, theta=10000.0))
+        layers = []
+        for i in range(3):
+            p = f"layers.{i}."
+            mixer = (PartSpec("toy_ema", dict(hidden_size=h, decay=0.5), p + "ema.") if i == 1 else
+                     PartSpec("gqa_attention", dict(hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=16, position=pos,
+                                                    window=9 if i == 2 else 0), p + "attn."))
+            layers.append(LayerSpec(PartSpec("pre_norm"), {
+                "mixer_norm": ("norm", PartSpec("rms_norm", norm, p + "n1.")), "mixer": ("mixer", mixer),
+                "feed_forward_norm": ("norm", PartSpec("rms_norm", norm, p + "n2.")),
+                "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=48), p + "mlp."))}))
+        return ModelSpec(
+            architecture="ToyForCausalLM", vocab_size=cfg["vocab_size"], hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=cfg["vocab_size"], hidden_size=h), "embed."),
+            layers=tuple(layers),
+            # layer 0 runs twice (two caches), the windowed layer 2 and the stateful layer 1 between
+            schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2), ScheduleEntry(0)),
+            final_norm=PartSpec("rms_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=cfg["vocab_size"], hidden_size=h, tied=True), "head."))
+
+    register_architecture("ToyForCausalLM", parse, build)
+    try:
+        import tempfile
+
+        raw = {"architectures": ["ToyForCausalLM"], "vocab_size": 61, "hidden_size": 32, "eps": 1e-5}
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, raw, seed=3, std=0.2, norm_jitter=0.1)
+
+            def make():
+                model = load_model(folder, dtype="float32")
+                specs = model.cache_specs()
+                assert [type(s).__name__ for s in specs] == ["PagedKVSpec", "StateSpec", "PagedKVSpec", "PagedKVSpec"]
+                store = CacheStore(model.rt, specs, num_pages=12, page_size=4, max_seqs=4)
+                assert len(store.groups) == 2 and store.stateful  # full attention and the window of 9
+                mgr = CacheManager(group_specs(store.groups), num_pages=12, page_size=4, max_seqs=4,
+                                   stateful=store.stateful, watermark=0.0)
+                assert not mgr.prefix_caching
+                return EngineCore(model, mgr, store, StepFunction(model, mgr, store))
+
+            toks = {"a": [5, 9, 2, 40, 33, 7, 7, 12, 60, 1, 18, 25, 3, 3, 44, 51, 9, 30, 2, 11, 17],
+                    "b": [8, 8, 1, 50, 23, 4, 19, 36, 2, 45, 13, 27]}
+            whole = {}
+            for rid, t in toks.items():
+                s = TraceSession(make())
+                whole[rid] = s.step([{"id": rid, "tokens": t, "want": list(range(len(t)))}]).cpu()
+            core = make()
+            s = TraceSession(core)
+            got = {"a": [], "b": []}
+            plan = [{"a": 5}, {"a": 2, "b": 3}, {"a": 1, "b": 1}, {"b": 6}, {"a": 9, "b": 1}, {"a": 1, "b": 1}, {"a": 3}]
+            fed = {"a": 0, "b": 0}
+            for stepplan in plan:
+                entries = []
+                for rid, n in stepplan.items():
+                    entries.append({"id": rid, "tokens": toks[rid][fed[rid]:fed[rid] + n], "want": list(range(n))})
+                out = s.step(entries).cpu()
+                row = 0
+                for rid, n in stepplan.items():
+                    got[rid].append(out[row:row + n])
+                    row += n
+                    fed[rid] += n
+                core.manager.check_invariants()
+            for rid in toks:
+                assert fed[rid] == len(toks[rid])
+                assert (torch.cat(got[rid]) - whole[rid]).abs().max() < 1e-4, rid
+            assert core.manager.stats().window_pages_released > 0  # the window gave pages back
+            s.step([], end=["a", "b"])
+            assert core.manager.stats().used_pages == 0
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        unregister_part("mixer", "toy_ema")
