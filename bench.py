@@ -135,6 +135,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="run only the 2,048-token prefill steps (for profiling) and print their time")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
@@ -148,9 +150,13 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
-    max_batch = max(args.batch, 1 if args.no_points else 64)
+    max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
     engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=8192)
 
+    if args.only_prefill:
+        t = prefill_run(engine, cfg, 2048, repeats=args.steps)
+        print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": 2048, "tok_s": round(2048 / t, 1)}))
+        return 0
     tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup)
     achieved = decode_bytes(cfg, args.batch, args.context, itemsize) / (ms * 1e-3) / 1e9
     line = {

@@ -18,8 +18,8 @@ __global__ void embedding_kernel(const T* __restrict__ table, const int* __restr
 // type before the weight multiplies it (reference: src/dli/model/llama.py:40-44).
 // With `delta`, the row is first replaced by x + delta (sum in 32-bit) and written to `sum_out`.
 template <typename T>
-__global__ void rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ delta,
-                                const float* __restrict__ weight, T* __restrict__ sum_out,
+__global__ void rms_norm_kernel(const T* x, const T* __restrict__ delta,
+                                const float* __restrict__ weight, T* sum_out,
                                 T* __restrict__ out, int width, float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
@@ -48,6 +48,74 @@ __global__ void rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ d
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     const float normed = round_to<T>(to_f32(xr[i]) * r);
     yr[i] = from_f32<T>(weight[i] * normed);
+  }
+}
+
+// Eight elements at a time (rows of a multiple of eight elements, 16-byte aligned).
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> { typedef __bf16 type __attribute__((ext_vector_type(8))); };
+template <> struct Vec8<float> { typedef float type __attribute__((ext_vector_type(8))); };
+
+template <typename T>
+__global__ void rms_norm_vec_kernel(const T* x, const T* __restrict__ delta,
+                                    const float* __restrict__ weight, T* sum_out,
+                                    T* __restrict__ out, int width, float eps) {
+  typedef typename Vec8<T>::type V;
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const V* xr = reinterpret_cast<const V*>(x + row * width);
+  const V* dr = delta != nullptr ? reinterpret_cast<const V*>(delta + row * width) : nullptr;
+  V* sr = delta != nullptr ? reinterpret_cast<V*>(sum_out + row * width) : nullptr;
+  const int chunks = width / 8;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+    V v = xr[c];
+    if (dr != nullptr) {
+      const V d = dr[c];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = from_f32<T>(to_f32((T)v[i]) + to_f32((T)d[i]));
+      sr[c] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float f = to_f32((T)v[i]);
+      ss += f * f;
+    }
+  }
+  const float r = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+  const V* src = dr != nullptr ? reinterpret_cast<const V*>(sum_out + row * width) : xr;
+  V* yr = reinterpret_cast<V*>(out + row * width);
+  for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+    const V v = src[c];  // re-read of this thread's own chunk
+    const float4 w0 = *reinterpret_cast<const float4*>(weight + c * 8);
+    const float4 w1 = *reinterpret_cast<const float4*>(weight + c * 8 + 4);
+    const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+    V y;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = from_f32<T>(wv[i] * round_to<T>(to_f32((T)v[i]) * r));
+    yr[c] = y;
+  }
+}
+
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t rows, int inter) {
+  typedef typename Vec8<T>::type V;
+  const int chunks = inter / 8;
+  const int64_t total = rows * chunks;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = idx / chunks;
+    const int c = (int)(idx - r * chunks);
+    const V g = *reinterpret_cast<const V*>(gu + r * 2 * inter + c * 8);
+    const V u = *reinterpret_cast<const V*>(gu + r * 2 * inter + inter + c * 8);
+    V o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float gf = to_f32((T)g[i]);
+      const float sg = gf / (1.f + expf(-gf));
+      o[i] = from_f32<T>(round_to<T>(sg) * to_f32((T)u[i]));
+    }
+    *reinterpret_cast<V*>(out + r * inter + c * 8) = o;
   }
 }
 
@@ -150,6 +218,13 @@ int dli_rms_norm(const void* x, const void* delta, const float* weight, void* su
   if (rows <= 0) return DLI_OK;
   if (width <= 0 || (delta != nullptr && sum_out == nullptr)) return DLI_ERR_ARGUMENT;
   const int threads = width >= 2048 ? 512 : 256;
+  const bool aligned = (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)sum_out | (uintptr_t)out | (uintptr_t)weight) % 32) == 0;
+  if (width % 8 == 0 && aligned) {
+    const int vthreads = width / 8 >= 256 ? 256 : (width / 8 >= 128 ? 128 : 64);
+    DISPATCH_DTYPE(is_bf16, (rms_norm_vec_kernel<T><<<rows, vthreads, 0, stream>>>(
+                                (const T*)x, (const T*)delta, weight, (T*)sum_out, (T*)out, width, eps)));
+    return dli_launch_status();
+  }
   DISPATCH_DTYPE(is_bf16, (rms_norm_kernel<T><<<rows, threads, 0, stream>>>(
                               (const T*)x, (const T*)delta, weight, (T*)sum_out, (T*)out, width, eps)));
   return dli_launch_status();
@@ -159,6 +234,10 @@ int dli_silu_mul(const void* gu, void* out, int rows, int inter, int is_bf16, hi
   if (rows <= 0) return DLI_OK;
   if (inter <= 0) return DLI_ERR_ARGUMENT;
   const int64_t total = (int64_t)rows * inter;
+  if (inter % 8 == 0 && (((uintptr_t)gu | (uintptr_t)out) % 32) == 0) {
+    DISPATCH_DTYPE(is_bf16, (silu_mul_vec_kernel<T><<<grid_for(total / 8, 256), 256, 0, stream>>>((const T*)gu, (T*)out, rows, inter)));
+    return dli_launch_status();
+  }
   DISPATCH_DTYPE(is_bf16, (silu_mul_kernel<T><<<grid_for(total, 256), 256, 0, stream>>>((const T*)gu, (T*)out, rows, inter)));
   return dli_launch_status();
 }
