@@ -40,6 +40,27 @@ __device__ __forceinline__ short bf16_bits(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Reductions over the four lanes l, l^16, l^32, l^48 (the lane groups that share a column) with
+// the gfx950 lane-swap instructions: after v_permlane32_swap of two copies of v, one copy holds
+// the lower half's values in both halves and the other the upper half's; v_permlane16_swap does
+// the same for neighbouring rows of 16 lanes.
+__device__ __forceinline__ float column_max(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const unsigned um = __float_as_uint(m);
+  const auto b = __builtin_amdgcn_permlane16_swap(um, um, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_sum(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const float m = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const unsigned um = __float_as_uint(m);
+  const auto b = __builtin_amdgcn_permlane16_swap(um, um, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Online-softmax state of one column tile (16 columns; this lane owns column lane%16).
 template <int DCH>
 struct ColumnTile {
@@ -74,9 +95,7 @@ __device__ __forceinline__ void attend_tile(ColumnTile<DCH>& st, const short4v (
       if (key > last_visible || key < first_visible) sv[i] = -INFINITY;
     }
   }
-  float tile_max = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, DLI_WAVE));
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, DLI_WAVE));
+  const float tile_max = column_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
   const float m_new = fmaxf(st.m, tile_max);
   const float m_safe = m_new == -INFINITY ? 0.f : m_new;
   const float alpha = fast_exp2(st.m - m_safe);
@@ -87,16 +106,16 @@ __device__ __forceinline__ void attend_tile(ColumnTile<DCH>& st, const short4v (
     p[i] = fast_exp2(sv[i] - m_safe);
     tile_sum += p[i];
   }
-  tile_sum += __shfl_xor(tile_sum, 16, DLI_WAVE);
-  tile_sum += __shfl_xor(tile_sum, 32, DLI_WAVE);
+  tile_sum = column_sum(tile_sum);
   st.l = st.l * alpha + tile_sum;
   st.m = m_new;
   const short4v pb = {bf16_bits(p[0]), bf16_bits(p[1]), bf16_bits(p[2]), bf16_bits(p[3])};
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // the running maximum rose somewhere
 #pragma unroll
-  for (int c = 0; c < DCH; ++c) {
-    st.o[c] *= alpha;
-    st.o[c] = mfma16(vreg[c], pb, st.o[c]);
+    for (int c = 0; c < DCH; ++c) st.o[c] *= alpha;
   }
+#pragma unroll
+  for (int c = 0; c < DCH; ++c) st.o[c] = mfma16(vreg[c], pb, st.o[c]);
 }
 
 template <int DCH>
@@ -334,6 +353,251 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------ prefill, shared tiles
+// The four waves of a workgroup share every key tile through LDS: a workgroup takes HW query heads
+// of one kv head (HW = 4, 2 or 1, whatever divides the group) times 4/HW blocks of 32 queries, so
+// each K/V tile is fetched from memory once for 128 query rows. Tiles of 32 keys are pipelined:
+// while tile i is consumed from LDS, tile i+1 already lies there, tile i+2 is being written there
+// from registers and tiles i+3.. are on their way from memory into registers.
+// Products use v_mfma_f32_16x16x32_bf16 (lane l: row/column l%16, k-indices 8*(l/16)..+7). For
+// P*V the eight k-indices of lane group g stand for the keys 4g..4g+3 and 16+4g..16+4g+3 of the
+// tile, which is how the two 16-key halves of S^T leave the first product.
+// Needs head_dim % 32 == 0.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+template <int DCH>
+__global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
+    const int* __restrict__ q_start, const int* __restrict__ kv_len,
+    const int* __restrict__ block_tables, int table_stride, const int* __restrict__ tile_entry,
+    const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
+    int window, int heads_per_wg) {
+  constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of the first product
+  constexpr int KPAD = D + 8, VPAD = 32 + 8;    // padded rows against bank conflicts
+  constexpr int KCH = (4 * D + 255) / 256;      // 16-byte chunks per thread and tile
+  constexpr int RD = 3;                         // tiles in flight from memory to registers
+  __shared__ __attribute__((aligned(16))) bf16_t ks[3][32][KPAD];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[3][D][VPAD];
+
+  const int e = tile_entry[blockIdx.x];
+  const int group = q_heads / kv_heads;
+  const int wg_per_kv = group / heads_per_wg;
+  const int kvh = blockIdx.y / wg_per_kv;
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int col = lane % 16, grp = lane / 16;
+  const int head = kvh * group + (blockIdx.y % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
+  const int tok0 = q_start[e];
+  const int q_len = q_start[e + 1] - tok0;
+  const int n_keys = kv_len[e];
+  const int first_pos = n_keys - q_len;
+  const int wg_q0 = tile_q0[blockIdx.x];
+  const int wg_rows = min((4 / heads_per_wg) * 32, q_len - wg_q0);
+  const int q0 = wg_q0 + (wave / heads_per_wg) * 32;  // this wave's first query
+  const int wave_rows = max(0, min(32, q_len - q0));
+  const int* table = block_tables + (int64_t)e * table_stride;
+
+  bf16x8 qreg[2][DK];
+  ColumnTile<DCH> st[2];
+  int pos[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    st[j].init();
+    const int qi = q0 + j * 16 + col;
+    pos[j] = qi < q_len ? first_pos + qi : -1;
+#pragma unroll
+    for (int c = 0; c < DK; ++c) qreg[j][c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (qi < q_len) {
+      const bf16_t* qp = q + (int64_t)(tok0 + qi) * q_stride + (int64_t)head * D + grp * 8;
+#pragma unroll
+      for (int c = 0; c < DK; ++c) qreg[j][c] = *reinterpret_cast<const bf16x8*>(qp + c * 32);
+    }
+  }
+  const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + wave_rows - 1;  // this wave's span
+  const int wg_pos_lo = first_pos + wg_q0, wg_pos_hi = first_pos + wg_q0 + wg_rows - 1;
+  const int begin = window > 0 ? max(0, wg_pos_lo - window + 1) / 32 * 32 : 0;
+  const int end = wg_pos_hi + 1;
+  const int n_tiles = (end - begin + 31) / 32;
+
+  // staging: each thread moves KCH chunks of K and KCH chunks of V^T per tile; RD tiles in flight
+  bf16x8 kst[RD][KCH], vst[RD][KCH];
+  // Tiles are fetched in order, so the page of the tile's first key is tracked by addition
+  // instead of division: `tile_page` indexes the block table, `tile_off` is the key's offset in it.
+  int tile_page = begin / page_size, tile_off = begin % page_size;
+  auto fetch = [&](int t, bf16x8 (&kq)[KCH], bf16x8 (&vq)[KCH]) {
+    const bool whole = t + 32 <= n_keys;  // every key of the tile exists
+#pragma unroll
+    for (int r = 0; r < KCH; ++r) {
+      const int c = threadIdx.x + r * 256;
+      kq[r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      vq[r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (4 * D % 256 == 0 || c < 4 * D) {
+        const int kk = c / (D / 8), part = c % (D / 8);
+        int kp = tile_page, ko = tile_off + kk;
+        while (ko >= page_size) { ko -= page_size; ++kp; }
+        if (whole || t + kk < n_keys) {
+          const int64_t page = table[kp];
+          kq[r] = *reinterpret_cast<const bf16x8*>(
+              k_pages + ((page * kv_heads + kvh) * page_size + ko) * D + part * 8);
+        }
+        const int d = c / 4, vk = (c % 4) * 8;
+        int vp = tile_page, vo = tile_off + vk;
+        while (vo >= page_size) { vo -= page_size; ++vp; }
+        if (whole || t + vk < n_keys) {
+          const int64_t page = table[vp];
+          vq[r] = *reinterpret_cast<const bf16x8*>(v_pages + ((page * kv_heads + kvh) * D + d) * page_size + vo);
+          if (!whole && t + vk + 8 > n_keys) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              if (t + vk + i >= n_keys) vq[r][i] = (bf16_t)0.f;
+          }
+        }
+      }
+    }
+    tile_off += 32;
+    while (tile_off >= page_size) { tile_off -= page_size; ++tile_page; }
+  };
+  auto stash = [&](int buf, const bf16x8 (&kq)[KCH], const bf16x8 (&vq)[KCH]) {
+#pragma unroll
+    for (int r = 0; r < KCH; ++r) {
+      const int c = threadIdx.x + r * 256;
+      if (c < 4 * D) {
+        *reinterpret_cast<bf16x8*>(&ks[buf][c / (D / 8)][(c % (D / 8)) * 8]) = kq[r];
+        *reinterpret_cast<bf16x8*>(&vs[buf][c / 4][(c % 4) * 8]) = vq[r];
+      }
+    }
+  };
+
+  // tiles 0 and 1 go straight to LDS; tile T >= 2 waits in register slot T % RD
+#pragma unroll
+  for (int T = 0; T < 2 + RD; ++T) {
+    if (T < n_tiles) fetch(begin + T * 32, kst[T % RD], vst[T % RD]);
+    if (T < 2) {
+      if (T < n_tiles) stash(T, kst[T % RD], vst[T % RD]);
+    }
+  }
+  __syncthreads();
+  for (int it0 = 0; it0 < n_tiles; it0 += RD) {
+#pragma unroll
+   for (int r = 0; r < RD; ++r) {
+    const int it = it0 + r;
+    if (it >= n_tiles) break;
+    const int t = begin + it * 32, buf = it % 3;
+    if (wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1)) {
+      const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
+      // all operand fragments of the tile are requested from LDS first, so that the reads of V
+      // overlap the first product and the softmax
+      bf16x8 kf0[DK], kf1[DK];
+#pragma unroll
+      for (int c = 0; c < DK; ++c) {
+        kf0[c] = *reinterpret_cast<const bf16x8*>(&ks[buf][col][c * 32 + grp * 8]);
+        kf1[c] = *reinterpret_cast<const bf16x8*>(&ks[buf][16 + col][c * 32 + grp * 8]);
+      }
+      typedef short short4a __attribute__((ext_vector_type(4)));
+      union VFrag {
+        bf16x8 v;
+        short4a h[2];
+      } vf[DCH];
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) {
+        vf[c].h[0] = *reinterpret_cast<const short4a*>(&vs[buf][c * 16 + col][4 * grp]);
+        vf[c].h[1] = *reinterpret_cast<const short4a*>(&vs[buf][c * 16 + col][16 + 4 * grp]);
+      }
+      // S^T of both column tiles, for the two halves of the tile: keys t+4g+i and t+16+4g+i
+      float4v sa[2], sb[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        sa[j] = float4v{0.f, 0.f, 0.f, 0.f};
+        sb[j] = float4v{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int c = 0; c < DK; ++c)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          sa[j] = mfma32(kf0[c], qreg[j][c], sa[j]);
+          sb[j] = mfma32(kf1[c], qreg[j][c], sb[j]);
+        }
+      float sv[2][8];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          sv[j][i] = sa[j][i];
+          sv[j][4 + i] = sb[j][i];
+        }
+      if (need_mask) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int low = window > 0 ? pos[j] - window + 1 : 0;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const int key = t + (i < 4 ? 4 * grp + i : 16 + 4 * grp + i - 4);
+            if (key > pos[j] || key < low) sv[j][i] = -INFINITY;
+          }
+        }
+      }
+      float alpha[2];
+      bf16x8 pb[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float tile_max = fmaxf(fmaxf(fmaxf(sv[j][0], sv[j][1]), fmaxf(sv[j][2], sv[j][3])),
+                               fmaxf(fmaxf(sv[j][4], sv[j][5]), fmaxf(sv[j][6], sv[j][7])));
+        tile_max = column_max(tile_max) * scale_log2e;  // the scale is positive
+        const float m_new = fmaxf(st[j].m, tile_max);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        alpha[j] = fast_exp2(st[j].m - m_safe);
+        float tile_sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float p = fast_exp2(fmaf(sv[j][i], scale_log2e, -m_safe));
+          tile_sum += p;
+          pb[j][i] = (bf16_t)p;
+        }
+        tile_sum = column_sum(tile_sum);
+        st[j].l = st[j].l * alpha[j] + tile_sum;
+        st[j].m = m_new;
+      }
+      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.f || alpha[1] != 1.f) != 0) {
+        // the running maximum rose somewhere: rescale what has been accumulated
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int c = 0; c < DCH; ++c) st[j].o[c] *= alpha[j];
+      }
+#pragma unroll
+      for (int c = 0; c < DCH; ++c)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
+    }
+    // tile it+2 leaves its register slot for LDS; the slot then receives tile it+2+RD
+    const int slot = (r + 2) % RD;
+    if (it + 2 < n_tiles) {
+      stash((it + 2) % 3, kst[slot], vst[slot]);
+      if (it + 2 + RD < n_tiles) fetch(begin + (it + 2 + RD) * 32, kst[slot], vst[slot]);
+    }
+    __syncthreads();
+   }
+  }
+
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int qi = q0 + j * 16 + col;
+    if (qi >= q_len) continue;
+    const float inv = st[j].l > 0.f ? 1.f / st[j].l : 0.f;
+    bf16_t* op = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * D + 4 * grp;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) {
+      const short4v packed = {bf16_bits(st[j].o[c][0] * inv), bf16_bits(st[j].o[c][1] * inv),
+                              bf16_bits(st[j].o[c][2] * inv), bf16_bits(st[j].o[c][3] * inv)};
+      *reinterpret_cast<short4v*>(op + c * 16) = packed;
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------ host side
 #define LOG2E 1.4426950408889634f
 
@@ -341,7 +605,19 @@ extern "C" int dli_attention_mfma_supports(int head_dim, int page_size) {
   return head_dim > 0 && head_dim % 16 == 0 && head_dim <= 128 && page_size > 0 && page_size % 16 == 0;
 }
 
-extern "C" int dli_attention_prefill_tile_rows() { return PF_TILE_ROWS; }
+// Query heads that one workgroup of the shared-tile kernel takes (4, 2 or 1), or 0 if the shape
+// has to take the plain kernel (head_dim not a multiple of 32).
+static int shared_heads_per_wg(int head_dim, int group) {
+  if (head_dim % 32 != 0) return 0;
+  return group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+}
+
+// Queries per tile of the tile list that dli_attention_prefill_bf16 expects for this shape.
+extern "C" int dli_attention_prefill_tile_rows(int head_dim, int q_heads, int kv_heads) {
+  if (kv_heads <= 0 || q_heads % kv_heads != 0) return DLI_ERR_ARGUMENT;
+  const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
+  return hw == 0 ? PF_TILE_ROWS : (4 / hw) * 32;
+}
 
 extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pages,
                                          const void* v_pages, void* out, int64_t out_stride,
@@ -389,6 +665,23 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || q_heads > 65535 || q_stride % 4 != 0 || out_stride % 4 != 0)
     return DLI_ERR_ARGUMENT;
+  const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
+  if (hw > 0) {
+    const dim3 sgrid(tiles, q_heads / hw);
+#define SHARED_CASE(N)                                                                            \
+  case N:                                                                                         \
+    attention_prefill_shared_kernel<N><<<sgrid, 256, 0, stream>>>(                                \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
+        out_stride, q_start, kv_len, block_tables, table_stride, tile_entry, tile_q0, q_heads,    \
+        kv_heads, page_size, scale * LOG2E, window, hw);                                          \
+    break;
+    switch (head_dim / 16) {
+      SHARED_CASE(2) SHARED_CASE(4) SHARED_CASE(6) SHARED_CASE(8)
+      default: return DLI_ERR_ARGUMENT;
+    }
+#undef SHARED_CASE
+    return dli_launch_status();
+  }
   const dim3 grid(tiles, q_heads);
 #define PREFILL_CASE(N)                                                                           \
   case N:                                                                                         \

@@ -28,6 +28,9 @@ ARCH = "gfx950"
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core accumulators stay in ordinary vector registers: no moves to and from the
+    # accumulation registers around the online softmax's rescaling
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
 ]
 LIB_STEM = "libdli_hip"

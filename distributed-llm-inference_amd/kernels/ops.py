@@ -48,7 +48,7 @@ _SIGNATURES = {
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
-    "dli_attention_prefill_tile_rows": [],
+    "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
@@ -414,8 +414,11 @@ def attention_mfma_supports(head_dim: int, page_size: int, dtype: torch.dtype) -
     return dtype == torch.bfloat16 and bool(library().dli_attention_mfma_supports(head_dim, page_size))
 
 
-def attention_prefill_tile_rows() -> int:
-    return int(library().dli_attention_prefill_tile_rows())
+def attention_prefill_tile_rows(head_dim: int, q_heads: int, kv_heads: int) -> int:
+    """Queries per tile of the tile list that :func:`attention_prefill` expects for this shape."""
+    rows = int(library().dli_attention_prefill_tile_rows(head_dim, q_heads, kv_heads))
+    _require(rows > 0, "query heads are not a multiple of kv heads")
+    return rows
 
 
 def _check_paged(q, k_pages, v_pages, out, q_heads):
@@ -469,7 +472,7 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
                       tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
                       window: int = 0) -> None:
     """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
-    :func:`attention_prefill_tile_rows` queries."""
+    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height)."""
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
     for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
         _dense(t, name, torch.int32, 1)

@@ -53,6 +53,6 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
         ops.attention_decode(q[:nd], k_pages, v_pages, out[:nd], ctx.kv_len, grp.block_tables, q_heads,
                              scale, window, splits, part_o, part_ml)
     if ctx.num_entries > nd:
-        tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(), first_entry=nd)
+        tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads), first_entry=nd)
         ops.attention_prefill(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
                               tile_entry, tile_q0, q_heads, scale, window)

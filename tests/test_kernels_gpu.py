@@ -190,7 +190,7 @@ def test_attention_generic(ops, dtype, qh, kvh, d, bs, window):
 
 
 MFMA_SHAPES = [(4, 4, 16, 16), (6, 2, 32, 16), (32, 8, 64, 16), (14, 2, 64, 32), (8, 8, 128, 16), (5, 1, 80, 16),
-               (3, 3, 48, 64), (40, 2, 64, 16), (7, 7, 112, 16)]
+               (3, 3, 48, 64), (40, 2, 64, 16), (7, 7, 112, 16), (12, 2, 96, 16), (9, 3, 64, 48), (16, 2, 128, 64)]
 
 
 @pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
@@ -221,7 +221,7 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
 def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window):
     lens = [(2, 2), (7, 7), (33, 33), (5, 40), (2, 131), (129, 129), (16, 16), (31, 300), (140, 333), (1, 50)]
     q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + bs)
-    te, tq = _tiles(q_start, ops.attention_prefill_tile_rows())
+    te, tq = _tiles(q_start, ops.attention_prefill_tile_rows(d, qh, kvh))
     dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
     out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
     scale = 1.0 / math.sqrt(d)
@@ -251,7 +251,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops):
     out = torch.zeros(q.shape, dtype=torch.bfloat16, device="cuda")
     ops.attention_decode(q[:1].cuda(), kp.cuda(), vp.cuda(), out[:1], dev(kv_len), dev(tables), qh, scale, 0, 4,
                          torch.empty(qh * 4 * d, device="cuda"), torch.empty(qh * 4 * 2, device="cuda"))
-    te, tq = _tiles(q_start, ops.attention_prefill_tile_rows())
+    te, tq = _tiles(q_start, ops.attention_prefill_tile_rows(d, qh, kvh))
     te, tq = [t for t in te if t == 1], [q0 for t, q0 in zip(te, tq) if t == 1]
     ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables),
                           dev(te), dev(tq), qh, scale, 0)
