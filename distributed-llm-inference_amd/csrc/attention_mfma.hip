@@ -354,11 +354,15 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 }
 
 // ------------------------------------------------------------------------------------ prefill, shared tiles
-// The four waves of a workgroup share every key tile through LDS: a workgroup takes HW query heads
-// of one kv head (HW = 4, 2 or 1, whatever divides the group) times 4/HW blocks of 32 queries, so
-// each K/V tile is fetched from memory once for 128 query rows. Tiles of 32 keys are pipelined:
-// while tile i is consumed from LDS, tile i+1 already lies there, tile i+2 is being written there
-// from registers and tiles i+3.. are on their way from memory into registers.
+// The waves of a workgroup share every key tile through LDS. Four waves take HW query heads of
+// one kv head (HW = 4, 2 or 1, whatever divides the group) times 4/HW blocks of 32 queries, so
+// each K/V tile is fetched from memory once for 128 query rows. With PAIR a workgroup has a second
+// set of four waves that takes the mirror tile of the same request (tile b of n pairs with tile
+// n-1-b): under a causal mask the two together always have the same number of key tiles to visit,
+// whatever b, so that all workgroups take equally long; the workgroups of the lower half of the
+// tile list leave at once. Tiles of 32 keys are pipelined: while tile i is consumed from LDS, tile
+// i+1 already lies there, tile i+2 is being written there from registers and tiles i+3.. are on
+// their way from memory into registers.
 // Products use v_mfma_f32_16x16x32_bf16 (lane l: row/column l%16, k-indices 8*(l/16)..+7). For
 // P*V the eight k-indices of lane group g stand for the keys 4g..4g+3 and 16+4g..16+4g+3 of the
 // tile, which is how the two 16-key halves of S^T leave the first product.
@@ -369,8 +373,8 @@ __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-template <int DCH>
-__global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
+template <int DCH, bool PAIR>
+__global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len,
@@ -379,25 +383,35 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
     int window, int heads_per_wg) {
   constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of the first product
   constexpr int KPAD = D + 8, VPAD = 32 + 8;    // padded rows against bank conflicts
-  constexpr int KCH = (4 * D + 255) / 256;      // 16-byte chunks per thread and tile
+  constexpr int NT = PAIR ? 512 : 256;          // threads
+  constexpr int CHUNKS = 8 * D;                 // 16-byte chunks of a tile: 4D of K, then 4D of V^T
+  constexpr int UCH = (CHUNKS + NT - 1) / NT;   // chunks per thread and tile
   constexpr int RD = 3;                         // tiles in flight from memory to registers
-  __shared__ __attribute__((aligned(16))) bf16_t ks[3][32][KPAD];
-  __shared__ __attribute__((aligned(16))) bf16_t vs[3][D][VPAD];
+  constexpr int K_ELEMS = 32 * KPAD, TILE_ELEMS = K_ELEMS + D * VPAD;
+  __shared__ __attribute__((aligned(16))) bf16_t lds[3][TILE_ELEMS];  // K rows, then V^T rows
 
   const int e = tile_entry[blockIdx.x];
+  const int tok0 = q_start[e];
+  const int q_len = q_start[e + 1] - tok0;
+  const int tile_rows = (4 / heads_per_wg) * 32;
+  const int q0_first = tile_q0[blockIdx.x];
+  int q0_second = -1;
+  if (PAIR) {
+    const int b = q0_first / tile_rows, mirror = (q_len + tile_rows - 1) / tile_rows - 1 - b;
+    if (b < mirror) return;  // the workgroup of the mirror tile does this one too
+    if (mirror < b) q0_second = mirror * tile_rows;
+  }
   const int group = q_heads / kv_heads;
   const int wg_per_kv = group / heads_per_wg;
   const int kvh = blockIdx.y / wg_per_kv;
-  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int lane = threadIdx.x % DLI_WAVE, wave = (threadIdx.x / DLI_WAVE) % 4;
+  const int set = threadIdx.x / 256;  // which of the workgroup's two tiles
   const int col = lane % 16, grp = lane / 16;
   const int head = kvh * group + (blockIdx.y % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
-  const int tok0 = q_start[e];
-  const int q_len = q_start[e + 1] - tok0;
   const int n_keys = kv_len[e];
   const int first_pos = n_keys - q_len;
-  const int wg_q0 = tile_q0[blockIdx.x];
-  const int wg_rows = min((4 / heads_per_wg) * 32, q_len - wg_q0);
-  const int q0 = wg_q0 + (wave / heads_per_wg) * 32;  // this wave's first query
+  const int set_q0 = set == 0 ? q0_first : q0_second;
+  const int q0 = set_q0 < 0 ? q_len : set_q0 + (wave / heads_per_wg) * 32;  // this wave's first query
   const int wave_rows = max(0, min(32, q_len - q0));
   const int* table = block_tables + (int64_t)e * table_stride;
 
@@ -418,56 +432,91 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
     }
   }
   const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + wave_rows - 1;  // this wave's span
-  const int wg_pos_lo = first_pos + wg_q0, wg_pos_hi = first_pos + wg_q0 + wg_rows - 1;
-  const int begin = window > 0 ? max(0, wg_pos_lo - window + 1) / 32 * 32 : 0;
-  const int end = wg_pos_hi + 1;
+  // the workgroup walks the keys that any of its queries sees
+  const int wg_q_lo = q0_second >= 0 ? q0_second : q0_first;
+  const int wg_q_hi = min(q_len, q0_first + tile_rows) - 1;
+  const int begin = window > 0 ? max(0, first_pos + wg_q_lo - window + 1) / 32 * 32 : 0;
+  const int end = first_pos + wg_q_hi + 1;
   const int n_tiles = (end - begin + 31) / 32;
 
-  // staging: each thread moves KCH chunks of K and KCH chunks of V^T per tile; RD tiles in flight
-  bf16x8 kst[RD][KCH], vst[RD][KCH];
+  // Staging: thread-constant description of the UCH chunks this thread moves per tile. Chunk u <
+  // 4D is 8 dims of key u/(D/8); chunk 4D+c is 8 keys of dim c/4.
+  const bf16_t* src_base[UCH];
+  int src_off[UCH], src_mul[UCH], lds_off[UCH];
+  bool second_half[UCH], is_v[UCH], live[UCH];
+  int v_key[UCH];
+#pragma unroll
+  for (int r = 0; r < UCH; ++r) {
+    const int u_raw = threadIdx.x + r * NT;
+    live[r] = CHUNKS % NT == 0 || u_raw < CHUNKS;
+    const int u = live[r] ? u_raw : CHUNKS - 1;
+    is_v[r] = u >= 4 * D;
+    if (!is_v[r]) {
+      const int kk = u / (D / 8), part = u % (D / 8);
+      second_half[r] = kk >= 16;
+      src_base[r] = k_pages;
+      src_mul[r] = D;
+      src_off[r] = (kk % 16) * D + part * 8;
+      lds_off[r] = kk * KPAD + part * 8;
+      v_key[r] = 0;
+    } else {
+      const int c = u - 4 * D, d = c / 4, vk = (c % 4) * 8;
+      second_half[r] = vk >= 16;
+      src_base[r] = v_pages;
+      src_mul[r] = 1;
+      src_off[r] = d * page_size + vk % 16;
+      lds_off[r] = K_ELEMS + d * VPAD + vk;
+      v_key[r] = vk;
+    }
+  }
+  bf16x8 stage[RD][UCH];
   // Tiles are fetched in order, so the page of the tile's first key is tracked by addition
   // instead of division: `tile_page` indexes the block table, `tile_off` is the key's offset in it.
+  // Tiles start at multiples of 32 and pages hold a multiple of 16 keys, so each half of a tile
+  // lies in one page: the two page numbers are the same for every lane and are read through the
+  // scalar unit one tile ahead (`page_a`, `page_b`), which keeps the table lookup out of the
+  // vector memory queue where it would wait behind the tiles in flight.
   int tile_page = begin / page_size, tile_off = begin % page_size;
-  auto fetch = [&](int t, bf16x8 (&kq)[KCH], bf16x8 (&vq)[KCH]) {
-    const bool whole = t + 32 <= n_keys;  // every key of the tile exists
-#pragma unroll
-    for (int r = 0; r < KCH; ++r) {
-      const int c = threadIdx.x + r * 256;
-      kq[r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      vq[r] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (4 * D % 256 == 0 || c < 4 * D) {
-        const int kk = c / (D / 8), part = c % (D / 8);
-        int kp = tile_page, ko = tile_off + kk;
-        while (ko >= page_size) { ko -= page_size; ++kp; }
-        if (whole || t + kk < n_keys) {
-          const int64_t page = table[kp];
-          kq[r] = *reinterpret_cast<const bf16x8*>(
-              k_pages + ((page * kv_heads + kvh) * page_size + ko) * D + part * 8);
-        }
-        const int d = c / 4, vk = (c % 4) * 8;
-        int vp = tile_page, vo = tile_off + vk;
-        while (vo >= page_size) { vo -= page_size; ++vp; }
-        if (whole || t + vk < n_keys) {
-          const int64_t page = table[vp];
-          vq[r] = *reinterpret_cast<const bf16x8*>(v_pages + ((page * kv_heads + kvh) * D + d) * page_size + vo);
-          if (!whole && t + vk + 8 > n_keys) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-              if (t + vk + i >= n_keys) vq[r][i] = (bf16_t)0.f;
-          }
-        }
-      }
-    }
+  int page_a = 0, page_b = 0, off_a = 0, off_b = 0;
+  auto lookup = [&](int t) {
+    // table entries exist only for pages that hold keys
+    off_a = tile_off;
+    const int second = tile_off + 16 >= page_size ? 1 : 0;
+    off_b = tile_off + 16 - (second ? page_size : 0);
+    page_a = t < n_keys ? table[tile_page] : 0;
+    page_b = t + 16 < n_keys ? table[tile_page + second] : 0;
     tile_off += 32;
     while (tile_off >= page_size) { tile_off -= page_size; ++tile_page; }
   };
-  auto stash = [&](int buf, const bf16x8 (&kq)[KCH], const bf16x8 (&vq)[KCH]) {
+  lookup(begin);
+  // Every fetch issues the same loads whatever the tile, also for tiles past the last one (their
+  // halves read page 0 and are never used): the count of loads in flight is then known at compile
+  // time and a tile is awaited without draining the younger ones behind it. Keys past the last one
+  // of a half-filled page may hold anything: K rows there are masked as later than every query, V
+  // columns are cleared on the way into LDS.
+  const int64_t page_elems = (int64_t)page_size * D;
+  auto fetch = [&](int t, bf16x8 (&sq)[UCH]) {
+    const int64_t pa = ((int64_t)page_a * kv_heads + kvh) * page_elems;
+    const int64_t pb = ((int64_t)page_b * kv_heads + kvh) * page_elems;
+    const int oa = off_a, ob = off_b;
+    lookup(t + 32);
 #pragma unroll
-    for (int r = 0; r < KCH; ++r) {
-      const int c = threadIdx.x + r * 256;
-      if (c < 4 * D) {
-        *reinterpret_cast<bf16x8*>(&ks[buf][c / (D / 8)][(c % (D / 8)) * 8]) = kq[r];
-        *reinterpret_cast<bf16x8*>(&vs[buf][c / 4][(c % 4) * 8]) = vq[r];
+    for (int r = 0; r < UCH; ++r) {
+      const int64_t pg = second_half[r] ? pb : pa;
+      const int of = second_half[r] ? ob : oa;
+      sq[r] = *reinterpret_cast<const bf16x8*>(src_base[r] + pg + of * src_mul[r] + src_off[r]);
+    }
+  };
+  auto stash = [&](int buf, int t, bf16x8 (&sq)[UCH]) {
+#pragma unroll
+    for (int r = 0; r < UCH; ++r) {
+      if (live[r]) {
+        if (t + 32 > n_keys && is_v[r]) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (t + v_key[r] + i >= n_keys) sq[r][i] = (bf16_t)0.f;
+        }
+        *reinterpret_cast<bf16x8*>(&lds[buf][lds_off[r]]) = sq[r];
       }
     }
   };
@@ -475,10 +524,8 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
   // tiles 0 and 1 go straight to LDS; tile T >= 2 waits in register slot T % RD
 #pragma unroll
   for (int T = 0; T < 2 + RD; ++T) {
-    if (T < n_tiles) fetch(begin + T * 32, kst[T % RD], vst[T % RD]);
-    if (T < 2) {
-      if (T < n_tiles) stash(T, kst[T % RD], vst[T % RD]);
-    }
+    fetch(begin + T * 32, stage[T % RD]);
+    if (T < 2) stash(T, begin + T * 32, stage[T % RD]);
   }
   __syncthreads();
   for (int it0 = 0; it0 < n_tiles; it0 += RD) {
@@ -489,13 +536,15 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
     const int t = begin + it * 32, buf = it % 3;
     if (wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1)) {
       const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
+      const bf16_t* ks = &lds[buf][0];
+      const bf16_t* vs = &lds[buf][K_ELEMS];
       // all operand fragments of the tile are requested from LDS first, so that the reads of V
       // overlap the first product and the softmax
       bf16x8 kf0[DK], kf1[DK];
 #pragma unroll
       for (int c = 0; c < DK; ++c) {
-        kf0[c] = *reinterpret_cast<const bf16x8*>(&ks[buf][col][c * 32 + grp * 8]);
-        kf1[c] = *reinterpret_cast<const bf16x8*>(&ks[buf][16 + col][c * 32 + grp * 8]);
+        kf0[c] = *reinterpret_cast<const bf16x8*>(ks + col * KPAD + c * 32 + grp * 8);
+        kf1[c] = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KPAD + c * 32 + grp * 8);
       }
       typedef short short4a __attribute__((ext_vector_type(4)));
       union VFrag {
@@ -504,8 +553,8 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
       } vf[DCH];
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
-        vf[c].h[0] = *reinterpret_cast<const short4a*>(&vs[buf][c * 16 + col][4 * grp]);
-        vf[c].h[1] = *reinterpret_cast<const short4a*>(&vs[buf][c * 16 + col][16 + 4 * grp]);
+        vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 4 * grp);
+        vf[c].h[1] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 16 + 4 * grp);
       }
       // S^T of both column tiles, for the two halves of the tile: keys t+4g+i and t+16+4g+i
       float4v sa[2], sb[2];
@@ -575,10 +624,8 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
     }
     // tile it+2 leaves its register slot for LDS; the slot then receives tile it+2+RD
     const int slot = (r + 2) % RD;
-    if (it + 2 < n_tiles) {
-      stash((it + 2) % 3, kst[slot], vst[slot]);
-      if (it + 2 + RD < n_tiles) fetch(begin + (it + 2 + RD) * 32, kst[slot], vst[slot]);
-    }
+    stash((it + 2) % 3, begin + (it + 2) * 32, stage[slot]);
+    fetch(begin + (it + 2 + RD) * 32, stage[slot]);
     __syncthreads();
    }
   }
@@ -660,7 +707,8 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
                                           const int* block_tables, int table_stride,
                                           const int* tile_entry, const int* tile_q0, int tiles,
                                           int q_heads, int kv_heads, int head_dim, int page_size,
-                                          float scale, int window, hipStream_t stream) {
+                                          float scale, int window, int pair_tiles,
+                                          hipStream_t stream) {
   if (tiles <= 0) return DLI_OK;
   if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || q_heads > 65535 || q_stride % 4 != 0 || out_stride % 4 != 0)
@@ -668,12 +716,22 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (hw > 0) {
     const dim3 sgrid(tiles, q_heads / hw);
+    // Mirror tiles are paired (pair_tiles 1, or -1 and the launch large enough) while that still
+    // leaves every compute unit a workgroup. The tile list has to hold all tiles of a request.
+    const bool pair = pair_tiles >= 0 ? pair_tiles != 0
+                                      : (int64_t)tiles * (q_heads / hw) >= 2 * (int64_t)dli_compute_units();
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \
-    attention_prefill_shared_kernel<N><<<sgrid, 256, 0, stream>>>(                                \
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
-        out_stride, q_start, kv_len, block_tables, table_stride, tile_entry, tile_q0, q_heads,    \
-        kv_heads, page_size, scale * LOG2E, window, hw);                                          \
+    if (pair)                                                                                     \
+      attention_prefill_shared_kernel<N, true><<<sgrid, 512, 0, stream>>>(                        \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
+          (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \
+          tile_q0, q_heads, kv_heads, page_size, scale * LOG2E, window, hw);                      \
+    else                                                                                          \
+      attention_prefill_shared_kernel<N, false><<<sgrid, 256, 0, stream>>>(                       \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
+          (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \
+          tile_q0, q_heads, kv_heads, page_size, scale * LOG2E, window, hw);                      \
     break;
     switch (head_dim / 16) {
       SHARED_CASE(2) SHARED_CASE(4) SHARED_CASE(6) SHARED_CASE(8)

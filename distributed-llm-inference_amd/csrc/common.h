@@ -49,3 +49,16 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 static inline int dli_launch_status() {
   return hipGetLastError() == hipSuccess ? DLI_OK : DLI_ERR_LAUNCH;
 }
+
+// Compute units of the current device (256 if the runtime does not say), asked once per device.
+static inline int dli_compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}

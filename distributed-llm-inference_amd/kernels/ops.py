@@ -52,7 +52,8 @@ _SIGNATURES = {
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                                   _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+                                   _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                                   _c_ptr],
     "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                               _c_int, _c_int, _c_ptr],
@@ -470,9 +471,12 @@ def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
 def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
                       tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
-                      window: int = 0) -> None:
+                      window: int = 0, pair_tiles: Optional[bool] = None) -> None:
     """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
-    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height)."""
+    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height:
+    every tile of every listed request, in ascending order within a request). ``pair_tiles``:
+    whether one workgroup takes a tile and its mirror within the request, which evens out the
+    causal mask's triangle; ``None`` lets the kernel decide by the size of the launch."""
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
     for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
         _dense(t, name, torch.int32, 1)
@@ -484,7 +488,8 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
     _check(library().dli_attention_prefill_bf16(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tile_entry.shape[0], q_heads,
-        kv_heads, head_dim, page_size, float(scale), int(window), _stream()), "attention_prefill")
+        kv_heads, head_dim, page_size, float(scale), int(window), -1 if pair_tiles is None else int(pair_tiles),
+        _stream()), "attention_prefill")
 
 # ----------------------------------------------------------------------------- sampling
 

@@ -218,15 +218,19 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
 
 @pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37])
-def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window):
-    lens = [(2, 2), (7, 7), (33, 33), (5, 40), (2, 131), (129, 129), (16, 16), (31, 300), (140, 333), (1, 50)]
+@pytest.mark.parametrize("pair", [False, True])
+def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window, pair):
+    """Portions of every shape against their caches; `pair`: a workgroup takes a tile and its mirror
+    tile of the same request (odd and even numbers of tiles, one tile only, half-filled last tiles)."""
+    lens = [(2, 2), (7, 7), (33, 33), (5, 40), (2, 131), (129, 129), (16, 16), (31, 300), (140, 333), (1, 50),
+            (257, 257), (200, 420)]
     q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + bs)
     te, tq = _tiles(q_start, ops.attention_prefill_tile_rows(d, qh, kvh))
     dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
     out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
     scale = 1.0 / math.sqrt(d)
     ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables),
-                          dev(te), dev(tq), qh, scale, window)
+                          dev(te), dev(tq), qh, scale, window, pair_tiles=pair)
     ref = ref_paged_attention(q, kp, vp, q_start, kv_len, tables, qh, scale, window)
     err = (out.cpu().double() - ref).abs().max().item()
     assert err < tol(torch.bfloat16), err
