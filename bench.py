@@ -63,7 +63,11 @@ def decode_run(engine, cfg, batch, context, steps, warmup):
     from dli_amd.sampling import SamplingParams
 
     gen = torch.Generator().manual_seed(batch)
+    # Requests admitted first decode a token a step while the others still prefill; the prompts are
+    # shortened by that many steps so that no request outgrows `context` while the clock runs.
+    budget = engine.scheduler.config.max_num_batched_tokens
     prompt_len = context - steps - warmup - 1
+    prompt_len -= -(-batch * prompt_len // budget) + 1
     ids = []
     for i in range(batch):
         prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).tolist()

@@ -1,0 +1,336 @@
+// Matrix product for at most 16 rows of activations (decode): y[m][n] = sum_k xhat[m][k] * w[n][k],
+// built around the memory system rather than the matrix cores: a decode product streams each
+// weight once and is bound by how many bytes a compute unit's vector cache can accept per tag
+// lookup, so every load here covers whole 64-byte runs.
+//
+// Products use v_mfma_f32_4x4x4_16B_bf16: sixteen independent 4x4x4 blocks per instruction. Lane
+// l belongs to block l/4; as operand A it supplies row l%4 and four k values, as operand B column
+// l%4 and four k values; the result gives it column l%4 and the four rows. Here the sixteen blocks
+// are sixteen consecutive runs of eight k (a "chunk" of 128 k), rows are four neighbouring
+// features (a "quad") and columns four activation rows: lane l loads the 16 bytes at k = chunk*128
+// + 8*(l/4) of its feature's weight row, so that sixteen neighbouring lanes read four rows times 64
+// contiguous bytes, and does two products (k halves) per quad and group of four activation rows.
+// The blocks' partial sums are added at the end: lanes l, l^16, l^32, l^48 by lane swaps, the rest
+// and the waves' shares of k through LDS, always in the same order.
+//
+// A workgroup has KS waves that split k among themselves and owns FQ quads of features. Few
+// quads and many waves suit products with few features (every compute unit still gets a
+// workgroup, and many loads are in flight on each); more quads read the activations less often.
+//
+// Fused in (template switches), as in the product for more rows:
+//   NORM          xhat = cast(norm_w[k] * cast(x[m][k] * rs[m])), rs[m] = rsqrt(sum_k x^2 / K + eps)
+//                 from the parts of the row sums of squares that the producer of x left
+//                 (RMSNorm: src/dli/model/llama.py:40-44)
+//   EPI_STORE     y (+ bias) stored as bf16
+//   EPI_SWIGLU    half of the quads are gate rows n, half up rows n + up_offset:
+//                 stores cast(silu(gate)) * up (src/dli/model/llama.py:190)
+//   EPI_RESIDUAL  stream[m][n] = cast(stream[m][n] + cast(y + bias)) in place, and this tile's part
+//                 of sum_n stream[m][n]^2 for the norm that follows
+//   EPI_F32       y stored as float32 (logits)
+#include "common.h"
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2, EPI_F32 = 3 };
+
+union Frag16 {
+  u32x4 raw;
+  short4v h[2];
+  bf16_t e[8];
+};
+
+__device__ __forceinline__ float4v mfma4(short4v a, short4v b, float4v c) {
+  return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
+}
+
+template <int KS, int FQ, int MG, int EPI, bool NORM>
+__global__ __launch_bounds__(KS * 64) void skinny4_kernel(
+    const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
+    const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
+    const bf16_t* __restrict__ bias, void* __restrict__ out, int64_t ldo,
+    bf16_t* __restrict__ stream, int64_t lds_, float* __restrict__ ssq_out, int M, int N, int K,
+    int up_offset) {
+  constexpr int PAIRS = FQ * MG;                        // (quad, row group) accumulators per lane
+  constexpr int OQ = EPI == EPI_SWIGLU ? FQ / 2 : FQ;   // quads of output features per tile
+  __shared__ float4v red[KS][PAIRS][16];
+  __shared__ float4v fin[PAIRS][4];
+  __shared__ float sqs[OQ][MG][4];
+
+  const int lane = threadIdx.x % 64, ks = threadIdx.x / 64;
+  const int r = lane % 4, blk = lane / 4;
+  const int tile = blockIdx.x;
+  const int n_tile = tile * 4 * OQ;  // first output feature of the tile
+
+  // weight rows of this lane, one per quad (clamped at the matrix's end: computed and dropped)
+  const bf16_t* wrow[FQ];
+#pragma unroll
+  for (int f = 0; f < FQ; ++f) {
+    const int oq = f % OQ;
+    const int n = min(n_tile + 4 * oq + r, N - 1) + (f / OQ) * up_offset;
+    wrow[f] = w + (int64_t)n * K;
+  }
+  // activations through a buffer resource that ends after the last row: rows that do not exist
+  // and k past the end read zeros and cause no memory traffic
+  const unsigned x_bytes = (unsigned)(((int64_t)(M - 1) * ldx + K) * 2);
+  const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, x_bytes, 0x00020000);
+  int xrow[MG];
+  float rs[MG];
+#pragma unroll
+  for (int g = 0; g < MG; ++g) {
+    const int m = 4 * g + r;
+    xrow[g] = m < M ? (int)(m * ldx * 2) : -1;
+    rs[g] = 1.f;
+  }
+  if constexpr (NORM) {
+    // rs[m] from the parts of sum x^2: block b adds the parts b, b+16, ..., the blocks are added
+    // in a fixed order
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+      const int m = min(4 * g + r, M - 1);
+      float sum = 0.f;
+      for (int p = blk; p < ssq_parts; p += 16) sum += ssq_in[(int64_t)p * M + m];
+      sum += __shfl_xor(sum, 4, 64);
+      sum += __shfl_xor(sum, 8, 64);
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      rs[g] = rsqrtf(sum / (float)K + eps);
+    }
+  }
+
+  float4v acc[FQ][MG];
+#pragma unroll
+  for (int f = 0; f < FQ; ++f)
+#pragma unroll
+    for (int g = 0; g < MG; ++g) acc[f][g] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // chunks of 128 k: this wave's share
+  const int chunks = (K + 127) / 128;
+  const int c0 = chunks * ks / KS, c1 = chunks * (ks + 1) / KS;
+
+  struct Stage {
+    Frag16 wf[FQ], xf[MG];
+    float4v g0, g1;
+  };
+  // Every turn of the loop issues the same loads (the last one reads its own chunk again), so the
+  // number of loads in flight is known at compile time and only the current chunk is waited for.
+  auto fetch = [&](int c, Stage& st) {
+    const int k = c * 128 + blk * 8;
+    const bool inside = k < K;  // the last chunk may reach past k; K % 8 == 0
+    const int kc = inside ? k : 0;
+#pragma unroll
+    for (int f = 0; f < FQ; ++f) st.wf[f].raw = *reinterpret_cast<const u32x4*>(wrow[f] + kc);
+#pragma unroll
+    for (int g = 0; g < MG; ++g)
+      st.xf[g].raw = __builtin_amdgcn_raw_buffer_load_b128(
+          xres, inside && xrow[g] >= 0 ? xrow[g] + k * 2 : (int)x_bytes, 0, 0);
+    if constexpr (NORM) {
+      st.g0 = *reinterpret_cast<const float4v*>(norm_w + kc);
+      st.g1 = *reinterpret_cast<const float4v*>(norm_w + kc + 4);
+    }
+  };
+  if (c0 < c1) {
+    Stage cur;
+    fetch(c0, cur);
+    for (int c = c0; c < c1; ++c) {
+      Stage nxt;
+      fetch(min(c + 1, c1 - 1), nxt);
+      if constexpr (NORM) {
+#pragma unroll
+        for (int g = 0; g < MG; ++g)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float normed = (float)(bf16_t)((float)cur.xf[g].e[i] * rs[g]);
+            cur.xf[g].e[i] = (bf16_t)((i < 4 ? cur.g0[i] : cur.g1[i - 4]) * normed);
+          }
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int f = 0; f < FQ; ++f)
+#pragma unroll
+          for (int g = 0; g < MG; ++g) acc[f][g] = mfma4(cur.wf[f].h[h], cur.xf[g].h[h], acc[f][g]);
+      cur = nxt;
+    }
+  }
+
+  // blocks l/4 that differ in their upper two bits are added by lane swaps, the remaining four
+  // blocks and the waves through LDS
+#pragma unroll
+  for (int f = 0; f < FQ; ++f)
+#pragma unroll
+    for (int g = 0; g < MG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = acc[f][g][i];
+        v += __shfl_xor(v, 32, 64);
+        v += __shfl_xor(v, 16, 64);
+        acc[f][g][i] = v;
+      }
+  if (lane < 16) {
+#pragma unroll
+    for (int f = 0; f < FQ; ++f)
+#pragma unroll
+      for (int g = 0; g < MG; ++g) red[ks][f * MG + g][lane] = acc[f][g];
+  }
+  __syncthreads();
+  // thread t < 4*PAIRS owns the four features of quad f = p / MG for activation row m = 4g + rr
+  const int t = threadIdx.x;
+  const bool owner = t < 4 * PAIRS;
+  const int p = t / 4, rr = t % 4;
+  float4v total = {0.f, 0.f, 0.f, 0.f};
+  if (owner) {
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) total += red[k][p][4 * b + rr];
+  }
+  if (EPI == EPI_SWIGLU) {
+    if (owner) fin[p][rr] = total;
+    __syncthreads();
+  }
+  const int f = p / MG, g = p % MG;
+  const int m = 4 * g + rr;
+  const int nb = n_tile + 4 * f;
+  float sq = 0.f;
+  if (owner && f < OQ && m < M && nb < N) {
+    const bool whole = nb + 3 < N;
+    float y[2][4];
+#pragma unroll
+    for (int a = 0; a < (EPI == EPI_SWIGLU ? 2 : 1); ++a) {
+      const float4v src = EPI == EPI_SWIGLU ? fin[(f + a * OQ) * MG + g][rr] : total;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        y[a][i] = src[i] + (bias != nullptr && nb + i < N ? (float)bias[nb + i + a * up_offset] : 0.f);
+    }
+    if (EPI == EPI_F32) {
+      float* op = reinterpret_cast<float*>(out) + (int64_t)m * ldo + nb;
+      if (whole && ldo % 4 == 0) {
+        *reinterpret_cast<float4v*>(op) = float4v{y[0][0], y[0][1], y[0][2], y[0][3]};
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nb + i < N) op[i] = y[0][i];
+      }
+    } else {
+      bf16_t* op = EPI == EPI_RESIDUAL ? stream + (int64_t)m * lds_ + nb
+                                       : reinterpret_cast<bf16_t*>(out) + (int64_t)m * ldo + nb;
+      const bool vec = whole && (EPI == EPI_RESIDUAL ? lds_ : ldo) % 4 == 0;
+      union Pack4 {
+        short4v v;
+        bf16_t e[4];
+      } old, res;
+      if (EPI == EPI_RESIDUAL) {
+        if (vec) {
+          old.v = *reinterpret_cast<const short4v*>(op);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) old.e[i] = nb + i < N ? op[i] : (bf16_t)0.f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (EPI == EPI_STORE) {
+          res.e[i] = (bf16_t)y[0][i];
+        } else if (EPI == EPI_SWIGLU) {
+          const float gt = (float)(bf16_t)y[0][i], up = (float)(bf16_t)y[1][i];
+          const float sg = (float)(bf16_t)(gt / (1.f + expf(-gt)));
+          res.e[i] = (bf16_t)(sg * up);
+        } else {  // EPI_RESIDUAL: the sum in 32-bit, rounded to the stream's type
+          res.e[i] = (bf16_t)((float)old.e[i] + (float)(bf16_t)y[0][i]);
+          if (nb + i < N) sq += (float)res.e[i] * (float)res.e[i];
+        }
+      }
+      if (vec) {
+        *reinterpret_cast<short4v*>(op) = res.v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nb + i < N) op[i] = res.e[i];
+      }
+    }
+  }
+  if (EPI == EPI_RESIDUAL) {
+    // the tile's part of the row's sum of squares: the quads' shares, added in quad order
+    if (owner) sqs[f][g][rr] = sq;
+    __syncthreads();
+    if (owner && f == 0 && m < M) {
+      float s = 0.f;
+#pragma unroll
+      for (int q = 0; q < OQ; ++q) s += sqs[q][g][rr];
+      ssq_out[(int64_t)tile * M + m] = s;
+    }
+  }
+}
+
+#define S4_PARAMS                                                                                 \
+  const void *x, int64_t ldx, const float *ssq_in, int ssq_parts, const float *norm_w, float eps,   \
+      const void *w, const void *bias, void *out, int64_t ldo, void *stream_buf, int64_t lds_,      \
+      float *ssq_out, int M, int N, int K, int up_offset, hipStream_t stream
+#define S4_ARGS \
+  x, ldx, ssq_in, ssq_parts, norm_w, eps, w, bias, out, ldo, stream_buf, lds_, ssq_out, M, N, K, up_offset, stream
+
+template <int KS, int FQ, int MG, int EPI, bool NORM>
+static void launch4(S4_PARAMS) {
+  constexpr int OQ = EPI == EPI_SWIGLU ? FQ / 2 : FQ;
+  const int tiles = (N + 4 * OQ - 1) / (4 * OQ);
+  skinny4_kernel<KS, FQ, MG, EPI, NORM><<<tiles, KS * 64, 0, stream>>>(
+      (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
+      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
+}
+
+template <int KS, int FQ, int EPI, bool NORM>
+static void dispatch_rows(int mg, S4_PARAMS) {
+  if (mg == 1) launch4<KS, FQ, 1, EPI, NORM>(S4_ARGS);
+  else if (mg == 2) launch4<KS, FQ, 2, EPI, NORM>(S4_ARGS);
+  else launch4<KS, FQ, 4, EPI, NORM>(S4_ARGS);
+}
+
+// shapes of the workgroup: 0: 4 waves x 4 quads, 1: 8 waves x 2 quads, 2: 16 waves x 2 quads
+template <int EPI, bool NORM>
+static int dispatch4(int shape, int mg, S4_PARAMS) {
+  switch (shape) {
+    case 0: dispatch_rows<4, 4, EPI, NORM>(mg, S4_ARGS); break;
+    case 1: dispatch_rows<8, 2, EPI, NORM>(mg, S4_ARGS); break;
+    default: dispatch_rows<16, 2, EPI, NORM>(mg, S4_ARGS); break;
+  }
+  return dli_launch_status();
+}
+
+extern "C" int dli_skinny4_max_rows() { return 16; }
+
+// Output features per tile of workgroup shape `shape`: the residual epilogue leaves one part of
+// each row's sum of squares per tile.
+extern "C" int dli_skinny4_tile_features(int shape, int epilogue) {
+  const int fq = shape == 0 ? 4 : 2;
+  return epilogue == EPI_SWIGLU ? 2 * fq : 4 * fq;
+}
+
+// epilogue: 0 store bf16, 1 swiglu (N = features of one half, up rows at +up_offset), 2 residual,
+// 3 store float32. norm_w == nullptr: no norm. shape: see dispatch4.
+extern "C" int dli_skinny4_gemm(const void* x, int64_t ldx, const float* ssq_in, int ssq_parts,
+                                const float* norm_w, float eps, const void* w, const void* bias,
+                                void* out, int64_t ldo, void* stream_buf, int64_t lds_,
+                                float* ssq_out, int M, int N, int K, int up_offset, int epilogue,
+                                int shape, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return DLI_OK;
+  if (M > 16 || K <= 0 || K % 8 != 0 || ldx % 8 != 0 || ldx < K || (int64_t)M * ldx * 2 >= (int64_t)1 << 31 ||
+      shape < 0 || shape > 2 || epilogue < 0 || epilogue > 3 ||
+      (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)) ||
+      (epilogue == EPI_RESIDUAL && (stream_buf == nullptr || ssq_out == nullptr || norm_w != nullptr)) ||
+      (epilogue != EPI_RESIDUAL && out == nullptr))
+    return DLI_ERR_ARGUMENT;
+  const int mg = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
+  const bool norm = norm_w != nullptr;
+  switch (epilogue) {
+    case EPI_STORE:
+      return norm ? dispatch4<EPI_STORE, true>(shape, mg, S4_ARGS) : dispatch4<EPI_STORE, false>(shape, mg, S4_ARGS);
+    case EPI_SWIGLU:
+      return norm ? dispatch4<EPI_SWIGLU, true>(shape, mg, S4_ARGS) : dispatch4<EPI_SWIGLU, false>(shape, mg, S4_ARGS);
+    case EPI_RESIDUAL:
+      return dispatch4<EPI_RESIDUAL, false>(shape, mg, S4_ARGS);
+    default:
+      return norm ? dispatch4<EPI_F32, true>(shape, mg, S4_ARGS) : dispatch4<EPI_F32, false>(shape, mg, S4_ARGS);
+  }
+}

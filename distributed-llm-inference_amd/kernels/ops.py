@@ -35,6 +35,10 @@ _SIGNATURES = {
     "dli_to_float": [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
     "dli_copy_pages": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_i64, _c_int, _c_ptr],
     "dli_fill": [_c_ptr, _c_float, _c_i64, _c_int, _c_ptr],
+    "dli_skinny4_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
+                         _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_skinny4_tile_features": [_c_int, _c_int],
+    "dli_touch": [_c_ptr, _c_i64, _c_int, _c_ptr],
     "dli_rope_kv_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_f32_nt": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int,
@@ -201,6 +205,16 @@ def fill(x: torch.Tensor, value: float) -> None:
     _check(library().dli_fill(_ptr(x), float(value), x.numel(), _is_bf16(x.dtype), _stream()), "fill")
 
 
+def touch(x: torch.Tensor, workgroups: int) -> None:
+    """Read all of ``x`` with ``workgroups`` workgroups and keep nothing: brings it into the
+    memory-side cache ahead of the kernel that streams it."""
+    _dense(x, "x")
+    nbytes = x.numel() * x.element_size()
+    _require(nbytes % 16 == 0 and x.data_ptr() % 16 == 0, "touch takes 16-byte aligned memory in 16-byte units")
+    _require(1 <= workgroups <= 65535, "workgroups out of range")
+    _check(library().dli_touch(_ptr(x), nbytes, int(workgroups), _stream()), "touch")
+
+
 def copy_pages(pool: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
     """Copy page ``src[i]`` onto page ``dst[i]`` in every layer, keys and values.
 
@@ -299,18 +313,55 @@ def skinny_gemm_shape(n: int, k: int) -> int:
     return 1 if k >= 4096 else 0
 
 
+_compute_units: dict[int, int] = {}
+
+
+def _units(device: torch.device) -> int:
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _compute_units:
+        _compute_units[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return _compute_units[index]
+
+
+def skinny_gemm_plan(rows: int, n: int, k: int, epilogue: int, device: torch.device,
+                     blocks4: Optional[int] = None) -> tuple[str, int, int]:
+    """How :func:`skinny_gemm` runs a product: ``(kernel, shape, parts)``.
+
+    ``"blocks4"`` is the 4x4-block kernel (at most 16 rows), ``"tiles16"`` the 16x16-tile kernel
+    (at most 64 rows); ``shape`` is that kernel's workgroup shape. ``parts`` is the number of parts
+    that the residual epilogue leaves of each row's sum of squares. The choice follows cold-cache
+    timings on MI355X: the block kernel reads whole cache lines of the weights and only the rows of
+    activations that exist, which wins for one to four rows; with more rows the activations'
+    traffic grows and the tile kernel, which reads them once per 16 features, is ahead.
+    """
+    if blocks4 is None and rows <= 16 and k % 8 == 0:
+        deep = k >= 4096 and n <= 4096   # long rows, few features: many waves on narrow tiles
+        if rows <= 4:
+            out_feats = n * (2 if epilogue == SKINNY_SWIGLU else 1)
+            blocks4 = 2 if deep else (1 if out_feats <= 16 * _units(device) else 0)
+        elif deep:
+            blocks4 = 1
+    if blocks4 is not None:
+        feats = int(library().dli_skinny4_tile_features(blocks4, epilogue))
+        return "blocks4", blocks4, -(-n // feats)
+    return "tiles16", skinny_gemm_shape(n, k), -(-n // 16)
+
+
 def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optional[torch.Tensor] = None,
                 bias: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
                 ssq_in: Optional[torch.Tensor] = None, stream: Optional[torch.Tensor] = None,
-                ssq_out: Optional[torch.Tensor] = None, shape: Optional[int] = None) -> None:
+                ssq_out: Optional[torch.Tensor] = None, shape: Optional[int] = None,
+                blocks4: Optional[int] = None) -> Optional[torch.Tensor]:
     """``y = xhat @ w.T`` for at most 64 rows of bfloat16 ``x``, with fused surroundings.
 
     ``norm_w``/``eps``/``ssq_in [parts, rows]``: xhat is the RMSNorm of x, the row sums of squares
     being given in parts. Epilogues: ``SKINNY_STORE`` (``out`` bfloat16 ``[rows, n]``),
     ``SKINNY_SWIGLU`` (``w`` is ``[2n, k]``: gate rows then up rows; ``out [rows, n]`` gets
-    ``silu(gate) * up``), ``SKINNY_RESIDUAL`` (``stream [rows, n]`` becomes ``stream + y`` in place
-    and ``ssq_out [ceil(n/16), rows]`` receives the parts of its row sums of squares),
-    ``SKINNY_F32`` (``out`` float32).
+    ``silu(gate) * up``), ``SKINNY_RESIDUAL`` (``stream [rows, n]`` becomes ``stream + y`` in place;
+    the parts of its row sums of squares are returned as ``[parts, rows]``, in ``ssq_out`` if that
+    is given with the shape :func:`skinny_gemm_plan` names), ``SKINNY_F32`` (``out`` float32).
+    ``shape`` forces the 16x16-tile kernel with that workgroup shape, ``blocks4`` the 4x4-block
+    kernel with that one (at most 16 rows).
     """
     _rows(x, "x", torch.bfloat16)
     _dense(w, "w", torch.bfloat16, 2)
@@ -325,6 +376,13 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
     if bias is not None:
         _dense(bias, "bias", torch.bfloat16, 1)
         _require(bias.shape[0] == w.shape[0], "bias length differs from rows of w")
+    if shape is not None:
+        _require(shape in (0, 1, 2, 3), "shape must be 0..3")
+        kernel, a, n_parts = "tiles16", shape, -(-n // 16)
+    else:
+        if blocks4 is not None:
+            _require(blocks4 in (0, 1, 2) and m <= 16 and k % 8 == 0, "blocks4 must be 0..2, with at most 16 rows")
+        kernel, a, n_parts = skinny_gemm_plan(m, n, k, epilogue, x.device, blocks4)
     parts = 0
     if norm_w is not None:
         _require(epilogue != SKINNY_RESIDUAL, "the residual epilogue takes no fused norm")
@@ -336,22 +394,30 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
         parts = ssq_in.shape[0]
     ldo = lds = 0
     if epilogue == SKINNY_RESIDUAL:
-        _require(stream is not None and ssq_out is not None, "the residual epilogue needs stream and ssq_out")
+        _require(stream is not None, "the residual epilogue needs stream")
         _rows(stream, "stream", torch.bfloat16)
+        _require(stream.shape == (m, n), "stream must be [rows, n]")
+        if ssq_out is None:
+            ssq_out = torch.empty(n_parts, m, device=x.device, dtype=torch.float32)
         _dense(ssq_out, "ssq_out", torch.float32, 2)
-        _require(stream.shape == (m, n) and ssq_out.shape == (-(-n // 16), m), "stream [rows, n], ssq_out [ceil(n/16), rows]")
+        _require(ssq_out.shape == (n_parts, m), f"ssq_out must be [{n_parts}, rows] for this product")
+        _require(stream.data_ptr() % 8 == 0, "stream must be 8-byte aligned")
         lds = stream.stride(0)
     else:
         _require(out is not None, "this epilogue needs out")
         _rows(out, "out", torch.float32 if epilogue == SKINNY_F32 else torch.bfloat16)
         _require(out.shape == (m, n), "out must be [rows, n]")
+        _require(out.data_ptr() % 16 == 0, "out must be 16-byte aligned")
         ldo = out.stride(0)
-    if shape is None:
-        shape = skinny_gemm_shape(n, k)
-    _require(shape in (0, 1, 2, 3), "shape must be 0..3")
-    _check(library().dli_skinny_gemm(
-        _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
-        _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, shape, _stream()), "skinny_gemm")
+    if kernel == "tiles16":
+        _check(library().dli_skinny_gemm(
+            _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
+            _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, a, _stream()), "skinny_gemm")
+    else:
+        _check(library().dli_skinny4_gemm(
+            _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
+            _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, a, _stream()), "skinny4_gemm")
+    return ssq_out if epilogue == SKINNY_RESIDUAL else None
 
 
 def embedding_ssq(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, ssq: torch.Tensor) -> None:

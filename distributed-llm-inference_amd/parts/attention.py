@@ -130,6 +130,4 @@ class GQAttention(Mixer):
                           cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         out = self.rt.empty(n, nh * d)
         paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
-        ssq = torch.empty(-(-self.hidden_size // 16), n, device=self.rt.device, dtype=torch.float32)
-        ops.skinny_gemm(out, self.w_o, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, ssq_out=ssq, bias=self.b_o)
-        stream.ssq = ssq
+        stream.ssq = ops.skinny_gemm(out, self.w_o, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, bias=self.b_o)

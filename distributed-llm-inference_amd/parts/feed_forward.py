@@ -60,6 +60,5 @@ class GatedMLP(FeedForward):
         act = self.rt.empty(n, self.intermediate_size)
         ops.skinny_gemm(stream.x, self.w_gate_up, epilogue=ops.SKINNY_SWIGLU, out=act, bias=self.b_gate_up,
                         norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
-        ssq = torch.empty(-(-self.hidden_size // 16), n, device=self.rt.device, dtype=torch.float32)
-        ops.skinny_gemm(act, self.w_down, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, ssq_out=ssq, bias=self.b_down)
-        stream.ssq = ssq
+        stream.ssq = ops.skinny_gemm(act, self.w_down, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x,
+                                     bias=self.b_down)

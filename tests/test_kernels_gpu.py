@@ -328,6 +328,64 @@ def test_skinny_gemm_norm_and_swiglu(ops, m, inter, k, shape, parts):
     assert (y.cpu().double() - gu).abs().max() < 3e-2 * max(1.0, gu.abs().max().item())
 
 
+@pytest.mark.parametrize("m", [1, 3, 4, 5, 8, 9, 16])
+@pytest.mark.parametrize("n,k", [(48, 64), (100, 192), (301, 160), (512, 2048), (64, 416), (1000, 96), (2048, 8192)])
+@pytest.mark.parametrize("blocks4", [0, 1, 2])
+def test_skinny4_gemm_epilogues(ops, m, n, k, blocks4):
+    """The 4x4-block product: store, float32 and residual epilogues at sizes that are no multiples
+    of its tiles and chunks, in every workgroup shape."""
+    torch.manual_seed(m * 1000 + n)
+    x = torch.randn(m, k, device="cuda").bfloat16()
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    bias = torch.randn(n, device="cuda").bfloat16()
+    ref = x.cpu().double() @ w.cpu().double().T + bias.cpu().double()
+    kw = dict(blocks4=blocks4)
+    for _ in range(1):
+        out = torch.full((m, n), 7.0, device="cuda", dtype=torch.bfloat16)
+        ops.skinny_gemm(x, w, epilogue=ops.SKINNY_STORE, out=out, bias=bias, **kw)
+        assert (out.cpu().double() - ref).abs().max() < 3e-2
+    out32 = torch.empty(m, n, device="cuda")
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_F32, out=out32, **kw)
+    assert (out32.cpu().double() - (ref - bias.cpu().double())).abs().max() < 1e-4 * math.sqrt(k)
+    # a row's result does not depend on the other rows (same row group size: same kernel)
+    again = torch.empty(m, n, device="cuda")
+    x2 = x.clone()
+    x2[: m - 1] = torch.randn(m - 1, k, device="cuda").bfloat16()
+    ops.skinny_gemm(x2, w, epilogue=ops.SKINNY_F32, out=again, **kw)
+    assert torch.equal(again[m - 1], out32[m - 1])
+    # residual: stream += y, with the parts of its row sums of squares
+    stream = torch.randn(m, n, device="cuda").bfloat16()
+    before = stream.clone()
+    ssq = ops.skinny_gemm(x, w, epilogue=ops.SKINNY_RESIDUAL, stream=stream, bias=bias, **kw)
+    want = (before.float() + out.float()).bfloat16()
+    assert torch.equal(stream, want)
+    assert ssq.shape[1] == m and torch.allclose(ssq.sum(0), stream.float().pow(2).sum(-1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("m", [1, 8, 13])
+@pytest.mark.parametrize("blocks4", [0, 1, 2])
+@pytest.mark.parametrize("inter,k,parts", [(160, 64, 1), (500, 192, 5), (8192, 2048, 128)])
+def test_skinny4_gemm_norm_and_swiglu(ops, m, inter, k, parts, blocks4):
+    torch.manual_seed(m + inter)
+    x = (torch.randn(m, k, device="cuda") * 2).bfloat16()
+    nw = (1 + 0.1 * torch.randn(k, device="cuda")).float()
+    w = (torch.randn(2 * inter, k, device="cuda") / math.sqrt(k)).bfloat16()
+    xs = x.float().pow(2)
+    cut = torch.linspace(0, k, parts + 1).long().tolist()
+    ssq = torch.stack([xs[:, a:b].sum(-1) for a, b in zip(cut[:-1], cut[1:])]).contiguous()
+    eps = 1e-5
+    xhat = _ref_norm_bf16(x, nw, eps)
+    gu = (xhat.cpu().double() @ w.cpu().double().T)
+    g, u = gu[:, :inter].bfloat16().double(), gu[:, inter:].bfloat16().double()
+    ref = (g * torch.sigmoid(g)).bfloat16().double() * u
+    out = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_SWIGLU, out=out, norm_w=nw, eps=eps, ssq_in=ssq, blocks4=blocks4)
+    assert (out.cpu().double() - ref).abs().max() < 2e-2 * max(1.0, ref.abs().max().item())
+    y = torch.empty(m, 2 * inter, device="cuda", dtype=torch.bfloat16)
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_STORE, out=y, norm_w=nw, eps=eps, ssq_in=ssq, blocks4=blocks4)
+    assert (y.cpu().double() - gu).abs().max() < 3e-2 * max(1.0, gu.abs().max().item())
+
+
 def test_embedding_with_sum_of_squares(ops):
     table = torch.randn(50, 96, device="cuda").bfloat16()
     ids = torch.tensor([4, 49, 0, 4], dtype=torch.int32, device="cuda")
