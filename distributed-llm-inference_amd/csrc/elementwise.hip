@@ -203,26 +203,6 @@ static inline int grid_for(int64_t total, int threads) {
     }                                 \
   } while (0)
 
-// Reads `bytes` of memory (a multiple of 16) and keeps nothing: it brings weights that a later
-// kernel will stream into the memory-side cache while other kernels are busy elsewhere. `sink`
-// is never written (the sum of real data is not the impossible value tested for).
-__global__ __launch_bounds__(256) void touch_kernel(const uint4* __restrict__ p, int64_t chunks,
-                                                    unsigned* __restrict__ sink) {
-  unsigned acc = 0;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + 3 * stride < chunks; i += 4 * stride) {
-    const uint4 a = p[i], b = p[i + stride];
-    const uint4 c = p[i + 2 * stride], d = p[i + 3 * stride];
-    acc += (a.x ^ a.y ^ a.z ^ a.w) + (b.x ^ b.y ^ b.z ^ b.w) + (c.x ^ c.y ^ c.z ^ c.w) + (d.x ^ d.y ^ d.z ^ d.w);
-  }
-  for (; i < chunks; i += stride) {
-    const uint4 a = p[i];
-    acc += a.x ^ a.y ^ a.z ^ a.w;
-  }
-  if (acc == 0x9e3779b9u && sink != nullptr && chunks < 0) *sink = acc;
-}
-
 extern "C" {
 
 int dli_embedding(const void* table, const int* ids, void* out, int rows, int width, int is_bf16,
@@ -297,13 +277,6 @@ int dli_copy_pages(void* pool, const int* src, const int* dst, int ops, int plan
 int dli_fill(void* x, float value, int64_t total, int is_bf16, hipStream_t stream) {
   if (total <= 0) return DLI_OK;
   DISPATCH_DTYPE(is_bf16, (fill_kernel<T><<<grid_for(total, 256), 256, 0, stream>>>((T*)x, value, total)));
-  return dli_launch_status();
-}
-
-int dli_touch(const void* p, int64_t bytes, int workgroups, hipStream_t stream) {
-  if (bytes <= 0) return DLI_OK;
-  if (bytes % 16 != 0 || workgroups <= 0 || workgroups > 65535) return DLI_ERR_ARGUMENT;
-  touch_kernel<<<workgroups, 256, 0, stream>>>((const uint4*)p, bytes / 16, nullptr);
   return dli_launch_status();
 }
 

@@ -38,7 +38,6 @@ _SIGNATURES = {
     "dli_skinny4_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
                          _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_skinny4_tile_features": [_c_int, _c_int],
-    "dli_touch": [_c_ptr, _c_i64, _c_int, _c_ptr],
     "dli_rope_kv_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_f32_nt": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int,
@@ -203,16 +202,6 @@ def to_float(x: torch.Tensor, out: torch.Tensor) -> None:
 def fill(x: torch.Tensor, value: float) -> None:
     _dense(x, "x")
     _check(library().dli_fill(_ptr(x), float(value), x.numel(), _is_bf16(x.dtype), _stream()), "fill")
-
-
-def touch(x: torch.Tensor, workgroups: int) -> None:
-    """Read all of ``x`` with ``workgroups`` workgroups and keep nothing: brings it into the
-    memory-side cache ahead of the kernel that streams it."""
-    _dense(x, "x")
-    nbytes = x.numel() * x.element_size()
-    _require(nbytes % 16 == 0 and x.data_ptr() % 16 == 0, "touch takes 16-byte aligned memory in 16-byte units")
-    _require(1 <= workgroups <= 65535, "workgroups out of range")
-    _check(library().dli_touch(_ptr(x), nbytes, int(workgroups), _stream()), "touch")
 
 
 def copy_pages(pool: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
