@@ -189,14 +189,37 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
 
   ColumnTile<DCH> st;
   st.init();
-  for (int t = k0 + wave * 16; t < k1; t += 64) {
-    const int64_t page = table[t / page_size];
-    const int off = t % page_size;
-    short4v kreg[DCH], vreg[DCH];
-    load_k<DCH>(kreg, k_pages, page, kv_heads, kvh, page_size, off, col, grp);
-    load_v<DCH>(vreg, v_pages, page, kv_heads, kvh, page_size, off, col, grp, t, k1);
-    const bool need_mask = t + 16 > k1 || t < first_visible;
-    attend_tile<DCH>(st, kreg, qreg, vreg, t, grp, k1 - 1, first_visible, scale_log2e, need_mask);
+  // A wave takes every fourth tile of 16 keys. The step is as long as its chain of dependent
+  // memory accesses, so the tiles are taken UN at a time: first all their block-table entries,
+  // then all their keys and values, then the arithmetic. Tiles past the end read page 0 and are
+  // skipped.
+  constexpr int UN = DCH <= 4 ? 4 : 2;
+  int tp = (k0 + wave * 16) / page_size, toff = (k0 + wave * 16) % page_size;
+  for (int t0 = k0 + wave * 16; t0 < k1; t0 += 64 * UN) {
+    int64_t page[UN];
+    int off[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int t = t0 + 64 * u;
+      page[u] = t < k1 ? table[tp] : 0;
+      off[u] = toff;
+      toff += 64;
+      while (toff >= page_size) { toff -= page_size; ++tp; }
+    }
+    short4v kreg[UN][DCH], vreg[UN][DCH];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      load_k<DCH>(kreg[u], k_pages, page[u], kv_heads, kvh, page_size, off[u], col, grp);
+      load_v<DCH>(vreg[u], v_pages, page[u], kv_heads, kvh, page_size, off[u], col, grp, t0 + 64 * u, k1);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int t = t0 + 64 * u;
+      if (t < k1) {
+        const bool need_mask = t + 16 > k1 || t < first_visible;
+        attend_tile<DCH>(st, kreg[u], qreg, vreg[u], t, grp, k1 - 1, first_visible, scale_log2e, need_mask);
+      }
+    }
   }
 
   // merge the four waves' states in wave 0
@@ -251,27 +274,61 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   }
 }
 
-// grid (q_heads, requests), 64 threads: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
-__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
-                                                             const float* __restrict__ part_ml,
-                                                             bf16_t* __restrict__ out,
-                                                             int64_t out_stride, int q_heads,
-                                                             int head_dim, int splits) {
-  const int head = blockIdx.x, e = blockIdx.y;
-  const int64_t base = ((int64_t)e * q_heads + head) * splits;
-  float m_all = -INFINITY;
-  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
-  const float m_safe = m_all == -INFINITY ? 0.f : m_all;
-  float l_all = 0.f;
-  for (int s = 0; s < splits; ++s)
-    l_all += part_ml[(base + s) * 2 + 1] * fast_exp2(part_ml[(base + s) * 2] - m_safe);
-  const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
-  for (int d = threadIdx.x; d < head_dim; d += 64) {
-    float acc = 0.f;
-    for (int s = 0; s < splits; ++s)
-      acc += part_o[(base + s) * head_dim + d] * fast_exp2(part_ml[(base + s) * 2] - m_safe);
-    out[(int64_t)e * out_stride + (int64_t)head * head_dim + d] = (bf16_t)(acc * inv);
+// One wave per (request, head), four to a workgroup: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+// Lane s reads the statistics of split s and every lane the partial outputs of up to SMAX splits
+// for its dims, all before anything is used: the kernel is one round trip to memory long. The
+// weights 2^(m_s - M) then go from lane to lane and the splits are added in their order.
+// head_dim <= 64 * DV; more than SMAX splits are taken SMAX at a time.
+template <int SMAX, int DV>
+__global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                              const float* __restrict__ part_ml,
+                                                              bf16_t* __restrict__ out,
+                                                              int64_t out_stride, int q_heads,
+                                                              int head_dim, int splits, int pairs) {
+  const int lane = threadIdx.x % DLI_WAVE;
+  const int pair = blockIdx.x * 4 + threadIdx.x / DLI_WAVE;  // request * q_heads + head
+  if (pair >= pairs) return;
+  const int e = pair / q_heads, head = pair % q_heads;
+  const int64_t base = (int64_t)pair * splits;
+  float m_run = -INFINITY, l_run = 0.f;
+  float acc[DV];
+#pragma unroll
+  for (int v = 0; v < DV; ++v) acc[v] = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += SMAX) {
+    const int n = min(SMAX, splits - s0);
+    float m_s = -INFINITY, l_s = 0.f;
+    if (lane < n) {
+      m_s = part_ml[(base + s0 + lane) * 2];
+      l_s = part_ml[(base + s0 + lane) * 2 + 1];
+    }
+    float po[SMAX][DV];
+#pragma unroll
+    for (int j = 0; j < SMAX; ++j)
+#pragma unroll
+      for (int v = 0; v < DV; ++v) {
+        const bool live = j < n && v * DLI_WAVE + lane < head_dim;
+        po[j][v] = live ? part_o[(base + s0 + j) * head_dim + v * DLI_WAVE + lane] : 0.f;
+      }
+    const float m_new = fmaxf(m_run, wave_max(m_s));
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float keep = fast_exp2(m_run - m_safe);  // rescales what earlier rounds left
+    const float weight = lane < n ? fast_exp2(m_s - m_safe) : 0.f;
+    l_run = l_run * keep + wave_sum(l_s * weight);
+#pragma unroll
+    for (int v = 0; v < DV; ++v) acc[v] *= keep;
+#pragma unroll
+    for (int j = 0; j < SMAX; ++j) {
+      const float wj = __shfl(weight, j, DLI_WAVE);
+#pragma unroll
+      for (int v = 0; v < DV; ++v) acc[v] += po[j][v] * wj;
+    }
+    m_run = m_new;
   }
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+#pragma unroll
+  for (int v = 0; v < DV; ++v)
+    if (v * DLI_WAVE + lane < head_dim)
+      out[(int64_t)e * out_stride + (int64_t)head * head_dim + v * DLI_WAVE + lane] = (bf16_t)(acc[v] * inv);
 }
 
 // ------------------------------------------------------------------------------------ prefill
@@ -695,8 +752,19 @@ extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const 
 #undef DECODE_CASE
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   if (splits > 1) {
-    attention_merge_kernel<<<dim3(q_heads, requests), 64, 0, stream>>>(
-        part_o, part_ml, (bf16_t*)out, out_stride, q_heads, head_dim, splits);
+    const int pairs = requests * q_heads;
+#define MERGE(S, V)                                                             \
+  attention_merge_kernel<S, V><<<(pairs + 3) / 4, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, \
+                                                                    out_stride, q_heads, head_dim, splits, pairs)
+    if (head_dim <= 64) {
+      if (splits <= 8) MERGE(8, 1);
+      else if (splits <= 16) MERGE(16, 1);
+      else MERGE(32, 1);
+    } else {
+      if (splits <= 8) MERGE(8, 2);
+      else MERGE(16, 2);
+    }
+#undef MERGE
   }
   return dli_launch_status();
 }
