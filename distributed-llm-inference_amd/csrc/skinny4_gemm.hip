@@ -84,17 +84,37 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     rs[g] = 1.f;
   }
   if constexpr (NORM) {
-    // rs[m] from the parts of sum x^2: block b adds the parts b, b+16, ..., the blocks are added
-    // in a fixed order
+    // rs[m] from the parts of sum x^2. The parts are dealt out to all blocks of all waves (block
+    // q of 16*KS takes the parts q, q + 16*KS, ...), eight loads at a time so that they share one
+    // trip to memory; a wave adds its blocks, the waves' sums meet in LDS and are added in wave
+    // order.
+    __shared__ float rsum[KS][MG][4];
 #pragma unroll
     for (int g = 0; g < MG; ++g) {
       const int m = min(4 * g + r, M - 1);
       float sum = 0.f;
-      for (int p = blk; p < ssq_parts; p += 16) sum += ssq_in[(int64_t)p * M + m];
+      for (int p0 = ks * 16 + blk; p0 < ssq_parts; p0 += 128 * KS) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int p = p0 + u * 16 * KS;
+          v[u] = p < ssq_parts ? ssq_in[(int64_t)p * M + m] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+      }
       sum += __shfl_xor(sum, 4, 64);
       sum += __shfl_xor(sum, 8, 64);
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
+      if (blk == 0) rsum[ks][g][r] = sum;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+      float sum = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < KS; ++wv) sum += rsum[wv][g][r];
       rs[g] = rsqrtf(sum / (float)K + eps);
     }
   }

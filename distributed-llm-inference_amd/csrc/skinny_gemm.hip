@@ -111,17 +111,36 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
     rs[t] = 1.f;
   }
   if constexpr (NORM) {
-    // rs[m] from the parts of sum x^2 that the producer of x left. Every wave computes the rows of
-    // its own lanes: lane group g adds the parts p = g, g+4, ... of row m = 16t + col, the four
-    // groups are added in a fixed order.
+    // rs[m] from the parts of sum x^2 that the producer of x left. The parts are dealt out to
+    // all lane groups of all waves (group q of W*4 takes the parts q, q + 4W, ...), eight loads
+    // at a time so that they share one trip to memory; a wave adds its four groups, the waves'
+    // sums meet in LDS and are added in wave order.
+    constexpr int W = KS * NS;
+    __shared__ float rsum[W][MT][16];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const int m = min(t * 16 + col, M - 1);
       float sum = 0.f;
-#pragma unroll 8
-      for (int p = grp; p < ssq_parts; p += 4) sum += ssq_in[(int64_t)p * M + m];
+      for (int p0 = wave * 4 + grp; p0 < ssq_parts; p0 += 32 * W) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int p = p0 + u * 4 * W;
+          v[u] = p < ssq_parts ? ssq_in[(int64_t)p * M + m] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+      }
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
+      if (grp == 0) rsum[wave][t][col] = sum;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float sum = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < W; ++wv) sum += rsum[wv][t][col];
       rs[t] = rsqrtf(sum / (float)K + eps);
     }
   }
