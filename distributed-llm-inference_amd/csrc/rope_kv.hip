@@ -11,9 +11,12 @@
 // Dimensions at and beyond rotary_dim pass through. inv_freq == nullptr means no rotation.
 #include "common.h"
 
-// One workgroup per token: cos/sin of the token's angles are computed once into LDS, then the
-// threads walk the token's q heads (rotated in place), k heads (rotated into the page) and v heads
-// (copied into the transposed page).
+// A token's work is a list of items: the rotary pairs of its q and k heads, the dimensions of k
+// beyond the rotary part, and the values of v. Each thread takes one item, workgroup y of a token
+// the items [256y, 256y + 256). A thread first asks for its operands, then the first threads of
+// the workgroup compute the token's cos/sin into LDS (every workgroup its own copy), then the
+// items are finished: what a thread reads does not wait for the angles, so the kernel is one trip
+// to memory long.
 #define ROPE_MAX_HALF 128
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(
@@ -24,55 +27,63 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   const int64_t token = blockIdx.x;
   T* row = qkv + token * row_stride;
+  const int half = rotary_dim / 2, rest = head_dim - rotary_dim;
+  const int n_pairs = (q_heads + kv_heads) * half, n_rest = kv_heads * rest, n_v = kv_heads * head_dim;
+  const int item = blockIdx.y * 256 + threadIdx.x;
+
+  // operands first
+  int kind = 3, head = 0, i = 0;  // 0 pair, 1 rest of k, 2 v, 3 nothing
+  float x1 = 0.f, x2 = 0.f;
+  if (item < n_pairs) {
+    kind = 0;
+    head = item / half;
+    i = item - head * half;
+    const T* h = row + (int64_t)head * head_dim;
+    x1 = to_f32(h[i]);
+    x2 = to_f32(h[i + half]);
+  } else if (item < n_pairs + n_rest) {
+    kind = 1;
+    head = (item - n_pairs) / rest;
+    i = rotary_dim + (item - n_pairs) - head * rest;
+    x1 = to_f32(row[(int64_t)(q_heads + head) * head_dim + i]);
+  } else if (item < n_pairs + n_rest + n_v) {
+    kind = 2;
+    head = (item - n_pairs - n_rest) / head_dim;
+    i = (item - n_pairs - n_rest) - head * head_dim;
+    x1 = to_f32(row[(int64_t)(q_heads + kv_heads + head) * head_dim + i]);
+  }
   const int slot = slots != nullptr ? slots[token] : -1;
-  const int64_t page = slot >= 0 ? slot / page_size : 0;
-  const int off = slot >= 0 ? slot % page_size : 0;
-  const int half = rotary_dim / 2;
   const float pos = (float)positions[token];
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
-    float c = 1.f, s = 0.f;
+  if (threadIdx.x < half) {
+    float c = 1.f, sv = 0.f;
     if (inv_freq != nullptr) {
-      sincosf(pos * inv_freq[i], &s, &c);
+      sincosf(pos * inv_freq[threadIdx.x], &sv, &c);
       c = round_to<T>(c);
-      s = round_to<T>(s);
+      sv = round_to<T>(sv);
     }
-    cs[i] = c;
-    sn[i] = s;
+    cs[threadIdx.x] = c;
+    sn[threadIdx.x] = sv;
   }
   __syncthreads();
   const bool cache = slot >= 0 && k_pages != nullptr && v_pages != nullptr;
-
-  // q and k heads: pairs (i, i + half) of the rotary part
-  const int rot_heads = q_heads + kv_heads;
-  if (half > 0) {
-    for (int idx = threadIdx.x; idx < rot_heads * half; idx += blockDim.x) {
-      const int head = idx / half, i = idx - head * half;
+  const int64_t page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  if (kind == 0) {
+    const T y1 = from_f32<T>(x1 * cs[i] - x2 * sn[i]);
+    const T y2 = from_f32<T>(x2 * cs[i] + x1 * sn[i]);
+    if (head < q_heads) {
       T* h = row + (int64_t)head * head_dim;
-      const float x1 = to_f32(h[i]), x2 = to_f32(h[i + half]);
-      const T y1 = from_f32<T>(x1 * cs[i] - x2 * sn[i]);
-      const T y2 = from_f32<T>(x2 * cs[i] + x1 * sn[i]);
-      if (head < q_heads) {
-        h[i] = y1;
-        h[i + half] = y2;
-      } else if (cache) {
-        T* kd = k_pages + ((page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
-        kd[i] = y1;
-        kd[i + half] = y2;
-      }
+      h[i] = y1;
+      h[i + half] = y2;
+    } else if (cache) {
+      T* kd = k_pages + ((page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
+      kd[i] = y1;
+      kd[i + half] = y2;
     }
-  }
-  if (!cache) return;
-  // the part of k beyond the rotary dimensions passes through
-  const int rest = head_dim - rotary_dim;
-  for (int idx = threadIdx.x; idx < kv_heads * rest; idx += blockDim.x) {
-    const int h = idx / rest, i = rotary_dim + idx - h * rest;
-    k_pages[((page * kv_heads + h) * page_size + off) * head_dim + i] = row[(int64_t)(q_heads + h) * head_dim + i];
-  }
-  // v heads into the transposed page
-  const T* v = row + (int64_t)(q_heads + kv_heads) * head_dim;
-  for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x) {
-    const int h = idx / head_dim, i = idx - h * head_dim;
-    v_pages[((page * kv_heads + h) * head_dim + i) * page_size + off] = v[idx];
+  } else if (kind == 1) {
+    if (cache) k_pages[((page * kv_heads + head) * page_size + off) * head_dim + i] = from_f32<T>(x1);
+  } else if (kind == 2) {
+    if (cache) v_pages[((page * kv_heads + head) * head_dim + i) * page_size + off] = from_f32<T>(x1);
   }
 }
 
@@ -85,12 +96,17 @@ extern "C" int dli_rope_kv_write(void* qkv, int64_t row_stride, const int* posit
       rotary_dim / 2 > ROPE_MAX_HALF || q_heads < 0 || kv_heads < 0 || page_size <= 0 ||
       q_heads + 2 * kv_heads <= 0)
     return DLI_ERR_ARGUMENT;
+  const int half = rotary_dim / 2;
+  const int items = (q_heads + kv_heads) * half + kv_heads * (head_dim - rotary_dim) + kv_heads * head_dim;
+  if (items <= 0) return DLI_OK;
+  const dim3 grid(tokens, (items + 255) / 256);
+  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
   if (is_bf16)
-    rope_kv_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>(
+    rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, positions, inv_freq, rotary_dim, slots, (bf16_t*)k_pages,
         (bf16_t*)v_pages, q_heads, kv_heads, head_dim, page_size);
   else
-    rope_kv_write_kernel<float><<<tokens, 256, 0, stream>>>(
+    rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
         (float*)qkv, row_stride, positions, inv_freq, rotary_dim, slots, (float*)k_pages,
         (float*)v_pages, q_heads, kv_heads, head_dim, page_size);
   return dli_launch_status();
