@@ -12,46 +12,58 @@
 #include "common.h"
 
 // A token's work is a list of items: the rotary pairs of its q and k heads, the dimensions of k
-// beyond the rotary part, and the values of v. Each thread takes one item, workgroup y of a token
-// the items [256y, 256y + 256). A thread first asks for its operands, then the first threads of
-// the workgroup compute the token's cos/sin into LDS (every workgroup its own copy), then the
-// items are finished: what a thread reads does not wait for the angles, so the kernel is one trip
-// to memory long.
+// beyond the rotary part, and the values of v. Workgroup y of a token takes the items y*256 + t,
+// (y + gridDim.y)*256 + t, ... With few tokens (decode) there are as many workgroups per token as
+// it takes to give each thread one item; with many (prefill) one workgroup per token, so that
+// the token's cos/sin are computed once. A thread asks for the operands of its first item before
+// the angles are computed (every workgroup its own copy in LDS): what it reads does not wait for
+// them, and with one item per thread the kernel is one trip to memory long.
 #define ROPE_MAX_HALF 128
+template <typename T>
+struct RopeItem {
+  int kind, head, i;  // kind: 0 pair, 1 rest of k, 2 v, 3 nothing
+  float x1, x2;
+};
+
+template <typename T>
+__device__ __forceinline__ RopeItem<T> rope_fetch(const T* __restrict__ row, int item, int half,
+                                                  int rest, int rotary_dim, int q_heads, int kv_heads,
+                                                  int head_dim) {
+  const int n_pairs = (q_heads + kv_heads) * half, n_rest = kv_heads * rest, n_v = kv_heads * head_dim;
+  RopeItem<T> it{3, 0, 0, 0.f, 0.f};
+  if (item < n_pairs) {
+    it.kind = 0;
+    it.head = item / half;
+    it.i = item - it.head * half;
+    const T* h = row + (int64_t)it.head * head_dim;
+    it.x1 = to_f32(h[it.i]);
+    it.x2 = to_f32(h[it.i + half]);
+  } else if (item < n_pairs + n_rest) {
+    it.kind = 1;
+    it.head = (item - n_pairs) / rest;
+    it.i = rotary_dim + (item - n_pairs) - it.head * rest;
+    it.x1 = to_f32(row[(int64_t)(q_heads + it.head) * head_dim + it.i]);
+  } else if (item < n_pairs + n_rest + n_v) {
+    it.kind = 2;
+    it.head = (item - n_pairs - n_rest) / head_dim;
+    it.i = (item - n_pairs - n_rest) - it.head * head_dim;
+    it.x1 = to_f32(row[(int64_t)(q_heads + kv_heads + it.head) * head_dim + it.i]);
+  }
+  return it;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions,
     const float* __restrict__ inv_freq, int rotary_dim, const int* __restrict__ slots,
     T* __restrict__ k_pages, T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim,
-    int page_size) {
+    int page_size, int items) {
   __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   const int64_t token = blockIdx.x;
   T* row = qkv + token * row_stride;
   const int half = rotary_dim / 2, rest = head_dim - rotary_dim;
-  const int n_pairs = (q_heads + kv_heads) * half, n_rest = kv_heads * rest, n_v = kv_heads * head_dim;
-  const int item = blockIdx.y * 256 + threadIdx.x;
-
-  // operands first
-  int kind = 3, head = 0, i = 0;  // 0 pair, 1 rest of k, 2 v, 3 nothing
-  float x1 = 0.f, x2 = 0.f;
-  if (item < n_pairs) {
-    kind = 0;
-    head = item / half;
-    i = item - head * half;
-    const T* h = row + (int64_t)head * head_dim;
-    x1 = to_f32(h[i]);
-    x2 = to_f32(h[i + half]);
-  } else if (item < n_pairs + n_rest) {
-    kind = 1;
-    head = (item - n_pairs) / rest;
-    i = rotary_dim + (item - n_pairs) - head * rest;
-    x1 = to_f32(row[(int64_t)(q_heads + head) * head_dim + i]);
-  } else if (item < n_pairs + n_rest + n_v) {
-    kind = 2;
-    head = (item - n_pairs - n_rest) / head_dim;
-    i = (item - n_pairs - n_rest) - head * head_dim;
-    x1 = to_f32(row[(int64_t)(q_heads + kv_heads + head) * head_dim + i]);
-  }
+  int item = blockIdx.y * 256 + threadIdx.x;
+  RopeItem<T> it = rope_fetch<T>(row, item, half, rest, rotary_dim, q_heads, kv_heads, head_dim);
   const int slot = slots != nullptr ? slots[token] : -1;
   const float pos = (float)positions[token];
   if (threadIdx.x < half) {
@@ -68,22 +80,27 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   const bool cache = slot >= 0 && k_pages != nullptr && v_pages != nullptr;
   const int64_t page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot % page_size : 0;
-  if (kind == 0) {
-    const T y1 = from_f32<T>(x1 * cs[i] - x2 * sn[i]);
-    const T y2 = from_f32<T>(x2 * cs[i] + x1 * sn[i]);
-    if (head < q_heads) {
-      T* h = row + (int64_t)head * head_dim;
-      h[i] = y1;
-      h[i + half] = y2;
-    } else if (cache) {
-      T* kd = k_pages + ((page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
-      kd[i] = y1;
-      kd[i + half] = y2;
+  while (true) {
+    if (it.kind == 0) {
+      const T y1 = from_f32<T>(it.x1 * cs[it.i] - it.x2 * sn[it.i]);
+      const T y2 = from_f32<T>(it.x2 * cs[it.i] + it.x1 * sn[it.i]);
+      if (it.head < q_heads) {
+        T* h = row + (int64_t)it.head * head_dim;
+        h[it.i] = y1;
+        h[it.i + half] = y2;
+      } else if (cache) {
+        T* kd = k_pages + ((page * kv_heads + (it.head - q_heads)) * page_size + off) * head_dim;
+        kd[it.i] = y1;
+        kd[it.i + half] = y2;
+      }
+    } else if (it.kind == 1) {
+      if (cache) k_pages[((page * kv_heads + it.head) * page_size + off) * head_dim + it.i] = from_f32<T>(it.x1);
+    } else if (it.kind == 2) {
+      if (cache) v_pages[((page * kv_heads + it.head) * head_dim + it.i) * page_size + off] = from_f32<T>(it.x1);
     }
-  } else if (kind == 1) {
-    if (cache) k_pages[((page * kv_heads + head) * page_size + off) * head_dim + i] = from_f32<T>(x1);
-  } else if (kind == 2) {
-    if (cache) v_pages[((page * kv_heads + head) * head_dim + i) * page_size + off] = from_f32<T>(x1);
+    item += gridDim.y * 256;
+    if (item >= items) break;
+    it = rope_fetch<T>(row, item, half, rest, rotary_dim, q_heads, kv_heads, head_dim);
   }
 }
 
@@ -99,15 +116,15 @@ extern "C" int dli_rope_kv_write(void* qkv, int64_t row_stride, const int* posit
   const int half = rotary_dim / 2;
   const int items = (q_heads + kv_heads) * half + kv_heads * (head_dim - rotary_dim) + kv_heads * head_dim;
   if (items <= 0) return DLI_OK;
-  const dim3 grid(tokens, (items + 255) / 256);
-  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
+  // a thread an item while that still leaves few workgroups; else one workgroup per token
+  const dim3 grid(tokens, tokens <= 64 ? min((items + 255) / 256, 64) : 1);
   if (is_bf16)
     rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, positions, inv_freq, rotary_dim, slots, (bf16_t*)k_pages,
-        (bf16_t*)v_pages, q_heads, kv_heads, head_dim, page_size);
+        (bf16_t*)v_pages, q_heads, kv_heads, head_dim, page_size, items);
   else
     rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
         (float*)qkv, row_stride, positions, inv_freq, rotary_dim, slots, (float*)k_pages,
-        (float*)v_pages, q_heads, kv_heads, head_dim, page_size);
+        (float*)v_pages, q_heads, kv_heads, head_dim, page_size, items);
   return dli_launch_status();
 }
