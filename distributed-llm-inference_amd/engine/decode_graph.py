@@ -173,46 +173,63 @@ class DecodeGraphs:
         v = cap.views
         limit = self.step_fn.store.num_pages
         token_ids, positions, kv_len, state_slots = v["token_ids"], v["positions"], v["kv_len"], v["state_slots"]
+        # The step's arrays are filled in bulk (one conversion per array instead of one per number):
+        # at large batches this loop is a visible part of the step.
+        toks = [int(e.tokens[0]) for e in entries]
+        starts = [e.start for e in entries]
+        if min(toks) < 0 or max(toks) >= self.step_fn.vocab_size:
+            bad = next(e for e, t in zip(entries, toks) if not 0 <= t < self.step_fn.vocab_size)
+            raise ValueError(f"request {bad.seq_id!r}: token id {int(bad.tokens[0])} outside the vocabulary")
+        token_ids[:n] = toks
+        positions[:n] = starts
+        np.add(positions[:n], 1, out=kv_len[:n])
         kv_len[n:] = 0
         token_ids[n:] = 0
         positions[n:] = 0
+        state_slots[:n] = [mgr.state_slot(e.seq_id) for e in entries]
         rows = []
         for i, e in enumerate(entries):
-            tok = int(e.tokens[0])
-            if not 0 <= tok < self.step_fn.vocab_size:
-                raise ValueError(f"request {e.seq_id!r}: token id {tok} outside the vocabulary")
-            token_ids[i] = tok
-            positions[i] = e.start
-            kv_len[i] = e.start + 1
-            state_slots[i] = mgr.state_slot(e.seq_id)
-            known = cap.rows[i]
-            for g in range(self.n_groups):
+            if e.want:
+                rows.extend(i for _ in e.want)
+        lengths = [[0] * self.n_groups for _ in range(n)]
+        for g in range(self.n_groups):
+            full = mgr.groups[g].kind == "full"
+            flat = v[f"tables{g}"]
+            slots, last_at, last_page = [], [], []
+            for i, e in enumerate(entries):
                 table = mgr.table_ref(e.seq_id, g)
                 page = table[e.start // ps]
                 if not 0 <= page < limit:
                     raise ValueError("a block table names a page outside the pool")
-                v[f"slots{g}"][i] = page * ps + e.start % ps
-                row = v[f"tables{g}"][i * width:(i + 1) * width]
-                full = mgr.groups[g].kind == "full"
-                # a request that keeps its row only appends pages (the last one may have been
-                # swapped by a copy-on-write): rewrite from the last page known
+                slots.append(page * ps + e.start % ps)
+                count = len(table)
+                lengths[i][g] = count
+                known = cap.rows[i]
+                if full and known is not None and known[0] == e.seq_id and known[1][g] == count:
+                    # the row is in place; only its last page may have been swapped by a copy-on-write
+                    last_at.append(i * width + count - 1)
+                    last_page.append(table[-1])
+                    continue
+                # a request that keeps its row only appends pages: rewrite from the last page known
                 lo = max(0, known[1][g] - 1) if (known is not None and known[0] == e.seq_id and full) else 0
-                row[lo:len(table)] = table[lo:]
+                row = flat[i * width:(i + 1) * width]
+                row[lo:count] = table[lo:]
                 if not full:
                     np.maximum(row, 0, out=row)  # pages that the window has passed are never read
-            cap.rows[i] = (e.seq_id, [len(mgr.table_ref(e.seq_id, g)) for g in range(self.n_groups)])
-            if e.want:
-                rows.extend(i for _ in e.want)
-        for g in range(self.n_groups):
+            v[f"slots{g}"][:n] = slots
             v[f"slots{g}"][n:] = -1
+            if last_at:
+                flat[last_at] = last_page
+        for i, e in enumerate(entries):
+            cap.rows[i] = (e.seq_id, lengths[i])
         for i in range(n, b):
             cap.rows[i] = None
         if sampled:
             temp, top_p = v["temperature"].view(np.float32), v["top_p"].view(np.float32)
             seeds, counters = v["seeds"].view(np.int64), v["counters"].view(np.int64)
             temp[n:] = 0.0
-            for i, (t, k, p, seed, draw) in enumerate(sampling):
-                temp[i], v["top_k"][i], top_p[i], seeds[i], counters[i] = t, k, p, seed, draw
+            ts, ks, pp, sd, dr = zip(*sampling)
+            temp[:n], v["top_k"][:n], top_p[:n], seeds[:n], counters[:n] = ts, ks, pp, sd, dr
         cap.dev.copy_(cap.host, non_blocking=True)
         cap.graph.replay()
         self.replays += 1

@@ -56,6 +56,15 @@ class Request:
     def all_token_ids(self) -> list[int]:
         return self.prompt_ids + self.output_ids
 
+    def token_slice(self, begin: int, end: int) -> list[int]:
+        """Tokens ``[begin, end)`` of prompt followed by output, without joining the two lists."""
+        n_prompt = len(self.prompt_ids)
+        if end <= n_prompt:
+            return self.prompt_ids[begin:end]
+        if begin >= n_prompt:
+            return self.output_ids[begin - n_prompt:end - n_prompt]
+        return self.prompt_ids[begin:] + self.output_ids[:end - n_prompt]
+
     @property
     def num_tokens(self) -> int:
         return len(self.prompt_ids) + len(self.output_ids)

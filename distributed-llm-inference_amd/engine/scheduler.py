@@ -230,6 +230,7 @@ class Scheduler:
         if missing <= 0:
             return []
         try:
-            return self.manager.append_slots(req.request_id, req.all_token_ids[-missing:])
+            total = req.num_tokens
+            return self.manager.append_slots(req.request_id, req.token_slice(total - missing, total))
         except NoFreePagesError:
             return None
