@@ -37,7 +37,7 @@ LLAMA_3_2_1B = {
 }
 
 
-def make_engine(raw, dtype, batch, context, block_size, budget):
+def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1):
     import torch
 
     from dli_amd.engine import LLMEngine, SchedulerConfig
@@ -52,11 +52,12 @@ def make_engine(raw, dtype, batch, context, block_size, budget):
     pages = batch * (-(-(context + SLACK) // block_size) + 1) + 8
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=False,
-        config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget))
+        config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
+                               decode_steps=decode_steps))
     return engine, cfg
 
 
-def decode_run(engine, cfg, batch, context, steps, warmup):
+def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     """Tokens a second and milliseconds a step of ``steps`` decode steps at about ``context``."""
     import torch
 
@@ -79,15 +80,27 @@ def decode_run(engine, cfg, batch, context, steps, warmup):
         engine.step()  # prefill, in portions under the token budget
         guard += 1
         assert guard < SLACK, "prefill took more steps than the pool has slack for"
-    for _ in range(warmup):
-        engine.step()
+    # An engine step may decode several tokens of every request (SchedulerConfig.decode_steps): the
+    # clock runs over exactly `steps` decode steps of the model, however many engine steps that is.
+    def advance(n):
+        done = 0
+        while done < n:
+            out = engine.step()
+            assert len(out) == batch and len({len(o.new_token_ids) for o in out}) == 1
+            done += len(out[0].new_token_ids)
+        return done
+
+    import dataclasses
+
+    per = max(d for d in (8, 4, 2, 1) if d <= max(1, decode_steps) and steps % d == 0)
+    engine.scheduler.config = dataclasses.replace(engine.scheduler.config, decode_steps=per)
+    advance(-(-warmup // per) * per)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        out = engine.step()
+    done = advance(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    assert len(out) == batch and len(engine.scheduler.running) == batch
+    assert done == steps and len(engine.scheduler.running) == batch
     for rid in ids:
         engine.abort(rid)
     return batch * steps / dt, dt / steps * 1e3
@@ -138,6 +151,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--decode-steps", type=int, default=4,
+                    help="decode steps that one engine step runs on the device before the host looks "
+                         "(reduced to a divisor of --steps)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run only the 2,048-token prefill steps (for profiling) and print their time")
@@ -155,13 +171,14 @@ def main() -> int:
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
     max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
-    engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=8192)
+    engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=8192,
+                              decode_steps=args.decode_steps)
 
     if args.only_prefill:
         t = prefill_run(engine, cfg, 2048, repeats=args.steps)
         print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": 2048, "tok_s": round(2048 / t, 1)}))
         return 0
-    tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup)
+    tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup, args.decode_steps)
     achieved = decode_bytes(cfg, args.batch, args.context, itemsize) / (ms * 1e-3) / 1e9
     line = {
         "metric": "decode tok/s at batch 8, Llama-3.2-1B shape",
@@ -175,7 +192,7 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "rms_norm_eps": cfg.rms_norm_eps, "rope": f"{cfg.rope.rope_type} theta {cfg.rope.theta:g} factor {cfg.rope.factor:g}",
             "tied_head": cfg.tie_word_embeddings, "kv_block_size": args.block_size, "prefill_tokens": 2048,
-            "sampling": "greedy",
+            "sampling": "greedy", "decode_steps_per_engine_step": engine.scheduler.config.decode_steps,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
@@ -187,7 +204,7 @@ def main() -> int:
         points = {}
         for b in (1, 64):
             steps = min(args.steps, 32)
-            points[f"decode_b{b}"] = round(decode_run(engine, cfg, b, args.context, steps, min(args.warmup, 4))[0], 1)
+            points[f"decode_b{b}"] = round(decode_run(engine, cfg, b, args.context, steps, min(args.warmup, 4), args.decode_steps)[0], 1)
         line["points"] = points
     print(json.dumps(line))
     return 0

@@ -117,6 +117,7 @@ class _Seq:
     page_hashes: list[PageHash] = field(default_factory=list)
     tail_tokens: list[int] = field(default_factory=list)
     num_registered: int = 0
+    reserved: int = 0  # tokens that the tables have room for, where that exceeds num_tokens
 
 
 class CacheManager:
@@ -294,11 +295,14 @@ class CacheManager:
         done on the device before the next write (copy-on-write of a shared partial page)."""
         seq = self._seq(seq_id)
         ps, pos, n = self.page_size, seq.num_tokens, len(token_ids)
-        needed = sum(1 for p in range(pos, pos + n) if p % ps == 0)
+        have = self._ceil(max(seq.num_tokens, seq.reserved))  # pages in place, some reserved ahead
+        needed = max(0, self._ceil(pos + n) - have)
         cows = []
         for g, pool in enumerate(self.pools):
-            last = seq.tables[g][-1] if seq.tables[g] else RELEASED
-            cow = pos % ps != 0 and last != RELEASED and pool.ref[last] > 1
+            # the partly filled page that the first new token goes into (pages behind it may be
+            # reserved ahead: those are never shared)
+            last = seq.tables[g][pos // ps] if pos % ps != 0 else RELEASED
+            cow = last != RELEASED and pool.ref[last] > 1
             cows.append(cow)
             if needed + cow > pool.num_available:
                 raise NoFreePagesError(f"append needs {needed + cow} pages in group {g}")
@@ -306,19 +310,43 @@ class CacheManager:
         for g, pool in enumerate(self.pools):
             table = seq.tables[g]
             if cows[g]:
-                old = table[-1]
+                old = table[pos // ps]
                 new = pool.take()
                 ops.append(CopyOp(src=old, dst=new, group=g))
-                table[-1] = new
+                table[pos // ps] = new
                 pool.decref(old)
                 self._stats.cow_copies += 1
-            for p in range(pos, pos + n):
-                if p % ps == 0:
-                    table.append(pool.take())
+            for _ in range(needed):
+                table.append(pool.take())
         seq.num_tokens += n
+        if seq.reserved <= seq.num_tokens:
+            seq.reserved = 0
         if self.prefix_caching:
             seq.tail_tokens.extend(token_ids)
         return ops
+
+    def reserve_ahead(self, seq_id: SeqId, extra_tokens: int) -> None:
+        """Make room for ``extra_tokens`` more tokens than the request has, without naming them:
+        the pages they will need are taken now, :meth:`append_slots` uses them later. For steps
+        that decode several tokens on the device before the host sees any of them.
+
+        Raises:
+            NoFreePagesError: not enough pages (nothing changed).
+        """
+        seq = self._seq(seq_id)
+        if extra_tokens <= 0:
+            return
+        target = seq.num_tokens + extra_tokens
+        have = self._ceil(max(seq.num_tokens, seq.reserved))
+        needed = self._ceil(target) - have
+        if needed > 0:
+            for g, pool in enumerate(self.pools):
+                if needed > pool.num_available:
+                    raise NoFreePagesError(f"reserving ahead needs {needed} pages in group {g}")
+            for g, pool in enumerate(self.pools):
+                for _ in range(needed):
+                    seq.tables[g].append(pool.take())
+        seq.reserved = max(seq.reserved, target)
 
     def mark_computed(self, seq_id: SeqId, num_computed_tokens: int) -> None:
         """Record that the keys of the first ``num_computed_tokens`` tokens are written.
@@ -343,12 +371,13 @@ class CacheManager:
         if child_id in self._seqs:
             raise SequenceError(f"sequence {child_id!r} already allocated")
         slot = self.slots.take()
+        held = self._ceil(parent.num_tokens)  # pages reserved ahead stay the parent's alone
         for g, pool in enumerate(self.pools):
-            for page in parent.tables[g]:
+            for page in parent.tables[g][:held]:
                 if page != RELEASED:
                     pool.incref(page)
         self._seqs[child_id] = _Seq(
-            tables=[list(t) for t in parent.tables], num_tokens=parent.num_tokens,
+            tables=[list(t[:held]) for t in parent.tables], num_tokens=parent.num_tokens,
             num_computed=parent.num_computed, namespace=parent.namespace, state_slot=slot,
             released=list(parent.released), page_hashes=list(parent.page_hashes),
             tail_tokens=list(parent.tail_tokens), num_registered=parent.num_registered)
@@ -378,7 +407,7 @@ class CacheManager:
             expected: Counter = Counter()
             for seq in self._seqs.values():
                 table = seq.tables[g]
-                assert len(table) == self._ceil(seq.num_tokens), "table size != ceil(tokens/page)"
+                assert len(table) == self._ceil(max(seq.num_tokens, seq.reserved)), "table size != ceil(tokens/page)"
                 assert 0 <= seq.num_computed <= seq.num_tokens, "computed outside [0, tokens]"
                 assert all(p == RELEASED for p in table[:seq.released[g]]), "released prefix holds a page"
                 assert all(p != RELEASED for p in table[seq.released[g]:]), "a live page is missing"

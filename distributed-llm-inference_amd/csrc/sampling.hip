@@ -236,3 +236,52 @@ extern "C" int dli_sample(const float* logits, int64_t row_stride, int rows, int
                                                      top_p, seeds, counters, part_val, part_idx, out);
   return dli_launch_status();
 }
+
+// Between two decode steps that run back to back on the device: row i's sampled token becomes
+// its next input, its position and key count grow by one, its draw counter moves on, and its
+// cache slot in each group of layers is looked up in its block table. Rows without keys
+// (padding) are left alone. `tokens_out` receives the sampled tokens of the step that has just
+// run; with advance == 0 nothing else is done (the last step of a run).
+#define ADVANCE_MAX_GROUPS 4
+struct AdvanceGroups {
+  int* slots[ADVANCE_MAX_GROUPS];
+  const int* tables[ADVANCE_MAX_GROUPS];
+};
+__global__ void decode_advance_kernel(const int* __restrict__ sampled, int* __restrict__ tokens_out,
+                                      int* __restrict__ token_ids, int* __restrict__ positions,
+                                      int* __restrict__ kv_len, uint64_t* __restrict__ counters,
+                                      AdvanceGroups groups, int n_groups, int table_stride,
+                                      int page_size, int rows, int advance) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows) return;
+  const int tok = sampled[i];
+  tokens_out[i] = tok;
+  if (!advance || kv_len[i] <= 0) return;
+  const int pos = positions[i] + 1;
+  token_ids[i] = tok;
+  positions[i] = pos;
+  kv_len[i] += 1;
+  counters[i] += 1;
+  for (int g = 0; g < n_groups; ++g) {
+    const int page = groups.tables[g][(int64_t)i * table_stride + pos / page_size];
+    groups.slots[g][i] = page * page_size + pos % page_size;
+  }
+}
+
+extern "C" int dli_decode_advance(const int* sampled, int* tokens_out, int* token_ids, int* positions,
+                                  int* kv_len, uint64_t* counters, int* const* slots,
+                                  const int* const* tables, int n_groups, int table_stride,
+                                  int page_size, int rows, int advance, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (n_groups < 0 || n_groups > ADVANCE_MAX_GROUPS || page_size <= 0 || table_stride <= 0)
+    return DLI_ERR_ARGUMENT;
+  AdvanceGroups groups;
+  for (int g = 0; g < ADVANCE_MAX_GROUPS; ++g) {
+    groups.slots[g] = g < n_groups ? slots[g] : nullptr;
+    groups.tables[g] = g < n_groups ? tables[g] : nullptr;
+  }
+  decode_advance_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(sampled, tokens_out, token_ids, positions,
+                                                                kv_len, counters, groups, n_groups,
+                                                                table_stride, page_size, rows, advance);
+  return dli_launch_status();
+}

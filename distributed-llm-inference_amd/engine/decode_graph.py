@@ -46,7 +46,7 @@ class _Captured:
     views: dict             # name -> numpy view into host
     width: int              # block-table entries per row
     rows: list              # per row: (request, pages already written into its table row)
-    tokens_host: Optional[torch.Tensor] = None  # pinned int32 [b]: sampled tokens (sampling graphs)
+    tokens_host: Optional[torch.Tensor] = None  # pinned int32 [steps * b]: sampled tokens (sampling graphs)
 
 
 class DecodeGraphs:
@@ -56,7 +56,7 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self.max_width = max(1, max_blocks_per_seq)
         self.n_groups = step_fn.manager.num_groups
-        self.captured: dict[tuple[int, int, int, bool], _Captured] = {}
+        self.captured: dict[tuple[int, int, int, bool, int], _Captured] = {}
         self.replays = 0
         self.enabled = self._supported()
 
@@ -72,11 +72,11 @@ class DecodeGraphs:
                 return False
         return True
 
-    def can_run(self, entries: Sequence[StepEntry]) -> bool:
+    def can_run(self, entries: Sequence[StepEntry], steps: int = 1) -> bool:
         if not self.enabled or not entries or len(entries) > self.max_batch:
             return False
         ps = self.step_fn.manager.page_size
-        return all(len(e.tokens) == 1 and e.start + 1 <= self.max_width * ps for e in entries)
+        return all(len(e.tokens) == 1 and e.start + steps <= self.max_width * ps for e in entries)
 
     # ------------------------------------------------------------------ capture
 
@@ -92,7 +92,7 @@ class DecodeGraphs:
             at += -(-n // 4) * 4  # 16-byte aligned starts
         return offsets, at
 
-    def _capture(self, b: int, splits: int, width: int, sampled: bool) -> _Captured:
+    def _capture(self, b: int, splits: int, width: int, sampled: bool, steps: int = 1) -> _Captured:
         dev_name = self.rt.device
         offsets, total = self._layout(b, width)
         host = torch.zeros(total, dtype=torch.int32).pin_memory()
@@ -127,19 +127,28 @@ class DecodeGraphs:
         views["temperature"].view(np.float32)[:] = 0.0  # padding rows are greedy
         views["top_p"].view(np.float32)[:] = 1.0
         views["top_k"][:] = -1
-        tokens_host = tokens_dev = scratch = None
+        tokens_host = tokens_dev = tokens_all = scratch = None
         if sampled:
-            tokens_host = torch.zeros(b, dtype=torch.int32).pin_memory()
+            tokens_host = torch.zeros(steps * b, dtype=torch.int32).pin_memory()
             tokens_dev = torch.zeros(b, dtype=torch.int32, device=dev_name)
+            tokens_all = torch.zeros(steps, b, dtype=torch.int32, device=dev_name)
             scratch = ops.sample_scratch(b, dev_name)
+        ps = self.step_fn.manager.page_size
 
         def body():
-            logits = model.forward(ctx, caches)
+            # `steps` decode steps back to back: after each, the sampled tokens become the next
+            # inputs and positions, lengths, slots and draw counters move on, all on the device
+            for j in range(steps):
+                logits = model.forward(ctx, caches)
+                if sampled:
+                    ops.sample(logits, dv["temperature"].view(torch.float32), dv["top_k"],
+                               dv["top_p"].view(torch.float32), dv["seeds"].view(torch.int64),
+                               dv["counters"].view(torch.int64), tokens_dev, scratch)
+                    ops.decode_advance(tokens_dev, tokens_all[j], dv["token_ids"], dv["positions"], dv["kv_len"],
+                                       dv["counters"].view(torch.int64), [g.slots for g in groups],
+                                       [g.block_tables for g in groups], ps, advance=j + 1 < steps)
             if sampled:
-                ops.sample(logits, dv["temperature"].view(torch.float32), dv["top_k"],
-                           dv["top_p"].view(torch.float32), dv["seeds"].view(torch.int64),
-                           dv["counters"].view(torch.int64), tokens_dev, scratch)
-                tokens_host.copy_(tokens_dev, non_blocking=True)
+                tokens_host.copy_(tokens_all.view(-1), non_blocking=True)
             return logits
 
         dev.copy_(host)
@@ -154,22 +163,26 @@ class DecodeGraphs:
 
     # ------------------------------------------------------------------ replay
 
-    def run(self, entries: Sequence[StepEntry], sampling: Optional[Sequence[tuple]] = None):
+    def run(self, entries: Sequence[StepEntry], sampling: Optional[Sequence[tuple]] = None, steps: int = 1):
         """A decode-only step. Without ``sampling``: logits ``[wanted, vocab]`` (a view of the
         graph's output: use it before the next step). With ``sampling``, one
         ``(temperature, top_k, top_p, seed, draw index)`` per entry: the graph samples too and the
-        chosen token ids come back as a list."""
+        chosen token ids come back as a list; with ``steps`` > 1 the graph runs that many decode
+        steps in a row and one list per step comes back (the block tables must already hold the
+        pages of all positions that will be written)."""
         mgr = self.step_fn.manager
         ps, n = mgr.page_size, len(entries)
         b = _bucket(n)
-        max_kv = max(e.start + 1 for e in entries)
+        max_kv = max(e.start + steps for e in entries)
         width = max(16, _bucket(-(-max_kv // ps)))
         splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv))
         sampled = sampling is not None
-        key = (b, splits, width, sampled)
+        if steps > 1 and not sampled:
+            raise ValueError("several steps in a row need the sampling parameters")
+        key = (b, splits, width, sampled, steps)
         cap = self.captured.get(key)
         if cap is None:
-            cap = self.captured[key] = self._capture(b, splits, width, sampled)
+            cap = self.captured[key] = self._capture(b, splits, width, sampled, steps)
         v = cap.views
         limit = self.step_fn.store.num_pages
         token_ids, positions, kv_len, state_slots = v["token_ids"], v["positions"], v["kv_len"], v["state_slots"]
@@ -205,15 +218,17 @@ class DecodeGraphs:
                 count = len(table)
                 lengths[i][g] = count
                 known = cap.rows[i]
-                if full and known is not None and known[0] == e.seq_id and known[1][g] == count:
-                    # the row is in place; only its last page may have been swapped by a copy-on-write
-                    last_at.append(i * width + count - 1)
-                    last_page.append(table[-1])
+                if full and known is not None and known[0] == e.seq_id:
+                    # A request that keeps its row only appends pages, and only the page it writes
+                    # next may have been swapped by a copy-on-write: rewrite from whichever of the
+                    # two comes first (a few entries, gathered for one assignment).
+                    lo = max(0, min(known[1][g] - 1, e.start // ps))
+                    for at in range(lo, count):
+                        last_at.append(i * width + at)
+                        last_page.append(table[at])
                     continue
-                # a request that keeps its row only appends pages: rewrite from the last page known
-                lo = max(0, known[1][g] - 1) if (known is not None and known[0] == e.seq_id and full) else 0
                 row = flat[i * width:(i + 1) * width]
-                row[lo:count] = table[lo:]
+                row[:count] = table
                 if not full:
                     np.maximum(row, 0, out=row)  # pages that the window has passed are never read
             v[f"slots{g}"][:n] = slots
@@ -235,7 +250,9 @@ class DecodeGraphs:
         self.replays += 1
         if sampled:
             torch.cuda.current_stream().synchronize()
-            return cap.tokens_host[:n].tolist()
+            if steps == 1:
+                return cap.tokens_host[:n].tolist()
+            return [row[:n] for row in cap.tokens_host.view(steps, b).tolist()]
         if rows == list(range(n)):
             return cap.logits[:n]
         if not rows:

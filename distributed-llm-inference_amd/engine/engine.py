@@ -7,6 +7,8 @@ a token for every request whose chunk reached its last known token, append it, f
 
 from __future__ import annotations
 
+import dataclasses
+
 import itertools
 import random
 import time
@@ -47,7 +49,12 @@ class ModelRunner:
 
         sampling = [sampling_tuple(c.request.params, c.request.seed, len(c.request.output_ids))
                     for c in sched.chunks if c.needs_logits]
-        return self.core.step.run(self._entries(sched), sched.copy_ops, sampling=sampling)
+        return self.core.step.run(self._entries(sched), sched.copy_ops, sampling=sampling, steps=sched.decode_steps)
+
+    @property
+    def max_decode_steps(self) -> int:
+        """Tokens per request that one step can decode on the device (1 without decode graphs)."""
+        return self.core.step.max_decode_steps
 
     def _entries(self, sched: SchedulerOutput) -> list:
         from .batch import StepEntry
@@ -109,7 +116,12 @@ class LLMEngine:
                  sampler: Optional[TokenSampler] = None) -> None:
         self.runner = runner
         self.manager = manager
-        self.scheduler = Scheduler(config or SchedulerConfig(), manager)
+        config = config or SchedulerConfig()
+        # several tokens per step need a runner that decodes and samples them on the device
+        can = getattr(runner, "max_decode_steps", 1) if sampler is None else 1
+        if config.decode_steps > can:
+            config = dataclasses.replace(config, decode_steps=max(1, can))
+        self.scheduler = Scheduler(config, manager)
         self.eos = frozenset(eos_token_ids)
         self._rng = random.Random(seed)
         self._arrivals = itertools.count()
@@ -189,16 +201,18 @@ class LLMEngine:
             else:
                 logits = self.runner.execute(sched)
             t2 = time.perf_counter()
+            k = sched.decode_steps
             for ch in sched.chunks:
-                ch.request.num_computed_tokens += ch.num_tokens
+                ch.request.num_computed_tokens += ch.num_tokens + k - 1
             if fused is None:
                 tokens = self._sample(
                     logits, [c.request.params for c in sampling], [c.request.seed for c in sampling],
                     [len(c.request.output_ids) for c in sampling])
-            if len(tokens) != len(sampling):
+            rounds = tokens if k > 1 else [tokens]  # one list of tokens per decoded position
+            if len(rounds) != k or any(len(r) != len(sampling) for r in rounds):
                 raise RuntimeError("the sampler returned a wrong number of tokens")
-            for ch, tok in zip(sampling, tokens):
-                outputs.append(self._append_token(ch.request, int(tok)))
+            for i, ch in enumerate(sampling):
+                outputs.append(self._append_tokens(ch.request, [int(r[i]) for r in rounds]))
         else:
             t2 = t1
         t3 = time.perf_counter()
@@ -229,13 +243,19 @@ class LLMEngine:
 
     # ------------------------------------------------------------------ internals
 
-    def _append_token(self, req: Request, tok: int) -> RequestOutput:
-        req.output_ids.append(tok)
+    def _append_tokens(self, req: Request, toks: Sequence[int]) -> RequestOutput:
+        """Take the tokens that a step decoded for the request, in order, up to the one that ends
+        it; what was decoded beyond that one is dropped."""
         reason: Optional[FinishReason] = None
-        if tok in req.params.stop_token_ids or (not req.params.ignore_eos and tok in self.eos):
-            reason = FinishReason.STOP
-        elif len(req.output_ids) >= req.params.max_tokens:
-            reason = FinishReason.LENGTH
-        if reason is not None:
-            self.scheduler.finish(req, reason)
-        return RequestOutput(req.request_id, [tok], reason is not None, reason)
+        taken: list[int] = []
+        for tok in toks:
+            req.output_ids.append(tok)
+            taken.append(tok)
+            if tok in req.params.stop_token_ids or (not req.params.ignore_eos and tok in self.eos):
+                reason = FinishReason.STOP
+            elif len(req.output_ids) >= req.params.max_tokens:
+                reason = FinishReason.LENGTH
+            if reason is not None:
+                self.scheduler.finish(req, reason)
+                break
+        return RequestOutput(req.request_id, taken, reason is not None, reason)

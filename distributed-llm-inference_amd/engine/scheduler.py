@@ -34,7 +34,10 @@ class SchedulerConfig:
 
     ``namespace`` scopes content reuse of cache pages (model and weights identity);
     ``tenant_weights`` gives tenants a weighted fair share of admissions; after ``aging_steps``
-    steps of waiting a request counts as INTERACTIVE.
+    steps of waiting a request counts as INTERACTIVE. ``decode_steps`` > 1 lets a step in which
+    every request decodes, nobody waits and the cache has room run up to that many tokens of each
+    request on the device before the host sees them (the reference has no counterpart; 1 keeps
+    its behaviour).
     """
 
     max_num_seqs: int = 64
@@ -42,10 +45,13 @@ class SchedulerConfig:
     namespace: bytes = b""
     tenant_weights: Mapping[str, float] = field(default_factory=dict)
     aging_steps: int = 200
+    decode_steps: int = 1
 
     def __post_init__(self) -> None:
         if self.max_num_seqs < 1 or self.max_num_batched_tokens < 1:
             raise ValueError("max_num_seqs and max_num_batched_tokens must be >= 1")
+        if self.decode_steps < 1:
+            raise ValueError("decode_steps must be >= 1")
         if self.aging_steps < 1:
             raise ValueError("aging_steps must be >= 1")
         if any(w <= 0 for w in self.tenant_weights.values()):
@@ -68,6 +74,7 @@ class SchedulerOutput:
     chunks: list[ScheduledChunk] = field(default_factory=list)
     copy_ops: list[CopyOp] = field(default_factory=list)
     preempted: list[Request] = field(default_factory=list)
+    decode_steps: int = 1  # tokens that each chunk's request decodes in this step (all chunks decode if > 1)
 
     @property
     def num_batched_tokens(self) -> int:
@@ -135,8 +142,30 @@ class Scheduler:
         left = self._serve_running(plan, self.config.max_num_batched_tokens)
         if not plan.preempted:  # memory that was just freed serves running requests first
             self._admit_waiting(plan, left)
+        plan.decode_steps = self._decode_steps(plan)
         self._step += 1
         return plan
+
+    def _decode_steps(self, plan: SchedulerOutput) -> int:
+        """How many tokens each request of the step may decode before the host looks again: more
+        than one only if the step is all decoding, nobody waits for admission, nothing was
+        preempted or has to be copied, and the pages for the extra tokens can be reserved now.
+        Never more than the request with the fewest tokens left may still produce."""
+        k = self.config.decode_steps
+        if k <= 1 or not plan.chunks or self.waiting or plan.preempted or plan.copy_ops:
+            return 1
+        for ch in plan.chunks:
+            if ch.num_tokens != 1 or not ch.needs_logits:
+                return 1
+            k = min(k, ch.request.params.max_tokens - len(ch.request.output_ids))
+        if k <= 1:
+            return 1
+        try:
+            for ch in plan.chunks:
+                self.manager.reserve_ahead(ch.request.request_id, k - 1)
+        except NoFreePagesError:
+            return 1  # what was reserved so far stays with its requests and is used later
+        return k
 
     def _serve_running(self, plan: SchedulerOutput, budget: int) -> int:
         """Give each running request its next token or portion; returns the budget left."""

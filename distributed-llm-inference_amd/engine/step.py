@@ -24,6 +24,9 @@ from ..parts.model import Model
 from .batch import GroupView, StepContext, StepEntry
 
 
+MAX_DECODE_STEPS = 8  # tokens per request that one graph replay may decode
+
+
 class StepError(ValueError):
     """A batch that the step function refuses (it would read or write outside a request's cache)."""
 
@@ -143,17 +146,30 @@ class StepFunction:
 
     # ------------------------------------------------------------------ the step
 
+    @property
+    def max_decode_steps(self) -> int:
+        """Tokens per request that :meth:`run` can decode in one call (``steps``)."""
+        return MAX_DECODE_STEPS if self.graphs is not None and self.graphs.enabled else 1
+
     def run(self, entries: Sequence[StepEntry], copy_ops: Sequence[CopyOp] = (),
-            sampling: Optional[Sequence[tuple]] = None):
+            sampling: Optional[Sequence[tuple]] = None, steps: int = 1):
         """Run one step. Returns float32 logits ``[wanted places, vocab]`` on the device, in the
         order of the entries and of each entry's ``want``.
 
         With ``sampling`` (one ``(temperature, top_k, top_p, seed, draw index)`` for each wanted
         place, temperature 0 meaning greedy) a token is chosen at every wanted place and the list
-        of token ids is returned instead."""
+        of token ids is returned instead.
+
+        ``steps`` > 1 (decode-only batches with ``sampling``, cache room reserved ahead with
+        ``CacheManager.reserve_ahead``): every request decodes that many tokens, each sampled
+        token being the next input on the device; returns one list of token ids per decoded
+        position. The tokens but the last are appended to the requests in the cache manager and
+        all positions that were run are marked computed."""
         self.store.copy_pages(copy_ops)  # before any write of this step (runner.py:56)
         if not entries:
             return torch.empty(0, self.vocab_size, device=self.rt.device, dtype=torch.float32)
+        if steps > 1:
+            return self._run_many(entries, copy_ops, sampling, steps)
         if self.graphs is not None and not copy_ops and self.graphs.can_run(entries):
             for e in entries:  # the same checks as build_context makes
                 if e.start != self.manager.num_computed_tokens(e.seq_id):
@@ -180,6 +196,32 @@ class StepFunction:
         if logits is None:
             return tokens
         return self._sample(logits, sampling)
+
+    def _run_many(self, entries: Sequence[StepEntry], copy_ops: Sequence[CopyOp],
+                  sampling: Optional[Sequence[tuple]], steps: int) -> list[list[int]]:
+        mgr, ps = self.manager, self.manager.page_size
+        if steps > self.max_decode_steps:
+            raise StepError(f"{steps} tokens per step asked for, {self.max_decode_steps} possible")
+        if copy_ops or sampling is None or len(sampling) != len(entries) or not self.graphs.can_run(entries, steps):
+            raise StepError("several tokens per step need a decode-only batch that samples every request")
+        if len({e.seq_id for e in entries}) != len(entries):
+            raise StepError("a request appears twice in one step")
+        for e in entries:
+            if e.start != mgr.num_computed_tokens(e.seq_id) or e.start + 1 != mgr.num_tokens(e.seq_id):
+                raise StepError(f"request {e.seq_id!r}: its last token must be the only one not computed")
+            if tuple(int(w) for w in e.want) != (0,):
+                raise StepError(f"request {e.seq_id!r}: the one token's logits must be wanted")
+            for g in range(mgr.num_groups):
+                if len(mgr.table_ref(e.seq_id, g)) * ps < e.start + steps:
+                    raise StepError(f"request {e.seq_id!r}: no cache room reserved for {steps} tokens")
+        rounds = self.graphs.run(entries, sampling, steps=steps)
+        for i, e in enumerate(entries):
+            for j in range(steps - 1):
+                if mgr.append_slots(e.seq_id, [rounds[j][i]]):
+                    raise StepError("a page reserved ahead was shared")
+            mgr.mark_computed(e.seq_id, e.start + steps)
+        self.steps_run += steps
+        return rounds
 
     def _sample(self, logits: torch.Tensor, sampling: Sequence[tuple]) -> list[int]:
         from ..kernels import ops

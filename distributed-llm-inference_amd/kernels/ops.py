@@ -9,7 +9,7 @@ stream; nothing here computes with torch.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Sequence
 
 import torch
 
@@ -45,6 +45,8 @@ _SIGNATURES = {
     "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                    _c_ptr],
     "dli_sample_scratch_per_row": [],
+    "dli_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                           _c_int, _c_int, _c_ptr],
     "dli_skinny_gemm_max_rows": [],
     "dli_skinny_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
                         _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -584,3 +586,37 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _check(library().dli_sample(_ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k),
                                 _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(scratch[0]), _ptr(scratch[1]),
                                 _ptr(out), _stream()), "sample")
+
+
+def decode_advance(sampled: torch.Tensor, tokens_out: torch.Tensor, token_ids: torch.Tensor,
+                   positions: torch.Tensor, kv_len: torch.Tensor, counters: torch.Tensor,
+                   slots: Sequence[torch.Tensor], tables: Sequence[torch.Tensor], page_size: int,
+                   advance: bool) -> None:
+    """Hand the sampled tokens of a decode step to the next one on the device.
+
+    ``tokens_out[i] = sampled[i]``; with ``advance`` every row that has keys gets its sampled token
+    as next input, position, key count and draw counter plus one, and in each group of layers the
+    cache slot of the new position from its block-table row (``tables[g]`` is ``[rows, width]``).
+    """
+    rows = sampled.shape[0]
+    for name, t in (("sampled", sampled), ("tokens_out", tokens_out), ("token_ids", token_ids),
+                    ("positions", positions), ("kv_len", kv_len)):
+        _dense(t, name, torch.int32, 1)
+        _require(t.shape[0] == rows, f"{name} must have one entry per row")
+    _dense(counters, "counters", torch.int64, 1)
+    _require(counters.shape[0] == rows, "counters must have one entry per row")
+    _require(len(slots) == len(tables) <= 4, "one slot vector and one table per group, at most 4 groups")
+    width = 1
+    for g, (sl, tb) in enumerate(zip(slots, tables)):
+        _dense(sl, f"slots[{g}]", torch.int32, 1)
+        _dense(tb, f"tables[{g}]", torch.int32, 2)
+        _require(sl.shape[0] == rows and tb.shape[0] == rows, "slots and tables must have one row per request")
+        _require(g == 0 or tb.shape[1] == width, "the groups' tables differ in width")
+        width = tb.shape[1]
+    n = len(slots)
+    slot_ptrs = (ctypes.c_void_p * 4)(*([t.data_ptr() for t in slots] + [None] * (4 - n)))
+    table_ptrs = (ctypes.c_void_p * 4)(*([t.data_ptr() for t in tables] + [None] * (4 - n)))
+    _check(library().dli_decode_advance(
+        _ptr(sampled), _ptr(tokens_out), _ptr(token_ids), _ptr(positions), _ptr(kv_len), _ptr(counters),
+        ctypes.cast(slot_ptrs, ctypes.c_void_p), ctypes.cast(table_ptrs, ctypes.c_void_p), n, width,
+        int(page_size), rows, int(bool(advance)), _stream()), "decode_advance")

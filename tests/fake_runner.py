@@ -49,6 +49,31 @@ class FakeRunner:
                 picks.append(next_token(ch.request.all_token_ids[:ch.start + ch.num_tokens]))
         return picks
 
+    # the interface of a runner that also samples, with several decoded tokens per step
+    max_decode_steps = 8
+
+    def execute_and_sample(self, sched):
+        k = sched.decode_steps
+        if k == 1:
+            return self.execute(sched)
+        self.calls.append(sched)
+        rounds = [[] for _ in range(k)]
+        for ch in sched.chunks:
+            rid = ch.request.request_id
+            assert ch.num_tokens == 1 and ch.needs_logits, "only decoding requests take several tokens a step"
+            assert self.manager.num_computed_tokens(rid) == ch.start == self.manager.num_tokens(rid) - 1
+            ps = self.manager.page_size
+            assert len(self.manager.table_ref(rid)) * ps >= ch.start + k, "no room reserved ahead"
+            history = ch.request.token_slice(0, ch.start + 1)
+            for j in range(k):
+                tok = next_token(history)
+                rounds[j].append(tok)
+                history.append(tok)
+                if j < k - 1:
+                    assert self.manager.append_slots(rid, [tok]) == []
+            self.manager.mark_computed(rid, ch.start + k)
+        return rounds
+
 
 def passthrough_sampler(logits, params, seeds, draws):
     assert len(logits) == len(params) == len(seeds) == len(draws)

@@ -367,3 +367,42 @@ def test_shadow_cache_never_serves_wrong_or_unwritten_content():
                 m.free(rid)
                 del live[rid]
         m.check_invariants()
+
+
+def test_reserving_ahead_takes_pages_now_and_appends_use_them():
+    m = CacheManager(num_pages=8, page_size=4, max_seqs=4, watermark=0.0)
+    m.allocate("a", [1, 2, 3, 4, 5])           # 2 pages
+    m.mark_computed("a", 4)
+    m.reserve_ahead("a", 7)                     # room for 12 tokens: 3 pages
+    assert len(m.block_table("a")) == 3 and m.num_tokens("a") == 5
+    m.check_invariants()
+    before = m.stats().free_pages
+    table = m.block_table("a")
+    for t in range(6):
+        assert m.append_slots("a", [t]) == []
+    assert m.block_table("a") == table and m.stats().free_pages == before, "appends took pages they had"
+    m.check_invariants()
+    assert m.append_slots("a", [9, 9]) == []    # 13 tokens: a 4th page
+    assert len(m.block_table("a")) == 4
+    m.check_invariants()
+    # nothing changes when the pool cannot serve the reservation
+    m.allocate("b", list(range(13)))            # 4 pages: the pool is full
+    with pytest.raises(NoFreePagesError):
+        m.reserve_ahead("a", 8)
+    assert len(m.block_table("a")) == 4
+    m.check_invariants()
+    m.free("b")
+    m.reserve_ahead("a", 8)                     # 21 tokens: 6 pages
+    assert len(m.block_table("a")) == 6
+    # a fork shares what is written, not what is reserved ahead
+    m.fork("a", "c")
+    assert len(m.block_table("c")) == 4
+    m.check_invariants()
+    ops = m.append_slots("a", [7])              # position 13 lies in a page that the fork shares
+    assert len(ops) == 1 and ops[0].src == m.block_table("c")[3] and ops[0].dst == m.block_table("a")[3]
+    m.check_invariants()
+    m.free("a")
+    m.free("c")
+    m.reset_prefix_cache()
+    m.check_invariants()
+    assert m.stats().free_pages == 8

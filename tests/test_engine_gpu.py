@@ -131,6 +131,46 @@ def test_graph_replay_equals_eager_steps(name, block):
         assert torch.equal(a, b), f"step {i}: graph replay differs from the eager step by {(a - b).abs().max()}"
 
 
+@pytest.mark.parametrize("name,block,k", [("A", 16, 4), ("C", 32, 3), ("B", 16, 8)])
+def test_several_decode_tokens_per_step_equal_one_per_step(name, block, k):
+    """Steps that decode `k` tokens of every request on the device (sampled tokens fed back there,
+    positions, slots and draw counters advanced by a kernel) against one token per step: greedy
+    and seeded sampling give the same tokens; limits that are no multiple of k, a stop token
+    inside a run, prompts that end at a page's edge, and pages reserved ahead that are returned."""
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    ps = prompts(name, [block - 1, block, 5, 2 * block + 3], seed=31)
+    limits = [7, 2 * block + 5, 1, 13]
+
+    def run(steps, stop=()):
+        eng = LLMEngine.for_model(str(model_folder(name)), dtype="bfloat16", num_blocks=64, block_size=block,
+                                  config=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=256, decode_steps=steps))
+        params = [SamplingParams(max_tokens=limits[0], stop_token_ids=tuple(stop)),
+                  SamplingParams(max_tokens=limits[1], temperature=0.8, top_k=12, seed=5),
+                  SamplingParams(max_tokens=limits[2]),
+                  SamplingParams(max_tokens=limits[3], temperature=1.1, top_p=0.9, seed=9)]
+        reqs = [eng.add_request(f"r{i}", p, q) for i, (p, q) in enumerate(zip(ps, params))]
+        many = 0
+        while eng.has_unfinished():
+            eng.step()
+            eng.core.manager.check_invariants()
+        many = sum(1 for s in eng.stats.steps if s.num_decode_tokens and s.num_seqs)
+        eng.core.manager.reset_prefix_cache()
+        st = eng.core.manager.stats()
+        assert st.free_pages == st.num_pages
+        return [r.output_ids for r in reqs], [r.finish_reason for r in reqs], len(eng.stats.steps)
+
+    one, why1, n1 = run(1)
+    some, whyk, nk = run(k)
+    assert one == some and why1 == whyk
+    assert nk < n1, "no step decoded several tokens"
+    stop = one[0][3]  # ends request 0 inside a run of k
+    one, why1, _ = run(1, [stop])
+    some, whyk, _ = run(k, [stop])
+    assert one == some and why1 == whyk and one[0][-1] == stop and len(one[0]) <= 4
+
+
 def test_shared_prefix_sampling_preemption_config_b():
     """Six prompts that share a 40-token prefix, sampled at temperature 0.8 with per-request seeds
     in a pool so small that requests are preempted: with and without content reuse of cache pages,

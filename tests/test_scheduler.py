@@ -252,3 +252,104 @@ def test_scheduler_config_is_validated():
     m = CacheManager(num_pages=4, page_size=4, max_seqs=2)
     with pytest.raises(ValueError, match="state slots"):
         LLMEngine(FakeRunner(m), m, SchedulerConfig(max_num_seqs=3), sampler=passthrough_sampler)
+
+
+# ------------------------------------------------------------------ several tokens per step
+
+def make_multi(decode_steps, num_pages=256, page_size=4, max_seqs=8, budget=32, eos=()):
+    """An engine whose runner decodes and samples by itself (the fake's hash of the history)."""
+    m = CacheManager(num_pages=num_pages, page_size=page_size, max_seqs=max(max_seqs, 8), watermark=0.0)
+    runner = FakeRunner(m)
+    eng = LLMEngine(runner, m, SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=budget,
+                                               decode_steps=decode_steps), eos_token_ids=eos)
+    return eng, runner, m
+
+
+@pytest.mark.parametrize("k", [2, 3, 8])
+def test_several_tokens_per_step_give_the_same_outputs(k):
+    eng, runner, m = make_multi(k)
+    rng = random.Random(k)
+    prompts = [[rng.randrange(50) for _ in range(rng.randrange(1, 40))] for _ in range(6)]
+    limits = [1, 2, 5, 16, 17, 23]
+    reqs = [eng.add_request(f"r{i}", p, SamplingParams(max_tokens=mt)) for i, (p, mt) in enumerate(zip(prompts, limits))]
+    run(eng)
+    for r, p in zip(reqs, prompts):
+        assert r.output_ids == alone(p, r.params.max_tokens), r.request_id
+        assert r.finish_reason is FinishReason.LENGTH
+    assert any(s.decode_steps > 1 for s in runner.calls), "no step took several tokens"
+    for s in runner.calls:  # never past a request's limit, never while somebody waits or a prompt runs
+        if s.decode_steps > 1:
+            assert all(c.num_tokens == 1 and c.needs_logits for c in s.chunks)
+    m.reset_prefix_cache()
+    m.check_invariants()
+    assert m.stats().free_pages == m.stats().num_pages and m.slots.num_free == m.slots.num_slots
+
+
+def test_stop_token_inside_a_run_of_tokens_ends_the_request_there():
+    prompt = [3, 1, 4, 1, 5]
+    full = alone(prompt, 30)
+    stop = full[6]
+    cut = full.index(stop) + 1
+    eng, _, m = make_multi(4)
+    r = eng.add_request("a", prompt, SamplingParams(max_tokens=30, stop_token_ids=(stop,)))
+    outs = []
+    while eng.has_unfinished():
+        outs.extend(eng.step())
+    assert r.output_ids == full[:cut] and r.finish_reason is FinishReason.STOP
+    assert [t for o in outs for t in o.new_token_ids] == full[:cut]
+    m.reset_prefix_cache()
+    m.check_invariants()
+    assert m.stats().free_pages == m.stats().num_pages
+
+
+def test_one_token_per_step_while_somebody_waits_or_pages_are_short():
+    eng, runner, m = make_multi(4, max_seqs=1)
+    eng.add_request("a", [1, 2, 3], SamplingParams(max_tokens=6))
+    eng.add_request("b", [4, 5], SamplingParams(max_tokens=6))  # waits: the cap is one request
+    while not eng.scheduler.running or eng.scheduler.waiting:
+        eng.step()
+        if eng.scheduler.waiting:
+            assert runner.calls[-1].decode_steps == 1
+    run(eng)
+    # pages: prompt of 6 and 9 tokens to come need 4 pages of 4; with exactly 4 there is no room to
+    # reserve ahead at first, and the outputs stay right
+    eng, runner, m = make_multi(8, num_pages=4, page_size=4)
+    r = eng.add_request("c", [1, 2, 3, 4, 5, 6], SamplingParams(max_tokens=9))
+    run(eng)
+    assert r.output_ids == alone([1, 2, 3, 4, 5, 6], 9)
+    m.check_invariants()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_scenarios_with_several_tokens_per_step(seed):
+    rng = random.Random(100 + seed)
+    pages, ps = rng.randrange(6, 40), rng.choice([1, 2, 4, 8])
+    budget, seqs = rng.choice([1, 2, 3, 8, 32, 128]), rng.randrange(1, 7)
+    eng, runner, m = make_multi(rng.choice([2, 4, 8]), num_pages=pages, page_size=ps, max_seqs=seqs, budget=budget)
+    expected, n, steps = {}, 0, 0
+    while steps < 20000:
+        if n < 25 and rng.random() < 0.3:
+            prompt = [rng.randrange(4) for _ in range(rng.randrange(1, 20))]
+            mt = rng.randrange(1, 12)
+            r = eng.add_request(f"q{n}", prompt, SamplingParams(max_tokens=mt))
+            if r.finish_reason is not FinishReason.CAPACITY:
+                expected[r] = alone(prompt, mt)
+            n += 1
+        if rng.random() < 0.03 and expected:
+            victim = rng.choice(list(expected))
+            if not victim.is_finished:
+                eng.abort(victim.request_id)
+                del expected[victim]
+        if not eng.has_unfinished():
+            if n >= 25:
+                break
+            continue
+        eng.step()
+        steps += 1
+        m.check_invariants()
+    assert steps < 20000, "liveness"
+    for r, out in expected.items():
+        assert r.output_ids == out
+    m.reset_prefix_cache()
+    m.check_invariants()
+    assert m.stats().free_pages == pages
