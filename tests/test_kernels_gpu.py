@@ -99,12 +99,14 @@ def test_gemm_f32(ops, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("qh,kvh,d,rd,bs", [(4, 4, 16, 16, 16), (6, 2, 32, 32, 8), (3, 1, 48, 32, 4), (2, 2, 80, 80, 16)])
-def test_rope_kv_write(ops, dtype, qh, kvh, d, rd, bs):
+@pytest.mark.parametrize("n", [11, 70])  # few tokens: one item per thread; many: one workgroup per token
+def test_rope_kv_write(ops, dtype, qh, kvh, d, rd, bs, n):
     torch.manual_seed(4)
-    n, pages = 11, 9
+    pages = max(9, -(-n // bs) + 2)
     qkv = torch.randn(n, (qh + 2 * kvh) * d, device="cuda").to(dtype)
     orig = qkv.clone()
-    positions = torch.tensor([0, 1, 2, 3, 500, 4095, 7, 8, 9, 10, 11], dtype=torch.int32, device="cuda")
+    positions = torch.tensor([0, 1, 2, 3, 500, 4095, 7, 8, 9, 10, 11] + list(range(100, 100 + n - 11)),
+                             dtype=torch.int32, device="cuda")
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rd, 2).float() / rd))).cuda()
     perm = torch.randperm(pages * bs)[:n]
     perm[5] = -1  # not cached
