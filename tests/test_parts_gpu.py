@@ -253,3 +253,117 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
     finally:
         unregister_architecture("ToyForCausalLM")
         unregister_part("mixer", "toy_ema")
+
+
+# ------------------------------------------------------------------ toy feed-forward with routing, toy position encoding
+
+def test_a_toy_routed_feed_forward_and_a_toy_position_encoding_are_registered_built_and_stepped():
+    """Two more parts defined here and nowhere in the framework: a feed-forward that routes each
+    row to one of three small experts (router logits and the choice in 32-bit), and a position
+    encoding that is no rotation (q_i is scaled by s^i and k_j by s^-j, so a score decays with the
+    distance i - j). A model that uses them in one layer and the built-in parts in the other steps
+    in portions and mixed batches exactly as each request does whole."""
+    from typing import Any, Mapping
+
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import (FeedForward, LayerSpec, ModelSpec, PartSpec, PositionEncoding, ScheduleEntry,
+                               WeightSpec, register_part, unregister_part)
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    @register_part("feed_forward", "toy_routed")
+    class ToyRouted(FeedForward):
+        def __init__(self, runtime, *, hidden_size: int, experts: int, expert_size: int) -> None:
+            super().__init__(runtime)
+            self.h, self.e, self.f = hidden_size, experts, expert_size
+            self.t = {}
+
+        def weight_specs(self):
+            return {"router.weight": WeightSpec((self.e, self.h), role="float32"),
+                    "up.weight": WeightSpec((self.e * self.f, self.h)),
+                    "down.weight": WeightSpec((self.e * self.h, self.f))}
+
+        def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+            self.t = dict(tensors)
+
+        def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
+            scores = torch.softmax(x.float() @ self.t["router.weight"].float().T, dim=-1)
+            weight, choice = scores.max(dim=-1)
+            up = self.t["up.weight"].float().view(self.e, self.f, self.h)
+            down = self.t["down.weight"].float().view(self.e, self.h, self.f)
+            out = torch.empty_like(x)
+            for r in range(x.shape[0]):  # a toy: one row after the other
+                e = int(choice[r])
+                out[r] = (weight[r] * (down[e] @ torch.relu(up[e] @ x[r].float()))).to(x.dtype)
+            return out
+
+    @register_part("position", "toy_decay")
+    class ToyDecay(PositionEncoding):
+        def __init__(self, runtime, *, base: float) -> None:
+            super().__init__(runtime)
+            self.base = base
+
+        def apply(self, q, k, positions) -> None:
+            s = torch.pow(torch.tensor(self.base, device=q.device), positions.float())[:, None, None]
+            q.mul_(s.to(q.dtype))
+            if k is not None:
+                k.div_(s.to(k.dtype))
+
+    def build(cfg):
+        h = cfg["hidden_size"]
+        norm = dict(width=h, eps=cfg["eps"])
+        attn = dict(hidden_size=h, num_heads=4, num_kv_heads=2, head_dim=16)
+        ffs = [PartSpec("toy_routed", dict(hidden_size=h, experts=3, expert_size=24), "layers.0.moe."),
+               PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=40), "layers.1.mlp.")]
+        poss = [PartSpec("toy_decay", dict(base=1.04)), PartSpec("rotary", dict(dim=16, theta=100.0))]
+        layers = [LayerSpec(PartSpec("pre_norm"), {
+            "mixer_norm": ("norm", PartSpec("rms_norm", norm, f"layers.{i}.n1.")),
+            "mixer": ("mixer", PartSpec("gqa_attention", dict(attn, position=poss[i]), f"layers.{i}.attn.")),
+            "feed_forward_norm": ("norm", PartSpec("rms_norm", norm, f"layers.{i}.n2.")),
+            "feed_forward": ("feed_forward", ffs[i])}) for i in range(2)]
+        return ModelSpec(
+            architecture="ToyRoutedForCausalLM", vocab_size=cfg["vocab_size"], hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=cfg["vocab_size"], hidden_size=h), "embed."),
+            layers=tuple(layers), schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+            final_norm=PartSpec("rms_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=cfg["vocab_size"], hidden_size=h, tied=False), "head."))
+
+    register_architecture("ToyRoutedForCausalLM", dict, build)
+    try:
+        import tempfile
+
+        raw = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 47, "hidden_size": 32, "eps": 1e-6}
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, raw, seed=8, std=0.25, norm_jitter=0.1)
+            make = lambda: build_core(load_model(folder, dtype="float32"), num_pages=14, page_size=4, max_seqs=4,
+                                      enable_prefix_caching=False, watermark=0.0)
+            toks = {"a": [5, 9, 2, 40, 33, 7, 7, 12, 46, 1, 18, 25, 3, 3, 44, 21, 9, 30, 2, 11, 17],
+                    "b": [8, 8, 1, 30, 23, 4, 19, 36, 2, 45, 13, 27]}
+            whole, routes = {}, set()
+            for rid, t in toks.items():
+                core = make()
+                whole[rid] = TraceSession(core).step([{"id": rid, "tokens": t, "want": list(range(len(t)))}]).cpu()
+                moe = core.model.layers[0].parts["feed_forward"]
+                x = torch.randn(64, 32, device="cuda")
+                routes |= set((x @ moe.t["router.weight"].float().T).argmax(-1).tolist())
+            assert len(routes) > 1, "the router always picks the same expert: the test would prove little"
+            core = make()
+            s = TraceSession(core)
+            got, fed = {"a": [], "b": []}, {"a": 0, "b": 0}
+            for stepplan in [{"a": 5}, {"a": 2, "b": 3}, {"a": 1, "b": 1}, {"b": 6}, {"a": 9, "b": 1}, {"a": 1, "b": 1}, {"a": 3}]:
+                entries = [{"id": rid, "tokens": toks[rid][fed[rid]:fed[rid] + n], "want": list(range(n))}
+                           for rid, n in stepplan.items()]
+                out = s.step(entries).cpu()
+                row = 0
+                for rid, n in stepplan.items():
+                    got[rid].append(out[row:row + n])
+                    row += n
+                    fed[rid] += n
+            for rid in toks:
+                assert fed[rid] == len(toks[rid])
+                assert (torch.cat(got[rid]) - whole[rid]).abs().max() < 1e-4, rid
+    finally:
+        unregister_architecture("ToyRoutedForCausalLM")
+        unregister_part("feed_forward", "toy_routed")
+        unregister_part("position", "toy_decay")
