@@ -202,10 +202,22 @@ class StepFunction:
         mgr, ps = self.manager, self.manager.page_size
         if steps > self.max_decode_steps:
             raise StepError(f"{steps} tokens per step asked for, {self.max_decode_steps} possible")
-        if copy_ops or sampling is None or len(sampling) != len(entries) or not self.graphs.can_run(entries, steps):
+        if copy_ops or sampling is None or len(sampling) != len(entries) or any(len(e.tokens) != 1 for e in entries):
             raise StepError("several tokens per step need a decode-only batch that samples every request")
         if len({e.seq_id for e in entries}) != len(entries):
             raise StepError("a request appears twice in one step")
+        if not self.graphs.can_run(entries, steps):
+            # longer than the graphs were sized for: the same tokens, one step at a time
+            rounds, cur = [], list(entries)
+            for j in range(steps):
+                toks = self.run(cur, (), [(t, k, p, seed, draw + j) for t, k, p, seed, draw in sampling])
+                rounds.append(toks)
+                if j + 1 < steps:
+                    for e, tok in zip(cur, toks):
+                        if mgr.append_slots(e.seq_id, [tok]):
+                            raise StepError("a page reserved ahead was shared")
+                    cur = [StepEntry(e.seq_id, (tok,), e.start + 1, (0,)) for e, tok in zip(cur, toks)]
+            return rounds
         for e in entries:
             if e.start != mgr.num_computed_tokens(e.seq_id) or e.start + 1 != mgr.num_tokens(e.seq_id):
                 raise StepError(f"request {e.seq_id!r}: its last token must be the only one not computed")

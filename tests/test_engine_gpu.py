@@ -131,12 +131,15 @@ def test_graph_replay_equals_eager_steps(name, block):
         assert torch.equal(a, b), f"step {i}: graph replay differs from the eager step by {(a - b).abs().max()}"
 
 
-@pytest.mark.parametrize("name,block,k", [("A", 16, 4), ("C", 32, 3), ("B", 16, 8)])
-def test_several_decode_tokens_per_step_equal_one_per_step(name, block, k):
+@pytest.mark.parametrize("name,block,k,graph_len", [("A", 16, 4, None), ("C", 32, 3, None), ("B", 16, 8, None),
+                                                   ("A", 16, 4, 40)])
+def test_several_decode_tokens_per_step_equal_one_per_step(name, block, k, graph_len):
     """Steps that decode `k` tokens of every request on the device (sampled tokens fed back there,
     positions, slots and draw counters advanced by a kernel) against one token per step: greedy
     and seeded sampling give the same tokens; limits that are no multiple of k, a stop token
-    inside a run, prompts that end at a page's edge, and pages reserved ahead that are returned."""
+    inside a run, prompts that end at a page's edge, and pages reserved ahead that are returned.
+    `graph_len`: the graphs are sized for shorter requests than some that come, whose tokens then
+    run one step at a time."""
     from dli_amd.engine import LLMEngine, SchedulerConfig
     from dli_amd.sampling import SamplingParams
 
@@ -145,6 +148,7 @@ def test_several_decode_tokens_per_step_equal_one_per_step(name, block, k):
 
     def run(steps, stop=()):
         eng = LLMEngine.for_model(str(model_folder(name)), dtype="bfloat16", num_blocks=64, block_size=block,
+                                  max_model_len=graph_len,
                                   config=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=256, decode_steps=steps))
         params = [SamplingParams(max_tokens=limits[0], stop_token_ids=tuple(stop)),
                   SamplingParams(max_tokens=limits[1], temperature=0.8, top_k=12, seed=5),
