@@ -1,0 +1,89 @@
+"""The engine at the layer sizes it serves (Llama-3.2-1B's widths, two layers) against the plain
+implementation: the kernels that the tiny configurations reach only through their kernel tests
+(head size 64 in groups of four, products of depth 2048 and 8192, decode graphs at batch 1 and 8)
+run here inside the whole model."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+import torch
+
+import plain_llama as P
+from test_model_gpu import check
+from tiny_configs import model_folder
+
+pytestmark = pytest.mark.gpu
+
+_plain: dict = {}
+
+
+def plain(tokens):
+    key = tuple(tokens)
+    if key not in _plain:
+        cfg, w = P.load_folder(model_folder("W"))
+        _plain[key] = P.forward_logits(w, cfg, tokens)
+    return _plain[key]
+
+
+def make_core(dtype, pages, page=16, graphs=0):
+    from dli_amd.engine.core import build_core
+
+    core = build_core(model_folder("W"), num_pages=pages, page_size=page, max_seqs=8, dtype=dtype,
+                      enable_prefix_caching=False, watermark=0.0)
+    if graphs:
+        core.step.enable_decode_graphs(graphs, pages * page)
+    return core
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_whole_prompt_then_decoding_at_serving_widths(dtype):
+    from dli_amd.trace import TraceSession
+
+    rng = random.Random(3)
+    toks = [rng.randrange(32003) for _ in range(150 if dtype == "bfloat16" else 70)]
+    ref = plain(toks)
+    core = make_core(dtype, pages=12, graphs=1)
+    s = TraceSession(core)
+    got = s.step([{"id": "w", "tokens": toks, "want": list(range(len(toks)))}], end=["w"])
+    check(got, ref, dtype, "wide whole")
+    head = len(toks) - 24
+    got = s.step([{"id": "d", "tokens": toks[:head], "want": [head - 1]}])
+    check(got, ref[head - 1:head], dtype, "wide prefix")
+    for i in range(head, len(toks)):  # one row: the 4x4-block products, through the decode graph in bfloat16
+        got = s.step([{"id": "d", "tokens": [toks[i]], "want": [0]}])
+        check(got, ref[i:i + 1], dtype, f"wide decode at {i}")
+    if dtype == "bfloat16":
+        assert core.step.graphs is not None and core.step.graphs.replays >= 24
+
+
+def test_eight_requests_decode_together_at_serving_widths():
+    """Prompts of different lengths go in as a mixed batch of portions, then all eight decode side
+    by side (the 16x16-tile products with their fused norm, SwiGLU and residual epilogues)."""
+    from dli_amd.trace import TraceSession
+
+    rng = random.Random(4)
+    lens = [37, 64, 50, 33, 71, 48, 40, 59]
+    toks = [[rng.randrange(32003) for _ in range(n + 10)] for n in lens]
+    core = make_core("bfloat16", pages=48, graphs=8)
+    s = TraceSession(core)
+    fed = [0] * 8
+    # prompts in two mixed steps of portions
+    for part in (0, 1):
+        entries = []
+        for r in range(8):
+            n = lens[r] // 2 if part == 0 else lens[r] - lens[r] // 2
+            entries.append({"id": r, "tokens": toks[r][fed[r]:fed[r] + n], "want": [n - 1] if part else []})
+            fed[r] += n
+        out = s.step(entries)
+    rows = torch.stack([plain(toks[r])[lens[r] - 1] for r in range(8)])
+    check(out, rows, "bfloat16", "wide mixed prompts")
+    for stepno in range(10):
+        entries = [{"id": r, "tokens": [toks[r][fed[r]]], "want": [0]} for r in range(8)]
+        out = s.step(entries)
+        rows = torch.stack([plain(toks[r])[fed[r]] for r in range(8)])
+        check(out, rows, "bfloat16", f"wide decode step {stepno}")
+        for r in range(8):
+            fed[r] += 1
+    assert core.step.graphs.replays >= 10

@@ -30,7 +30,18 @@ TINY_C = {
     "rope_scaling": {"type": "linear", "factor": 2.0}, "attention_bias": True, "mlp_bias": True,
     "tie_word_embeddings": False, "hidden_act": "silu",
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# the layer sizes of Llama-3.2-1B (width 2048, 32 heads of 64 on 8 kv heads, feed-forward 8192,
+# llama3 rope, tied head) with two layers and a quarter of the vocabulary (odd on purpose): the
+# kernels meet the shapes they serve
+WIDE = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 32003, "hidden_size": 2048,
+    "intermediate_size": 8192, "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 64, "rms_norm_eps": 1e-5, "max_position_embeddings": 131072, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": True, "hidden_act": "silu",
+}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "W": WIDE}
 
 _made: dict = {}
 _tmp = None
@@ -40,7 +51,7 @@ _tmp = None
 # have a spread of about one, so attention is far from uniform (a key in the wrong place, a wrong
 # rotation or a wrong mask changes the logits) without being so sharp that bfloat16's rounding of a
 # score is blown up into a different distribution.
-STD = {"A": 0.15, "B": 0.085, "C": 0.085}
+STD = {"A": 0.15, "B": 0.085, "C": 0.085, "W": 0.0265}
 
 
 def model_folder(name: str, seed: int = 11, std: float | None = None, norm_jitter: float = 0.1) -> Path:
