@@ -17,6 +17,11 @@
 // quads and many waves suit products with few features (every compute unit still gets a
 // workgroup, and many loads are in flight on each); more quads read the activations less often.
 //
+// With XL the activations go through LDS: all threads of the workgroup read x once (whole lines),
+// apply the norm there and then, and leave xhat in LDS, from where the waves take their fragments.
+// The loop then holds no loads but the weights' and no arithmetic but the products. Used when
+// rows * k fits (64 KB) and the product has many tiles (see launch4).
+//
 // Fused in (template switches), as in the product for more rows:
 //   NORM          xhat = cast(norm_w[k] * cast(x[m][k] * rs[m])), rs[m] = rsqrt(sum_k x^2 / K + eps)
 //                 from the parts of the row sums of squares that the producer of x left
@@ -45,7 +50,7 @@ __device__ __forceinline__ float4v mfma4(short4v a, short4v b, float4v c) {
   return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
 }
 
-template <int KS, int FQ, int MG, int EPI, bool NORM>
+template <int KS, int FQ, int MG, int EPI, bool NORM, bool XL>
 __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
     const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
@@ -57,6 +62,7 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
   __shared__ float4v red[KS][PAIRS][16];
   __shared__ float4v fin[PAIRS][4];
   __shared__ float sqs[OQ][MG][4];
+  extern __shared__ __attribute__((aligned(16))) bf16_t xs[];  // XL: xhat, rows of XPAD(K) values
 
   const int lane = threadIdx.x % 64, ks = threadIdx.x / 64;
   const int r = lane % 4, blk = lane / 4;
@@ -83,6 +89,42 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     xrow[g] = m < M ? (int)(m * ldx * 2) : -1;
     rs[g] = 1.f;
   }
+  float4v acc[FQ][MG];
+#pragma unroll
+  for (int f = 0; f < FQ; ++f)
+#pragma unroll
+    for (int g = 0; g < MG; ++g) acc[f][g] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // chunks of 128 k: this wave's share
+  const int chunks = (K + 127) / 128;
+  const int c0 = chunks * ks / KS, c1 = chunks * (ks + 1) / KS;
+
+  struct Stage {
+    Frag16 wf[FQ], xf[MG];
+    float4v g0, g1;
+  };
+  const int xpad = chunks * 128 + 32;  // XL: values per row of xs; rows 64 bytes apart in the banks
+  // Every turn of the loop issues the same loads (the last one reads its own chunk again), so the
+  // number of loads in flight is known at compile time and only the current chunk is waited for.
+  auto fetch = [&](int c, Stage& st) __attribute__((always_inline)) {
+    const int k = c * 128 + blk * 8;
+    const bool inside = k < K;  // the last chunk may reach past k; K % 8 == 0
+    const int kc = inside ? k : 0;
+#pragma unroll
+    for (int f = 0; f < FQ; ++f) st.wf[f].raw = *reinterpret_cast<const u32x4*>(wrow[f] + kc);
+    if constexpr (!XL) {
+#pragma unroll
+      for (int g = 0; g < MG; ++g)
+        st.xf[g].raw = __builtin_amdgcn_raw_buffer_load_b128(
+            xres, inside && xrow[g] >= 0 ? xrow[g] + k * 2 : (int)x_bytes, 0, 0);
+      if constexpr (NORM) {
+        st.g0 = *reinterpret_cast<const float4v*>(norm_w + kc);
+        st.g1 = *reinterpret_cast<const float4v*>(norm_w + kc + 4);
+      }
+    }
+  };
+  Stage cur;
+  if (XL && c0 < c1) fetch(c0, cur);  // the first weights are on their way while x is staged
   if constexpr (NORM) {
     // rs[m] from the parts of sum x^2. The parts are dealt out to all blocks of all waves (block
     // q of 16*KS takes the parts q, q + 16*KS, ...), eight loads at a time so that they share one
@@ -119,44 +161,51 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     }
   }
 
-  float4v acc[FQ][MG];
-#pragma unroll
-  for (int f = 0; f < FQ; ++f)
-#pragma unroll
-    for (int g = 0; g < MG; ++g) acc[f][g] = float4v{0.f, 0.f, 0.f, 0.f};
-
-  // chunks of 128 k: this wave's share
-  const int chunks = (K + 127) / 128;
-  const int c0 = chunks * ks / KS, c1 = chunks * (ks + 1) / KS;
-
-  struct Stage {
-    Frag16 wf[FQ], xf[MG];
-    float4v g0, g1;
-  };
-  // Every turn of the loop issues the same loads (the last one reads its own chunk again), so the
-  // number of loads in flight is known at compile time and only the current chunk is waited for.
-  auto fetch = [&](int c, Stage& st) {
-    const int k = c * 128 + blk * 8;
-    const bool inside = k < K;  // the last chunk may reach past k; K % 8 == 0
-    const int kc = inside ? k : 0;
-#pragma unroll
-    for (int f = 0; f < FQ; ++f) st.wf[f].raw = *reinterpret_cast<const u32x4*>(wrow[f] + kc);
-#pragma unroll
-    for (int g = 0; g < MG; ++g)
-      st.xf[g].raw = __builtin_amdgcn_raw_buffer_load_b128(
-          xres, inside && xrow[g] >= 0 ? xrow[g] + k * 2 : (int)x_bytes, 0, 0);
+  if (!XL && c0 < c1) fetch(c0, cur);
+  if constexpr (XL) {
+    // thread t stages the 8 values at k = 8*(t % (chunks*16)) of row t / (chunks*16), and so on
+    __shared__ float rs_row[4 * MG];
     if constexpr (NORM) {
-      st.g0 = *reinterpret_cast<const float4v*>(norm_w + kc);
-      st.g1 = *reinterpret_cast<const float4v*>(norm_w + kc + 4);
+      if (ks == 0 && blk == 0) {
+#pragma unroll
+        for (int g = 0; g < MG; ++g) rs_row[4 * g + r] = rs[g];
+      }
+      __syncthreads();
     }
-  };
+    const int per_row = chunks * 16;
+    for (int idx = threadIdx.x; idx < M * per_row; idx += KS * 64) {
+      const int m = idx / per_row, k = (idx - m * per_row) * 8;
+      Frag16 v;
+      v.raw = u32x4{0, 0, 0, 0};
+      if (k < K) {
+        v.raw = *reinterpret_cast<const u32x4*>(x + (int64_t)m * ldx + k);
+        if constexpr (NORM) {
+          const float4v g0 = *reinterpret_cast<const float4v*>(norm_w + k);
+          const float4v g1 = *reinterpret_cast<const float4v*>(norm_w + k + 4);
+          const float rsm = rs_row[m];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float normed = (float)(bf16_t)((float)v.e[i] * rsm);
+            v.e[i] = (bf16_t)((i < 4 ? g0[i] : g1[i - 4]) * normed);
+          }
+        }
+      }
+      *reinterpret_cast<u32x4*>(xs + (int64_t)m * xpad + k) = v.raw;
+    }
+    __syncthreads();
+  }
   if (c0 < c1) {
-    Stage cur;
-    fetch(c0, cur);
     for (int c = c0; c < c1; ++c) {
       Stage nxt;
       fetch(min(c + 1, c1 - 1), nxt);
-      if constexpr (NORM) {
+      if constexpr (XL) {
+#pragma unroll
+        for (int g = 0; g < MG; ++g) {
+          const int m = 4 * g + r;
+          cur.xf[g].raw = u32x4{0, 0, 0, 0};
+          if (m < M) cur.xf[g].raw = *reinterpret_cast<const u32x4*>(xs + (int64_t)m * xpad + c * 128 + blk * 8);
+        }
+      } else if constexpr (NORM) {
 #pragma unroll
         for (int g = 0; g < MG; ++g)
 #pragma unroll
@@ -295,9 +344,18 @@ template <int KS, int FQ, int MG, int EPI, bool NORM>
 static void launch4(S4_PARAMS) {
   constexpr int OQ = EPI == EPI_SWIGLU ? FQ / 2 : FQ;
   const int tiles = (N + 4 * OQ - 1) / (4 * OQ);
-  skinny4_kernel<KS, FQ, MG, EPI, NORM><<<tiles, KS * 64, 0, stream>>>(
-      (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
-      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
+  // The activations are staged through LDS when they fit 64 KB there and the product has many
+  // tiles: staging costs a workgroup a barrier and a trip to memory before its first product, which
+  // pays when each compute unit works through several workgroups, and does not for a short kernel.
+  const int64_t x_lds = (int64_t)M * ((K + 127) / 128 * 128 + 32) * 2;
+  if (x_lds <= 64 * 1024 && tiles >= 4 * dli_compute_units())
+    skinny4_kernel<KS, FQ, MG, EPI, NORM, true><<<tiles, KS * 64, (size_t)x_lds, stream>>>(
+        (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
+        out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
+  else
+    skinny4_kernel<KS, FQ, MG, EPI, NORM, false><<<tiles, KS * 64, 0, stream>>>(
+        (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
+        out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
 }
 
 template <int KS, int FQ, int EPI, bool NORM>
