@@ -167,6 +167,30 @@ __global__ __launch_bounds__(256) void rope_kv_write_token_kernel(
   }
 }
 
+// cos and sin of every token's angles, rounded to the activation type as the rotation uses them:
+// table[t][0][i] = cos(pos[t] * inv_freq[i]), table[t][1][i] = sin(...), float32. Computed once a
+// step for kernels that rotate on the fly in every layer.
+template <typename T>
+__global__ void rope_angles_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                   float* __restrict__ table, int half) {
+  const int64_t token = blockIdx.x;
+  const float pos = (float)positions[token];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float sv, cv;
+    sincosf(pos * inv_freq[i], &sv, &cv);
+    table[(token * 2 + 0) * half + i] = round_to<T>(cv);
+    table[(token * 2 + 1) * half + i] = round_to<T>(sv);
+  }
+}
+
+extern "C" int dli_rope_angles(const int* positions, const float* inv_freq, float* table, int tokens,
+                               int half, int is_bf16, hipStream_t stream) {
+  if (tokens <= 0 || half <= 0) return DLI_OK;
+  if (is_bf16) rope_angles_kernel<bf16_t><<<tokens, 64, 0, stream>>>(positions, inv_freq, table, half);
+  else rope_angles_kernel<float><<<tokens, 64, 0, stream>>>(positions, inv_freq, table, half);
+  return dli_launch_status();
+}
+
 extern "C" int dli_rope_kv_write(void* qkv, int64_t row_stride, const int* positions,
                                  const float* inv_freq, int rotary_dim, const int* slots,
                                  void* k_pages, void* v_pages, int tokens, int q_heads, int kv_heads,

@@ -59,6 +59,7 @@ class StepContext:
     state_slots_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     seq_ids: list = field(default_factory=list)
     _tiles: dict = field(default_factory=dict)
+    _angles: dict = field(default_factory=dict)
 
     @property
     def max_kv_len(self) -> int:
@@ -70,6 +71,23 @@ class StepContext:
 
     def entry_rows(self, e: int) -> tuple[int, int]:
         return int(self.q_start_host[e]), int(self.q_start_host[e + 1])
+
+    def begin_forward(self) -> None:
+        """Called at the start of every forward pass over this context: forgets what was derived
+        from arrays that may have changed on the device since the last pass (positions move when a
+        graph runs several decode steps on one context)."""
+        self._angles.clear()
+
+    def rope_angles(self, inv_freq: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        """cos/sin of the step's positions for the rotary table ``inv_freq``, ``[tokens, 2, half]``:
+        made at the first call of a forward pass and shared by all layers that use that table."""
+        key = (inv_freq.data_ptr(), dtype)
+        hit = self._angles.get(key)
+        if hit is None:
+            from ..kernels import ops
+
+            hit = self._angles[key] = ops.rope_angles(self.positions, inv_freq, dtype)
+        return hit
 
     def is_fresh(self, e: int) -> bool:
         """The entry starts its request at position 0 (per-request state must be reset)."""

@@ -17,6 +17,8 @@ The reference replays CUDA graphs of batched decode in fixed buckets the same wa
 
 from __future__ import annotations
 
+import gc
+
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
@@ -157,8 +159,19 @@ class DecodeGraphs:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = body()
+        # No cyclic garbage collection while the stream is capturing: a dead cycle that holds
+        # device memory or an older graph (an engine that was dropped) would be destroyed in the
+        # middle of the capture, and freeing those is not allowed there (the process aborts).
+        # Such cycles are collected before the capture instead.
+        collecting = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                logits = body()
+        finally:
+            if collecting:
+                gc.enable()
         return _Captured(graph, ctx, host, dev, logits, views, width, [None] * b, tokens_host)
 
     # ------------------------------------------------------------------ replay

@@ -56,6 +56,10 @@ _SIGNATURES = {
     "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "dli_rope_angles": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_attention_decode_rope_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
+                                       _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                                       _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                    _c_ptr],
@@ -523,6 +527,62 @@ def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml),
         _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size,
         float(scale), int(window), int(splits), _stream()), "attention_decode")
+
+
+def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """``[tokens, 2, half]`` float32: cos and sin of ``float(position) * inv_freq``, rounded to
+    ``dtype`` as the rotation kernels round them. One table serves every layer of a step."""
+    _dense(positions, "positions", torch.int32, 1)
+    _dense(inv_freq, "inv_freq", torch.float32, 1)
+    n, half = positions.shape[0], inv_freq.shape[0]
+    table = torch.empty(n, 2, half, device=positions.device, dtype=torch.float32)
+    _check(library().dli_rope_angles(_ptr(positions), _ptr(inv_freq), _ptr(table), n, half, _is_bf16(dtype),
+                                     _stream()), "rope_angles")
+    return table
+
+
+def attention_decode_rope(qkv: torch.Tensor, angles: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                          out: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor, q_heads: int,
+                          scale: float, window: int = 0, splits: int = 1, part_o: Optional[torch.Tensor] = None,
+                          part_ml: Optional[torch.Tensor] = None) -> None:
+    """:func:`attention_decode` with the rotation of q and k and the cache write of the decoded
+    tokens inside: ``qkv [rows, (q_heads + 2*kv_heads) * head_dim]`` is the fused projection as
+    the product left it; ``angles [rows, 2, head_dim/2]`` comes from :func:`rope_angles` (the
+    rotation covers the whole head); row ``e`` is the token at position ``kv_len[e] - 1``, whose
+    page the block table names already. The token's rotated key and its value are written into
+    the pages."""
+    _dense(k_pages, "k_pages", torch.bfloat16, 4)
+    _dense(v_pages, "v_pages", torch.bfloat16, 4)
+    pages, kv_heads, page_size, head_dim = k_pages.shape
+    _require(v_pages.shape == (pages, kv_heads, head_dim, page_size),
+             "v_pages must be [pages, kv_heads, head_dim, page_size]")
+    _rows(qkv, "qkv", torch.bfloat16)
+    _rows(out, "out", torch.bfloat16)
+    rows = qkv.shape[0]
+    _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
+    _require(qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim and out.shape == (rows, q_heads * head_dim),
+             "qkv must be [rows, (q_heads + 2*kv_heads)*head_dim] and out [rows, q_heads*head_dim]")
+    _require(qkv.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and qkv.data_ptr() % 8 == 0 and out.data_ptr() % 8 == 0,
+             "qkv/out rows must be 8-byte aligned")
+    _require(bool(library().dli_attention_mfma_supports(head_dim, page_size)),
+             f"the matrix-core attention takes head_dim 16..128 in steps of 16 and pages of a multiple of 16, "
+             f"not head_dim {head_dim}, page size {page_size}")
+    _dense(angles, "angles", torch.float32, 3)
+    _require(angles.shape == (rows, 2, head_dim // 2), "angles must be [rows, 2, head_dim/2]: the rotation covers the whole head")
+    _dense(kv_len, "kv_len", torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    _require(kv_len.shape[0] >= rows and block_tables.shape[0] >= rows, "one kv_len and table row per request")
+    _require(1 <= splits <= 65535 and rows <= 65535, "splits and requests must fit the grid")
+    if splits > 1:
+        _require(part_o is not None and part_ml is not None, "splits > 1 needs the partial-result buffers")
+        _dense(part_o, "part_o", torch.float32)
+        _dense(part_ml, "part_ml", torch.float32)
+        _require(part_o.numel() >= rows * q_heads * splits * head_dim and part_ml.numel() >= rows * q_heads * splits * 2,
+                 "partial-result buffers are too small")
+    _check(library().dli_attention_decode_rope_bf16(
+        _ptr(qkv), qkv.stride(0), _ptr(angles), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0),
+        _ptr(part_o), _ptr(part_ml), _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads,
+        kv_heads, head_dim, page_size, float(scale), int(window), int(splits), _stream()), "attention_decode_rope")
 
 
 def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,

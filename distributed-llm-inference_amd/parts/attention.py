@@ -20,11 +20,16 @@ from typing import Any, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .attention_kernels import paged_attention
+from .attention_kernels import decode_attention_with_rope, paged_attention
 from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
 from .linear import linear
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
+
+# Decode steps of at most this many rows rotate q and k and write the cache inside the attention
+# kernel; larger ones run the rotation kernel first (measured: the fused form saves a launch's
+# latency at one row and loses to the separate kernel once every compute unit has work).
+ROPE_IN_ATTENTION_MAX_ROWS = 2
 
 
 @register_part("mixer", "gqa_attention")
@@ -126,8 +131,13 @@ class GQAttention(Mixer):
             inv_freq, rotary_dim = None, 0
         else:
             inv_freq, rotary_dim = table
-        ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
-                          cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         out = self.rt.empty(n, nh * d)
-        paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        if nkv and inv_freq is not None and rotary_dim == d and n <= ROPE_IN_ATTENTION_MAX_ROWS:
+            # rotation and cache write happen inside the attention kernel
+            decode_attention_with_rope(qkv, inv_freq, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale,
+                                       self.window)
+        else:
+            ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
+                              cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
+            paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         stream.ssq = ops.skinny_gemm(out, self.w_o, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, bias=self.b_o)

@@ -43,16 +43,33 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
         return
     nd = ctx.num_decode
     if nd > 0:
-        group = q_heads // kv_heads
-        splits = getattr(ctx, "forced_splits", None) or choose_splits(
-            nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len)
-        part_o = part_ml = None
-        if splits > 1:
-            part_o = torch.empty(nd * q_heads * splits * head_dim, device=q.device, dtype=torch.float32)
-            part_ml = torch.empty(nd * q_heads * splits * 2, device=q.device, dtype=torch.float32)
+        splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device)
         ops.attention_decode(q[:nd], k_pages, v_pages, out[:nd], ctx.kv_len, grp.block_tables, q_heads,
                              scale, window, splits, part_o, part_ml)
     if ctx.num_entries > nd:
         tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads), first_entry=nd)
         ops.attention_prefill(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
                               tile_entry, tile_q0, q_heads, scale, window)
+
+
+def _decode_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, head_dim: int, device: torch.device):
+    group = q_heads // kv_heads
+    splits = getattr(ctx, "forced_splits", None) or choose_splits(
+        nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty(nd * q_heads * splits * head_dim, device=device, dtype=torch.float32)
+        part_ml = torch.empty(nd * q_heads * splits * 2, device=device, dtype=torch.float32)
+    return splits, part_o, part_ml
+
+
+def decode_attention_with_rope(qkv: torch.Tensor, inv_freq: torch.Tensor, k_pages: torch.Tensor,
+                               v_pages: torch.Tensor, out: torch.Tensor, ctx: Any, grp: Any, q_heads: int,
+                               scale: float, window: int = 0) -> None:
+    """A decode-only step's attention with rotation and cache write inside the attention kernel:
+    ``qkv`` is the fused projection, unrotated; the tokens' keys and values reach the pages here.
+    The angles' cos and sin are computed once per step and rotary table, for all layers."""
+    _, kv_heads, _, head_dim = k_pages.shape
+    splits, part_o, part_ml = _decode_splits(ctx, ctx.num_decode, q_heads, kv_heads, head_dim, qkv.device)
+    ops.attention_decode_rope(qkv, ctx.rope_angles(inv_freq, qkv.dtype), k_pages, v_pages, out, ctx.kv_len,
+                              grp.block_tables, q_heads, scale, window, splits, part_o, part_ml)

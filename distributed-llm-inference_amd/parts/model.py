@@ -136,6 +136,7 @@ class Model:
 
     def forward(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
         """Run the step's tokens through the schedule; float32 logits ``[wanted rows, vocab]``."""
+        ctx.begin_forward()
         if self._streams(ctx):
             return self._forward_stream(ctx, caches)
         x = self.embedding.forward(ctx.token_ids)

@@ -45,6 +45,9 @@ def rotary_inverse_frequencies(dim: int, theta: float, rope_type: str = "default
     return inv.astype(np.float32)
 
 
+_TABLES: dict = {}
+
+
 @register_part("position", "rotary")
 class Rotary(PositionEncoding):
     def __init__(self, runtime: Runtime, *, dim: int, theta: float, rope_type: str = "default",
@@ -58,7 +61,13 @@ class Rotary(PositionEncoding):
         self._table: Optional[torch.Tensor] = None
 
     def finalize(self) -> None:
-        self._table = torch.from_numpy(self.inv_freq_host.copy()).to(self.rt.device)
+        # equal tables share one device tensor, so that what a step derives from a table (the cos
+        # and sin of its positions) is derived once for all layers
+        key = (str(self.rt.device), self.inv_freq_host.tobytes())
+        hit = _TABLES.get(key)
+        if hit is None:
+            hit = _TABLES[key] = torch.from_numpy(self.inv_freq_host.copy()).to(self.rt.device)
+        self._table = hit
 
     def rotary_table(self) -> Optional[tuple[torch.Tensor, int]]:
         if self._table is None:

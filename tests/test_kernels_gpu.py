@@ -218,6 +218,41 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
     assert err < tol(torch.bfloat16), err
 
 
+@pytest.mark.parametrize("qh,kvh,d,bs", [(8, 2, 64, 16), (32, 8, 64, 16), (6, 2, 32, 16), (20, 1, 48, 32), (4, 4, 128, 16)])
+@pytest.mark.parametrize("splits", [1, 4, 16])
+@pytest.mark.parametrize("window", [0, 45])
+def test_attention_decode_with_rotation_and_cache_write_inside(ops, qh, kvh, d, bs, splits, window):
+    """The decode kernel that rotates q and k and writes the new token's key and value itself,
+    against the separate rotation kernel followed by the plain decode kernel: same outputs, same
+    pages (a rounding of the rotated values apart), nothing else touched."""
+    rng = torch.Generator().manual_seed(d + bs + splits)
+    lens = [(1, n) for n in [1, 2, bs, bs + 1, 3 * bs - 1, 16, 17, 33] + [int(x) for x in torch.randint(1, 30 * bs, (5,), generator=rng)]]
+    _, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + splits, poison=False)
+    n = len(lens)
+    qkv = torch.randn(n, (qh + 2 * kvh) * d, generator=rng).bfloat16().cuda()
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d))).cuda()
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    positions = dev([k - 1 for k in kv_len])
+    slots = dev([tables[e][(kv_len[e] - 1) // bs] * bs + (kv_len[e] - 1) % bs for e in range(n)])
+    scale = 1.0 / math.sqrt(d)
+    parts = lambda: (torch.full((n * qh * splits * d,), float("nan"), device="cuda"),
+                     torch.full((n * qh * splits * 2,), float("nan"), device="cuda"))
+    # separate kernels
+    kp1, vp1, qkv1 = kp.cuda().clone(), vp.cuda().clone(), qkv.clone()
+    ops.rope_kv_write(qkv1, positions, inv_freq, d, slots, kp1, vp1, qh, kvh, d)
+    out1 = torch.zeros(n, qh * d, dtype=torch.bfloat16, device="cuda")
+    ops.attention_decode(qkv1[:, :qh * d], kp1, vp1, out1, dev(kv_len), dev(tables), qh, scale, window, splits, *parts())
+    # one kernel
+    kp2, vp2 = kp.cuda().clone(), vp.cuda().clone()
+    out2 = torch.zeros(n, qh * d, dtype=torch.bfloat16, device="cuda")
+    ops.attention_decode_rope(qkv, ops.rope_angles(positions, inv_freq, torch.bfloat16), kp2, vp2, out2, dev(kv_len), dev(tables), qh, scale, window, splits, *parts())
+    assert torch.equal(vp1, vp2)
+    assert (kp1.float() - kp2.float()).abs().max() <= 2 ** -7 * kp1.float().abs().max()
+    changed = (kp2 != kp.cuda()).any(dim=-1).sum().item()
+    assert changed <= n * kvh, "keys other than the new tokens' were written"
+    assert (out1.float() - out2.float()).abs().max() < tol(torch.bfloat16)
+
+
 @pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("pair", [False, True])
