@@ -99,16 +99,22 @@ def test_gemm_f32(ops, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("qh,kvh,d,rd,bs", [(4, 4, 16, 16, 16), (6, 2, 32, 32, 8), (3, 1, 48, 32, 4), (2, 2, 80, 80, 16)])
-@pytest.mark.parametrize("n", [11, 70])  # few tokens: one item per thread; many: one workgroup per token
-def test_rope_kv_write(ops, dtype, qh, kvh, d, rd, bs, n):
+# few tokens: one item per thread; many: a workgroup per 8 tokens, which writes v in runs where the
+# slots are consecutive and aligned in a page (and element by element where they are not)
+@pytest.mark.parametrize("n,slots_as", [(11, "scattered"), (70, "scattered"), (203, "consecutive"), (150, "offset")])
+def test_rope_kv_write(ops, dtype, qh, kvh, d, rd, bs, n, slots_as):
     torch.manual_seed(4)
-    pages = max(9, -(-n // bs) + 2)
+    pages = max(9, -(-n // bs) + 3)
     qkv = torch.randn(n, (qh + 2 * kvh) * d, device="cuda").to(dtype)
     orig = qkv.clone()
     positions = torch.tensor([0, 1, 2, 3, 500, 4095, 7, 8, 9, 10, 11] + list(range(100, 100 + n - 11)),
                              dtype=torch.int32, device="cuda")
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rd, 2).float() / rd))).cuda()
-    perm = torch.randperm(pages * bs)[:n]
+    if slots_as == "scattered":
+        perm = torch.randperm(pages * bs)[:n]
+    else:  # a prompt's portion: consecutive slots, from a page's start or from inside a page
+        first = bs if slots_as == "consecutive" else bs + 3
+        perm = torch.arange(first, first + n)
     perm[5] = -1  # not cached
     slots = perm.to(torch.int32).cuda()
     k_pages = torch.full((pages, kvh, bs, d), 7.0, device="cuda").to(dtype)
