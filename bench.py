@@ -36,6 +36,16 @@ LLAMA_3_2_1B = {
     "tie_word_embeddings": True, "hidden_act": "silu",
 }
 
+# the other shapes that the baseline's configurations name, for measurements beside the default one
+LLAMA_3_2_3B = dict(LLAMA_3_2_1B, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, head_dim=128)
+SMOLLM2_1_7B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 49152, "hidden_size": 2048,
+    "intermediate_size": 8192, "num_hidden_layers": 24, "num_attention_heads": 32, "num_key_value_heads": 32,
+    "head_dim": 64, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "rope_theta": 130000.0,
+    "tie_word_embeddings": True, "hidden_act": "silu",
+}
+SHAPES = {"Llama-3.2-1B": LLAMA_3_2_1B, "Llama-3.2-3B": LLAMA_3_2_3B, "SmolLM2-1.7B": SMOLLM2_1_7B}
+
 
 def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1):
     import torch
@@ -148,6 +158,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--shape", default="Llama-3.2-1B", choices=sorted(SHAPES),
+                    help="layer sizes (the default is the configuration that the headline number is quoted on)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
@@ -164,7 +176,7 @@ def main() -> int:
 
     import torch
 
-    raw = dict(LLAMA_3_2_1B)
+    raw = dict(SHAPES[args.shape])
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -181,12 +193,12 @@ def main() -> int:
     tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup, args.decode_steps)
     achieved = decode_bytes(cfg, args.batch, args.context, itemsize) / (ms * 1e-3) / 1e9
     line = {
-        "metric": "decode tok/s at batch 8, Llama-3.2-1B shape",
+        "metric": f"decode tok/s at batch {args.batch}, {args.shape} shape",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
         "config": {
-            "model": "Llama-3.2-1B shape", "global_batch": args.batch, "seq_len": args.context,
+            "model": f"{args.shape} shape", "global_batch": args.batch, "seq_len": args.context,
             "parallelism": "single GPU", "layers": cfg.num_layers, "layers_of_config": full_layers,
             "hidden": cfg.hidden_size, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
