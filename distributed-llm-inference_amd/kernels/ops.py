@@ -301,9 +301,7 @@ def skinny_gemm_shape(n: int, k: int) -> int:
     waves of a workgroup split k (8 ways when k is long), with many they split the tiles so that
     the activations are read once per 8 tiles."""
     tiles = -(-n // 16)
-    if tiles >= 2048:
-        return 2
-    if tiles >= 768:
+    if tiles >= 768:   # a vocabulary: 2 k-waves x 2 n-waves x 2 tiles was ahead of 4 n-waves x 2 tiles
         return 3
     return 1 if k >= 4096 else 0
 

@@ -32,7 +32,16 @@ class LinearHead(Head):
         if self.tied:
             self.weight = table
 
+    FEW_ROWS = 16  # up to here the decode product streams the table faster than the library does
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        rows = x.shape[0]
+        if (self.rt.is_bf16 and 0 < rows <= self.FEW_ROWS and x.dtype == torch.bfloat16
+                and ops.skinny_gemm_supports(rows, self.hidden_size, self.rt.dtype)):
+            # the usual case of a prompt's step: logits for its last row only
+            out = torch.empty(rows, self.vocab_size, device=self.rt.device, dtype=torch.float32)
+            ops.skinny_gemm(x, self.weight, epilogue=ops.SKINNY_F32, out=out)
+            return out
         logits = linear(self.rt, x, self.weight)
         if logits.dtype == torch.float32:
             return logits
