@@ -22,6 +22,12 @@ template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return
 // Round through the storage type: what a value becomes when it is written as T and read back.
 template <typename T> __device__ __forceinline__ float round_to(float x) { return to_f32(from_f32<T>(x)); }
 
+// silu(g) = g * sigmoid(g) in 32-bit (reference: src/dli/model/llama.py:190). Faster forms of the
+// exponential and the division were tried for bfloat16 and changed no timing: the kernels that
+// use it wait for memory.
+template <typename T> __device__ __forceinline__ float silu(float g) { return g / (1.f + expf(-g)); }
+
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int m = DLI_WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, DLI_WAVE);

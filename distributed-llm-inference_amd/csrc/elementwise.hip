@@ -68,6 +68,41 @@ __global__ void rms_norm_vec_kernel(const T* x, const T* __restrict__ delta,
   V* sr = delta != nullptr ? reinterpret_cast<V*>(sum_out + row * width) : nullptr;
   const int chunks = width / 8;
   float ss = 0.f;
+  if (chunks <= (int)blockDim.x) {
+    // one chunk a thread: it stays in registers across the reduction, and the weights are asked
+    // for together with it, so the row is one trip to memory long
+    const int c = threadIdx.x;
+    const bool mine = c < chunks;
+    V v;
+    float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w1 = w0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = from_f32<T>(0.f);
+    if (mine) {
+      v = xr[c];
+      w0 = *reinterpret_cast<const float4*>(weight + c * 8);
+      w1 = *reinterpret_cast<const float4*>(weight + c * 8 + 4);
+      if (dr != nullptr) {
+        const V d = dr[c];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = from_f32<T>(to_f32((T)v[i]) + to_f32((T)d[i]));
+        sr[c] = v;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float f = to_f32((T)v[i]);
+        ss += f * f;
+      }
+    }
+    const float r = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+    if (mine) {
+      const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+      V y;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = from_f32<T>(wv[i] * round_to<T>(to_f32((T)v[i]) * r));
+      reinterpret_cast<V*>(out + row * width)[c] = y;
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
     V v = xr[c];
     if (dr != nullptr) {
@@ -112,7 +147,7 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ ou
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float gf = to_f32((T)g[i]);
-      const float sg = gf / (1.f + expf(-gf));
+      const float sg = silu<T>(gf);
       o[i] = from_f32<T>(round_to<T>(sg) * to_f32((T)u[i]));
     }
     *reinterpret_cast<V*>(out + r * inter + c * 8) = o;
@@ -130,7 +165,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
     const int c = (int)(idx - r * inter);
     const float g = to_f32(gu[r * 2 * inter + c]);
     const float u = to_f32(gu[r * 2 * inter + inter + c]);
-    const float s = g / (1.f + expf(-g));
+    const float s = silu<T>(g);
     out[idx] = from_f32<T>(round_to<T>(s) * u);
   }
 }

@@ -304,7 +304,7 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
           res.e[i] = (bf16_t)y[0][i];
         } else if (EPI == EPI_SWIGLU) {
           const float gt = (float)(bf16_t)y[0][i], up = (float)(bf16_t)y[1][i];
-          const float sg = (float)(bf16_t)(gt / (1.f + expf(-gt)));
+          const float sg = (float)(bf16_t)silu<bf16_t>(gt);
           res.e[i] = (bf16_t)(sg * up);
         } else {  // EPI_RESIDUAL: the sum in 32-bit, rounded to the stream's type
           res.e[i] = (bf16_t)((float)old.e[i] + (float)(bf16_t)y[0][i]);

@@ -288,7 +288,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
             reinterpret_cast<float*>(out)[(int64_t)m * ldo + n] = y[0][i];
           } else if (EPI == EPI_SWIGLU) {
             const float g = (float)(bf16_t)y[0][i], u = (float)(bf16_t)y[NA - 1][i];
-            const float sg = (float)(bf16_t)(g / (1.f + expf(-g)));
+            const float sg = (float)(bf16_t)silu<bf16_t>(g);
             reinterpret_cast<bf16_t*>(out)[(int64_t)m * ldo + n] = (bf16_t)(sg * u);
           } else {  // EPI_RESIDUAL
             bf16_t* sp = stream + (int64_t)m * lds_ + n;

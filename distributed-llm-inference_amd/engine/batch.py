@@ -19,6 +19,24 @@ import numpy as np
 import torch
 
 
+def upload(arrays: Sequence[np.ndarray], device: torch.device) -> list[torch.Tensor]:
+    """The host arrays as device tensors of the same shapes and types, all views of one buffer
+    that one asynchronous copy from pinned memory fills; each starts on a 16-byte boundary. A
+    copy from pageable memory would make the host wait for the work already queued on the GPU,
+    which then idles while the host catches up with its launches."""
+    starts, at = [], 0
+    for a in arrays:
+        starts.append(at)
+        at += -(-a.nbytes // 16) * 16
+    host = torch.empty(max(at, 16), dtype=torch.uint8, pin_memory=True)
+    flat = host.numpy()
+    for a, s0 in zip(arrays, starts):
+        flat[s0:s0 + a.nbytes] = np.ascontiguousarray(a).reshape(-1).view(np.uint8)
+    buf = host.to(device, non_blocking=True)
+    return [buf[s0:s0 + a.nbytes].view(torch.from_numpy(np.empty(0, a.dtype)).dtype).view(a.shape)
+            for a, s0 in zip(arrays, starts)]
+
+
 @dataclass
 class StepEntry:
     """``tokens`` continue request ``seq_id`` at absolute position ``start``; ``want`` lists the
@@ -109,7 +127,6 @@ class StepContext:
                 for q0 in range(0, length, rows_per_tile):
                     ent.append(e)
                     q0s.append(q0)
-            both = torch.tensor([ent, q0s], dtype=torch.int32).to(self.device, non_blocking=False)
-            hit = (both[0].contiguous(), both[1].contiguous())
+            hit = tuple(upload([np.asarray(ent, np.int32), np.asarray(q0s, np.int32)], self.device))
             self._tiles[key] = hit
         return hit

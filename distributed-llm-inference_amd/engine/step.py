@@ -21,7 +21,7 @@ import torch
 from ..cache.manager import RELEASED, CacheManager, CopyOp
 from ..cache.store import CacheStore
 from ..parts.model import Model
-from .batch import GroupView, StepContext, StepEntry
+from .batch import GroupView, StepContext, StepEntry, upload
 
 
 MAX_DECODE_STEPS = 8  # tokens per request that one graph replay may decode
@@ -81,9 +81,10 @@ class StepFunction:
                     f"{mgr.num_computed_tokens(e.seq_id)} tokens are computed")
             if e.start + n > mgr.num_tokens(e.seq_id):
                 raise StepError(f"request {e.seq_id!r}: no cache slots reserved up to {e.start + n}")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise StepError(f"request {e.seq_id!r}: token id {t} outside the vocabulary")
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size:
+                bad = int(ids[(ids < 0) | (ids >= self.vocab_size)][0])
+                raise StepError(f"request {e.seq_id!r}: token id {bad} outside the vocabulary")
             for wnt in e.want:
                 if not 0 <= int(wnt) < n:
                     raise StepError(f"request {e.seq_id!r}: wanted place {wnt} outside its {n} tokens")
@@ -122,8 +123,14 @@ class StepFunction:
             [first_row[i] + int(w) for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
 
         dev = self.rt.device
-        to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-        groups: list[GroupView] = []
+        # every integer array of the step goes to the device in one copy from pinned memory
+        pending: list[np.ndarray] = []
+
+        def to_dev(a: np.ndarray) -> int:
+            pending.append(np.ascontiguousarray(a, dtype=np.int32))
+            return len(pending) - 1
+
+        group_arrays: list[tuple[int, int, int]] = []
         for g in range(n_groups):
             width = max((len(t) for t in tables[g]), default=1) or 1
             host = np.zeros((max(len(entries), 1), width), np.int32)
@@ -136,13 +143,16 @@ class StepFunction:
                 host[k, :len(t)] = row
             if total and (slots[g].min() < 0 or slots[g].max() >= limit * ps):
                 raise StepError("a cache slot lies outside the pool")
-            groups.append(GroupView(to_dev(slots[g]), to_dev(host), width))
+            group_arrays.append((to_dev(slots[g]), to_dev(host), width))
+        named = {name: to_dev(a) for name, a in (
+            ("token_ids", token_ids), ("positions", positions), ("q_start", q_start), ("kv_len", kv_len),
+            ("state_slots", state_slots), ("logit_rows", logit_rows))}
+        views = upload(pending, dev)
+        groups = [GroupView(views[s_], views[t_], width) for s_, t_, width in group_arrays]
         return StepContext(
             device=dev, page_size=ps, num_tokens=total, num_entries=len(entries), num_decode=num_decode,
-            token_ids=to_dev(token_ids), positions=to_dev(positions), q_start=to_dev(q_start),
-            kv_len=to_dev(kv_len), state_slots=to_dev(state_slots), logit_rows=to_dev(logit_rows),
             groups=groups, q_start_host=q_start, kv_len_host=kv_len, state_slots_host=state_slots,
-            seq_ids=[entries[i].seq_id for i in order])
+            seq_ids=[entries[i].seq_id for i in order], **{name: views[i] for name, i in named.items()})
 
     # ------------------------------------------------------------------ the step
 
@@ -244,9 +254,10 @@ class StepFunction:
         if rows == 0:
             return []
         dev = logits.device
-        floats = torch.tensor([[s[0] for s in sampling], [s[2] for s in sampling]], dtype=torch.float32).to(dev)
-        top_k = torch.tensor([s[1] for s in sampling], dtype=torch.int32).to(dev)
-        longs = torch.tensor([[s[3] for s in sampling], [s[4] for s in sampling]], dtype=torch.int64).to(dev)
+        temperature, top_p, top_k, seeds, counters = upload(
+            [np.asarray([s[0] for s in sampling], np.float32), np.asarray([s[2] for s in sampling], np.float32),
+             np.asarray([s[1] for s in sampling], np.int32), np.asarray([s[3] for s in sampling], np.int64),
+             np.asarray([s[4] for s in sampling], np.int64)], dev)
         out = torch.empty(rows, dtype=torch.int32, device=dev)
-        ops.sample(logits, floats[0], top_k, floats[1], longs[0], longs[1], out)
+        ops.sample(logits, temperature, top_k, top_p, seeds, counters, out)
         return out.cpu().tolist()

@@ -40,7 +40,7 @@ def test_embedding_and_gather_rows(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,eps", [(64, 1e-5), (192, 1e-6), (2050, 1e-5), (7, 1e-2)])
+@pytest.mark.parametrize("width,eps", [(64, 1e-5), (192, 1e-6), (2048, 1e-5), (2050, 1e-5), (4104, 1e-5), (7, 1e-2)])
 def test_rms_norm(ops, dtype, width, eps):
     torch.manual_seed(1)
     x = (torch.randn(9, width, device="cuda") * 3).to(dtype)
