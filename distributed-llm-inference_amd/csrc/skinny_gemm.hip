@@ -10,6 +10,12 @@
 // four runs of eight: the same permutation of k for both operands, so the sum is unchanged and a
 // lane reads 64 contiguous bytes of its weight row.
 //
+// TILED: the weights are stored tile by tile instead of row by row, as
+//   t[tile][block][q][g][c][8] = w[16*tile + c][128*block + 32*g + 8*q + (0..7)],
+// so that the 16 features x 128 k of one tile and block are 4 KB of consecutive memory in the
+// order in which the lanes take them (lane = 16*g + c) and every load of a wave is 1 KB of
+// consecutive bytes. Needs K % 128 == 0 and whole tiles (N % 16 == 0, gate and up parts included).
+//
 // Fused in (template switches):
 //   NORM     xhat = cast(norm_w[k] * cast(x[m][k] * rs[m])), rs[m] = rsqrt(sum_k x^2 / K + eps),
 //            the row sums of squares being handed over in parts by the kernel that wrote x
@@ -74,7 +80,7 @@ __device__ __forceinline__ bf16x8 finish_x(const XFrag<NORM>& f, float rs) {
 // KS waves split k, NS groups of waves split the workgroup's tiles, each wave owns NT tiles:
 // a workgroup computes NS*NT tiles of 16 features with KS*NS waves. The activation fragments are
 // loaded once per block of k and reused for the wave's NT tiles.
-template <int KS, int NS, int NT, int MT, int EPI, bool NORM>
+template <int KS, int NS, int NT, int MT, int EPI, bool NORM, bool TILED>
 __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
     const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
@@ -96,9 +102,19 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
-      const int n = min((tile0 + j) * 16 + col, N - 1) + a * up_offset;
-      wrow[j][a] = w + (int64_t)n * K;
+      if constexpr (TILED) {
+        // the tile's first block, at this lane's 16 bytes of a 1 KB load
+        const int tile = min(tile0 + j, (N - 1) / 16) + a * (up_offset / 16);
+        wrow[j][a] = w + (int64_t)tile * 16 * K + lane * 8;
+      } else {
+        const int n = min((tile0 + j) * 16 + col, N - 1) + a * up_offset;
+        wrow[j][a] = w + (int64_t)n * K + grp * 32;
+      }
     }
+  // where a lane finds its eight k values of product q in the block that starts at step s
+  auto w_at = [&](const bf16_t* base, int s, int q) __attribute__((always_inline)) {
+    return reinterpret_cast<const bf16x8*>(TILED ? base + (s / 4) * 2048 + q * 512 : base + s * 32 + q * 8);
+  };
 
   const bf16_t* xrow[MT];
   bool live[MT];
@@ -155,7 +171,8 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
 
   // this wave's share of the k steps of 32
   const int steps = K / 32;
-  const int s_begin = (int)((int64_t)steps * ks / KS), s_end = (int)((int64_t)steps * (ks + 1) / KS);
+  const int s_begin = TILED ? 4 * (int)((int64_t)(steps / 4) * ks / KS) : (int)((int64_t)steps * ks / KS);
+  const int s_end = TILED ? 4 * (int)((int64_t)(steps / 4) * (ks + 1) / KS) : (int)((int64_t)steps * (ks + 1) / KS);
   int s = s_begin;
   // blocks of 128: lane group g reads k in [32g, 32g + 32). The weights of the next block are
   // requested before the products of the current one, so two blocks are in flight per wave.
@@ -168,7 +185,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
       for (int a = 0; a < NA; ++a)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          af[j][a][q] = *reinterpret_cast<const bf16x8*>(wrow[j][a] + s * 32 + grp * 32 + q * 8);
+          af[j][a][q] = *w_at(wrow[j][a], s, q);
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -186,7 +203,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
         for (int a = 0; a < NA; ++a)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            nf[j][a][q] = *reinterpret_cast<const bf16x8*>(wrow[j][a] + kb + 128 + q * 8);
+            nf[j][a][q] = *w_at(wrow[j][a], s + 4, q);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -216,7 +233,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
         for (int q = 0; q < 4; ++q) xf[t][q] = nx[t][q];
     }
   }
-  for (; s < s_end; ++s) {  // single steps: lane group g reads k in [8g, 8g + 8)
+  for (; !TILED && s < s_end; ++s) {  // single steps: lane group g reads k in [8g, 8g + 8)
     const int kb = s * 32 + grp * 8;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -225,7 +242,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
       for (int j = 0; j < NT; ++j)
 #pragma unroll
         for (int a = 0; a < NA; ++a)
-          acc[j][a][t] = mfma32(*reinterpret_cast<const bf16x8*>(wrow[j][a] + kb), bf, acc[j][a][t]);
+          acc[j][a][t] = mfma32(*reinterpret_cast<const bf16x8*>(wrow[j][a] - grp * 32 + kb), bf, acc[j][a][t]);
     }
   }
 
@@ -331,11 +348,11 @@ __global__ void embedding_ssq_kernel(const bf16_t* __restrict__ table, const int
 #define SK_ARGS \
   x, ldx, ssq_in, ssq_parts, norm_w, eps, w, bias, out, ldo, stream_buf, lds_, ssq_out, M, N, K, up_offset, stream
 
-template <int KS, int NS, int NT, int MT, int EPI, bool NORM>
+template <int KS, int NS, int NT, int MT, int EPI, bool NORM, bool TILED>
 static void launch_skinny(SK_PARAMS) {
   const int tiles = (N + 15) / 16;
   const int groups = (tiles + NS * NT - 1) / (NS * NT);
-  skinny_gemm_kernel<KS, NS, NT, MT, EPI, NORM><<<groups, KS * NS * 64, 0, stream>>>(
+  skinny_gemm_kernel<KS, NS, NT, MT, EPI, NORM, TILED><<<groups, KS * NS * 64, 0, stream>>>(
       (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
       out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
 }
@@ -343,21 +360,23 @@ static void launch_skinny(SK_PARAMS) {
 // shapes of the workgroup: 0: 4 k-waves x 1 tile (few tiles, short k); 1: 8 k-waves x 1 tile (few
 // tiles, long k); 2: 4 n-waves x 2 tiles, no k split (many tiles: the activations are read once
 // per 8 tiles); 3: 2 k-waves x 2 n-waves x 2 tiles
-template <int MT, int EPI, bool NORM>
+template <int MT, int EPI, bool NORM, bool TILED>
 static void dispatch_shape(int shape, SK_PARAMS) {
   switch (shape) {
-    case 0: launch_skinny<4, 1, 1, MT, EPI, NORM>(SK_ARGS); break;
-    case 1: launch_skinny<8, 1, 1, MT, EPI, NORM>(SK_ARGS); break;
-    case 2: launch_skinny<1, 4, 2, MT, EPI, NORM>(SK_ARGS); break;
-    default: launch_skinny<2, 2, 2, MT, EPI, NORM>(SK_ARGS); break;
+    case 0: launch_skinny<4, 1, 1, MT, EPI, NORM, TILED>(SK_ARGS); break;
+    case 1: launch_skinny<8, 1, 1, MT, EPI, NORM, TILED>(SK_ARGS); break;
+    case 2: launch_skinny<1, 4, 2, MT, EPI, NORM, TILED>(SK_ARGS); break;
+    default: launch_skinny<2, 2, 2, MT, EPI, NORM, TILED>(SK_ARGS); break;
   }
 }
 
+// tiled weights serve the decode steps of few rows: one row tile only
 template <int EPI, bool NORM>
-static int dispatch_skinny(int shape, int mt, SK_PARAMS) {
-  if (mt == 1) dispatch_shape<1, EPI, NORM>(shape, SK_ARGS);
-  else if (mt == 2) dispatch_shape<2, EPI, NORM>(shape, SK_ARGS);
-  else dispatch_shape<4, EPI, NORM>(shape, SK_ARGS);
+static int dispatch_skinny(int shape, int mt, bool tiled, SK_PARAMS) {
+  if (tiled) dispatch_shape<1, EPI, NORM, true>(shape, SK_ARGS);
+  else if (mt == 1) dispatch_shape<1, EPI, NORM, false>(shape, SK_ARGS);
+  else if (mt == 2) dispatch_shape<2, EPI, NORM, false>(shape, SK_ARGS);
+  else dispatch_shape<4, EPI, NORM, false>(shape, SK_ARGS);
   return dli_launch_status();
 }
 
@@ -365,12 +384,14 @@ extern "C" int dli_skinny_gemm_max_rows() { return 64; }
 
 // epilogue: 0 store bf16, 1 swiglu (N = features of one half, up rows at +up_offset), 2 residual,
 // 3 store float32. norm_w == nullptr: no norm. shape: the workgroup shape, see dispatch_shape.
+// tiled: w is in the tile order described at the top (at most 16 rows, K % 128 == 0, whole tiles).
 extern "C" int dli_skinny_gemm(const void* x, int64_t ldx, const float* ssq_in, int ssq_parts,
                                const float* norm_w, float eps, const void* w, const void* bias,
                                void* out, int64_t ldo, void* stream_buf, int64_t lds_,
                                float* ssq_out, int M, int N, int K, int up_offset, int epilogue,
-                               int shape, hipStream_t stream) {
+                               int shape, int tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return DLI_OK;
+  if (tiled && (M > 16 || K % 128 != 0 || N % 16 != 0 || up_offset % 16 != 0)) return DLI_ERR_ARGUMENT;
   if (M > 64 || K <= 0 || K % 32 != 0 || ldx % 8 != 0 || shape < 0 || shape > 3 || epilogue < 0 ||
       epilogue > 3 || (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)) ||
       (epilogue == EPI_RESIDUAL && (stream_buf == nullptr || ssq_out == nullptr || norm_w != nullptr)) ||
@@ -380,13 +401,13 @@ extern "C" int dli_skinny_gemm(const void* x, int64_t ldx, const float* ssq_in, 
   const bool norm = norm_w != nullptr;
   switch (epilogue) {
     case EPI_STORE:
-      return norm ? dispatch_skinny<EPI_STORE, true>(shape, mt, SK_ARGS) : dispatch_skinny<EPI_STORE, false>(shape, mt, SK_ARGS);
+      return norm ? dispatch_skinny<EPI_STORE, true>(shape, mt, tiled != 0, SK_ARGS) : dispatch_skinny<EPI_STORE, false>(shape, mt, tiled != 0, SK_ARGS);
     case EPI_SWIGLU:
-      return norm ? dispatch_skinny<EPI_SWIGLU, true>(shape, mt, SK_ARGS) : dispatch_skinny<EPI_SWIGLU, false>(shape, mt, SK_ARGS);
+      return norm ? dispatch_skinny<EPI_SWIGLU, true>(shape, mt, tiled != 0, SK_ARGS) : dispatch_skinny<EPI_SWIGLU, false>(shape, mt, tiled != 0, SK_ARGS);
     case EPI_RESIDUAL:
-      return dispatch_skinny<EPI_RESIDUAL, false>(shape, mt, SK_ARGS);
+      return dispatch_skinny<EPI_RESIDUAL, false>(shape, mt, tiled != 0, SK_ARGS);
     default:
-      return norm ? dispatch_skinny<EPI_F32, true>(shape, mt, SK_ARGS) : dispatch_skinny<EPI_F32, false>(shape, mt, SK_ARGS);
+      return norm ? dispatch_skinny<EPI_F32, true>(shape, mt, tiled != 0, SK_ARGS) : dispatch_skinny<EPI_F32, false>(shape, mt, tiled != 0, SK_ARGS);
   }
 }
 

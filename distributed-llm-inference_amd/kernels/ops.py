@@ -49,7 +49,7 @@ _SIGNATURES = {
                            _c_int, _c_int, _c_ptr],
     "dli_skinny_gemm_max_rows": [],
     "dli_skinny_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
-                        _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                        _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
@@ -296,14 +296,38 @@ def skinny_gemm_supports(rows: int, k: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and 0 < rows <= 64 and k > 0 and k % 32 == 0
 
 
-def skinny_gemm_shape(n: int, k: int) -> int:
+def skinny_gemm_shape(n: int, k: int, tiled: bool = False) -> int:
     """Workgroup shape for ``n`` output features of depth ``k``: with few tiles of 16 features the
-    waves of a workgroup split k (8 ways when k is long), with many they split the tiles so that
-    the activations are read once per 8 tiles."""
+    waves of a workgroup split k (8 ways when k is long, or when there are fewer tiles than
+    compute units and the weights are tiled), with many they split the tiles so that the
+    activations are read once per 8 tiles. From cold-cache timings on MI355X."""
     tiles = -(-n // 16)
-    if tiles >= 768:   # a vocabulary: 2 k-waves x 2 n-waves x 2 tiles was ahead of 4 n-waves x 2 tiles
-        return 3
+    if tiles >= 768:   # a vocabulary
+        return 2 if tiled else 3
+    if tiled and tiles <= 256:
+        return 1
     return 1 if k >= 4096 else 0
+
+
+def tiled_weights_help(w_rows: int, k: int, epilogue: int, device: torch.device) -> bool:
+    """Whether a second copy of a ``[w_rows, k]`` weight in tile order (:func:`tile_weights`)
+    would be used: the sizes allow it and steps of 5 to 16 rows run this product on the
+    16x16-tile kernel."""
+    n = w_rows // 2 if epilogue == SKINNY_SWIGLU else w_rows
+    if k % 128 != 0 or n % 16 != 0 or n == 0:
+        return False
+    return skinny_gemm_plan(8, n, k, epilogue, device)[0] == "tiles16"
+
+
+def tile_weights(w: torch.Tensor) -> torch.Tensor:
+    """``w [n, k]`` (bfloat16, n % 16 == 0, k % 128 == 0) in the order in which the 16x16-tile
+    kernel's lanes read it: ``t[tile][block][q][g][c][8] = w[16*tile + c][128*block + 32*g + 8*q + ...]``,
+    so that each load of a wave is 1 KB of consecutive memory. Same number of elements, flat."""
+    _dense(w, "w", torch.bfloat16, 2)
+    n, k = w.shape
+    _require(n % 16 == 0 and k % 128 == 0, "tile order needs n % 16 == 0 and k % 128 == 0")
+    t = w.view(n // 16, 16, k // 128, 4, 4, 8)       # tile, c, block, g, q, 8
+    return t.permute(0, 2, 4, 3, 1, 5).contiguous().view(-1)
 
 
 _compute_units: dict[int, int] = {}
@@ -344,7 +368,7 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
                 bias: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
                 ssq_in: Optional[torch.Tensor] = None, stream: Optional[torch.Tensor] = None,
                 ssq_out: Optional[torch.Tensor] = None, shape: Optional[int] = None,
-                blocks4: Optional[int] = None) -> Optional[torch.Tensor]:
+                blocks4: Optional[int] = None, w_tiled: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """``y = xhat @ w.T`` for at most 64 rows of bfloat16 ``x``, with fused surroundings.
 
     ``norm_w``/``eps``/``ssq_in [parts, rows]``: xhat is the RMSNorm of x, the row sums of squares
@@ -354,7 +378,8 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
     the parts of its row sums of squares are returned as ``[parts, rows]``, in ``ssq_out`` if that
     is given with the shape :func:`skinny_gemm_plan` names), ``SKINNY_F32`` (``out`` float32).
     ``shape`` forces the 16x16-tile kernel with that workgroup shape, ``blocks4`` the 4x4-block
-    kernel with that one (at most 16 rows).
+    kernel with that one (at most 16 rows). ``w_tiled``: the same weights in tile order
+    (:func:`tile_weights`), read instead of ``w`` when the 16x16-tile kernel runs at most 16 rows.
     """
     _rows(x, "x", torch.bfloat16)
     _dense(w, "w", torch.bfloat16, 2)
@@ -376,6 +401,13 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
         if blocks4 is not None:
             _require(blocks4 in (0, 1, 2) and m <= 16 and k % 8 == 0, "blocks4 must be 0..2, with at most 16 rows")
         kernel, a, n_parts = skinny_gemm_plan(m, n, k, epilogue, x.device, blocks4)
+    tiled = w_tiled is not None and kernel == "tiles16" and m <= 16
+    if tiled:
+        _dense(w_tiled, "w_tiled", torch.bfloat16, 1)
+        _require(w_tiled.numel() == w.numel() and k % 128 == 0 and n % 16 == 0 and w_tiled.data_ptr() % 16 == 0,
+                 "w_tiled must hold the same weights in tile order (n % 16 == 0, k % 128 == 0)")
+        if shape is None:
+            a = skinny_gemm_shape(n, k, tiled=True)
     parts = 0
     if norm_w is not None:
         _require(epilogue != SKINNY_RESIDUAL, "the residual epilogue takes no fused norm")
@@ -404,8 +436,9 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
         ldo = out.stride(0)
     if kernel == "tiles16":
         _check(library().dli_skinny_gemm(
-            _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
-            _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, a, _stream()), "skinny_gemm")
+            _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w_tiled if tiled else w),
+            _ptr(bias), _ptr(out), ldo, _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, a,
+            int(tiled), _stream()), "skinny_gemm")
     else:
         _check(library().dli_skinny4_gemm(
             _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,

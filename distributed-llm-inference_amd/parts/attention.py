@@ -22,7 +22,7 @@ import torch
 from ..kernels import ops
 from .attention_kernels import decode_attention_with_rope, paged_attention
 from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
-from .linear import linear
+from .linear import decode_copy, linear
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
 
@@ -50,6 +50,7 @@ class GQAttention(Mixer):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.position = build_part("position", position or PartSpec("none"), runtime)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self.w_qkv_tiled = self.w_o_tiled = None
 
     # -- weights
     def weight_specs(self) -> dict[str, WeightSpec]:
@@ -70,6 +71,10 @@ class GQAttention(Mixer):
                       if self.qkv_bias else None)
         self.w_o = tensors["o_proj.weight"]
         self.b_o = tensors.get("o_proj.bias") if self.o_bias else None
+
+    def finalize(self) -> None:
+        self.w_qkv_tiled = decode_copy(self.rt, self.w_qkv, ops.SKINNY_STORE)
+        self.w_o_tiled = decode_copy(self.rt, self.w_o, ops.SKINNY_RESIDUAL)
 
     def sub_parts(self) -> dict[str, Part]:
         return {"position": self.position}
@@ -121,8 +126,8 @@ class GQAttention(Mixer):
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
-        ops.skinny_gemm(stream.x, self.w_qkv, epilogue=ops.SKINNY_STORE, out=qkv, bias=self.b_qkv,
-                        norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        ops.skinny_gemm(stream.x, self.w_qkv, w_tiled=self.w_qkv_tiled, epilogue=ops.SKINNY_STORE, out=qkv,
+                        bias=self.b_qkv, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         table = self.position.rotary_table()
         if table is None:
             q_view = qkv[:, :nh * d].view(n, nh, d)
@@ -140,4 +145,5 @@ class GQAttention(Mixer):
             ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
                               cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
             paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
-        stream.ssq = ops.skinny_gemm(out, self.w_o, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x, bias=self.b_o)
+        stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
+                                     stream=stream.x, bias=self.b_o)

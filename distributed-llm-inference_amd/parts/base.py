@@ -25,6 +25,9 @@ class Runtime:
 
     device: torch.device
     dtype: torch.dtype  # torch.float32 (true 32-bit path) or torch.bfloat16 (serving)
+    # bfloat16 only: keep a second copy of each matrix in the order in which the decode kernels
+    # read it (faster decode steps of 5 to 16 rows, twice the weight memory)
+    decode_weight_copy: bool = True
 
     @property
     def is_bf16(self) -> bool:

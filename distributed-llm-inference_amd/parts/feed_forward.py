@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import DecodeStream, FeedForward, Norm, Runtime
-from .linear import linear
+from .linear import decode_copy, linear
 from .registry import register_part
 from .spec import WeightSpec
 
@@ -24,6 +24,7 @@ class GatedMLP(FeedForward):
             raise ValueError(f"gated_mlp has no kernel for activation {activation!r} (only 'silu')")
         self.hidden_size, self.intermediate_size, self.bias = hidden_size, intermediate_size, bias
         self.w_gate_up = self.b_gate_up = self.w_down = self.b_down = None
+        self.w_gate_up_tiled = self.w_down_tiled = None
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         h, i = self.hidden_size, self.intermediate_size
@@ -40,6 +41,10 @@ class GatedMLP(FeedForward):
         if self.bias:
             self.b_gate_up = torch.cat([tensors["gate_proj.bias"], tensors["up_proj.bias"]], 0).contiguous()
             self.b_down = tensors["down_proj.bias"]
+
+    def finalize(self) -> None:
+        self.w_gate_up_tiled = decode_copy(self.rt, self.w_gate_up, ops.SKINNY_SWIGLU)
+        self.w_down_tiled = decode_copy(self.rt, self.w_down, ops.SKINNY_RESIDUAL)
 
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         gate_up = linear(self.rt, x, self.w_gate_up, self.b_gate_up)
@@ -58,7 +63,7 @@ class GatedMLP(FeedForward):
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
         act = self.rt.empty(n, self.intermediate_size)
-        ops.skinny_gemm(stream.x, self.w_gate_up, epilogue=ops.SKINNY_SWIGLU, out=act, bias=self.b_gate_up,
-                        norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
-        stream.ssq = ops.skinny_gemm(act, self.w_down, epilogue=ops.SKINNY_RESIDUAL, stream=stream.x,
-                                     bias=self.b_down)
+        ops.skinny_gemm(stream.x, self.w_gate_up, w_tiled=self.w_gate_up_tiled, epilogue=ops.SKINNY_SWIGLU, out=act,
+                        bias=self.b_gate_up, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        stream.ssq = ops.skinny_gemm(act, self.w_down, w_tiled=self.w_down_tiled, epilogue=ops.SKINNY_RESIDUAL,
+                                     stream=stream.x, bias=self.b_down)

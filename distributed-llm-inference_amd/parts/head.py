@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from .base import DecodeStream, Head, Norm, Runtime
-from .linear import linear
+from .linear import decode_copy, linear
 from .registry import register_part
 from .spec import WeightSpec
 
@@ -20,6 +20,7 @@ class LinearHead(Head):
         super().__init__(runtime)
         self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
         self.weight: Optional[torch.Tensor] = None
+        self.weight_tiled: Optional[torch.Tensor] = None
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {} if self.tied else {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
@@ -32,6 +33,9 @@ class LinearHead(Head):
         if self.tied:
             self.weight = table
 
+    def finalize(self) -> None:
+        self.weight_tiled = decode_copy(self.rt, self.weight, ops.SKINNY_F32)
+
     FEW_ROWS = 16  # up to here the decode product streams the table faster than the library does
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -40,7 +44,7 @@ class LinearHead(Head):
                 and ops.skinny_gemm_supports(rows, self.hidden_size, self.rt.dtype)):
             # the usual case of a prompt's step: logits for its last row only
             out = torch.empty(rows, self.vocab_size, device=self.rt.device, dtype=torch.float32)
-            ops.skinny_gemm(x, self.weight, epilogue=ops.SKINNY_F32, out=out)
+            ops.skinny_gemm(x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out)
             return out
         logits = linear(self.rt, x, self.weight)
         if logits.dtype == torch.float32:
@@ -56,6 +60,6 @@ class LinearHead(Head):
         """Logits of every row of the stream, the final norm computed inside the product."""
         norm_w, eps = norm.fused_params()
         out = torch.empty(stream.x.shape[0], self.vocab_size, device=self.rt.device, dtype=torch.float32)
-        ops.skinny_gemm(stream.x, self.weight, epilogue=ops.SKINNY_F32, out=out, norm_w=norm_w, eps=eps,
-                        ssq_in=stream.ssq)
+        ops.skinny_gemm(stream.x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out,
+                        norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         return out

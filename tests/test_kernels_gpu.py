@@ -371,6 +371,63 @@ def test_skinny_gemm_norm_and_swiglu(ops, m, inter, k, shape, parts):
     assert (y.cpu().double() - gu).abs().max() < 3e-2 * max(1.0, gu.abs().max().item())
 
 
+@pytest.mark.parametrize("m", [1, 5, 8, 16])
+@pytest.mark.parametrize("shape", [None, 0, 1, 2, 3])
+@pytest.mark.parametrize("n,k", [(96, 128), (112, 384), (2048, 2048), (1008, 640)])
+def test_skinny_gemm_with_weights_in_tile_order(ops, m, n, k, shape):
+    """The second copy of the weights, tile by tile, gives what the row-major weights give (the
+    same products; only the split of k over the waves may differ), for every epilogue."""
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m, k, device="cuda").bfloat16()
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    wt = ops.tile_weights(w)
+    assert wt.numel() == w.numel() and not torch.equal(wt.view(n, k), w)
+    # element (feature 16*tile + c, k 128*block + 32*g + 8*q + i) sits at [tile][block][q][g][c][i]
+    assert wt.view(n // 16, k // 128, 4, 4, 16, 8)[1, 0, 2, 3, 5, 6] == w[16 + 5, 32 * 3 + 8 * 2 + 6]
+    bias = torch.randn(n, device="cuda").bfloat16()
+    ref = x.cpu().double() @ w.cpu().double().T
+    kw = {} if shape is None else {"shape": shape}
+    plain32, tiled32 = torch.empty(m, n, device="cuda"), torch.empty(m, n, device="cuda")
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_F32, out=plain32, **kw)
+    ops.skinny_gemm(x, w, w_tiled=wt, epilogue=ops.SKINNY_F32, out=tiled32, **kw)
+    assert (tiled32.cpu().double() - ref).abs().max() < 1e-4 * math.sqrt(k)
+    assert (tiled32 - plain32).abs().max() < 1e-5 * math.sqrt(k)
+    # residual with bias and the parts of the sums of squares
+    stream = torch.randn(m, n, device="cuda").bfloat16()
+    before = stream.clone()
+    ssq = ops.skinny_gemm(x, w, w_tiled=wt, epilogue=ops.SKINNY_RESIDUAL, stream=stream, bias=bias, **kw)
+    y = (tiled32 + bias.float()).bfloat16()
+    assert torch.equal(stream, (before.float() + y.float()).bfloat16())
+    assert torch.allclose(ssq.sum(0), stream.float().pow(2).sum(-1), rtol=1e-5)
+    # norm prologue and SwiGLU epilogue: gate rows then up rows, both halves whole tiles
+    if n % 32 == 0:
+        nw = (1 + 0.1 * torch.randn(k, device="cuda")).float()
+        ssq_in = x.float().pow(2).sum(-1)[None].contiguous()
+        a = torch.empty(m, n // 2, device="cuda", dtype=torch.bfloat16)
+        b = torch.empty(m, n // 2, device="cuda", dtype=torch.bfloat16)
+        ops.skinny_gemm(x, w, epilogue=ops.SKINNY_SWIGLU, out=a, norm_w=nw, eps=1e-5, ssq_in=ssq_in, **kw)
+        ops.skinny_gemm(x, w, w_tiled=wt, epilogue=ops.SKINNY_SWIGLU, out=b, norm_w=nw, eps=1e-5, ssq_in=ssq_in, **kw)
+        assert (a.float() - b.float()).abs().max() <= 2e-2 * max(1.0, a.float().abs().max().item())
+        xhat = _ref_norm_bf16(x, nw, 1e-5)
+        gu = xhat.cpu().double() @ w.cpu().double().T
+        g, u = gu[:, :n // 2].bfloat16().double(), gu[:, n // 2:].bfloat16().double()
+        want = (g * torch.sigmoid(g)).bfloat16().double() * u
+        assert (b.cpu().double() - want).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
+
+
+def test_tiled_weights_are_refused_where_they_do_not_fit(ops):
+    w = torch.zeros(40, 128, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelArgumentError):
+        ops.tile_weights(w)                       # 40 features: no whole tiles
+    with pytest.raises(ops.KernelArgumentError):
+        ops.tile_weights(torch.zeros(48, 96, device="cuda", dtype=torch.bfloat16))  # k % 128 != 0
+    assert not ops.tiled_weights_help(40, 128, ops.SKINNY_STORE, w.device)
+    assert not ops.tiled_weights_help(48, 96, ops.SKINNY_STORE, w.device)
+    assert not ops.tiled_weights_help(48, 128, ops.SKINNY_SWIGLU, w.device)   # halves of 24 features
+    assert ops.tiled_weights_help(2048, 2048, ops.SKINNY_RESIDUAL, w.device)
+    assert not ops.tiled_weights_help(2048, 8192, ops.SKINNY_RESIDUAL, w.device)  # the block kernel's at every size
+
+
 @pytest.mark.parametrize("m", [1, 3, 4, 5, 8, 9, 16])
 @pytest.mark.parametrize("n,k", [(48, 64), (100, 192), (301, 160), (512, 2048), (64, 416), (1000, 96), (2048, 8192)])
 @pytest.mark.parametrize("blocks4", [0, 1, 2])
