@@ -359,13 +359,14 @@ static void launch_skinny(SK_PARAMS) {
 
 // shapes of the workgroup: 0: 4 k-waves x 1 tile (few tiles, short k); 1: 8 k-waves x 1 tile (few
 // tiles, long k); 2: 4 n-waves x 2 tiles, no k split (many tiles: the activations are read once
-// per 8 tiles); 3: 2 k-waves x 2 n-waves x 2 tiles
+// per 8 tiles); 3: 2 k-waves x 2 n-waves x 2 tiles; 4: 4 k-waves x 2 tiles (many tiles in tile order)
 template <int MT, int EPI, bool NORM, bool TILED>
 static void dispatch_shape(int shape, SK_PARAMS) {
   switch (shape) {
     case 0: launch_skinny<4, 1, 1, MT, EPI, NORM, TILED>(SK_ARGS); break;
     case 1: launch_skinny<8, 1, 1, MT, EPI, NORM, TILED>(SK_ARGS); break;
     case 2: launch_skinny<1, 4, 2, MT, EPI, NORM, TILED>(SK_ARGS); break;
+    case 4: launch_skinny<4, 1, 2, MT, EPI, NORM, TILED>(SK_ARGS); break;
     default: launch_skinny<2, 2, 2, MT, EPI, NORM, TILED>(SK_ARGS); break;
   }
 }
@@ -392,7 +393,7 @@ extern "C" int dli_skinny_gemm(const void* x, int64_t ldx, const float* ssq_in, 
                                int shape, int tiled, hipStream_t stream) {
   if (M <= 0 || N <= 0) return DLI_OK;
   if (tiled && (M > 16 || K % 128 != 0 || N % 16 != 0 || up_offset % 16 != 0)) return DLI_ERR_ARGUMENT;
-  if (M > 64 || K <= 0 || K % 32 != 0 || ldx % 8 != 0 || shape < 0 || shape > 3 || epilogue < 0 ||
+  if (M > 64 || K <= 0 || K % 32 != 0 || ldx % 8 != 0 || shape < 0 || shape > 4 || epilogue < 0 ||
       epilogue > 3 || (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)) ||
       (epilogue == EPI_RESIDUAL && (stream_buf == nullptr || ssq_out == nullptr || norm_w != nullptr)) ||
       (epilogue != EPI_RESIDUAL && out == nullptr))

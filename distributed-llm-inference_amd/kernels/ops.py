@@ -302,10 +302,10 @@ def skinny_gemm_shape(n: int, k: int, tiled: bool = False) -> int:
     compute units and the weights are tiled), with many they split the tiles so that the
     activations are read once per 8 tiles. From cold-cache timings on MI355X."""
     tiles = -(-n // 16)
+    if tiled:          # fewer tiles than compute units: 8 k-waves; else 4 k-waves on two tiles each
+        return 1 if tiles <= 256 else 4
     if tiles >= 768:   # a vocabulary
-        return 2 if tiled else 3
-    if tiled and tiles <= 256:
-        return 1
+        return 3
     return 1 if k >= 4096 else 0
 
 
@@ -395,7 +395,7 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
         _dense(bias, "bias", torch.bfloat16, 1)
         _require(bias.shape[0] == w.shape[0], "bias length differs from rows of w")
     if shape is not None:
-        _require(shape in (0, 1, 2, 3), "shape must be 0..3")
+        _require(shape in (0, 1, 2, 3, 4), "shape must be 0..4")
         kernel, a, n_parts = "tiles16", shape, -(-n // 16)
     else:
         if blocks4 is not None:

@@ -320,7 +320,7 @@ def _ref_norm_bf16(x, w, eps):
 
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 40, 64])
 @pytest.mark.parametrize("n,k,shape", [(48, 64, 0), (100, 192, 2), (301, 160, 1), (512, 2048, 1), (64, 416, 3),
-                                       (1000, 96, 2), (2048, 8192, 1)])
+                                       (1000, 96, 2), (2048, 8192, 1), (1000, 416, 4)])
 def test_skinny_gemm_epilogues(ops, m, n, k, shape):
     torch.manual_seed(m * 1000 + n)
     x = torch.randn(m, k, device="cuda").bfloat16()
@@ -372,7 +372,7 @@ def test_skinny_gemm_norm_and_swiglu(ops, m, inter, k, shape, parts):
 
 
 @pytest.mark.parametrize("m", [1, 5, 8, 16])
-@pytest.mark.parametrize("shape", [None, 0, 1, 2, 3])
+@pytest.mark.parametrize("shape", [None, 0, 1, 2, 3, 4])
 @pytest.mark.parametrize("n,k", [(96, 128), (112, 384), (2048, 2048), (1008, 640)])
 def test_skinny_gemm_with_weights_in_tile_order(ops, m, n, k, shape):
     """The second copy of the weights, tile by tile, gives what the row-major weights give (the
