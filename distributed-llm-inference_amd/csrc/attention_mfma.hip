@@ -149,42 +149,13 @@ __device__ __forceinline__ void load_v(short4v (&vreg)[DCH], const bf16_t* __res
 
 // ------------------------------------------------------------------------------------ decode
 // grid (splits, kv_heads * head_tiles, requests); 256 threads. Request e's single query is row e.
-// Rotation of four neighbouring dimensions d0.. of a head by the angles whose cos and sin (rounded
-// to bfloat16 as the separate rotation kernel rounds them) lie at cs/sn: dimension i pairs with
-// i + half; `other` holds the partners' values.
-__device__ __forceinline__ short4v rotate4(short4v own, short4v other, int d0, int half,
-                                           const float* __restrict__ cs, const float* __restrict__ sn) {
-  union {
-    short4v v;
-    bf16_t e[4];
-  } a, b, y;
-  a.v = own;
-  b.v = other;
-  const bool first = d0 < half;
-  const int i0 = first ? d0 : d0 - half;
-  const float4v c4 = *reinterpret_cast<const float4v*>(cs + i0), s4 = *reinterpret_cast<const float4v*>(sn + i0);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float x = (float)a.e[j], p = (float)b.e[j];
-    y.e[j] = first ? (bf16_t)(x * c4[j] - p * s4[j]) : (bf16_t)(x * c4[j] + p * s4[j]);
-  }
-  return y.v;
-}
-
-// With ROPE the kernel also does what otherwise a kernel before it does for a decoded token:
-// `q` then points at the rows of the fused q,k,v projection as it left the product (q heads, k
-// heads, v heads); the query is rotated as it is loaded; the token's own key and value are
-// rotated and put into the tile that holds its position from registers (the cache is not read
-// for them), and the workgroup of a kv head's first head tile also writes them into the pages
-// for the steps to come. cos and sin of the tokens' angles come from a table made once a step
-// (`angles[e][0][i]`, `angles[e][1][i]`, i < head_dim/2). Needs rotary_dim == head_dim.
-template <int DCH, bool ROPE>
+template <int DCH>
 __global__ __launch_bounds__(256) void attention_decode_kernel(
-    const bf16_t* __restrict__ q, int64_t q_stride, bf16_t* __restrict__ k_pages,
-    bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ kv_len,
     const int* __restrict__ block_tables, int table_stride, int q_heads, int kv_heads, int page_size,
-    float scale_log2e, int window, int splits, const float* __restrict__ angles) {
+    float scale_log2e, int window, int splits) {
   constexpr int D = DCH * 16;
   __shared__ float sm_o[3][D][16];
   __shared__ float sm_m[3][16], sm_l[3][16];
@@ -215,23 +186,6 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
 #pragma unroll
     for (int c = 0; c < DCH; ++c) qreg[c] = *reinterpret_cast<const short4v*>(qp + c * 4);
   }
-  const int pos = n_keys - 1;  // ROPE: the position of the token that is being decoded
-  const float* cs = ROPE ? angles + (int64_t)e * D : nullptr;  // D/2 cos, then D/2 sin
-  const float* sn = ROPE ? cs + D / 2 : nullptr;
-  if (ROPE) {
-    // lane group g holds the dimensions [g*D/4, (g+1)*D/4): the partners of groups 0,1 are in 2,3
-#pragma unroll
-    for (int c = 0; c < DCH; ++c) {
-      union {
-        short4v v;
-        unsigned u[2];
-      } own, other;
-      own.v = qreg[c];
-      other.u[0] = __shfl_xor(own.u[0], 32, DLI_WAVE);
-      other.u[1] = __shfl_xor(own.u[1], 32, DLI_WAVE);
-      qreg[c] = rotate4(own.v, other.v, grp * (D / 4) + 4 * c, D / 2, cs, sn);
-    }
-  }
 
   ColumnTile<DCH> st;
   st.init();
@@ -257,40 +211,6 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     for (int u = 0; u < UN; ++u) {
       load_k<DCH>(kreg[u], k_pages, page[u], kv_heads, kvh, page_size, off[u], col, grp);
       load_v<DCH>(vreg[u], v_pages, page[u], kv_heads, kvh, page_size, off[u], col, grp, t0 + 64 * u, k1);
-    }
-    if (ROPE) {
-#pragma unroll
-      for (int u = 0; u < UN; ++u) {
-        const int t = t0 + 64 * u;
-        if (t <= pos && pos < t + 16 && pos < k1) {  // this wave's tile holds the new token's slot
-          const int r = pos - t;
-          const bool writes = ht == 0;
-          const bf16_t* kraw = q + (int64_t)e * q_stride + (int64_t)(q_heads + kvh) * D;
-          const bf16_t* vraw = kraw + (int64_t)kv_heads * D;
-          if (col == r) {
-            bf16_t* kd = k_pages + ((page[u] * kv_heads + kvh) * page_size + off[u] + r) * D;
-#pragma unroll
-            for (int c = 0; c < DCH; ++c) {
-              const int d0 = grp * (D / 4) + 4 * c;
-              const short4v own = *reinterpret_cast<const short4v*>(kraw + d0);
-              const short4v other = *reinterpret_cast<const short4v*>(kraw + (d0 < D / 2 ? d0 + D / 2 : d0 - D / 2));
-              kreg[u][c] = rotate4(own, other, d0, D / 2, cs, sn);
-              if (writes) *reinterpret_cast<short4v*>(kd + d0) = kreg[u][c];
-            }
-          }
-          if (grp == r / 4) {
-#pragma unroll
-            for (int c = 0; c < DCH; ++c) {
-              const bf16_t val = vraw[c * 16 + col];
-              const short bits = *reinterpret_cast<const short*>(&val);
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-                if (j == r % 4) vreg[u][c][j] = bits;
-              if (writes) v_pages[((page[u] * kv_heads + kvh) * D + c * 16 + col) * page_size + off[u] + r] = val;
-            }
-          }
-        }
-      }
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
@@ -803,11 +723,12 @@ extern "C" int dli_attention_prefill_tile_rows(int head_dim, int q_heads, int kv
   return hw == 0 ? PF_TILE_ROWS : (4 / hw) * 32;
 }
 
-static int launch_decode(const void* q, int64_t q_stride, void* k_pages, void* v_pages, void* out,
-                         int64_t out_stride, float* part_o, float* part_ml, const int* kv_len,
-                         const int* block_tables, int table_stride, int requests, int q_heads,
-                         int kv_heads, int head_dim, int page_size, float scale, int window, int splits,
-                         const float* angles, hipStream_t stream) {
+extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pages,
+                                         const void* v_pages, void* out, int64_t out_stride,
+                                         float* part_o, float* part_ml, const int* kv_len,
+                                         const int* block_tables, int table_stride, int requests,
+                                         int q_heads, int kv_heads, int head_dim, int page_size,
+                                         float scale, int window, int splits, hipStream_t stream) {
   if (requests <= 0) return DLI_OK;
   if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || splits < 1 || splits > 65535 || requests > 65535 ||
@@ -816,14 +737,12 @@ static int launch_decode(const void* q, int64_t q_stride, void* k_pages, void* v
     return DLI_ERR_ARGUMENT;
   const int head_tiles = (q_heads / kv_heads + 15) / 16;
   const dim3 grid(splits, kv_heads * head_tiles, requests);
-#define DECODE_ARGS                                                                                 \
-  (const bf16_t*)q, q_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out, out_stride, part_o, \
-      part_ml, kv_len, block_tables, table_stride, q_heads, kv_heads, page_size, scale * LOG2E,     \
-      window, splits, angles
-#define DECODE_CASE(N)                                                                         \
-  case N:                                                                                      \
-    if (angles != nullptr) attention_decode_kernel<N, true><<<grid, 256, 0, stream>>>(DECODE_ARGS); \
-    else attention_decode_kernel<N, false><<<grid, 256, 0, stream>>>(DECODE_ARGS);            \
+#define DECODE_CASE(N)                                                                            \
+  case N:                                                                                         \
+    attention_decode_kernel<N><<<grid, 256, 0, stream>>>(                                         \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
+        out_stride, part_o, part_ml, kv_len, block_tables, table_stride, q_heads, kv_heads,       \
+        page_size, scale * LOG2E, window, splits);                                                \
     break;
   switch (head_dim / 16) {
     DECODE_CASE(1) DECODE_CASE(2) DECODE_CASE(3) DECODE_CASE(4)
@@ -831,7 +750,6 @@ static int launch_decode(const void* q, int64_t q_stride, void* k_pages, void* v
     default: return DLI_ERR_ARGUMENT;
   }
 #undef DECODE_CASE
-#undef DECODE_ARGS
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   if (splits > 1) {
     const int pairs = requests * q_heads;
@@ -849,36 +767,6 @@ static int launch_decode(const void* q, int64_t q_stride, void* k_pages, void* v
 #undef MERGE
   }
   return dli_launch_status();
-}
-
-extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pages,
-                                         const void* v_pages, void* out, int64_t out_stride,
-                                         float* part_o, float* part_ml, const int* kv_len,
-                                         const int* block_tables, int table_stride, int requests,
-                                         int q_heads, int kv_heads, int head_dim, int page_size,
-                                         float scale, int window, int splits, hipStream_t stream) {
-  return launch_decode(q, q_stride, const_cast<void*>(k_pages), const_cast<void*>(v_pages), out, out_stride,
-                       part_o, part_ml, kv_len, block_tables, table_stride, requests, q_heads, kv_heads,
-                       head_dim, page_size, scale, window, splits, nullptr, stream);
-}
-
-// The decode step's attention with the rotation of q and k and the cache write of the decoded
-// tokens done inside: `qkv` are the rows of the fused projection (q heads, k heads, v heads, each
-// of head_dim values; row e is request e's one token at position kv_len[e] - 1, whose page is in
-// the block table already), `angles` [requests][2][head_dim/2] cos and sin of the tokens' angles
-// (dli_rope_angles) for a rotation over the whole head. k_pages and v_pages are written at the
-// tokens' slots.
-extern "C" int dli_attention_decode_rope_bf16(const void* qkv, int64_t row_stride, const float* angles,
-                                              void* k_pages, void* v_pages, void* out,
-                                              int64_t out_stride, float* part_o, float* part_ml,
-                                              const int* kv_len, const int* block_tables,
-                                              int table_stride, int requests, int q_heads, int kv_heads,
-                                              int head_dim, int page_size, float scale, int window,
-                                              int splits, hipStream_t stream) {
-  if (angles == nullptr) return DLI_ERR_ARGUMENT;
-  return launch_decode(qkv, row_stride, k_pages, v_pages, out, out_stride, part_o, part_ml, kv_len,
-                       block_tables, table_stride, requests, q_heads, kv_heads, head_dim, page_size, scale,
-                       window, splits, angles, stream);
 }
 
 extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages,

@@ -26,12 +26,30 @@
 //   EPI_RESIDUAL  stream[m][n] = cast(stream[m][n] + cast(y + bias)) in place (the residual sum, in
 //                 32-bit), and this tile's part of sum_n stream[m][n]^2 for the norm that follows
 //   EPI_F32       y stored as float32 (logits)
+//   EPI_QKV       the fused q/k/v projection of a decode step with what follows it: rotary
+//                 rotation of the q and k heads (src/dli/model/rope.py:50-70) and the write of the
+//                 rotated keys and the values into the cache pages, so that no rotation kernel
+//                 runs. TILED only, and the tile order of the q and k heads is a special one: tile
+//                 t of a head holds its dimensions 8t..8t+7 and half+8t..half+8t+7, i.e. eight
+//                 rotary pairs, whose partners sit 32 lanes apart in the product's result. q is
+//                 stored to out in the usual order; k and v go to the pages only.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2, EPI_F32 = 3 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2, EPI_F32 = 3, EPI_QKV = 4 };
+
+// What EPI_QKV needs beside the product: cos/sin of the rows' positions ([rows][2][head_dim/2]
+// float32, rounded to bfloat16 values), the rows' cache slots (negative: not cached), the pages
+// (K page [kv_heads][page_size][head_dim], V page [kv_heads][head_dim][page_size]) and the heads.
+struct QkvRope {
+  const float* angles;
+  const int* slots;
+  bf16_t* k_pages;
+  bf16_t* v_pages;
+  int q_heads, kv_heads, head_dim, page_size;
+};
 
 __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -86,7 +104,8 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
     const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
     const bf16_t* __restrict__ bias, void* __restrict__ out, int64_t ldo,
     bf16_t* __restrict__ stream, int64_t lds_, float* __restrict__ ssq_out, int M, int N, int K,
-    int up_offset) {
+    int up_offset, QkvRope qr) {
+  static_assert(EPI != EPI_QKV || (TILED && MT == 1), "the q/k/v epilogue reads tiled weights, at most 16 rows");
   constexpr int NA = EPI == EPI_SWIGLU ? 2 : 1;  // weight row sets per tile (gate and up)
   constexpr int KR = KS > 1 ? KS - 1 : 1;
   __shared__ float red[KR][NS][NT][NA][MT][4][64];  // k-split waves 1.. hand their tiles to wave 0
@@ -293,6 +312,50 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
           y[a][i] = acc[j][a][t][i];
           if (bias != nullptr && nb + i < N) y[a][i] += (float)bias[nb + i + a * up_offset];
         }
+      if constexpr (EPI == EPI_QKV) {
+        // all lanes take part in the exchange of partners; rows beyond M hold zeros
+        const int d = qr.head_dim, half = d / 2;
+        const int head = tile * 16 / d, t_in = (tile * 16 - head * d) / 16;
+        const bool rotary = head < qr.q_heads + qr.kv_heads;
+        const int mm = min(m, M - 1);
+        const int slot = qr.slots[mm];
+        float v[4], partner[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i] = (float)(bf16_t)y[0][i];
+          partner[i] = __shfl_xor(v[i], 32, 64);
+        }
+        if (rotary) {
+          const int j = 8 * t_in + 4 * (grp & 1);  // first of this lane's four rotary pairs
+          const float4v cs = *reinterpret_cast<const float4v*>(qr.angles + ((int64_t)mm * 2 + 0) * half + j);
+          const float4v sn = *reinterpret_cast<const float4v*>(qr.angles + ((int64_t)mm * 2 + 1) * half + j);
+          bf16_t r[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            r[i] = grp < 2 ? (bf16_t)(v[i] * cs[i] - partner[i] * sn[i]) : (bf16_t)(v[i] * cs[i] + partner[i] * sn[i]);
+          const int dim = (grp < 2 ? 0 : half) + j;
+          bf16_t* dst = nullptr;
+          if (head < qr.q_heads) {
+            dst = reinterpret_cast<bf16_t*>(out) + (int64_t)m * ldo + head * d + dim;
+          } else if (slot >= 0) {
+            const int64_t page = slot / qr.page_size;
+            const int off = slot - (int)page * qr.page_size;
+            dst = qr.k_pages + ((page * qr.kv_heads + (head - qr.q_heads)) * qr.page_size + off) * d + dim;
+          }
+          if (m < M && dst != nullptr) {
+            typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+            *reinterpret_cast<bf16x4*>(dst) = bf16x4{r[0], r[1], r[2], r[3]};
+          }
+        } else if (m < M && slot >= 0) {
+          const int64_t page = slot / qr.page_size;
+          const int off = slot - (int)page * qr.page_size;
+          const int hv = head - qr.q_heads - qr.kv_heads;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            qr.v_pages[((page * qr.kv_heads + hv) * d + 16 * t_in + 4 * grp + i) * qr.page_size + off] = (bf16_t)v[i];
+        }
+        continue;
+      }
       float sq = 0.f;
       if (m < M) {
 #pragma unroll
@@ -344,9 +407,9 @@ __global__ void embedding_ssq_kernel(const bf16_t* __restrict__ table, const int
 #define SK_PARAMS                                                                                 \
   const void *x, int64_t ldx, const float *ssq_in, int ssq_parts, const float *norm_w, float eps,   \
       const void *w, const void *bias, void *out, int64_t ldo, void *stream_buf, int64_t lds_,      \
-      float *ssq_out, int M, int N, int K, int up_offset, hipStream_t stream
+      float *ssq_out, int M, int N, int K, int up_offset, QkvRope qr, hipStream_t stream
 #define SK_ARGS \
-  x, ldx, ssq_in, ssq_parts, norm_w, eps, w, bias, out, ldo, stream_buf, lds_, ssq_out, M, N, K, up_offset, stream
+  x, ldx, ssq_in, ssq_parts, norm_w, eps, w, bias, out, ldo, stream_buf, lds_, ssq_out, M, N, K, up_offset, qr, stream
 
 template <int KS, int NS, int NT, int MT, int EPI, bool NORM, bool TILED>
 static void launch_skinny(SK_PARAMS) {
@@ -354,7 +417,7 @@ static void launch_skinny(SK_PARAMS) {
   const int groups = (tiles + NS * NT - 1) / (NS * NT);
   skinny_gemm_kernel<KS, NS, NT, MT, EPI, NORM, TILED><<<groups, KS * NS * 64, 0, stream>>>(
       (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
-      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
+      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset, qr);
 }
 
 // shapes of the workgroup: 0: 4 k-waves x 1 tile (few tiles, short k); 1: 8 k-waves x 1 tile (few
@@ -391,6 +454,7 @@ extern "C" int dli_skinny_gemm(const void* x, int64_t ldx, const float* ssq_in, 
                                void* out, int64_t ldo, void* stream_buf, int64_t lds_,
                                float* ssq_out, int M, int N, int K, int up_offset, int epilogue,
                                int shape, int tiled, hipStream_t stream) {
+  const QkvRope qr{};
   if (M <= 0 || N <= 0) return DLI_OK;
   if (tiled && (M > 16 || K % 128 != 0 || N % 16 != 0 || up_offset % 16 != 0)) return DLI_ERR_ARGUMENT;
   if (M > 64 || K <= 0 || K % 32 != 0 || ldx % 8 != 0 || shape < 0 || shape > 4 || epilogue < 0 ||
@@ -410,6 +474,34 @@ extern "C" int dli_skinny_gemm(const void* x, int64_t ldx, const float* ssq_in, 
     default:
       return norm ? dispatch_skinny<EPI_F32, true>(shape, mt, tiled != 0, SK_ARGS) : dispatch_skinny<EPI_F32, false>(shape, mt, tiled != 0, SK_ARGS);
   }
+}
+
+// The fused q/k/v projection of a decode step with rotation and cache write inside (EPI_QKV):
+// w_tiled is the [(q_heads + 2*kv_heads) * head_dim, K] matrix in tile order with the q and k
+// heads' tiles made of rotary pairs (see the top), bias (optional) in the same feature order.
+// q goes to out[row][head*head_dim + dim] (row stride ldo), rotated; rotated k and v go to the
+// pages at slots[row]. angles: [M][2][head_dim/2] float32 cos/sin of the rows' positions.
+extern "C" int dli_skinny_gemm_qkv_rope(const void* x, int64_t ldx, const float* ssq_in, int ssq_parts,
+                                        const float* norm_w, float eps, const void* w_tiled,
+                                        const void* bias, void* out, int64_t ldo, const float* angles,
+                                        const int* slots, void* k_pages, void* v_pages, int M, int K,
+                                        int q_heads, int kv_heads, int head_dim, int page_size,
+                                        int shape, hipStream_t stream) {
+  if (M <= 0) return DLI_OK;
+  if (M > 16 || K <= 0 || K % 128 != 0 || ldx % 8 != 0 || ldo % 8 != 0 || shape < 0 || shape > 4 ||
+      q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 16 != 0 || page_size <= 0 ||
+      out == nullptr || angles == nullptr || slots == nullptr || k_pages == nullptr ||
+      v_pages == nullptr || (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)))
+    return DLI_ERR_ARGUMENT;
+  const QkvRope qr{angles, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, q_heads, kv_heads, head_dim, page_size};
+  const int N = (q_heads + 2 * kv_heads) * head_dim, up_offset = 0;
+  void* stream_buf = nullptr;
+  float* ssq_out = nullptr;
+  const int64_t lds_ = 0;
+  const void* w = w_tiled;
+  if (norm_w != nullptr) dispatch_shape<1, EPI_QKV, true, true>(shape, SK_ARGS);
+  else dispatch_shape<1, EPI_QKV, false, true>(shape, SK_ARGS);
+  return dli_launch_status();
 }
 
 extern "C" int dli_embedding_ssq(const void* table, const int* ids, void* out, float* ssq, int rows,

@@ -50,6 +50,9 @@ _SIGNATURES = {
     "dli_skinny_gemm_max_rows": [],
     "dli_skinny_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
                         _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_skinny_gemm_qkv_rope": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64,
+                                 _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                 _c_int, _c_ptr],
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
@@ -57,9 +60,6 @@ _SIGNATURES = {
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_rope_angles": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "dli_attention_decode_rope_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
-                                       _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                                       _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                    _c_ptr],
@@ -446,6 +446,79 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
     return ssq_out if epilogue == SKINNY_RESIDUAL else None
 
 
+def qkv_rope_feature_order(q_heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
+    """The order of the fused projection's features in which :func:`skinny_gemm_qkv_rope` wants
+    its weights and bias: tile ``t`` of a q or k head holds the head's dimensions ``8t..8t+7`` and
+    ``half+8t..half+8t+7`` (eight rotary pairs); v heads keep their order. int64 ``[features]``."""
+    _require(head_dim % 16 == 0 and q_heads > 0 and kv_heads > 0, "heads of a multiple of 16 dimensions")
+    half = head_dim // 2
+    within = torch.tensor([(8 * (f // 16) + f % 8) + (half if f % 16 >= 8 else 0) for f in range(head_dim)])
+    heads = []
+    for h in range(q_heads + 2 * kv_heads):
+        local = within if h < q_heads + kv_heads else torch.arange(head_dim)
+        heads.append(h * head_dim + local)
+    return torch.cat(heads)
+
+
+def tile_weights_qkv_rope(w: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
+    """The fused q/k/v matrix in tile order (:func:`tile_weights`) with the features in
+    :func:`qkv_rope_feature_order`."""
+    _dense(w, "w", torch.bfloat16, 2)
+    _require(w.shape[0] == (q_heads + 2 * kv_heads) * head_dim, "w must hold the q, k and v heads")
+    order = qkv_rope_feature_order(q_heads, kv_heads, head_dim).to(w.device)
+    return tile_weights(w[order].contiguous())
+
+
+def skinny_gemm_qkv_rope(x: torch.Tensor, w_tiled: torch.Tensor, q_out: torch.Tensor, angles: torch.Tensor,
+                         slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, q_heads: int, *,
+                         bias: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None,
+                         eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None,
+                         shape: Optional[int] = None) -> None:
+    """The fused q/k/v projection of at most 16 decode rows with rotation and cache write inside:
+    ``q_out[row, head*head_dim + dim]`` (a ``[rows, >= q_heads*head_dim]`` bfloat16 buffer) gets the
+    rotated queries; the rotated keys and the values go to the pages at ``slots[row]`` (negative:
+    not cached). ``w_tiled`` comes from :func:`tile_weights_qkv_rope`, ``bias`` (optional) is in
+    :func:`qkv_rope_feature_order`, ``angles [rows, 2, head_dim/2]`` from :func:`rope_angles`.
+    ``norm_w``/``eps``/``ssq_in`` as in :func:`skinny_gemm`."""
+    _rows(x, "x", torch.bfloat16)
+    m, k = x.shape
+    _dense(k_pages, "k_pages", torch.bfloat16, 4)
+    _dense(v_pages, "v_pages", torch.bfloat16, 4)
+    pages, kv_heads, page_size, head_dim = k_pages.shape
+    _require(v_pages.shape == (pages, kv_heads, head_dim, page_size), "v_pages must be [pages, kv_heads, head_dim, page_size]")
+    n = (q_heads + 2 * kv_heads) * head_dim
+    _require(0 < m <= 16 and k % 128 == 0 and head_dim % 16 == 0 and q_heads > 0,
+             f"this product takes 1..16 rows, k % 128 == 0 and head_dim % 16 == 0, not {m} x {k}, {head_dim}")
+    _dense(w_tiled, "w_tiled", torch.bfloat16, 1)
+    _require(w_tiled.numel() == n * k and w_tiled.data_ptr() % 16 == 0, "w_tiled must hold [(q + 2 kv) * head_dim, k]")
+    _require(x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0, "x must be 16-byte aligned")
+    _rows(q_out, "q_out", torch.bfloat16)
+    _require(q_out.shape[0] == m and q_out.shape[1] >= q_heads * head_dim and q_out.stride(0) % 8 == 0
+             and q_out.data_ptr() % 16 == 0, "q_out must be [rows, >= q_heads * head_dim], 16-byte aligned")
+    _dense(angles, "angles", torch.float32, 3)
+    _require(angles.shape == (m, 2, head_dim // 2) and angles.data_ptr() % 16 == 0, "angles must be [rows, 2, head_dim/2]")
+    _dense(slots, "slots", torch.int32, 1)
+    _require(slots.shape[0] == m, "one slot per row")
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == n, "bias length differs from the features")
+    parts = 0
+    if norm_w is not None:
+        _dense(norm_w, "norm_w", torch.float32, 1)
+        _require(norm_w.shape[0] == k and norm_w.data_ptr() % 16 == 0, "norm weight must have k aligned values")
+        _require(ssq_in is not None, "a fused norm needs the sums of squares")
+        _dense(ssq_in, "ssq_in", torch.float32, 2)
+        _require(ssq_in.shape[1] == m and ssq_in.shape[0] >= 1, "ssq_in must be [parts, rows]")
+        parts = ssq_in.shape[0]
+    if shape is None:
+        shape = skinny_gemm_shape(n, k, tiled=True)
+    _require(shape in (0, 1, 2, 3, 4), "shape must be 0..4")
+    _check(library().dli_skinny_gemm_qkv_rope(
+        _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w_tiled), _ptr(bias), _ptr(q_out),
+        q_out.stride(0), _ptr(angles), _ptr(slots), _ptr(k_pages), _ptr(v_pages), m, k, q_heads, kv_heads, head_dim,
+        page_size, shape, _stream()), "skinny_gemm_qkv_rope")
+
+
 def embedding_ssq(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, ssq: torch.Tensor) -> None:
     """``out[t] = table[ids[t]]`` and ``ssq[0, t] = sum(out[t]^2)`` (bfloat16 table)."""
     _dense(table, "table", torch.bfloat16, 2)
@@ -570,50 +643,6 @@ def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, dtype: torch.dt
     _check(library().dli_rope_angles(_ptr(positions), _ptr(inv_freq), _ptr(table), n, half, _is_bf16(dtype),
                                      _stream()), "rope_angles")
     return table
-
-
-def attention_decode_rope(qkv: torch.Tensor, angles: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
-                          out: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor, q_heads: int,
-                          scale: float, window: int = 0, splits: int = 1, part_o: Optional[torch.Tensor] = None,
-                          part_ml: Optional[torch.Tensor] = None) -> None:
-    """:func:`attention_decode` with the rotation of q and k and the cache write of the decoded
-    tokens inside: ``qkv [rows, (q_heads + 2*kv_heads) * head_dim]`` is the fused projection as
-    the product left it; ``angles [rows, 2, head_dim/2]`` comes from :func:`rope_angles` (the
-    rotation covers the whole head); row ``e`` is the token at position ``kv_len[e] - 1``, whose
-    page the block table names already. The token's rotated key and its value are written into
-    the pages."""
-    _dense(k_pages, "k_pages", torch.bfloat16, 4)
-    _dense(v_pages, "v_pages", torch.bfloat16, 4)
-    pages, kv_heads, page_size, head_dim = k_pages.shape
-    _require(v_pages.shape == (pages, kv_heads, head_dim, page_size),
-             "v_pages must be [pages, kv_heads, head_dim, page_size]")
-    _rows(qkv, "qkv", torch.bfloat16)
-    _rows(out, "out", torch.bfloat16)
-    rows = qkv.shape[0]
-    _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
-    _require(qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim and out.shape == (rows, q_heads * head_dim),
-             "qkv must be [rows, (q_heads + 2*kv_heads)*head_dim] and out [rows, q_heads*head_dim]")
-    _require(qkv.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and qkv.data_ptr() % 8 == 0 and out.data_ptr() % 8 == 0,
-             "qkv/out rows must be 8-byte aligned")
-    _require(bool(library().dli_attention_mfma_supports(head_dim, page_size)),
-             f"the matrix-core attention takes head_dim 16..128 in steps of 16 and pages of a multiple of 16, "
-             f"not head_dim {head_dim}, page size {page_size}")
-    _dense(angles, "angles", torch.float32, 3)
-    _require(angles.shape == (rows, 2, head_dim // 2), "angles must be [rows, 2, head_dim/2]: the rotation covers the whole head")
-    _dense(kv_len, "kv_len", torch.int32, 1)
-    _dense(block_tables, "block_tables", torch.int32, 2)
-    _require(kv_len.shape[0] >= rows and block_tables.shape[0] >= rows, "one kv_len and table row per request")
-    _require(1 <= splits <= 65535 and rows <= 65535, "splits and requests must fit the grid")
-    if splits > 1:
-        _require(part_o is not None and part_ml is not None, "splits > 1 needs the partial-result buffers")
-        _dense(part_o, "part_o", torch.float32)
-        _dense(part_ml, "part_ml", torch.float32)
-        _require(part_o.numel() >= rows * q_heads * splits * head_dim and part_ml.numel() >= rows * q_heads * splits * 2,
-                 "partial-result buffers are too small")
-    _check(library().dli_attention_decode_rope_bf16(
-        _ptr(qkv), qkv.stride(0), _ptr(angles), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0),
-        _ptr(part_o), _ptr(part_ml), _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads,
-        kv_heads, head_dim, page_size, float(scale), int(window), int(splits), _stream()), "attention_decode_rope")
 
 
 def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,

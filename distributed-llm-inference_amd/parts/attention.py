@@ -20,16 +20,17 @@ from typing import Any, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .attention_kernels import decode_attention_with_rope, paged_attention
+from .attention_kernels import paged_attention
 from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
 from .linear import decode_copy, linear
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
 
-# Decode steps of at most this many rows rotate q and k and write the cache inside the attention
-# kernel; larger ones run the rotation kernel first (measured: the fused form saves a launch's
-# latency at one row and loses to the separate kernel once every compute unit has work).
-ROPE_IN_ATTENTION_MAX_ROWS = 2
+# Decode steps with this many rows rotate and write the cache in the epilogue of the q/k/v
+# product, which reads a copy of the matrix whose tiles hold whole rotary pairs: no rotation
+# kernel runs. (A variant that rotated inside the attention kernel instead, repeating the rotation
+# in every split of the keys, was slower from four rows on and no faster below.)
+ROPE_IN_PRODUCT_ROWS = range(1, 17)
 
 
 @register_part("mixer", "gqa_attention")
@@ -51,6 +52,7 @@ class GQAttention(Mixer):
         self.position = build_part("position", position or PartSpec("none"), runtime)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self.w_qkv_tiled = self.w_o_tiled = None
+        self.w_qkv_rope = self.b_qkv_rope = None  # tile order with rotary pairs, for the product that rotates
 
     # -- weights
     def weight_specs(self) -> dict[str, WeightSpec]:
@@ -75,6 +77,17 @@ class GQAttention(Mixer):
     def finalize(self) -> None:
         self.w_qkv_tiled = decode_copy(self.rt, self.w_qkv, ops.SKINNY_STORE)
         self.w_o_tiled = decode_copy(self.rt, self.w_o, ops.SKINNY_RESIDUAL)
+        table = self.position.rotary_table()
+        if (self.w_qkv_tiled is not None and not self.shares_kv and table is not None
+                and table[1] == self.head_dim):
+            # the rotation covers the whole head: the product can rotate in its epilogue, and
+            # this order of the features replaces the plain tile order
+            nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+            self.w_qkv_rope = ops.tile_weights_qkv_rope(self.w_qkv, nh, nkv, d)
+            if self.b_qkv is not None:
+                order = ops.qkv_rope_feature_order(nh, nkv, d).to(self.b_qkv.device)
+                self.b_qkv_rope = self.b_qkv[order].contiguous()
+            self.w_qkv_tiled = None  # every step that would read it takes the other copy
 
     def sub_parts(self) -> dict[str, Part]:
         return {"position": self.position}
@@ -126,6 +139,16 @@ class GQAttention(Mixer):
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
+        if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS:
+            # product, rotation and cache write in one kernel; only q comes back
+            angles = ctx.rope_angles(self.position.rotary_table()[0], qkv.dtype)
+            ops.skinny_gemm_qkv_rope(stream.x, self.w_qkv_rope, qkv, angles, grp.slots, cache.k_pages, cache.v_pages,
+                                     nh, bias=self.b_qkv_rope, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+            out = self.rt.empty(n, nh * d)
+            paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+            stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
+                                         stream=stream.x, bias=self.b_o)
+            return
         ops.skinny_gemm(stream.x, self.w_qkv, w_tiled=self.w_qkv_tiled, epilogue=ops.SKINNY_STORE, out=qkv,
                         bias=self.b_qkv, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         table = self.position.rotary_table()
@@ -137,13 +160,8 @@ class GQAttention(Mixer):
         else:
             inv_freq, rotary_dim = table
         out = self.rt.empty(n, nh * d)
-        if nkv and inv_freq is not None and rotary_dim == d and n <= ROPE_IN_ATTENTION_MAX_ROWS:
-            # rotation and cache write happen inside the attention kernel
-            decode_attention_with_rope(qkv, inv_freq, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale,
-                                       self.window)
-        else:
-            ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
-                              cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
-            paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
+                          cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
+        paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
                                      stream=stream.x, bias=self.b_o)

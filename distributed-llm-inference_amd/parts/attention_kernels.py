@@ -61,15 +61,3 @@ def _decode_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, head_dim: int
         part_o = torch.empty(nd * q_heads * splits * head_dim, device=device, dtype=torch.float32)
         part_ml = torch.empty(nd * q_heads * splits * 2, device=device, dtype=torch.float32)
     return splits, part_o, part_ml
-
-
-def decode_attention_with_rope(qkv: torch.Tensor, inv_freq: torch.Tensor, k_pages: torch.Tensor,
-                               v_pages: torch.Tensor, out: torch.Tensor, ctx: Any, grp: Any, q_heads: int,
-                               scale: float, window: int = 0) -> None:
-    """A decode-only step's attention with rotation and cache write inside the attention kernel:
-    ``qkv`` is the fused projection, unrotated; the tokens' keys and values reach the pages here.
-    The angles' cos and sin are computed once per step and rotary table, for all layers."""
-    _, kv_heads, _, head_dim = k_pages.shape
-    splits, part_o, part_ml = _decode_splits(ctx, ctx.num_decode, q_heads, kv_heads, head_dim, qkv.device)
-    ops.attention_decode_rope(qkv, ctx.rope_angles(inv_freq, qkv.dtype), k_pages, v_pages, out, ctx.kv_len,
-                              grp.block_tables, q_heads, scale, window, splits, part_o, part_ml)

@@ -224,41 +224,6 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
     assert err < tol(torch.bfloat16), err
 
 
-@pytest.mark.parametrize("qh,kvh,d,bs", [(8, 2, 64, 16), (32, 8, 64, 16), (6, 2, 32, 16), (20, 1, 48, 32), (4, 4, 128, 16)])
-@pytest.mark.parametrize("splits", [1, 4, 16])
-@pytest.mark.parametrize("window", [0, 45])
-def test_attention_decode_with_rotation_and_cache_write_inside(ops, qh, kvh, d, bs, splits, window):
-    """The decode kernel that rotates q and k and writes the new token's key and value itself,
-    against the separate rotation kernel followed by the plain decode kernel: same outputs, same
-    pages (a rounding of the rotated values apart), nothing else touched."""
-    rng = torch.Generator().manual_seed(d + bs + splits)
-    lens = [(1, n) for n in [1, 2, bs, bs + 1, 3 * bs - 1, 16, 17, 33] + [int(x) for x in torch.randint(1, 30 * bs, (5,), generator=rng)]]
-    _, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + splits, poison=False)
-    n = len(lens)
-    qkv = torch.randn(n, (qh + 2 * kvh) * d, generator=rng).bfloat16().cuda()
-    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d))).cuda()
-    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
-    positions = dev([k - 1 for k in kv_len])
-    slots = dev([tables[e][(kv_len[e] - 1) // bs] * bs + (kv_len[e] - 1) % bs for e in range(n)])
-    scale = 1.0 / math.sqrt(d)
-    parts = lambda: (torch.full((n * qh * splits * d,), float("nan"), device="cuda"),
-                     torch.full((n * qh * splits * 2,), float("nan"), device="cuda"))
-    # separate kernels
-    kp1, vp1, qkv1 = kp.cuda().clone(), vp.cuda().clone(), qkv.clone()
-    ops.rope_kv_write(qkv1, positions, inv_freq, d, slots, kp1, vp1, qh, kvh, d)
-    out1 = torch.zeros(n, qh * d, dtype=torch.bfloat16, device="cuda")
-    ops.attention_decode(qkv1[:, :qh * d], kp1, vp1, out1, dev(kv_len), dev(tables), qh, scale, window, splits, *parts())
-    # one kernel
-    kp2, vp2 = kp.cuda().clone(), vp.cuda().clone()
-    out2 = torch.zeros(n, qh * d, dtype=torch.bfloat16, device="cuda")
-    ops.attention_decode_rope(qkv, ops.rope_angles(positions, inv_freq, torch.bfloat16), kp2, vp2, out2, dev(kv_len), dev(tables), qh, scale, window, splits, *parts())
-    assert torch.equal(vp1, vp2)
-    assert (kp1.float() - kp2.float()).abs().max() <= 2 ** -7 * kp1.float().abs().max()
-    changed = (kp2 != kp.cuda()).any(dim=-1).sum().item()
-    assert changed <= n * kvh, "keys other than the new tokens' were written"
-    assert (out1.float() - out2.float()).abs().max() < tol(torch.bfloat16)
-
-
 @pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("pair", [False, True])
@@ -413,6 +378,64 @@ def test_skinny_gemm_with_weights_in_tile_order(ops, m, n, k, shape):
         g, u = gu[:, :n // 2].bfloat16().double(), gu[:, n // 2:].bfloat16().double()
         want = (g * torch.sigmoid(g)).bfloat16().double() * u
         assert (b.cpu().double() - want).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 16])
+@pytest.mark.parametrize("qh,kvh,d,k,bs,shape", [(4, 4, 16, 128, 16, None), (6, 2, 32, 384, 8, 0), (5, 1, 48, 256, 4, 4),
+                                                 (32, 8, 64, 2048, 16, None), (3, 3, 128, 640, 16, 3)])
+def test_skinny_gemm_qkv_with_rotation_and_cache_write(ops, m, qh, kvh, d, k, bs, shape):
+    """The fused projection that rotates q and k and writes the cache itself against: norm,
+    product, rotation (kernel_refs.ref_rope) and a write by slot, each done plainly."""
+    torch.manual_seed(m + qh + d)
+    n = (qh + 2 * kvh) * d
+    x = (torch.randn(m, k, device="cuda") * 2).bfloat16()
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    bias = torch.randn(n, device="cuda").bfloat16()
+    nw = (1 + 0.1 * torch.randn(k, device="cuda")).float()
+    ssq = x.float().pow(2).sum(-1)[None].contiguous()
+    positions = torch.tensor([0, 1, 4095, 77, 500, 3, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18][:m], dtype=torch.int32, device="cuda")
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d))).cuda()
+    pages = 6
+    perm = torch.randperm(pages * bs)[:m]
+    if m > 2:
+        perm[2] = -1  # not cached
+    slots = perm.to(torch.int32).cuda()
+    k_pages = torch.full((pages, kvh, bs, d), 7.0, device="cuda").bfloat16()
+    v_pages = torch.full((pages, kvh, d, bs), 7.0, device="cuda").bfloat16()
+    order = ops.qkv_rope_feature_order(qh, kvh, d)
+    assert sorted(order.tolist()) == list(range(n))
+    wt = ops.tile_weights_qkv_rope(w, qh, kvh, d)
+    q_out = torch.full((m, n), 7.0, device="cuda", dtype=torch.bfloat16)
+    angles = ops.rope_angles(positions, inv_freq, torch.bfloat16)
+    ops.skinny_gemm_qkv_rope(x, wt, q_out, angles, slots, k_pages, v_pages, qh, bias=bias[order.cuda()].contiguous(),
+                             norm_w=nw, eps=1e-5, ssq_in=ssq, shape=shape)
+    xhat = _ref_norm_bf16(x, nw, 1e-5)
+    y = (xhat.cpu().double() @ w.cpu().double().T + bias.cpu().double()).bfloat16().view(m, qh + 2 * kvh, d)
+    q_ref = ref_rope(y[:, :qh], positions.cpu(), inv_freq.cpu(), d)
+    k_ref = ref_rope(y[:, qh:qh + kvh], positions.cpu(), inv_freq.cpu(), d)
+    scale = max(1.0, y.float().abs().max().item())
+    t = 3e-2 * scale
+    got = q_out.cpu().view(m, qh + 2 * kvh, d)
+    assert (got[:, :qh].double() - q_ref).abs().max() < t
+    assert (got[:, qh:] == 7.0).all()   # k and v go to the pages only
+    kp, vp = k_pages.cpu(), v_pages.cpu()
+    written = torch.zeros(pages * bs, dtype=torch.bool)
+    for row in range(m):
+        s_ = int(perm[row])
+        if s_ < 0:
+            continue
+        written[s_] = True
+        assert (kp[s_ // bs, :, s_ % bs, :].double() - k_ref[row]).abs().max() < t
+        assert (vp[s_ // bs, :, :, s_ % bs].double() - y[row, qh + kvh:].double()).abs().max() < t
+    for s_ in range(pages * bs):
+        if not written[s_]:
+            assert (kp[s_ // bs, :, s_ % bs, :] == 7.0).all() and (vp[s_ // bs, :, :, s_ % bs] == 7.0).all()
+    # the same numbers as the separate kernels give: product, then rotation and cache write
+    qkv = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    ops.skinny_gemm(x, w, epilogue=ops.SKINNY_STORE, out=qkv, bias=bias, norm_w=nw, eps=1e-5, ssq_in=ssq, shape=0)
+    k2, v2 = torch.zeros_like(k_pages), torch.zeros_like(v_pages)
+    ops.rope_kv_write(qkv, positions, inv_freq, d, slots, k2, v2, qh, kvh, d)
+    assert (qkv[:, :qh * d].float() - q_out[:, :qh * d].float()).abs().max() <= 2e-2 * scale
 
 
 def test_tiled_weights_are_refused_where_they_do_not_fit(ops):
