@@ -341,7 +341,7 @@ def _units(device: torch.device) -> int:
 
 
 def skinny_gemm_plan(rows: int, n: int, k: int, epilogue: int, device: torch.device,
-                     blocks4: Optional[int] = None) -> tuple[str, int, int]:
+                     blocks4: Optional[int] = None, tiled: bool = False) -> tuple[str, int, int]:
     """How :func:`skinny_gemm` runs a product: ``(kernel, shape, parts)``.
 
     ``"blocks4"`` is the 4x4-block kernel (at most 16 rows), ``"tiles16"`` the 16x16-tile kernel
@@ -350,18 +350,25 @@ def skinny_gemm_plan(rows: int, n: int, k: int, epilogue: int, device: torch.dev
     timings on MI355X: the block kernel reads whole cache lines of the weights and only the rows of
     activations that exist, which wins for one to four rows; with more rows the activations'
     traffic grows and the tile kernel, which reads them once per 16 features, is ahead.
+    ``tiled``: a copy of the weights in tile order is at hand (at most 16 rows); the tile kernel
+    then reads whole lines too and takes over from three rows on, and below that where the
+    product has few features.
     """
     if blocks4 is None and rows <= 16 and k % 8 == 0:
         deep = k >= 4096 and n <= 4096   # long rows, few features: many waves on narrow tiles
         if rows <= 4:
             out_feats = n * (2 if epilogue == SKINNY_SWIGLU else 1)
-            blocks4 = 2 if deep else (1 if out_feats <= 16 * _units(device) else 0)
+            few = out_feats <= 16 * _units(device)
+            if deep:
+                blocks4 = 2
+            elif not (tiled and (rows >= 3 or few)):
+                blocks4 = 1 if few else 0
         elif deep:
             blocks4 = 1
     if blocks4 is not None:
         feats = int(library().dli_skinny4_tile_features(blocks4, epilogue))
         return "blocks4", blocks4, -(-n // feats)
-    return "tiles16", skinny_gemm_shape(n, k), -(-n // 16)
+    return "tiles16", skinny_gemm_shape(n, k, tiled and rows <= 16), -(-n // 16)
 
 
 def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optional[torch.Tensor] = None,
@@ -400,14 +407,13 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
     else:
         if blocks4 is not None:
             _require(blocks4 in (0, 1, 2) and m <= 16 and k % 8 == 0, "blocks4 must be 0..2, with at most 16 rows")
-        kernel, a, n_parts = skinny_gemm_plan(m, n, k, epilogue, x.device, blocks4)
+        kernel, a, n_parts = skinny_gemm_plan(m, n, k, epilogue, x.device, blocks4,
+                                              tiled=w_tiled is not None and m <= 16)
     tiled = w_tiled is not None and kernel == "tiles16" and m <= 16
     if tiled:
         _dense(w_tiled, "w_tiled", torch.bfloat16, 1)
         _require(w_tiled.numel() == w.numel() and k % 128 == 0 and n % 16 == 0 and w_tiled.data_ptr() % 16 == 0,
                  "w_tiled must hold the same weights in tile order (n % 16 == 0, k % 128 == 0)")
-        if shape is None:
-            a = skinny_gemm_shape(n, k, tiled=True)
     parts = 0
     if norm_w is not None:
         _require(epilogue != SKINNY_RESIDUAL, "the residual epilogue takes no fused norm")
