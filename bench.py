@@ -77,14 +77,16 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     # Requests admitted first decode a token a step while the others still prefill; the prompts are
     # shortened by that many steps so that no request outgrows `context` while the clock runs.
     budget = engine.scheduler.config.max_num_batched_tokens
-    prompt_len = context - steps - warmup - 1
+    per = max(d for d in (8, 4, 2, 1) if d <= max(1, decode_steps) and steps % d == 0)
+    warm = -(-warmup // per) * per   # whole engine steps
+    prompt_len = context - steps - warm - per - 1   # the last engine step reserves `per` slots ahead
     prompt_len -= -(-batch * prompt_len // budget) + 1
     ids = []
     for i in range(batch):
         prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).tolist()
         ids.append(f"b{batch}-{i}")
         # requests that were admitted first decode a few tokens while the others still prefill
-        engine.add_request(ids[-1], prompt, SamplingParams(max_tokens=steps + warmup + 1 + SLACK, ignore_eos=True))
+        engine.add_request(ids[-1], prompt, SamplingParams(max_tokens=steps + warm + per + 1 + SLACK, ignore_eos=True))
     guard = 0
     while engine.scheduler.waiting or any(r.num_computed_tokens < prompt_len for r in engine.scheduler.running):
         engine.step()  # prefill, in portions under the token budget
@@ -102,9 +104,8 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
 
     import dataclasses
 
-    per = max(d for d in (8, 4, 2, 1) if d <= max(1, decode_steps) and steps % d == 0)
     engine.scheduler.config = dataclasses.replace(engine.scheduler.config, decode_steps=per)
-    advance(-(-warmup // per) * per)
+    advance(warm)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     done = advance(steps)
@@ -163,7 +164,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
-    ap.add_argument("--decode-steps", type=int, default=4,
+    ap.add_argument("--decode-steps", type=int, default=8,
                     help="decode steps that one engine step runs on the device before the host looks "
                          "(reduced to a divisor of --steps)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
