@@ -81,10 +81,6 @@ class StepFunction:
                     f"{mgr.num_computed_tokens(e.seq_id)} tokens are computed")
             if e.start + n > mgr.num_tokens(e.seq_id):
                 raise StepError(f"request {e.seq_id!r}: no cache slots reserved up to {e.start + n}")
-            ids = np.asarray(e.tokens, dtype=np.int64)
-            if int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size:
-                bad = int(ids[(ids < 0) | (ids >= self.vocab_size)][0])
-                raise StepError(f"request {e.seq_id!r}: token id {bad} outside the vocabulary")
             for wnt in e.want:
                 if not 0 <= int(wnt) < n:
                     raise StepError(f"request {e.seq_id!r}: wanted place {wnt} outside its {n} tokens")
@@ -99,26 +95,31 @@ class StepFunction:
             first_row[i] = int(q_start[k])
             q_start[k + 1] = q_start[k] + len(entries[i].tokens)
         total = int(q_start[-1])
-        token_ids = np.empty(total, np.int32)
+        token_ids = np.empty(total, np.int64)
         positions = np.empty(total, np.int32)
         kv_len = np.empty(len(entries), np.int32)
         state_slots = np.empty(len(entries), np.int32)
         n_groups = mgr.num_groups
-        slots = [np.empty(total, np.int32) for _ in range(n_groups)]
-        tables: list[list[tuple[int, ...]]] = [[] for _ in range(n_groups)]
+        slots = [np.empty(total, np.int64) for _ in range(n_groups)]
+        tables: list[list[np.ndarray]] = [[] for _ in range(n_groups)]
         for k, i in enumerate(order):
             e = entries[i]
             r0, n = int(q_start[k]), len(e.tokens)
-            token_ids[r0:r0 + n] = np.asarray(e.tokens, dtype=np.int32)
-            positions[r0:r0 + n] = np.arange(e.start, e.start + n, dtype=np.int32)
+            token_ids[r0:r0 + n] = e.tokens
+            pos = np.arange(e.start, e.start + n, dtype=np.int64)
+            positions[r0:r0 + n] = pos
             kv_len[k] = e.start + n
             state_slots[k] = mgr.state_slot(e.seq_id)
             for g in range(n_groups):
-                slots[g][r0:r0 + n] = mgr.slot_mapping(e.seq_id, e.start, e.start + n, g)
-                table = mgr.block_table(e.seq_id, g)
-                if len(table) * ps < e.start + n:
+                table = np.asarray(mgr.table_ref(e.seq_id, g), dtype=np.int64)
+                if table.size * ps < e.start + n:
                     raise StepError(f"request {e.seq_id!r}: block table shorter than its keys")
+                # a page that the window has passed gives a negative slot, refused below
+                slots[g][r0:r0 + n] = table[pos // ps] * ps + pos % ps
                 tables[g].append(table)
+        if total and (int(token_ids.min()) < 0 or int(token_ids.max()) >= self.vocab_size):
+            bad = int(token_ids[(token_ids < 0) | (token_ids >= self.vocab_size)][0])
+            raise StepError(f"token id {bad} outside the vocabulary")
         logit_rows = np.asarray(
             [first_row[i] + int(w) for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
 
@@ -133,16 +134,15 @@ class StepFunction:
         group_arrays: list[tuple[int, int, int]] = []
         for g in range(n_groups):
             width = max((len(t) for t in tables[g]), default=1) or 1
-            host = np.zeros((max(len(entries), 1), width), np.int32)
-            limit = self.store.num_pages
+            host = np.zeros((max(len(entries), 1), width), np.int64)
             for k, t in enumerate(tables[g]):
-                row = np.asarray(t, dtype=np.int64)
-                row = np.where(row == RELEASED, 0, row)  # pages that the window has passed: never read
-                if row.size and (row.min() < 0 or row.max() >= limit):
-                    raise StepError("a block table names a page outside the pool")
-                host[k, :len(t)] = row
-            if total and (slots[g].min() < 0 or slots[g].max() >= limit * ps):
-                raise StepError("a cache slot lies outside the pool")
+                host[k, :t.size] = t
+            host[host == RELEASED] = 0  # pages that the window has passed: never read
+            limit = self.store.num_pages
+            if host.size and (int(host.min()) < 0 or int(host.max()) >= limit):
+                raise StepError("a block table names a page outside the pool")
+            if total and (int(slots[g].min()) < 0 or int(slots[g].max()) >= limit * ps):
+                raise StepError("a cache slot lies outside the pool, or in a page that the window has passed")
             group_arrays.append((to_dev(slots[g]), to_dev(host), width))
         named = {name: to_dev(a) for name, a in (
             ("token_ids", token_ids), ("positions", positions), ("q_start", q_start), ("kv_len", kv_len),

@@ -94,7 +94,14 @@ def _check(status: int, name: str) -> None:
     raise KernelLaunchError(f"{name}: launch failed (status {status})")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> _c_ptr:
+    """The current stream's handle. The raw getter skips the Stream object that
+    ``torch.cuda.current_stream()`` builds at every call (a hundred calls a step)."""
+    if _raw_stream is not None:
+        return _c_ptr(_raw_stream(torch.cuda.current_device()))
     return _c_ptr(torch.cuda.current_stream().cuda_stream)
 
 
@@ -116,16 +123,19 @@ def _require(cond: bool, msg: str) -> None:
 
 
 def _dense(t: torch.Tensor, name: str, dtype: Optional[torch.dtype] = None, ndim: Optional[int] = None) -> None:
+    # the messages are put together only when a check fails: this runs hundreds of times a step
+    if t.is_cuda and t.is_contiguous() and (dtype is None or t.dtype == dtype) and (ndim is None or t.dim() == ndim):
+        return
     _require(t.is_cuda, f"{name} is not on the GPU")
     _require(t.is_contiguous(), f"{name} is not contiguous")
-    if dtype is not None:
-        _require(t.dtype == dtype, f"{name} has type {t.dtype}, expected {dtype}")
-    if ndim is not None:
-        _require(t.dim() == ndim, f"{name} has {t.dim()} dimensions, expected {ndim}")
+    _require(dtype is None or t.dtype == dtype, f"{name} has type {t.dtype}, expected {dtype}")
+    _require(ndim is None or t.dim() == ndim, f"{name} has {t.dim()} dimensions, expected {ndim}")
 
 
 def _rows(t: torch.Tensor, name: str, dtype: torch.dtype) -> None:
     """A 2-D operand whose rows are contiguous (a row stride larger than the width is allowed)."""
+    if t.is_cuda and t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= t.shape[1] and t.dtype == dtype:
+        return
     _require(t.is_cuda, f"{name} is not on the GPU")
     _require(t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= t.shape[1],
              f"{name} is not a matrix with contiguous rows")

@@ -210,3 +210,34 @@ def test_long_decoding(dtype):
     for i in range(20, len(toks)):
         got = s.step([{"id": 0, "tokens": [toks[i]], "want": [0]}])
         check(got, ref[i:i + 1], dtype, f"decode at {i}")
+
+
+def test_step_function_refuses_entries_that_do_not_fit_the_cache_state():
+    """What the step function checks before anything reaches the GPU: one entry per request, the
+    portion continues what is computed, slots are reserved, ids lie in the vocabulary, wanted
+    places lie in the portion. A refused step leaves the request as it was."""
+    from dli_amd.engine.batch import StepEntry
+    from dli_amd.engine.step import StepError
+
+    core = make_core("A", "float32", num_pages=8, page_size=16)
+    mgr, step = core.manager, core.step
+    toks = prompts_for("A", [20])[0]
+    mgr.allocate("r", toks, respect_watermark=False)
+    bad = [
+        ([StepEntry("r", toks[:4], 0, [0]), StepEntry("r", toks[4:8], 4, [0])], "twice"),
+        ([StepEntry("r", [], 0, [])], "no tokens"),
+        ([StepEntry("r", toks[4:8], 4, [0])], "computed"),            # skips the first four
+        ([StepEntry("r", toks + [1, 2], 0, [0])], "reserved"),         # more than was allocated
+        ([StepEntry("r", [toks[0], 256], 0, [0])], "vocabulary"),     # the vocabulary has 256 ids
+        ([StepEntry("r", [toks[0], -1], 0, [0])], "vocabulary"),
+        ([StepEntry("r", toks[:4], 0, [4])], "wanted"),
+    ]
+    for entries, word in bad:
+        with pytest.raises(StepError, match=word):
+            step.run(entries)
+        assert mgr.num_computed_tokens("r") == 0
+    # the same request still runs, and gives the plain implementation's logits
+    got = step.run([StepEntry("r", toks, 0, list(range(len(toks))))])
+    check(got, plain_logits("A", toks), "float32", "after refusals")
+    mgr.free("r")
+    mgr.check_invariants()
