@@ -159,8 +159,11 @@ def build(force: bool = False, verbose: bool = True) -> Path:
     with ThreadPoolExecutor(max_workers=workers) as pool:
         list(pool.map(compile_one, jobs))
     tmp_lib = lib.with_suffix(f".tmp{os.getpid()}.so")
-    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp_lib), *map(str, objects)],
-         lib.name)
+    # the vendor's matrix-product library (gemm_lt.hip calls it) lies beside the compiler
+    rocm_lib = Path(os.path.realpath(hipcc)).parent.parent / "lib"
+    link = [f"-L{rocm_lib}", f"-Wl,-rpath,{rocm_lib}"] if rocm_lib.is_dir() else []
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp_lib), *map(str, objects), *link,
+          "-lhipblaslt"], lib.name)
     os.replace(tmp_lib, lib)
     keep = {lib.name, *(o.name for o in objects)}
     for stale in list(out_dir.glob(f"{LIB_STEM}-*.so")) + list(out_dir.glob("*.o")):

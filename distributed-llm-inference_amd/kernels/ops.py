@@ -53,6 +53,8 @@ _SIGNATURES = {
     "dli_skinny_gemm_qkv_rope": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64,
                                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_ptr],
+    "dli_gemm_bf16": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64,
+                      _c_int, _c_ptr],
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
@@ -460,6 +462,36 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
             _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
             _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, a, _stream()), "skinny4_gemm")
     return ssq_out if epilogue == SKINNY_RESIDUAL else None
+
+
+_GEMM_WORKSPACE_BYTES = 64 << 20
+_gemm_workspaces: dict[int, torch.Tensor] = {}
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> bool:
+    """``out = x @ w.T (+ bias)`` for bfloat16 matrices with contiguous rows through the vendor
+    library, 32-bit accumulation, the bias added before the one rounding. The library's choice
+    of kernel is looked up once per shape. Returns False where the library has no kernel for the
+    shape (nothing was computed then)."""
+    _rows(x, "x", torch.bfloat16)
+    _rows(w, "w", torch.bfloat16)
+    _rows(out, "out", torch.bfloat16)
+    rows, k = x.shape
+    feats = w.shape[0]
+    _require(w.shape[1] == k and out.shape == (rows, feats), "x [n, k], w [m, k] and out [n, m] do not fit")
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == feats, "bias length differs from rows of w")
+    index = x.device.index if x.device.index is not None else torch.cuda.current_device()
+    workspace = _gemm_workspaces.get(index)
+    if workspace is None:
+        workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+    status = library().dli_gemm_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(bias), _ptr(out), out.stride(0),
+                                     rows, feats, k, _ptr(workspace), _GEMM_WORKSPACE_BYTES, index, _stream())
+    if status == -1:
+        return False
+    _check(status, "gemm_bf16")
+    return True
 
 
 def qkv_rope_feature_order(q_heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
