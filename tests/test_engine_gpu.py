@@ -40,7 +40,7 @@ def assert_same_or_near_tie(name, prompt, got, want, margin):
 
 
 @pytest.mark.parametrize("name,dtype,block", [("A", "float32", 16), ("B", "float32", 8), ("A", "bfloat16", 16),
-                                              ("B", "bfloat16", 16), ("C", "bfloat16", 32)])
+                                              ("B", "bfloat16", 16), ("C", "bfloat16", 32), ("D", "bfloat16", 16)])
 def test_greedy_generation_through_the_entry_point(name, dtype, block):
     from dli_amd.engine.generate import greedy_generate
 
@@ -75,7 +75,7 @@ def test_engine_equals_single_requests_in_three_regimes(regime):
     assert eng.manager.stats().used_pages == 0
 
 
-@pytest.mark.parametrize("name,block", [("A", 16), ("C", 32)])
+@pytest.mark.parametrize("name,block", [("A", 16), ("C", 32), ("D", 16)])
 def test_graph_replay_equals_eager_steps(name, block):
     """Decode steps through HIP graphs against the same steps run eagerly: logits of every step
     must agree, with other work and synchronisations between the replays, batch sizes that
@@ -132,7 +132,7 @@ def test_graph_replay_equals_eager_steps(name, block):
 
 
 @pytest.mark.parametrize("name,block,k,graph_len", [("A", 16, 4, None), ("C", 32, 3, None), ("B", 16, 8, None),
-                                                   ("A", 16, 4, 40)])
+                                                   ("A", 16, 4, 40), ("D", 16, 8, None)])
 def test_several_decode_tokens_per_step_equal_one_per_step(name, block, k, graph_len):
     """Steps that decode `k` tokens of every request on the device (sampled tokens fed back there,
     positions, slots and draw counters advanced by a kernel) against one token per step: greedy

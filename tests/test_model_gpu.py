@@ -69,7 +69,7 @@ def prompts_for(name: str, lengths, seed=5):
 
 
 CASES = [("A", 16, "float32"), ("A", 16, "bfloat16"), ("B", 8, "float32"), ("B", 8, "bfloat16"),
-         ("C", 4, "float32"), ("C", 32, "bfloat16")]
+         ("C", 4, "float32"), ("C", 32, "bfloat16"), ("D", 16, "bfloat16")]
 
 
 @pytest.mark.parametrize("name,page,dtype", CASES)

@@ -41,7 +41,18 @@ WIDE = {
                      "original_max_position_embeddings": 8192},
     "tie_word_embeddings": True, "hidden_act": "silu",
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "W": WIDE}
+# sizes that tile (width and feed-forward multiples of 128, vocabulary a multiple of 16): decode
+# steps read the tile-ordered copies of the weights and rotate in the q/k/v product, as at the
+# serving sizes, but on a model small enough for every way of cutting and batching
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 512, "hidden_size": 256,
+    "intermediate_size": 384, "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2,
+    "head_dim": 32, "rms_norm_eps": 1e-5, "max_position_embeddings": 2048, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 128},
+    "attention_bias": True, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "W": WIDE}
 
 _made: dict = {}
 _tmp = None
@@ -51,7 +62,7 @@ _tmp = None
 # have a spread of about one, so attention is far from uniform (a key in the wrong place, a wrong
 # rotation or a wrong mask changes the logits) without being so sharp that bfloat16's rounding of a
 # score is blown up into a different distribution.
-STD = {"A": 0.15, "B": 0.085, "C": 0.085, "W": 0.0265}
+STD = {"A": 0.15, "B": 0.085, "C": 0.085, "D": 0.075, "W": 0.0265}
 
 
 def model_folder(name: str, seed: int = 11, std: float | None = None, norm_jitter: float = 0.1) -> Path:
