@@ -14,14 +14,16 @@ import torch
 from ..kernels import ops
 
 NUM_CUS = 256            # MI355X
-WORKGROUPS_WANTED = 4 * NUM_CUS
+# from decode steps at 4K keys, batch 1 to 64: two workgroups per compute unit and at most 16 runs
+# of keys were ahead of more of either (the partial results cost a merge that grows with them)
+WORKGROUPS_WANTED = 2 * NUM_CUS
 MIN_KEYS_PER_SPLIT = 128
-MAX_SPLITS = 64
+MAX_SPLITS = 16
 
 
 def choose_splits(requests: int, kv_head_tiles: int, max_keys: int) -> int:
     """How many runs to cut each request's keys into for the decode kernel: enough workgroups
-    to fill the GPU about four times over, never runs under 128 keys (reference's rule of the
+    to give every compute unit two workgroups, never runs under 128 keys (reference's rule of the
     same kind: src/dli/model/paged_attention.py:63-74)."""
     programs = max(1, requests * kv_head_tiles)
     want = -(-WORKGROUPS_WANTED // programs)
