@@ -663,7 +663,8 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
           tile_sum += p;
           pb[j][i] = (bf16_t)p;
         }
-        tile_sum = column_sum(tile_sum);
+        // l stays a per-lane partial sum (the lanes of a column share m, hence alpha): the
+        // four partial sums of a column are added once, after the last tile
         st[j].l = st[j].l * alpha[j] + tile_sum;
         st[j].m = m_new;
       }
@@ -689,9 +690,10 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
 
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
+    const float l_sum = column_sum(st[j].l);  // every lane takes part
     const int qi = q0 + j * 16 + col;
     if (qi >= q_len) continue;
-    const float inv = st[j].l > 0.f ? 1.f / st[j].l : 0.f;
+    const float inv = l_sum > 0.f ? 1.f / l_sum : 0.f;
     bf16_t* op = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * D + 4 * grp;
 #pragma unroll
     for (int c = 0; c < DCH; ++c) {
