@@ -14,11 +14,14 @@ import torch
 from ..kernels import ops
 
 NUM_CUS = 256            # MI355X
-# from decode steps at 4K keys, batch 1 to 64: two workgroups per compute unit and at most 16 runs
-# of keys were ahead of more of either (the partial results cost a merge that grows with them)
+# From decode steps at batch 1 to 64: two workgroups per compute unit, and at 4K keys at most 16
+# runs, were ahead of more of either (the partial results cost a merge that grows with them); a
+# request with 32K keys did better with 64 runs than with 16, so the limit grows with the keys.
 WORKGROUPS_WANTED = 2 * NUM_CUS
 MIN_KEYS_PER_SPLIT = 128
-MAX_SPLITS = 16
+FEW_SPLITS = 16          # the limit up to 8K keys
+KEYS_PER_EXTRA_SPLIT = 512
+MAX_SPLITS = 64
 
 
 def choose_splits(requests: int, kv_head_tiles: int, max_keys: int) -> int:
@@ -28,7 +31,8 @@ def choose_splits(requests: int, kv_head_tiles: int, max_keys: int) -> int:
     programs = max(1, requests * kv_head_tiles)
     want = -(-WORKGROUPS_WANTED // programs)
     most = max(1, max_keys // MIN_KEYS_PER_SPLIT)
-    return max(1, min(want, most, MAX_SPLITS))
+    limit = min(MAX_SPLITS, max(FEW_SPLITS, max_keys // KEYS_PER_EXTRA_SPLIT))
+    return max(1, min(want, most, limit))
 
 
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,

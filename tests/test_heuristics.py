@@ -4,7 +4,7 @@ src/dli/model/paged_attention.py:63-74, tests/unit/model/test_paged_attention_gp
 
 from __future__ import annotations
 
-from dli_amd.parts.attention_kernels import MAX_SPLITS, MIN_KEYS_PER_SPLIT, choose_splits
+from dli_amd.parts.attention_kernels import FEW_SPLITS, MAX_SPLITS, MIN_KEYS_PER_SPLIT, choose_splits
 
 
 def test_enough_programs_already_means_one_run():
@@ -14,6 +14,8 @@ def test_enough_programs_already_means_one_run():
 
 def test_one_request_with_a_long_context_is_cut():
     assert choose_splits(requests=1, kv_head_tiles=8, max_keys=4096) > 1
+    assert choose_splits(requests=1, kv_head_tiles=8, max_keys=4096) == FEW_SPLITS
+    assert choose_splits(requests=1, kv_head_tiles=8, max_keys=16384) == 32   # the limit grows with the keys
     assert choose_splits(requests=1, kv_head_tiles=8, max_keys=1 << 20) == MAX_SPLITS
 
 
