@@ -241,3 +241,25 @@ def test_step_function_refuses_entries_that_do_not_fit_the_cache_state():
     check(got, plain_logits("A", toks), "float32", "after refusals")
     mgr.free("r")
     mgr.check_invariants()
+
+
+@pytest.mark.parametrize("name,page,dtype", [("D", 16, "bfloat16"), ("A", 16, "float32"), ("B", 16, "bfloat16")])
+def test_long_context_in_portions_then_decoding(name, page, dtype):
+    """2,600 tokens: the prompt in portions of 512 (each attends to hundreds of cached keys in
+    many pages), then 40 tokens one by one, where the decode attention cuts the keys into
+    several runs and the block table is 160 pages wide."""
+    from dli_amd.trace import TraceSession
+
+    toks = prompts_for(name, [2600], seed=31)[0]
+    ref = plain_logits(name, toks)
+    core = make_core(name, dtype, num_pages=-(-len(toks) // page) + 1, page_size=page)
+    s = TraceSession(core)
+    head = len(toks) - 40
+    for pos in range(0, head, 512):
+        n = min(512, head - pos)
+        want = [0, n // 2, n - 1]
+        got = s.step([{"id": "r", "tokens": toks[pos:pos + n], "want": want}])
+        check(got, ref[[pos + w for w in want]], dtype, f"{name} portion at {pos}")
+    for i in range(head, len(toks)):
+        got = s.step([{"id": "r", "tokens": [toks[i]], "want": [0]}])
+        check(got, ref[i:i + 1], dtype, f"{name} decode at {i}")
