@@ -49,6 +49,33 @@ class StepEntry:
 
 
 @dataclass
+class HostBatch:
+    """A checked step laid out on the host: single-token entries first, then portions (``order``
+    maps the layout's entries to the caller's). What the device-side context is made from, by an
+    upload or by a copy into a captured graph's arrays."""
+
+    order: list                   # layout entry -> index in the caller's list
+    seq_ids: list
+    num_decode: int
+    token_ids: np.ndarray         # int64 [tokens]
+    positions: np.ndarray         # int32 [tokens]
+    q_start: np.ndarray           # int32 [entries + 1]
+    kv_len: np.ndarray            # int32 [entries]
+    state_slots: np.ndarray       # int32 [entries]
+    logit_rows: np.ndarray        # int32 [k], in the caller's order of entries and wants
+    slots: list                   # per group: int64 [tokens]
+    tables: list                  # per group: one int64 array of pages per entry
+
+    @property
+    def num_tokens(self) -> int:
+        return int(self.q_start[-1])
+
+    @property
+    def num_entries(self) -> int:
+        return len(self.order)
+
+
+@dataclass
 class GroupView:
     """Addresses of one cache group for this step."""
 

@@ -21,7 +21,7 @@ import torch
 from ..cache.manager import RELEASED, CacheManager, CopyOp
 from ..cache.store import CacheStore
 from ..parts.model import Model
-from .batch import GroupView, StepContext, StepEntry, upload
+from .batch import GroupView, HostBatch, StepContext, StepEntry, upload
 
 
 MAX_DECODE_STEPS = 8  # tokens per request that one graph replay may decode
@@ -66,6 +66,10 @@ class StepFunction:
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         """Check the entries against the cache manager and lay the batch out on the device."""
+        return self.upload_context(self.lay_out(entries))
+
+    def lay_out(self, entries: Sequence[StepEntry]) -> HostBatch:
+        """Check the entries against the cache manager and lay the batch out in host arrays."""
         mgr, ps = self.manager, self.manager.page_size
         seen = set()
         for e in entries:
@@ -122,7 +126,21 @@ class StepFunction:
             raise StepError(f"token id {bad} outside the vocabulary")
         logit_rows = np.asarray(
             [first_row[i] + int(w) for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
+        limit = self.store.num_pages
+        for g in range(n_groups):
+            if total and (int(slots[g].min()) < 0 or int(slots[g].max()) >= limit * ps):
+                raise StepError("a cache slot lies outside the pool, or in a page that the window has passed")
+            pages = np.concatenate(tables[g]) if tables[g] else np.zeros(0, np.int64)
+            if pages.size and (int(pages.min()) < RELEASED or int(pages.max()) >= limit):
+                raise StepError("a block table names a page outside the pool")
+        return HostBatch(order=order, seq_ids=[entries[i].seq_id for i in order], num_decode=num_decode,
+                         token_ids=token_ids, positions=positions, q_start=q_start, kv_len=kv_len,
+                         state_slots=state_slots, logit_rows=logit_rows, slots=slots, tables=tables)
 
+    def upload_context(self, batch: HostBatch) -> StepContext:
+        """The device-side context of a laid-out step (one copy from pinned memory)."""
+        n_groups, total, entries = self.manager.num_groups, batch.num_tokens, batch.order
+        tables, slots = batch.tables, batch.slots
         dev = self.rt.device
         # every integer array of the step goes to the device in one copy from pinned memory
         pending: list[np.ndarray] = []
@@ -138,21 +156,16 @@ class StepFunction:
             for k, t in enumerate(tables[g]):
                 host[k, :t.size] = t
             host[host == RELEASED] = 0  # pages that the window has passed: never read
-            limit = self.store.num_pages
-            if host.size and (int(host.min()) < 0 or int(host.max()) >= limit):
-                raise StepError("a block table names a page outside the pool")
-            if total and (int(slots[g].min()) < 0 or int(slots[g].max()) >= limit * ps):
-                raise StepError("a cache slot lies outside the pool, or in a page that the window has passed")
             group_arrays.append((to_dev(slots[g]), to_dev(host), width))
         named = {name: to_dev(a) for name, a in (
-            ("token_ids", token_ids), ("positions", positions), ("q_start", q_start), ("kv_len", kv_len),
-            ("state_slots", state_slots), ("logit_rows", logit_rows))}
+            ("token_ids", batch.token_ids), ("positions", batch.positions), ("q_start", batch.q_start),
+            ("kv_len", batch.kv_len), ("state_slots", batch.state_slots), ("logit_rows", batch.logit_rows))}
         views = upload(pending, dev)
         groups = [GroupView(views[s_], views[t_], width) for s_, t_, width in group_arrays]
         return StepContext(
-            device=dev, page_size=ps, num_tokens=total, num_entries=len(entries), num_decode=num_decode,
-            groups=groups, q_start_host=q_start, kv_len_host=kv_len, state_slots_host=state_slots,
-            seq_ids=[entries[i].seq_id for i in order], **{name: views[i] for name, i in named.items()})
+            device=dev, page_size=self.manager.page_size, num_tokens=total, num_entries=len(entries),
+            num_decode=batch.num_decode, groups=groups, q_start_host=batch.q_start, kv_len_host=batch.kv_len,
+            state_slots_host=batch.state_slots, seq_ids=batch.seq_ids, **{name: views[i] for name, i in named.items()})
 
     # ------------------------------------------------------------------ the step
 
@@ -196,8 +209,7 @@ class StepFunction:
             if use_graph_sampler:
                 tokens, logits = logits, None
         else:
-            ctx = self.build_context(entries)
-            logits = self.model.forward(ctx, self.caches)
+            logits = self.model.forward(self.build_context(entries), self.caches)
         for e in entries:
             self.manager.mark_computed(e.seq_id, e.start + len(e.tokens))
         self.steps_run += 1

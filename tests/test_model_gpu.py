@@ -30,11 +30,17 @@ MEAN_RTOL = 3e-2
 WORST: dict = {}  # largest error / bound seen per dtype (printed in the terminal summary)
 
 
+GRAPHS = False  # set by the tests that replay the same traces through captured graphs
+
+
 def make_core(name: str, dtype: str, num_pages: int, page_size: int):
     from dli_amd.engine.core import build_core
 
-    return build_core(model_folder(name), num_pages=num_pages, page_size=page_size, max_seqs=8,
+    core = build_core(model_folder(name), num_pages=num_pages, page_size=page_size, max_seqs=8,
                       dtype=dtype, enable_prefix_caching=False, watermark=0.0)
+    if GRAPHS:
+        core.step.enable_decode_graphs(8, num_pages * page_size)  # as serving does
+    return core
 
 
 def check(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str) -> None:
@@ -263,3 +269,26 @@ def test_long_context_in_portions_then_decoding(name, page, dtype):
     for i in range(head, len(toks)):
         got = s.step([{"id": "r", "tokens": [toks[i]], "want": [0]}])
         check(got, ref[i:i + 1], dtype, f"{name} decode at {i}")
+
+
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 16), ("D", 16)])
+def test_the_same_traces_with_decode_graphs_on(name, page, monkeypatch):
+    """Serving replays decode-only steps as HIP graphs of a padded, fixed shape. The traces above
+    once more with that switched on (as bin/trace_run has it): the logits must still be the plain
+    implementation's, and the single-token steps must really have gone through the graphs."""
+    import test_model_gpu as this
+
+    monkeypatch.setattr(this, "GRAPHS", True)
+    real = this.make_core
+    cores: list = []
+
+    def remembering(*a, **k):
+        cores.append(real(*a, **k))
+        return cores[-1]
+
+    monkeypatch.setattr(this, "make_core", remembering)
+    test_portions_of_changing_size(name, page, "bfloat16")
+    test_mixed_batches_with_pages_used_again(name, page, "bfloat16")
+    test_most_in_one_step_then_last_32_one_by_one(name, page, "bfloat16")
+    assert all(core.step.graphs is not None for core in cores)
+    assert sum(core.step.graphs.replays for core in cores) > 60
