@@ -138,14 +138,15 @@ class LLMEngine:
                   eviction_policy: str = "lru", enable_prefix_caching: bool = True,
                   eos_token_ids: Collection[int] = (), seed: int = 0, dtype: str = "bfloat16",
                   device: str = "cuda", cuda_graphs: bool = True,
-                  max_model_len: Optional[int] = None) -> "LLMEngine":
+                  max_model_len: Optional[int] = None, decode_weight_copy: bool = True) -> "LLMEngine":
         """Engine for a loaded model or a model folder.
 
         ``num_blocks`` pages of ``block_size`` tokens, or as many as ``kv_cache_gb`` GiB hold
         (default 1 GiB), as the reference's server takes them (src/dli/server/__main__.py:150-156).
         ``cuda_graphs``: replay decode-only steps through HIP graphs (the reference's option of
         this name replays CUDA graphs; here it is on by default and falls back to eager steps for
-        shapes whose decode path is not captured).
+        shapes whose decode path is not captured). ``decode_weight_copy`` (when ``model`` is a
+        folder): see :func:`load_model`.
         """
         from ..weights.loader import load_model
         from .core import build_core, pages_for_budget
@@ -153,7 +154,7 @@ class LLMEngine:
         if num_blocks is not None and kv_cache_gb is not None:
             raise ValueError("give num_blocks or kv_cache_gb, not both")
         if isinstance(model, (str, Path)):
-            model = load_model(model, dtype=dtype, device=device)
+            model = load_model(model, dtype=dtype, device=device, decode_weight_copy=decode_weight_copy)
         if num_blocks is None:
             gib = 1.0 if kv_cache_gb is None else kv_cache_gb
             num_blocks = pages_for_budget(model, block_size, int(gib * 2 ** 30))

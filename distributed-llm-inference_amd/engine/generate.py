@@ -36,7 +36,8 @@ def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
              dtype: str = "bfloat16", num_blocks: Optional[int] = None, kv_cache_gb: Optional[float] = None,
              block_size: int = 16, max_num_seqs: int = 64, max_num_batched_tokens: int = 512,
              enable_prefix_caching: bool = True, eos_token_ids: Collection[int] = (), seed: int = 0,
-             cuda_graphs: bool = True, device: str = "cuda", decode_steps: int = 1) -> list[list[int]]:
+             cuda_graphs: bool = True, device: str = "cuda", decode_steps: int = 1,
+             decode_weight_copy: bool = True) -> list[list[int]]:
     """Load ``model`` (a folder or a loaded model), run ``prompts`` to completion, return token ids.
     ``decode_steps`` > 1: decoding steps run that many tokens of every request on the device
     before the host looks (same tokens, fewer round trips)."""
@@ -45,5 +46,5 @@ def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
         config=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=max_num_batched_tokens,
                                decode_steps=decode_steps),
         enable_prefix_caching=enable_prefix_caching, eos_token_ids=eos_token_ids, seed=seed,
-        cuda_graphs=cuda_graphs, device=device)
+        cuda_graphs=cuda_graphs, device=device, decode_weight_copy=decode_weight_copy)
     return engine.generate(prompts, params)

@@ -265,3 +265,21 @@ def test_trace_run_program(tmp_path):
         input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": a, "want": [0]}], "end": []}) + "\n",
         capture_output=True, text=True, timeout=300)
     assert proc.returncode != 0 and "NoFreePagesError" in proc.stderr
+
+
+def test_generation_without_the_decode_copy_of_the_weights():
+    """The second, tile-ordered copy of the matrices is an option: without it the decode steps
+    read the row-major matrices (and run the rotation kernel), and greedy generation gives the
+    plain implementation's tokens either way."""
+    from dli_amd.engine.generate import generate
+    from dli_amd.sampling import SamplingParams
+
+    name = "D"
+    ps = prompts(name, [9, 40], seed=23)
+    want = [plain_greedy(name, p, 20) for p in ps]
+    for copy in (True, False):
+        got = generate(str(model_folder(name)), ps, SamplingParams(max_tokens=20), dtype="bfloat16", num_blocks=32,
+                       enable_prefix_caching=False, decode_weight_copy=copy)
+        for g, w, p in zip(got, want, ps):
+            assert len(g) == 20
+            assert_same_or_near_tie(name, p, g, w, margin=0.25)
