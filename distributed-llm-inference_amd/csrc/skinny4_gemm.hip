@@ -69,6 +69,27 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
   const int tile = blockIdx.x;
   const int n_tile = tile * 4 * OQ;  // first output feature of the tile
 
+  // EPI_RESIDUAL: the stream values that this thread will add to at the end are asked for now, so
+  // that the epilogue does not wait for a trip to memory of its own (same thread, same places)
+  union Pack4 {
+    short4v v;
+    bf16_t e[4];
+  } old;
+  old.v = short4v{0, 0, 0, 0};
+  if (EPI == EPI_RESIDUAL) {
+    const int t0 = threadIdx.x, p0 = t0 / 4, f0 = p0 / MG;
+    const int m0 = 4 * (p0 % MG) + t0 % 4, nb0 = n_tile + 4 * f0;
+    if (t0 < 4 * PAIRS && f0 < OQ && m0 < M && nb0 < N) {
+      const bf16_t* sp = stream + (int64_t)m0 * lds_ + nb0;
+      if (nb0 + 3 < N && lds_ % 4 == 0) {
+        old.v = *reinterpret_cast<const short4v*>(sp);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) old.e[i] = nb0 + i < N ? sp[i] : (bf16_t)0.f;
+      }
+    }
+  }
+
   // weight rows of this lane, one per quad (clamped at the matrix's end: computed and dropped)
   const bf16_t* wrow[FQ];
 #pragma unroll
@@ -286,18 +307,7 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
       bf16_t* op = EPI == EPI_RESIDUAL ? stream + (int64_t)m * lds_ + nb
                                        : reinterpret_cast<bf16_t*>(out) + (int64_t)m * ldo + nb;
       const bool vec = whole && (EPI == EPI_RESIDUAL ? lds_ : ldo) % 4 == 0;
-      union Pack4 {
-        short4v v;
-        bf16_t e[4];
-      } old, res;
-      if (EPI == EPI_RESIDUAL) {
-        if (vec) {
-          old.v = *reinterpret_cast<const short4v*>(op);
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) old.e[i] = nb + i < N ? op[i] : (bf16_t)0.f;
-        }
-      }
+      Pack4 res;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (EPI == EPI_STORE) {

@@ -135,6 +135,24 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
     return reinterpret_cast<const bf16x8*>(TILED ? base + (s / 4) * 2048 + q * 512 : base + s * 32 + q * 8);
   };
 
+  // EPI_RESIDUAL: the stream values that this lane will add to at the end (lane holds
+  // y[m = 16t + col][n = 16*tile + 4*grp + i]) are asked for now, so that the epilogue does not
+  // wait for a trip to memory of its own
+  float old_s[EPI == EPI_RESIDUAL ? NT : 1][EPI == EPI_RESIDUAL ? MT : 1][4];
+  if constexpr (EPI == EPI_RESIDUAL) {
+    if (ks == 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int n = (tile0 + j) * 16 + 4 * grp + i, m = t * 16 + col;
+            old_s[j][t][i] = m < M && n < N ? (float)stream[(int64_t)m * lds_ + n] : 0.f;
+          }
+    }
+  }
+
   const bf16_t* xrow[MT];
   bool live[MT];
   float rs[MT];
@@ -372,7 +390,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
             reinterpret_cast<bf16_t*>(out)[(int64_t)m * ldo + n] = (bf16_t)(sg * u);
           } else {  // EPI_RESIDUAL
             bf16_t* sp = stream + (int64_t)m * lds_ + n;
-            const bf16_t summed = (bf16_t)((float)*sp + (float)(bf16_t)y[0][i]);
+            const bf16_t summed = (bf16_t)(old_s[EPI == EPI_RESIDUAL ? j : 0][EPI == EPI_RESIDUAL ? t : 0][i] + (float)(bf16_t)y[0][i]);
             *sp = summed;
             sq += (float)summed * (float)summed;
           }
