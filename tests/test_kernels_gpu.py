@@ -276,6 +276,30 @@ def test_attention_finds_one_far_key_among_hundreds(ops):
                 assert (got[h] - want).abs().max() < 0.05, (e, row, h)
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 48, 64), (100, 301, 160), (512, 2048, 2048), (70, 1000, 96), (2048, 96, 4104)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_library_product_called_directly(ops, m, n, k, with_bias):
+    """The vendor library's bfloat16 product behind the engine's own binding (descriptors and the
+    chosen kernel cached per shape): against a float64 product, with the bias inside, with row
+    strides larger than the widths, and the second call of a shape like the first."""
+    torch.manual_seed(m + n + k)
+    xb = torch.randn(m, k + 8, device="cuda").bfloat16()
+    x = xb[:, :k]                     # rows contiguous, stride k + 8
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    bias = torch.randn(n, device="cuda").bfloat16() if with_bias else None
+    outb = torch.full((m, n + 16), 7.0, device="cuda", dtype=torch.bfloat16)
+    out = outb[:, :n]
+    if not ops.gemm_bf16(x, w, out, bias):
+        pytest.skip("the library offers no kernel for this shape: the engine then goes through torch.mm")
+    ref = x.cpu().double() @ w.cpu().double().T + (bias.cpu().double() if with_bias else 0.0)
+    bound = 2.0 ** -8 * ref.abs().max().item() + 1e-2
+    assert (out.cpu().double() - ref).abs().max() < bound
+    assert (outb[:, n:] == 7.0).all()   # nothing beyond the row's width is touched
+    again = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    assert ops.gemm_bf16(x, w, again, bias)
+    assert torch.equal(again, out)
+
+
 def _ref_norm_bf16(x, w, eps):
     """RMSNorm with the engine's rounding: cast(w * cast(x * r))."""
     xf = x.float()
