@@ -77,9 +77,22 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     # Requests admitted first decode a token a step while the others still prefill; the prompts are
     # shortened by that many steps so that no request outgrows `context` while the clock runs.
     budget = engine.scheduler.config.max_num_batched_tokens
-    per = max(d for d in (8, 4, 2, 1) if d <= max(1, decode_steps) and steps % d == 0)
-    warm = -(-warmup // per) * per   # whole engine steps
-    prompt_len = context - steps - warm - per - 1   # the last engine step reserves `per` slots ahead
+    # An engine step may decode several tokens of every request (SchedulerConfig.decode_steps): the
+    # clock runs over exactly `steps` decode steps of the model, cut into engine steps of 8, 4, 2 or 1
+    # (the largest first), and the warm-up runs every such size once so that its graph exists.
+    def chunks_of(n):
+        out = []
+        while n > 0:
+            out.append(max(d for d in (8, 4, 2, 1) if d <= min(n, max(1, decode_steps))))
+            n -= out[-1]
+        return out
+
+    timed = chunks_of(steps)
+    warm_chunks = sorted(set(timed), reverse=True)
+    while sum(warm_chunks) < warmup:
+        warm_chunks.append(timed[0])
+    warm, per = sum(warm_chunks), timed[0]
+    prompt_len = context - steps - warm - per - 1   # an engine step reserves up to `per` slots ahead
     prompt_len -= -(-batch * prompt_len // budget) + 1
     ids = []
     for i in range(batch):
@@ -92,29 +105,27 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
         engine.step()  # prefill, in portions under the token budget
         guard += 1
         assert guard < SLACK, "prefill took more steps than the pool has slack for"
-    # An engine step may decode several tokens of every request (SchedulerConfig.decode_steps): the
-    # clock runs over exactly `steps` decode steps of the model, however many engine steps that is.
-    def advance(n):
-        done = 0
-        while done < n:
-            out = engine.step()
-            assert len(out) == batch and len({len(o.new_token_ids) for o in out}) == 1
-            done += len(out[0].new_token_ids)
-        return done
-
     import dataclasses
 
-    engine.scheduler.config = dataclasses.replace(engine.scheduler.config, decode_steps=per)
-    advance(warm)
+    def advance(chunks):
+        done = 0
+        for n in chunks:
+            engine.scheduler.config = dataclasses.replace(engine.scheduler.config, decode_steps=n)
+            out = engine.step()
+            assert len(out) == batch and all(len(o.new_token_ids) == n for o in out)
+            done += n
+        return done
+
+    advance(warm_chunks)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    done = advance(steps)
+    done = advance(timed)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert done == steps and len(engine.scheduler.running) == batch
     for rid in ids:
         engine.abort(rid)
-    return batch * steps / dt, dt / steps * 1e3
+    return batch * steps / dt, dt / steps * 1e3, per
 
 
 def prefill_run(engine, cfg, tokens, repeats=3):
@@ -166,7 +177,7 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--decode-steps", type=int, default=8,
                     help="decode steps that one engine step runs on the device before the host looks "
-                         "(reduced to a divisor of --steps)")
+                         "(the timed steps are cut into engine steps of at most this many)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run only the 2,048-token prefill steps (for profiling) and print their time")
@@ -191,7 +202,8 @@ def main() -> int:
         t = prefill_run(engine, cfg, 2048, repeats=args.steps)
         print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": 2048, "tok_s": round(2048 / t, 1)}))
         return 0
-    tok_s, ms = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup, args.decode_steps)
+    tok_s, ms, per_engine_step = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup,
+                                            args.decode_steps)
     achieved = decode_bytes(cfg, args.batch, args.context, itemsize) / (ms * 1e-3) / 1e9
     line = {
         "metric": f"decode tok/s at batch {args.batch}, {args.shape} shape",
@@ -205,7 +217,7 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "rms_norm_eps": cfg.rms_norm_eps, "rope": f"{cfg.rope.rope_type} theta {cfg.rope.theta:g} factor {cfg.rope.factor:g}",
             "tied_head": cfg.tie_word_embeddings, "kv_block_size": args.block_size, "prefill_tokens": 2048,
-            "sampling": "greedy", "decode_steps_per_engine_step": engine.scheduler.config.decode_steps,
+            "sampling": "greedy", "decode_steps_per_engine_step": per_engine_step,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
