@@ -144,24 +144,20 @@ class GQAttention(Mixer):
             angles = ctx.rope_angles(self.position.rotary_table()[0], qkv.dtype)
             ops.skinny_gemm_qkv_rope(stream.x, self.w_qkv_rope, qkv, angles, grp.slots, cache.k_pages, cache.v_pages,
                                      nh, bias=self.b_qkv_rope, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
-            out = self.rt.empty(n, nh * d)
-            paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
-            stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
-                                         stream=stream.x, bias=self.b_o)
-            return
-        ops.skinny_gemm(stream.x, self.w_qkv, w_tiled=self.w_qkv_tiled, epilogue=ops.SKINNY_STORE, out=qkv,
-                        bias=self.b_qkv, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
-        table = self.position.rotary_table()
-        if table is None:
-            q_view = qkv[:, :nh * d].view(n, nh, d)
-            k_view = qkv[:, nh * d:(nh + nkv) * d].view(n, nkv, d) if nkv else None
-            self.position.apply(q_view, k_view, ctx.positions)
-            inv_freq, rotary_dim = None, 0
         else:
-            inv_freq, rotary_dim = table
+            ops.skinny_gemm(stream.x, self.w_qkv, w_tiled=self.w_qkv_tiled, epilogue=ops.SKINNY_STORE, out=qkv,
+                            bias=self.b_qkv, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+            table = self.position.rotary_table()
+            if table is None:
+                q_view = qkv[:, :nh * d].view(n, nh, d)
+                k_view = qkv[:, nh * d:(nh + nkv) * d].view(n, nkv, d) if nkv else None
+                self.position.apply(q_view, k_view, ctx.positions)
+                inv_freq, rotary_dim = None, 0
+            else:
+                inv_freq, rotary_dim = table
+            ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
+                              cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         out = self.rt.empty(n, nh * d)
-        ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
-                          cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
                                      stream=stream.x, bias=self.b_o)
