@@ -447,11 +447,21 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   constexpr int K_ELEMS = 32 * KPAD, TILE_ELEMS = K_ELEMS + D * VPAD;
   __shared__ __attribute__((aligned(16))) bf16_t lds[3][TILE_ELEMS];  // K rows, then V^T rows
 
-  const int e = tile_entry[blockIdx.x];
+  // Workgroups are dealt to the eight XCDs in turn by their linear index, and each XCD has an L2
+  // of its own: the tiles of one kv head are therefore given to one XCD (when the heads divide
+  // evenly), so that a head's keys and values are fetched into one L2 instead of all eight.
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (gridDim.y % 8 == 0) {
+    const int linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int slot = linear / 8;
+    by = linear % 8 + 8 * (slot / (int)gridDim.x);
+    bx = slot % (int)gridDim.x;
+  }
+  const int e = tile_entry[bx];
   const int tok0 = q_start[e];
   const int q_len = q_start[e + 1] - tok0;
   const int tile_rows = (4 / heads_per_wg) * 32;
-  const int q0_first = tile_q0[blockIdx.x];
+  const int q0_first = tile_q0[bx];
   int q0_second = -1;
   if (PAIR) {
     const int b = q0_first / tile_rows, mirror = (q_len + tile_rows - 1) / tile_rows - 1 - b;
@@ -460,11 +470,11 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   }
   const int group = q_heads / kv_heads;
   const int wg_per_kv = group / heads_per_wg;
-  const int kvh = blockIdx.y / wg_per_kv;
+  const int kvh = by / wg_per_kv;
   const int lane = threadIdx.x % DLI_WAVE, wave = (threadIdx.x / DLI_WAVE) % 4;
   const int set = threadIdx.x / 256;  // which of the workgroup's two tiles
   const int col = lane % 16, grp = lane / 16;
-  const int head = kvh * group + (blockIdx.y % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
+  const int head = kvh * group + (by % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
   const int n_keys = kv_len[e];
   const int first_pos = n_keys - q_len;
   const int set_q0 = set == 0 ? q0_first : q0_second;
@@ -786,10 +796,12 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (hw > 0) {
     const dim3 sgrid(tiles, q_heads / hw);
-    // Mirror tiles are paired (pair_tiles 1, or -1 and the launch large enough) while that still
-    // leaves every compute unit a workgroup. The tile list has to hold all tiles of a request.
-    const bool pair = pair_tiles >= 0 ? pair_tiles != 0
-                                      : (int64_t)tiles * (q_heads / hw) >= 2 * (int64_t)dli_compute_units();
+    // Mirror tiles are paired (pair_tiles 1, or -1 and a launch of one to eight workgroups per
+    // compute unit: with fewer, pairing leaves units idle; with more, the queue of workgroups
+    // evens the causal triangle out by itself and single tiles were faster, measured at 16K
+    // tokens). The tile list has to hold all tiles of a request.
+    const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
+    const bool pair = pair_tiles >= 0 ? pair_tiles != 0 : (launch >= units && launch <= 8 * units);
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \
     if (pair)                                                                                     \
