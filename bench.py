@@ -47,7 +47,7 @@ SMOLLM2_1_7B = {
 SHAPES = {"Llama-3.2-1B": LLAMA_3_2_1B, "Llama-3.2-3B": LLAMA_3_2_3B, "SmolLM2-1.7B": SMOLLM2_1_7B}
 
 
-def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1):
+def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, num_pages=None):
     import torch
 
     from dli_amd.engine import LLMEngine, SchedulerConfig
@@ -59,7 +59,7 @@ def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1):
     model, cfg = build_model(raw, rt)
     model.config = cfg
     fill_random_on_device(model, seed=0, std=0.02)
-    pages = batch * (-(-(context + SLACK) // block_size) + 1) + 8
+    pages = num_pages or batch * (-(-(context + SLACK) // block_size) + 1) + 8
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=False,
         config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
@@ -149,6 +149,39 @@ def prefill_run(engine, cfg, tokens, repeats=3):
     return best
 
 
+def serving_run(raw, dtype, requests, budget, decode_steps, rounds=2):
+    """Continuous batching of ``requests`` requests with prompts of 128 to 2,048 random tokens and 256
+    generated tokens each under a budget of ``budget`` tokens a step (the workload that the baseline
+    names for the 3B sizes). The first round also captures the decode graphs; the last one is reported."""
+    import random
+
+    import torch
+
+    from dli_amd.sampling import SamplingParams
+
+    pages = requests * (-(-(2048 + 256) // 16) + 1) + 8
+    engine, cfg = make_engine(raw, dtype, requests, 2048 + 256 - SLACK, 16, budget, decode_steps, num_pages=pages)
+    rng = random.Random(0)
+    result = {}
+    for rnd in range(rounds):
+        lens = [rng.randint(128, 2048) for _ in range(requests)]
+        for i, n in enumerate(lens):
+            engine.add_request(f"s{rnd}-{i}", [rng.randrange(cfg.vocab_size) for _ in range(n)],
+                               SamplingParams(max_tokens=256, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = generated = 0
+        while engine.has_unfinished():
+            generated += sum(len(o.new_token_ids) for o in engine.step())
+            steps += 1
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        result = {"requests": requests, "prompt_tokens": sum(lens), "generated_tokens": generated,
+                  "seconds": round(dt, 4), "engine_steps": steps, "generated_tok_s": round(generated / dt, 1),
+                  "total_tok_s": round((sum(lens) + generated) / dt, 1)}
+    return result, cfg
+
+
 def prefill_flops(cfg, tokens):
     h, d = cfg.hidden_size, cfg.head_dim
     q, kv = cfg.num_heads * d, cfg.num_kv_heads * d
@@ -179,6 +212,10 @@ def main() -> int:
                     help="decode steps that one engine step runs on the device before the host looks "
                          "(the timed steps are cut into engine steps of at most this many)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
+    ap.add_argument("--serving", action="store_true",
+                    help="instead of the decode steps: 64 requests with prompts of 128 to 2,048 tokens and 256 "
+                         "generated tokens each, batched continuously under --budget tokens a step")
+    ap.add_argument("--budget", type=int, default=2048, help="tokens a step for --serving")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run only the 2,048-token prefill steps (for profiling) and print their time")
     args = ap.parse_args()
@@ -194,6 +231,16 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
+    if args.serving:
+        got, cfg = serving_run(raw, args.dtype, 64, args.budget, min(args.decode_steps, 8))
+        print(json.dumps({
+            "metric": f"continuous batching, {args.shape} shape: generated tok/s", "value": got["generated_tok_s"],
+            "unit": "tok/s", "n_gpus": 1, "higher_is_better": True, "dtype": short,
+            "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
+            "config": {"model": f"{args.shape} shape", "layers": cfg.num_layers, "budget_tokens_per_step": args.budget,
+                       "prompt_lengths": "uniform 128..2048", "max_tokens": 256, "kv_block_size": 16,
+                       "decode_steps_per_engine_step": min(args.decode_steps, 8)}, **got}))
+        return 0
     max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
     engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=8192,
                               decode_steps=args.decode_steps)
