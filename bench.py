@@ -47,7 +47,8 @@ SMOLLM2_1_7B = {
 SHAPES = {"Llama-3.2-1B": LLAMA_3_2_1B, "Llama-3.2-3B": LLAMA_3_2_3B, "SmolLM2-1.7B": SMOLLM2_1_7B}
 
 
-def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, num_pages=None):
+def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, num_pages=None,
+                prefix_caching=False):
     import torch
 
     from dli_amd.engine import LLMEngine, SchedulerConfig
@@ -61,7 +62,7 @@ def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, 
     fill_random_on_device(model, seed=0, std=0.02)
     pages = num_pages or batch * (-(-(context + SLACK) // block_size) + 1) + 8
     engine = LLMEngine.for_model(
-        model, num_blocks=pages, block_size=block_size, enable_prefix_caching=False,
+        model, num_blocks=pages, block_size=block_size, enable_prefix_caching=prefix_caching,
         config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
                                decode_steps=decode_steps))
     return engine, cfg
@@ -149,25 +150,33 @@ def prefill_run(engine, cfg, tokens, repeats=3):
     return best
 
 
-def serving_run(raw, dtype, requests, budget, decode_steps, rounds=2):
-    """Continuous batching of ``requests`` requests with prompts of 128 to 2,048 random tokens and 256
-    generated tokens each under a budget of ``budget`` tokens a step (the workload that the baseline
-    names for the 3B sizes). The first round also captures the decode graphs; the last one is reported."""
+def serving_run(raw, dtype, workload, budget, decode_steps, rounds=2):
+    """Requests batched continuously under a budget of ``budget`` tokens a step. ``mixed``: 64 requests
+    with prompts of 128 to 2,048 random tokens and 256 generated tokens each (the workload that the
+    baseline names for the 3B sizes). ``shared-prefix``: 32 requests that share a prefix of 1,024 tokens
+    and go on with 64 to 512 tokens of their own, 128 generated tokens each, with reuse of cached pages
+    on (the one it names for SmolLM2-1.7B). The first round also captures the decode graphs (and, for
+    the shared prefix, fills the cache with it); the last one is reported."""
     import random
 
     import torch
 
     from dli_amd.sampling import SamplingParams
 
-    pages = requests * (-(-(2048 + 256) // 16) + 1) + 8
-    engine, cfg = make_engine(raw, dtype, requests, 2048 + 256 - SLACK, 16, budget, decode_steps, num_pages=pages)
+    shared = workload == "shared-prefix"
+    requests, longest, out_tokens = (32, 1024 + 512, 128) if shared else (64, 2048, 256)
+    pages = requests * (-(-(longest + out_tokens) // 16) + 1) + 8
+    engine, cfg = make_engine(raw, dtype, requests, longest + out_tokens - SLACK, 16, budget, decode_steps,
+                              num_pages=pages, prefix_caching=shared)
     rng = random.Random(0)
+    prefix = [rng.randrange(cfg.vocab_size) for _ in range(1024)] if shared else []
     result = {}
     for rnd in range(rounds):
-        lens = [rng.randint(128, 2048) for _ in range(requests)]
+        lens = [rng.randint(64, 512) if shared else rng.randint(128, 2048) for _ in range(requests)]
+        before = engine.manager.stats()
         for i, n in enumerate(lens):
-            engine.add_request(f"s{rnd}-{i}", [rng.randrange(cfg.vocab_size) for _ in range(n)],
-                               SamplingParams(max_tokens=256, ignore_eos=True))
+            engine.add_request(f"s{rnd}-{i}", prefix + [rng.randrange(cfg.vocab_size) for _ in range(n)],
+                               SamplingParams(max_tokens=out_tokens, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         steps = generated = 0
@@ -176,9 +185,12 @@ def serving_run(raw, dtype, requests, budget, decode_steps, rounds=2):
             steps += 1
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        result = {"requests": requests, "prompt_tokens": sum(lens), "generated_tokens": generated,
+        after = engine.manager.stats()
+        prompt_tokens = sum(lens) + len(prefix) * requests
+        result = {"requests": requests, "prompt_tokens": prompt_tokens, "generated_tokens": generated,
+                  "prompt_tokens_from_cache": after.prompt_tokens_hit - before.prompt_tokens_hit,
                   "seconds": round(dt, 4), "engine_steps": steps, "generated_tok_s": round(generated / dt, 1),
-                  "total_tok_s": round((sum(lens) + generated) / dt, 1)}
+                  "total_tok_s": round((prompt_tokens + generated) / dt, 1)}
     return result, cfg
 
 
@@ -212,9 +224,11 @@ def main() -> int:
                     help="decode steps that one engine step runs on the device before the host looks "
                          "(the timed steps are cut into engine steps of at most this many)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
-    ap.add_argument("--serving", action="store_true",
-                    help="instead of the decode steps: 64 requests with prompts of 128 to 2,048 tokens and 256 "
-                         "generated tokens each, batched continuously under --budget tokens a step")
+    ap.add_argument("--serving", nargs="?", const="mixed", default=None, choices=["mixed", "shared-prefix"],
+                    help="instead of the decode steps, requests batched continuously under --budget tokens a "
+                         "step. mixed: 64 requests, prompts of 128 to 2,048 tokens, 256 generated tokens each; "
+                         "shared-prefix: 32 requests that share 1,024 tokens and add 64 to 512 of their own, "
+                         "128 generated tokens each, with reuse of cached pages")
     ap.add_argument("--budget", type=int, default=2048, help="tokens a step for --serving")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run only the 2,048-token prefill steps (for profiling) and print their time")
@@ -232,13 +246,14 @@ def main() -> int:
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
     if args.serving:
-        got, cfg = serving_run(raw, args.dtype, 64, args.budget, min(args.decode_steps, 8))
+        got, cfg = serving_run(raw, args.dtype, args.serving, args.budget, min(args.decode_steps, 8))
         print(json.dumps({
-            "metric": f"continuous batching, {args.shape} shape: generated tok/s", "value": got["generated_tok_s"],
+            "metric": f"continuous batching ({args.serving}), {args.shape} shape: generated tok/s",
+            "value": got["generated_tok_s"],
             "unit": "tok/s", "n_gpus": 1, "higher_is_better": True, "dtype": short,
             "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
             "config": {"model": f"{args.shape} shape", "layers": cfg.num_layers, "budget_tokens_per_step": args.budget,
-                       "prompt_lengths": "uniform 128..2048", "max_tokens": 256, "kv_block_size": 16,
+                       "workload": args.serving, "kv_block_size": 16,
                        "decode_steps_per_engine_step": min(args.decode_steps, 8)}, **got}))
         return 0
     max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
