@@ -315,6 +315,8 @@ def skinny_gemm_shape(n: int, k: int, tiled: bool = False) -> int:
     activations are read once per 8 tiles. From cold-cache timings on MI355X."""
     tiles = -(-n // 16)
     if tiled:          # fewer tiles than compute units: 8 k-waves; else 4 k-waves on two tiles each
+        if tiles >= 768 and k >= 3072:
+            return 2   # a vocabulary with long rows: no split of k
         return 1 if tiles <= 256 else 4
     if tiles >= 768:   # a vocabulary
         return 3
@@ -367,7 +369,9 @@ def skinny_gemm_plan(rows: int, n: int, k: int, epilogue: int, device: torch.dev
     product has few features.
     """
     if blocks4 is None and rows <= 16 and k % 8 == 0:
-        deep = k >= 4096 and n <= 4096   # long rows, few features: many waves on narrow tiles
+        # long rows and so few features that tiles of 16 would leave half the compute units idle
+        # (2048 at the 1B sizes; not 3072 at the 3B sizes, where the tile kernel is ahead from 4 rows on)
+        deep = k >= 4096 and -(-n // 16) * 2 <= _units(device)
         if rows <= 4:
             out_feats = n * (2 if epilogue == SKINNY_SWIGLU else 1)
             few = out_feats <= 16 * _units(device)

@@ -473,6 +473,7 @@ def test_tiled_weights_are_refused_where_they_do_not_fit(ops):
     assert not ops.tiled_weights_help(48, 128, ops.SKINNY_SWIGLU, w.device)   # halves of 24 features
     assert ops.tiled_weights_help(2048, 2048, ops.SKINNY_RESIDUAL, w.device)
     assert not ops.tiled_weights_help(2048, 8192, ops.SKINNY_RESIDUAL, w.device)  # the block kernel's at every size
+    assert ops.tiled_weights_help(3072, 8192, ops.SKINNY_RESIDUAL, w.device)      # enough tiles for the tile kernel
 
 
 @pytest.mark.parametrize("m", [1, 3, 4, 5, 8, 9, 16])
