@@ -315,7 +315,7 @@ def skinny_gemm_shape(n: int, k: int, tiled: bool = False) -> int:
     activations are read once per 8 tiles. From cold-cache timings on MI355X."""
     tiles = -(-n // 16)
     if tiled:          # fewer tiles than compute units: 8 k-waves; else 4 k-waves on two tiles each
-        if tiles >= 768 and k >= 3072:
+        if tiles >= 2048 and k >= 3072:
             return 2   # a vocabulary with long rows: no split of k
         return 1 if tiles <= 256 else 4
     if tiles >= 768:   # a vocabulary
