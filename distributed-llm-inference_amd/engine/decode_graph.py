@@ -25,10 +25,10 @@ from typing import Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache.manager import RELEASED
 from ..kernels import ops
 from ..parts.attention_kernels import choose_splits
 from .batch import GroupView, StepContext, StepEntry
+from .table_rows import TableRows
 
 
 def _bucket(n: int) -> int:
@@ -47,7 +47,7 @@ class _Captured:
     logits: torch.Tensor
     views: dict             # name -> numpy view into host
     width: int              # block-table entries per row
-    rows: list              # per row: (request, pages already written into its table row)
+    rows: TableRows         # what the block-table rows hold, so that a replay patches them
     tokens_host: Optional[torch.Tensor] = None  # pinned int32 [steps * b]: sampled tokens (sampling graphs)
 
 
@@ -172,7 +172,7 @@ class DecodeGraphs:
         finally:
             if collecting:
                 gc.enable()
-        return _Captured(graph, ctx, host, dev, logits, views, width, [None] * b, tokens_host)
+        return _Captured(graph, ctx, host, dev, logits, views, width, TableRows(b, width, self.n_groups), tokens_host)
 
     # ------------------------------------------------------------------ replay
 
@@ -217,41 +217,10 @@ class DecodeGraphs:
         for i, e in enumerate(entries):
             if e.want:
                 rows.extend(i for _ in e.want)
-        lengths = [[0] * self.n_groups for _ in range(n)]
         for g in range(self.n_groups):
-            full = mgr.groups[g].kind == "full"
-            flat = v[f"tables{g}"]
-            slots, last_at, last_page = [], [], []
-            for i, e in enumerate(entries):
-                table = mgr.table_ref(e.seq_id, g)
-                page = table[e.start // ps]
-                if not 0 <= page < limit:
-                    raise ValueError("a block table names a page outside the pool")
-                slots.append(page * ps + e.start % ps)
-                count = len(table)
-                lengths[i][g] = count
-                known = cap.rows[i]
-                if full and known is not None and known[0] == e.seq_id:
-                    # A request that keeps its row only appends pages, and only the page it writes
-                    # next may have been swapped by a copy-on-write: rewrite from whichever of the
-                    # two comes first (a few entries, gathered for one assignment).
-                    lo = max(0, min(known[1][g] - 1, e.start // ps))
-                    for at in range(lo, count):
-                        last_at.append(i * width + at)
-                        last_page.append(table[at])
-                    continue
-                row = flat[i * width:(i + 1) * width]
-                row[:count] = table
-                if not full:
-                    np.maximum(row, 0, out=row)  # pages that the window has passed are never read
+            slots = cap.rows.fill(mgr, entries, g, v[f"tables{g}"], limit)
             v[f"slots{g}"][:n] = slots
             v[f"slots{g}"][n:] = -1
-            if last_at:
-                flat[last_at] = last_page
-        for i, e in enumerate(entries):
-            cap.rows[i] = (e.seq_id, lengths[i])
-        for i in range(n, b):
-            cap.rows[i] = None
         if sampled:
             temp, top_p = v["temperature"].view(np.float32), v["top_p"].view(np.float32)
             seeds, counters = v["seeds"].view(np.int64), v["counters"].view(np.int64)

@@ -206,7 +206,33 @@ def test_shared_prefix_sampling_preemption_config_b():
     assert all(len(o) == 32 for o in alone) and len({tuple(o) for o in alone}) > 1
 
 
-def test_seeded_request_is_the_same_alone_and_in_a_busy_batch_bf16():
+def assert_same_or_near_cell_edge(name, prompt, a, b, params, seed, tol):
+    """Two runs of one seeded request: the same tokens, or at the first difference the request's
+    uniform draw (host Philox) lies within ``tol`` of the edge between the two tokens' cells of the
+    plain cumulative distribution (then rounding decides and the runs part there)."""
+    from test_sampling_gpu import philox_uniform
+
+    cfg, w = P.load_folder(model_folder(name))
+    for j, (x, y) in enumerate(zip(a, b)):
+        if x == y:
+            continue
+        logits = P.forward_logits(w, cfg, list(prompt) + list(a[:j]))[-1]
+        probs = P.sampling_probabilities(logits, params.temperature, params.top_k, params.top_p)
+        cdf = torch.cumsum(probs, 0)
+        u = philox_uniform(seed, j)
+        for tok in (x, y):
+            lo, hi = float(cdf[tok] - probs[tok]), float(cdf[tok])
+            assert lo - tol <= u <= hi + tol, f"draw {j}: token {tok} has cell [{lo}, {hi}], the draw is {u}"
+        return
+    assert len(a) == len(b)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_seeded_request_is_the_same_alone_and_in_a_busy_batch(dtype):
+    """The reference's tests/unit/model/test_engine_tiny.py:89-107, in both precisions. bfloat16
+    runs the matrix-core kernels, graph replay and the sampler inside the graph; there the kernels
+    chosen depend on the batch, so logits agree to rounding and a draw at the very edge of a
+    token's cell may fall to the neighbour."""
     from dli_amd.engine import LLMEngine, SchedulerConfig
     from dli_amd.sampling import SamplingParams
 
@@ -215,12 +241,54 @@ def test_seeded_request_is_the_same_alone_and_in_a_busy_batch_bf16():
     sp = SamplingParams(max_tokens=20, temperature=0.9, top_k=40, top_p=0.95, seed=7)
 
     def run(which):
-        eng = LLMEngine.for_model(str(model_folder(name)), dtype="float32", num_blocks=64, block_size=16,
+        eng = LLMEngine.for_model(str(model_folder(name)), dtype=dtype, num_blocks=64, block_size=16,
                                   config=SchedulerConfig(max_num_seqs=8, max_num_batched_tokens=64))
         pars = [sp if i == 2 else SamplingParams(max_tokens=25, temperature=1.0, seed=50 + i) for i in which]
-        return eng.generate([ps[i] for i in which], pars)[which.index(2)]
+        out = eng.generate([ps[i] for i in which], pars)[which.index(2)]
+        if dtype == "bfloat16":
+            assert eng.core.step.graphs is not None and eng.core.step.graphs.replays > 0
+        return out
 
-    assert run([2]) == run([0, 1, 2, 3, 4]) == run([2, 4])
+    alone, busy, pair = run([2]), run([0, 1, 2, 3, 4]), run([2, 4])
+    if dtype == "float32":
+        assert alone == busy == pair
+    else:
+        assert len(alone) == 20
+        assert_same_or_near_cell_edge(name, ps[2], alone, busy, sp, 7, 0.02)
+        assert_same_or_near_cell_edge(name, ps[2], alone, pair, sp, 7, 0.02)
+
+
+@pytest.mark.parametrize("name", ["A", "D"])
+@pytest.mark.parametrize("reuse", [False, True])
+def test_graph_replay_under_preemption_bf16(name, reuse):
+    """bfloat16 with graph replay in a pool so small that requests lose their pages and recompute:
+    a request that comes back under its id holds other pages, and the block-table row that the
+    captured graph kept for it must show them (the reference's
+    tests/unit/engine/test_preemption.py:32-45 with tests/unit/model/test_cuda_graph_gpu.py:129-150).
+    With content reuse on, the pool is small enough for idle cached pages to be reclaimed. Each
+    request's tokens are the plain implementation's, up to near-ties."""
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    ps = prompts(name, [40, 23, 55, 31, 47, 18, 60, 12], seed=37)
+    eng = LLMEngine.for_model(str(model_folder(name)), dtype="bfloat16", num_blocks=14, block_size=16,
+                              enable_prefix_caching=reuse,
+                              config=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=64))
+    assert eng.core.step.graphs is not None
+    reqs = [eng.add_request(f"r{i}", p, SamplingParams(max_tokens=44)) for i, p in enumerate(ps)]
+    while eng.has_unfinished():
+        eng.step()
+        eng.manager.check_invariants()
+    assert eng.core.step.graphs.replays > 0
+    assert sum(s.num_preempted for s in eng.stats.steps) > 0
+    assert max(r.num_preemptions for r in reqs) > 0
+    if reuse:
+        assert eng.manager.stats().evictions > 0
+    for p, r in zip(ps, reqs):
+        assert len(r.output_ids) == 44
+        assert_same_or_near_tie(name, p, r.output_ids, plain_greedy(name, p, 44), margin=0.25)
+    eng.manager.reset_prefix_cache()
+    assert eng.manager.stats().used_pages == 0
 
 
 def test_trace_run_program(tmp_path):
