@@ -259,6 +259,53 @@ def test_seeded_request_is_the_same_alone_and_in_a_busy_batch(dtype):
 
 
 @pytest.mark.parametrize("name", ["A", "D"])
+def test_graph_row_of_a_request_that_lost_its_pages_and_came_back(name):
+    """The schedule in which a captured graph's block-table row goes stale if it is keyed by the
+    request's id: B decodes in row 1 of the two-request graph and gives back its pages; C takes
+    them and writes its own keys there; A decodes alone meanwhile (the one-request graph, so the
+    other graph's row 1 is not touched); B comes back under its id with other pages and decodes
+    beside A in the two-request graph again. Every logit row is the plain implementation's."""
+    from test_model_gpu import check, plain_logits
+    from dli_amd.engine.core import build_core
+    from dli_amd.trace import TraceSession
+
+    page = 16
+    a, b, c, d = prompts(name, [120, 100, 80, 96], seed=43)
+    core = build_core(model_folder(name), num_pages=15, page_size=page, max_seqs=4, dtype="bfloat16",
+                      enable_prefix_caching=False, watermark=0.0)
+    core.step.enable_decode_graphs(4, 15 * page)
+    s = TraceSession(core)
+    ref_a, ref_b = plain_logits(name, a), plain_logits(name, b)
+    fed_a, fed_b = 50, 70
+    s.step([{"id": "A", "tokens": a[:fed_a], "want": []}])
+    s.step([{"id": "B", "tokens": b[:fed_b], "want": []}])
+
+    def decode_both(steps):
+        nonlocal fed_a, fed_b
+        for _ in range(steps):
+            got = s.step([{"id": "A", "tokens": [a[fed_a]], "want": [0]}, {"id": "B", "tokens": [b[fed_b]], "want": [0]}])
+            check(got, torch.stack([ref_a[fed_a], ref_b[fed_b]]), "bfloat16", f"{name} A at {fed_a}, B at {fed_b}")
+            fed_a, fed_b = fed_a + 1, fed_b + 1
+
+    decode_both(4)
+    replays = core.step.graphs.replays
+    assert replays == 4
+    old_pages = core.manager.block_table("B")
+    s.step([{"id": "D", "tokens": d, "want": []}], end=["B"])  # D fills the pool; B gives back its pages
+    s.step([{"id": "C", "tokens": c, "want": []}], end=["D"])  # C's keys now lie in the pages that were B's
+    assert set(core.manager.block_table("C")) == set(old_pages)
+    for _ in range(3):                                        # A alone: the one-request graph
+        got = s.step([{"id": "A", "tokens": [a[fed_a]], "want": [0]}])
+        check(got, ref_a[fed_a:fed_a + 1], "bfloat16", f"{name} A alone at {fed_a}")
+        fed_a += 1
+    s.step([{"id": "B", "tokens": b[:fed_b], "want": []}])   # B again, recomputed, in other pages
+    assert core.manager.block_table("B")[:4] != old_pages[:4]
+    decode_both(6)
+    assert core.step.graphs.replays == replays + 3 + 6
+    core.manager.check_invariants()
+
+
+@pytest.mark.parametrize("name", ["A", "D"])
 @pytest.mark.parametrize("reuse", [False, True])
 def test_graph_replay_under_preemption_bf16(name, reuse):
     """bfloat16 with graph replay in a pool so small that requests lose their pages and recompute:
