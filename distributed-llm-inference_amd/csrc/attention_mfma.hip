@@ -25,6 +25,7 @@
 // P is rounded to bfloat16 for the second product while the running sum keeps the unrounded
 // values (as the reference's kernel does: src/dli/model/paged_attention.py:128-168).
 #include "common.h"
+#include "no_alloc.h"
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
@@ -779,6 +780,58 @@ extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const 
 #undef MERGE
   }
   return dli_launch_status();
+}
+
+// ---------------------------------------------------------------- decode without an allocation
+// The split-key partial results of dli_attention_decode_bf16_static live in this array instead
+// of a buffer that the caller brings. Each GPU holds its own copy at its own address; host code
+// never uses the array's name as an address, only what hipGetSymbolAddress returned for the
+// current device.
+static __device__ __align__(256) float scratch[DLI_STATIC_SCRATCH_FLOATS];
+
+// The array's address on the current device (asked once per device), or nullptr.
+static float* static_scratch() {
+  static float* of_device[64] = {nullptr};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  if (of_device[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return nullptr;
+    of_device[dev] = static_cast<float*>(ptr);
+  }
+  return of_device[dev];
+}
+
+extern "C" int64_t dli_attention_decode_static_floats(int requests, int q_heads, int head_dim, int splits) {
+  if (requests <= 0 || q_heads <= 0 || head_dim <= 0 || splits <= 1) return 0;
+  const int64_t slots = (int64_t)requests * q_heads * splits;
+  return (slots * head_dim + 63) / 64 * 64 + slots * 2;
+}
+
+extern "C" int dli_attention_decode_bf16_static(const void* q, int64_t q_stride, const void* k_pages,
+                                                const void* v_pages, void* out, int64_t out_stride,
+                                                const int* kv_len, const int* block_tables,
+                                                int table_stride, int requests, int q_heads,
+                                                int kv_heads, int head_dim, int page_size, float scale,
+                                                int window, int splits, hipStream_t stream) {
+  if (requests <= 0) return DLI_OK;
+  if (q_heads <= 0 || head_dim <= 0 || splits < 1) return DLI_ERR_ARGUMENT;
+  float* part_o = nullptr;
+  float* part_ml = nullptr;
+  if (splits > 1) {
+    if (dli_attention_decode_static_floats(requests, q_heads, head_dim, splits) > DLI_STATIC_SCRATCH_FLOATS)
+      return DLI_ERR_SCRATCH;
+    float* base = static_scratch();
+    if (base == nullptr) return DLI_ERR_LAUNCH;
+    const int64_t slots = (int64_t)requests * q_heads * splits;
+    part_o = base;
+    part_ml = base + (slots * head_dim + 63) / 64 * 64;
+  }
+  // Nothing has to start at zero: every (request, head, split) writes its partial result and its
+  // statistics before the merge reads them.
+  return dli_attention_decode_bf16(q, q_stride, k_pages, v_pages, out, out_stride, part_o, part_ml, kv_len,
+                                   block_tables, table_stride, requests, q_heads, kv_heads, head_dim, page_size,
+                                   scale, window, splits, stream);
 }
 
 extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages,

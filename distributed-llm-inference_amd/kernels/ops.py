@@ -61,6 +61,8 @@ _SIGNATURES = {
     "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "dli_attention_decode_bf16_static": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int,
+                                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_rope_angles": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
@@ -683,6 +685,32 @@ def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml),
         _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size,
         float(scale), int(window), int(splits), _stream()), "attention_decode")
+
+
+STATIC_SCRATCH_FLOATS = 2 * 1024 * 1024  # csrc/no_alloc.h: DLI_STATIC_SCRATCH_FLOATS
+
+
+def attention_decode_static(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                            kv_len: torch.Tensor, block_tables: torch.Tensor, q_heads: int, scale: float,
+                            window: int = 0, splits: int = 1) -> None:
+    """:func:`attention_decode` for callers that cannot allocate: the partial results of the key
+    splits live in a static device array of :data:`STATIC_SCRATCH_FLOATS` floats inside the
+    library (one per GPU, shared by every call on it: calls that overlap on one GPU race)."""
+    kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
+    rows = q.shape[0]
+    _dense(kv_len, "kv_len", torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    _require(kv_len.shape[0] >= rows and block_tables.shape[0] >= rows, "one kv_len and table row per request")
+    _require(1 <= splits <= 65535 and rows <= 65535, "splits and requests must fit the grid")
+    status = library().dli_attention_decode_bf16_static(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(kv_len),
+        _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size, float(scale),
+        int(window), int(splits), _stream())
+    if status == -3:
+        raise KernelArgumentError(
+            f"attention_decode_static: {rows} requests x {q_heads} heads x {splits} splits x {head_dim} need more "
+            f"than the {STATIC_SCRATCH_FLOATS} floats of static scratch")
+    _check(status, "attention_decode_static")
 
 
 def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
