@@ -48,19 +48,25 @@ class TraceSession:
         from .engine.batch import StepEntry
 
         mgr = self.core.manager
-        batch = []
+        batch, copies = [], []
         for ent in entries:
             rid, tokens = ent.get("id"), [int(t) for t in ent.get("tokens") or []]
             want = [int(w) for w in ent.get("want") or []]
             if rid is None or not tokens:
                 raise TraceError("an entry needs an id and at least one token")
             if rid not in self.fed:
-                mgr.allocate(rid, tokens, respect_watermark=False)
-                self.fed[rid] = 0
+                # On a core with content reuse the leading pages may be another request's, already
+                # computed: only the rest of the tokens runs, and nothing can be wanted before it.
+                skip = mgr.allocate(rid, tokens, respect_watermark=False).num_cached_tokens
+                if any(w < skip for w in want):
+                    mgr.free(rid)
+                    raise TraceError(f"request {rid!r}: logits wanted at a place whose page was reused")
+                self.fed[rid] = skip
+                tokens, want = tokens[skip:], [w - skip for w in want]
             else:
-                mgr.append_slots(rid, tokens)
+                copies.extend(mgr.append_slots(rid, tokens))
             batch.append(StepEntry(rid, tokens, self.fed[rid], want))
-        logits = self.core.step.run(batch)
+        logits = self.core.step.run(batch, copies)
         for e in batch:
             self.fed[e.seq_id] += len(e.tokens)
         for rid in end:
@@ -68,6 +74,17 @@ class TraceSession:
                 mgr.free(rid)
                 del self.fed[rid]
         return logits
+
+
+    def fork(self, parent: Any, child: Any) -> None:
+        """``child`` continues from everything ``parent`` has been fed, sharing its pages; the
+        first write of either into a shared, partly filled page copies that page first."""
+        if self.core.store.stateful:
+            raise TraceError("a model with per-request state cannot be forked here")
+        if parent not in self.fed or child in self.fed:
+            raise TraceError(f"cannot fork {parent!r} into {child!r}")
+        self.core.manager.fork(parent, child)
+        self.fed[child] = self.fed[parent]
 
 
 class TraceRunner:
