@@ -170,6 +170,119 @@ def test_whole_model_properties(name):
     assert head.shape == (cfg["vocab_size"], cfg["hidden_size"])
 
 
+# ------------------------------------------------------------------ layer composition
+# The arrangement of a block (which norm feeds which branch, where the two sums sit, the final norm
+# and the head; model/llama.py:194-213,299-305) pinned by library routines and by what a wrong
+# arrangement would change.
+
+def _library_rotate(x, positions, inv_freq):
+    """Rotation of ``x [heads, n, d]`` written as a complex product on pairs (i, i + d/2)."""
+    half = x.shape[-1] // 2
+    z = torch.complex(x[..., :half], x[..., half:]) * torch.polar(
+        torch.ones(len(positions), half, dtype=x.dtype), positions[:, None].to(x.dtype) * inv_freq.to(x.dtype))
+    return torch.cat([z.real, z.imag], dim=-1)
+
+
+def _library_layer(h, w, i, cfg, positions):
+    """One block composed from library routines, every sum written out."""
+    s = P.model_sizes(cfg)
+    nh, nkv, d, eps = s["num_heads"], s["num_kv_heads"], s["head_dim"], s["eps"]
+    n, p = h.shape[0], f"model.layers.{i}."
+    inv_freq = P.inverse_frequencies(P.rope_settings(cfg), d)
+    a = F.rms_norm(h, (h.shape[-1],), w[p + "input_layernorm.weight"], eps)
+    q = F.linear(a, w[p + "self_attn.q_proj.weight"], w.get(p + "self_attn.q_proj.bias"))
+    k = F.linear(a, w[p + "self_attn.k_proj.weight"], w.get(p + "self_attn.k_proj.bias"))
+    v = F.linear(a, w[p + "self_attn.v_proj.weight"], w.get(p + "self_attn.v_proj.bias"))
+    q = _library_rotate(q.view(n, nh, d).transpose(0, 1), positions, inv_freq)
+    k = _library_rotate(k.view(n, nkv, d).transpose(0, 1), positions, inv_freq)
+    v = v.view(n, nkv, d).transpose(0, 1)
+    k, v = (t.repeat_interleave(nh // nkv, dim=0) for t in (k, v))
+    o = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+    o = F.linear(o.transpose(0, 1).reshape(n, nh * d), w[p + "self_attn.o_proj.weight"],
+                 w.get(p + "self_attn.o_proj.bias"))
+    h = h + o
+    m = F.rms_norm(h, (h.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
+    gate = F.linear(m, w[p + "mlp.gate_proj.weight"], w.get(p + "mlp.gate_proj.bias"))
+    up = F.linear(m, w[p + "mlp.up_proj.weight"], w.get(p + "mlp.up_proj.bias"))
+    return h + F.linear(F.silu(gate) * up, w[p + "mlp.down_proj.weight"], w.get(p + "mlp.down_proj.bias"))
+
+
+def _without_branches(w, keep=()):
+    """The weights with every layer's o_proj and down_proj (and their biases) zeroed, except the
+    layers in ``keep``: such a layer adds nothing to the residual stream."""
+    out = dict(w)
+    for name, t in w.items():
+        if ("o_proj" in name or "down_proj" in name) and not any(f"layers.{i}." in name for i in keep):
+            out[name] = torch.zeros_like(t)
+    return out
+
+
+def _head(w, cfg):
+    return w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_dead_branches_leave_embedding_final_norm_and_head(name):
+    cfg, w = P.load_folder(model_folder(name))
+    w = {k: t.to(F64) for k, t in w.items()}
+    toks = [7, 2, 9, 9, 30, 1, 17]
+    dead = _without_branches(w)
+    e = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    want = F.linear(F.rms_norm(e, (e.shape[-1],), w["model.norm.weight"], cfg["rms_norm_eps"]), _head(w, cfg))
+    got = P.forward_logits(dead, cfg, toks)
+    assert torch.allclose(got, want, atol=1e-10)
+    # the final norm is there: a scale of the embedding rows cancels (up to eps) ...
+    scaled = dict(dead)
+    scaled["model.embed_tokens.weight"] = dead["model.embed_tokens.weight"] * 3.0
+    if not cfg["tie_word_embeddings"]:
+        assert torch.allclose(P.forward_logits(scaled, cfg, toks), got, rtol=2e-3, atol=1e-3)
+        assert not torch.allclose(P.forward_logits(scaled, cfg, toks), 3.0 * got, rtol=2e-3, atol=1e-3)
+    else:  # ... and with a tied head it is the head that scales
+        assert torch.allclose(P.forward_logits(scaled, cfg, toks), 3.0 * got, rtol=2e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_one_live_layer_equals_the_library_composition(name):
+    cfg, w = P.load_folder(model_folder(name))
+    w = {k: t.to(F64) for k, t in w.items()}
+    toks = [4, 250, 3, 3, 91, 18, 5, 77, 6]
+    positions = torch.arange(len(toks))
+    e = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    for i in range(cfg["num_hidden_layers"]):
+        live = _without_branches(w, keep=(i,))
+        h = _library_layer(e, live, i, cfg, positions)
+        want = F.linear(F.rms_norm(h, (h.shape[-1],), w["model.norm.weight"], cfg["rms_norm_eps"]), _head(w, cfg))
+        got = P.forward_logits(live, cfg, toks)
+        assert torch.allclose(got, want, atol=1e-6), (name, i)
+        assert not torch.allclose(got, P.forward_logits(_without_branches(w), cfg, toks), atol=1e-3)
+    # all layers live: the blocks chained (the plain rotation takes its angles in 32-bit as the
+    # reference does, rope.py:58-60; the library composition here takes them in 64-bit)
+    h = e
+    for i in range(cfg["num_hidden_layers"]):
+        h = _library_layer(h, w, i, cfg, positions)
+    want = F.linear(F.rms_norm(h, (h.shape[-1],), w["model.norm.weight"], cfg["rms_norm_eps"]), _head(w, cfg))
+    assert torch.allclose(P.forward_logits(w, cfg, toks), want, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_each_norm_feeds_its_own_branch(name):
+    cfg, w = P.load_folder(model_folder(name))
+    toks = [4, 250, 3, 3, 91, 18]
+    base = P.forward_logits(w, cfg, toks)
+    a, b = "model.layers.0.input_layernorm.weight", "model.layers.0.post_attention_layernorm.weight"
+    swapped = dict(w)
+    swapped[a], swapped[b] = w[b], w[a]
+    assert (P.forward_logits(swapped, cfg, toks) - base).abs().max() > 1e-3
+    # with the feed-forward dead, only the norm before the attention matters, and the other way round
+    for dead, silent, heard in (("down_proj", b, a), ("o_proj", a, b)):
+        part = {k: (torch.zeros_like(t) if f"layers.0." in k and dead in k else t) for k, t in w.items()}
+        ref = P.forward_logits(part, cfg, toks)
+        for which, changes in ((silent, False), (heard, True)):
+            mod = dict(part)
+            mod[which] = part[which] * 1.5
+            assert ((P.forward_logits(mod, cfg, toks) - ref).abs().max() > 1e-3) == changes, (dead, which)
+
+
 def test_greedy_generation_recomputes_and_breaks_ties_low():
     cfg, w = P.load_folder(model_folder("A"))
     out = P.greedy_generate(w, cfg, [5, 6, 7], 6)
