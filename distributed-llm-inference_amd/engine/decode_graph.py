@@ -188,7 +188,7 @@ class DecodeGraphs:
         b = _bucket(n)
         max_kv = max(e.start + steps for e in entries)
         width = max(16, _bucket(-(-max_kv // ps)))
-        splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv))
+        splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv, ops.compute_units(self.step_fn.rt.device)))
         sampled = sampling is not None
         if steps > 1 and not sampled:
             raise ValueError("several steps in a row need the sampling parameters")

@@ -43,14 +43,9 @@ class StepFunction:
         self.vocab_size = model.spec.vocab_size
         self.steps_run = 0
         self.graphs = None  # DecodeGraphs, when the engine enables graph replay of decode steps
-        tiles = [1]
-        for i, cache in enumerate(store.layers):
-            if cache is not None and cache.kind == "paged":
-                mixer = self.model.layers[self.model.spec.schedule[i].layer].parts.get("mixer")
-                kv_heads = cache.k_pages.shape[1]
-                q_heads = int(getattr(mixer, "num_heads", kv_heads))
-                tiles.append(kv_heads * -(-(q_heads // kv_heads) // 16))
-        self.decode_head_tiles = max(tiles)  # workgroups per request and key split in decode attention
+        # workgroups per request and key split in the decode kernels of the parts that keep pages
+        self.decode_head_tiles = max([1] + [int(part.decode_head_tiles()) for part in model.cache_owners()
+                                            if part is not None and hasattr(part, "decode_head_tiles")])
 
     def enable_decode_graphs(self, max_batch: int, max_model_len: int) -> None:
         """Replay decode-only steps through HIP graphs (bfloat16 with the matrix-core decode path

@@ -349,6 +349,11 @@ def tile_weights(w: torch.Tensor) -> torch.Tensor:
 _compute_units: dict[int, int] = {}
 
 
+def compute_units(device: torch.device) -> int:
+    """Compute units of the device (256 on MI355X)."""
+    return _units(device)
+
+
 def _units(device: torch.device) -> int:
     index = device.index if device.index is not None else torch.cuda.current_device()
     if index not in _compute_units:

@@ -78,8 +78,15 @@ class GQAttention(Mixer):
         self.w_qkv_tiled = decode_copy(self.rt, self.w_qkv, ops.SKINNY_STORE)
         self.w_o_tiled = decode_copy(self.rt, self.w_o, ops.SKINNY_RESIDUAL)
         table = self.position.rotary_table()
+        if table is not None and table.pairing != "half":
+            raise ops.KernelArgumentError(
+                f"the attention kernels rotate pairs (i, i + dim/2); the position encoding asks for "
+                f"the pairing {table.pairing!r} (give it an apply() instead of a rotary table)")
+        if table is not None and (table.dim % 2 or not 0 < table.dim <= self.head_dim):
+            raise ops.KernelArgumentError(
+                f"rotary dimension {table.dim} does not fit heads of {self.head_dim}")
         if (self.w_qkv_tiled is not None and not self.shares_kv and table is not None
-                and table[1] == self.head_dim):
+                and table.dim == self.head_dim):
             # the rotation covers the whole head: the product can rotate in its epilogue, and
             # this order of the features replaces the plain tile order
             nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
@@ -94,6 +101,10 @@ class GQAttention(Mixer):
 
     def cache_spec(self) -> Optional[PagedKVSpec]:
         return None if self.shares_kv else PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    def decode_head_tiles(self) -> int:
+        # the decode kernel gives a workgroup up to 16 query heads of one kv head
+        return self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 16)
 
     # -- step
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
@@ -113,7 +124,7 @@ class GQAttention(Mixer):
             self.position.apply(q_view, k_view, ctx.positions)
             inv_freq, rotary_dim = None, 0
         else:
-            inv_freq, rotary_dim = table
+            inv_freq, rotary_dim = table.inv_freq, table.dim
         ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
                           cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         q = qkv[:, :nh * d]
@@ -141,7 +152,7 @@ class GQAttention(Mixer):
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
         if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS:
             # product, rotation and cache write in one kernel; only q comes back
-            angles = ctx.rope_angles(self.position.rotary_table()[0], qkv.dtype)
+            angles = ctx.rope_angles(self.position.rotary_table().inv_freq, qkv.dtype)
             ops.skinny_gemm_qkv_rope(stream.x, self.w_qkv_rope, qkv, angles, grp.slots, cache.k_pages, cache.v_pages,
                                      nh, bias=self.b_qkv_rope, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         else:
@@ -154,7 +165,7 @@ class GQAttention(Mixer):
                 self.position.apply(q_view, k_view, ctx.positions)
                 inv_freq, rotary_dim = None, 0
             else:
-                inv_freq, rotary_dim = table
+                inv_freq, rotary_dim = table.inv_freq, table.dim
             ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
                               cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         out = self.rt.empty(n, nh * d)

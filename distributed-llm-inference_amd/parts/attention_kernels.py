@@ -13,23 +13,22 @@ import torch
 
 from ..kernels import ops
 
-NUM_CUS = 256            # MI355X
 # From decode steps at batch 1 to 64: two workgroups per compute unit, and at 4K keys at most 16
 # runs, were ahead of more of either (the partial results cost a merge that grows with them); a
 # request with 32K keys did better with 64 runs than with 16, so the limit grows with the keys.
-WORKGROUPS_WANTED = 2 * NUM_CUS
+WORKGROUPS_PER_UNIT = 2
 MIN_KEYS_PER_SPLIT = 128
 FEW_SPLITS = 16          # the limit up to 8K keys
 KEYS_PER_EXTRA_SPLIT = 512
 MAX_SPLITS = 64
 
 
-def choose_splits(requests: int, kv_head_tiles: int, max_keys: int) -> int:
+def choose_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int = 256) -> int:
     """How many runs to cut each request's keys into for the decode kernel: enough workgroups
     to give every compute unit two workgroups, never runs under 128 keys (reference's rule of the
-    same kind: src/dli/model/paged_attention.py:63-74)."""
+    same kind: src/dli/model/paged_attention.py:63-74). ``units``: the device's compute units."""
     programs = max(1, requests * kv_head_tiles)
-    want = -(-WORKGROUPS_WANTED // programs)
+    want = -(-WORKGROUPS_PER_UNIT * units // programs)
     most = max(1, max_keys // MIN_KEYS_PER_SPLIT)
     limit = min(MAX_SPLITS, max(FEW_SPLITS, max_keys // KEYS_PER_EXTRA_SPLIT))
     return max(1, min(want, most, limit))
@@ -61,7 +60,7 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
 def _decode_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, head_dim: int, device: torch.device):
     group = q_heads // kv_heads
     splits = getattr(ctx, "forced_splits", None) or choose_splits(
-        nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len)
+        nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len, ops.compute_units(device))
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty(nd * q_heads * splits * head_dim, device=device, dtype=torch.float32)

@@ -12,7 +12,7 @@ of the step laid end to end; what belongs to which request is in the :class:`Ste
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Mapping, Optional
+from typing import Any, Mapping, Optional, NamedTuple
 
 import torch
 
@@ -122,16 +122,29 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class RotaryTable(NamedTuple):
+    """What a rotary encoding hands to the mixer whose kernels rotate.
+
+    ``inv_freq`` float32 ``[dim/2]``; the first ``dim`` components of every head are rotated.
+    ``pairing`` says which components form a rotated pair: ``"half"`` pairs component ``i`` with
+    ``i + dim/2`` (reference: src/dli/model/rope.py:63-70); a mixer refuses a pairing that its
+    kernels do not implement instead of rotating wrongly."""
+
+    inv_freq: torch.Tensor
+    dim: int
+    pairing: str = "half"
+
+
 class PositionEncoding(Part):
     """How positions enter a mixer.
 
-    A rotary encoding exposes :meth:`rotary_table`: inverse frequencies ``[rotary_dim/2]``
-    (float32); the attention mixer then rotates inside its fused cache-write kernel. Any other
-    encoding returns ``None`` there and implements :meth:`apply`, which rewrites q and k
-    (``[tokens, heads, head_dim]`` views) before keys are cached.
+    A rotary encoding exposes :meth:`rotary_table` (a :class:`RotaryTable`); the attention mixer
+    then rotates inside its fused cache-write kernel. Any other encoding returns ``None`` there
+    and implements :meth:`apply`, which rewrites q and k (``[tokens, heads, head_dim]`` views)
+    before keys are cached.
     """
 
-    def rotary_table(self) -> Optional[tuple[torch.Tensor, int]]:
+    def rotary_table(self) -> Optional[RotaryTable]:
         return None
 
     def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], positions: torch.Tensor) -> None:
@@ -150,6 +163,11 @@ class Mixer(Part):
 
     def cache_spec(self) -> Optional[PagedKVSpec | StateSpec]:
         return None
+
+    def decode_head_tiles(self) -> int:
+        """Workgroups that one request's decoded token gives the mixer's kernel per split of its
+        keys (1 where that means nothing); the step function sizes key splits with the largest."""
+        return 1
 
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
         raise NotImplementedError

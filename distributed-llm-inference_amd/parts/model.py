@@ -91,11 +91,21 @@ class Model:
 
     def cache_specs(self) -> list[Optional[Any]]:
         """What each schedule entry keeps per request (``None``: nothing of its own)."""
-        out = []
+        return [None if owner is None or entry.cache_of is not None else owner.cache_spec()
+                for entry, owner in zip(self.spec.schedule, self.cache_owners())]
+
+    def cache_owners(self) -> list[Optional[Part]]:
+        """Per schedule entry, the part of its layer that keeps something per request: whichever
+        part, in whatever role, answers ``cache_spec()`` with a spec. A schedule entry has one
+        cache, so a layer with two such parts is refused."""
+        out: list[Optional[Part]] = []
         for entry in self.spec.schedule:
-            mixer = self.layers[entry.layer].parts.get("mixer")
-            own = entry.cache_of is None and mixer is not None
-            out.append(mixer.cache_spec() if own else None)
+            owners = [(role, part) for role, part in self.layers[entry.layer].parts.items()
+                      if callable(getattr(part, "cache_spec", None)) and part.cache_spec() is not None]
+            if len(owners) > 1:
+                raise ValueError(f"layer {entry.layer}: the parts {[r for r, _ in owners]} each keep a cache; "
+                                 f"a schedule entry has one (put them in entries of their own)")
+            out.append(owners[0][1] if owners else None)
         return out
 
     def bind_caches(self, layer_caches: Sequence[Any]) -> list[Any]:

@@ -17,7 +17,7 @@ from typing import Optional
 import numpy as np
 import torch
 
-from .base import PositionEncoding, Runtime
+from .base import PositionEncoding, RotaryTable, Runtime
 from .registry import register_part
 
 
@@ -69,10 +69,10 @@ class Rotary(PositionEncoding):
             hit = _TABLES[key] = torch.from_numpy(self.inv_freq_host.copy()).to(self.rt.device)
         self._table = hit
 
-    def rotary_table(self) -> Optional[tuple[torch.Tensor, int]]:
+    def rotary_table(self) -> Optional[RotaryTable]:
         if self._table is None:
             self.finalize()
-        return self._table, self.dim
+        return RotaryTable(self._table, self.dim, "half")
 
 
 @register_part("position", "none")

@@ -142,9 +142,13 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     p.add_argument("--out", required=True, help="folder that receives <step>.f32")
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens that live requests hold at any time (each rounded up to 64)")
+    p.add_argument("--page-size", type=int, default=PAGE_SIZE,
+                   help=f"token slots of a cache page (default {PAGE_SIZE}; the pool is --max-tokens / this)")
     args = p.parse_args(argv)
     try:
-        runner = TraceRunner(args.model, args.dtype, args.out, args.max_tokens)
+        if args.page_size < 1 or 64 % args.page_size:
+            raise TraceError("--page-size must divide the 64 tokens that a request's count is rounded up to")
+        runner = TraceRunner(args.model, args.dtype, args.out, args.max_tokens, page_size=args.page_size)
         runner.replay(sys.stdin, sys.stdout)
     except Exception as exc:  # one clear line, non-zero exit
         print(f"trace_run: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)

@@ -382,6 +382,63 @@ def test_trace_run_program(tmp_path):
     assert proc.returncode != 0 and "NoFreePagesError" in proc.stderr
 
 
+def test_generate_command_line(tmp_path):
+    """``python -m dli_amd random-weights`` then ``... generate`` as a user runs them (the reference's
+    flag names, src/dli/server/__main__.py:65-124): the printed ids are the plain implementation's."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from tiny_configs import TINY_B
+
+    root = Path(__file__).resolve().parent.parent
+    env = dict(os.environ, PYTHONPATH=str(root) + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(TINY_B))
+    folder = tmp_path / "model"
+    proc = subprocess.run([sys.executable, "-m", "dli_amd", "random-weights", "--config", str(cfg_file), "--out",
+                           str(folder), "--seed", "9", "--std", "0.085", "--norm-jitter", "0.1"],
+                          capture_output=True, text=True, timeout=300, env=env, cwd=tmp_path)
+    assert proc.returncode == 0, proc.stderr
+    assert Path(proc.stdout.strip().splitlines()[-1]) == folder and (folder / "model.safetensors").exists()
+    cfg, w = P.load_folder(folder)
+    ps = [[11, 5, 300, 42, 7, 7, 129], list(range(3, 3 + 41))]
+    (tmp_path / "prompts.txt").write_text(json.dumps(ps[1]) + "\n")
+    for dtype, block, extra in (("float32", 8, ["--no-prefix-caching"]), ("bfloat16", 16, ["--max-num-batched-tokens", "24"]),
+                                ("auto", 16, ["--no-cuda-graphs", "--num-blocks", "12"])):
+        proc = subprocess.run(
+            [sys.executable, "-m", "dli_amd", "generate", "--model", str(folder), "--dtype", dtype, "--block-size",
+             str(block), "--max-tokens", "12", "--prompt-ids", " ".join(map(str, ps[0])), "--prompt-file",
+             str(tmp_path / "prompts.txt"), *extra],
+            capture_output=True, text=True, timeout=300, env=env, cwd=tmp_path)
+        assert proc.returncode == 0, proc.stderr
+        got = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("[")]
+        assert len(got) == 2 and all(len(g) == 12 for g in got), proc.stdout
+        for g, prompt in zip(got, ps):
+            want = P.greedy_generate(w, cfg, prompt, 12)
+            if dtype == "float32":
+                assert g == want
+            else:
+                toks = list(prompt)
+                for a, b in zip(g, want):
+                    if a != b:
+                        logits = P.forward_logits(w, cfg, toks)[-1]
+                        assert 0 <= (logits[b] - logits[a]).item() < 0.25
+                        break
+                    toks.append(b)
+    # a stop token ends a request early; the option's name is the reference's
+    stop = P.greedy_generate(w, cfg, ps[0], 12)[4]
+    proc = subprocess.run(
+        [sys.executable, "-m", "dli_amd", "generate", "--model", str(folder), "--dtype", "float32", "--block-size", "8",
+         "--max-tokens", "12", "--prompt-ids", ",".join(map(str, ps[0])), "--stop-token-ids", str(stop)],
+        capture_output=True, text=True, timeout=300, env=env, cwd=tmp_path)
+    assert proc.returncode == 0, proc.stderr
+    out = json.loads([l for l in proc.stdout.splitlines() if l.startswith("[")][0])
+    assert out[-1] == stop and len(out) <= 5
+
+
 def test_generation_without_the_decode_copy_of_the_weights():
     """The second, tile-ordered copy of the matrices is an option: without it the decode steps
     read the row-major matrices (and run the rotation kernel), and greedy generation gives the

@@ -300,6 +300,27 @@ def test_library_product_called_directly(ops, m, n, k, with_bias):
     assert torch.equal(again, out)
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_linear_where_the_direct_library_call_finds_no_kernel(ops, monkeypatch, with_bias):
+    """``parts.linear`` goes through ``torch.mm`` (and the engine's bias kernel) for a shape that
+    the direct call refuses; the refusal is forced here so that this branch runs on every box."""
+    from dli_amd.parts import linear as L
+    from dli_amd.parts.base import Runtime
+
+    calls = []
+    monkeypatch.setattr(L.ops, "gemm_bf16", lambda *a: calls.append(1) and False)
+    torch.manual_seed(5)
+    m, n, k = 37, 200, 136
+    x = torch.randn(m, k, device="cuda").bfloat16()
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    bias = torch.randn(n, device="cuda").bfloat16() if with_bias else None
+    rt = Runtime(device=torch.device("cuda"), dtype=torch.bfloat16)
+    out = L.linear(rt, x, w, bias)
+    assert calls == [1] and out.dtype == torch.bfloat16
+    ref = x.cpu().double() @ w.cpu().double().T + (bias.cpu().double() if with_bias else 0.0)
+    assert (out.cpu().double() - ref).abs().max() < 2.0 ** -7 * ref.abs().max().item() + 1e-2
+
+
 def _ref_norm_bf16(x, w, eps):
     """RMSNorm with the engine's rounding: cast(w * cast(x * r))."""
     xf = x.float()

@@ -48,8 +48,8 @@ def test_rotary_part_alone(raw):
     cfg = LlamaConfig.from_hf_dict(raw)
     spec = build_llama_spec(cfg).layers[0].parts["mixer"][1].params["position"]
     part = build_part("position", spec, rt())
-    table, dim = part.rotary_table()
-    assert dim == cfg.head_dim
+    table, dim, pairing = part.rotary_table()
+    assert dim == cfg.head_dim and pairing == "half"
     ref = P.inverse_frequencies(P.rope_settings(raw), cfg.head_dim)
     assert torch.allclose(table.cpu(), ref, rtol=2e-7, atol=0)
 
@@ -253,6 +253,54 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
     finally:
         unregister_architecture("ToyForCausalLM")
         unregister_part("mixer", "toy_ema")
+
+
+def test_a_rotary_table_with_another_pairing_is_refused_and_any_role_may_own_the_cache():
+    """The attention kernels rotate pairs (i, i + dim/2): a position encoding whose table names
+    another pairing is refused when the mixer is finalized, not rotated wrongly. And the part of
+    a layer that keeps a cache is found by what it answers to ``cache_spec()``, not by its role's
+    name; two such parts in one layer are refused."""
+    from dli_amd.kernels.ops import KernelArgumentError
+    from dli_amd.parts import (LayerSpec, ModelSpec, PartSpec, PositionEncoding, RotaryTable, ScheduleEntry,
+                               build_part, register_part, unregister_part)
+    from dli_amd.parts.model import Model
+
+    @register_part("position", "toy_adjacent_rotary")
+    class Adjacent(PositionEncoding):
+        def __init__(self, runtime, *, dim: int) -> None:
+            super().__init__(runtime)
+            self.dim = dim
+
+        def rotary_table(self):
+            return RotaryTable(torch.ones(self.dim // 2, device=self.rt.device), self.dim, "adjacent")
+
+    try:
+        attn = dict(hidden_size=32, num_heads=2, num_kv_heads=1, head_dim=16)
+        bad = build_part("mixer", PartSpec("gqa_attention", dict(attn, position=PartSpec("toy_adjacent_rotary", dict(dim=16)))), rt())
+        with pytest.raises(KernelArgumentError, match="adjacent"):
+            bad.finalize()
+        norm = dict(width=32, eps=1e-5)
+        mixer = PartSpec("gqa_attention", dict(attn, position=PartSpec("rotary", dict(dim=16, theta=1e4))), "a.")
+
+        def spec(parts):
+            return ModelSpec(
+                architecture="Toy", vocab_size=40, hidden_size=32,
+                embedding=PartSpec("token_embedding", dict(vocab_size=40, hidden_size=32), "embed."),
+                layers=(LayerSpec(PartSpec("pre_norm"), parts),), schedule=(ScheduleEntry(0),),
+                final_norm=PartSpec("rms_norm", norm, "norm."),
+                head=PartSpec("linear_head", dict(vocab_size=40, hidden_size=32, tied=True), "head."))
+
+        base = {"mixer_norm": ("norm", PartSpec("rms_norm", norm, "n1.")), "mixer": ("mixer", mixer),
+                "feed_forward_norm": ("norm", PartSpec("rms_norm", norm, "n2.")),
+                "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=32, intermediate_size=48), "mlp."))}
+        model = Model(spec(base), rt())
+        assert model.cache_owners() == [model.layers[0].parts["mixer"]]
+        assert type(model.cache_specs()[0]).__name__ == "PagedKVSpec"
+        two = dict(base, second_mixer=("mixer", PartSpec("gqa_attention", dict(attn), "b.")))
+        with pytest.raises(ValueError, match="each keep a cache"):
+            Model(spec(two), rt()).cache_specs()
+    finally:
+        unregister_part("position", "toy_adjacent_rotary")
 
 
 # ------------------------------------------------------------------ toy feed-forward with routing, toy position encoding
