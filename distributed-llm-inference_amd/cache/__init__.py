@@ -4,11 +4,11 @@ from .manager import (
     RELEASED, Allocation, CacheManager, CacheStats, CopyOp, GroupSpec, NoFreePagesError, SequenceError,
 )
 from .page_identity import ROOT_PARENT, chain_hashes, page_hash
-from .reclaim import CostAwarePolicy, LRUPolicy, make_policy
+from .reclaim import OldestFirst, ReclaimOrder, ReusedLast, make_order
 from .state_slots import NoFreeSlotError, StateSlots
 
 __all__ = [
-    "RELEASED", "Allocation", "CacheManager", "CacheStats", "CopyOp", "CostAwarePolicy", "GroupSpec",
-    "LRUPolicy", "NoFreePagesError", "NoFreeSlotError", "ROOT_PARENT", "SequenceError", "StateSlots",
-    "chain_hashes", "make_policy", "page_hash",
+    "RELEASED", "Allocation", "CacheManager", "CacheStats", "CopyOp", "GroupSpec",
+    "NoFreePagesError", "NoFreeSlotError", "OldestFirst", "ROOT_PARENT", "ReclaimOrder", "ReusedLast",
+    "SequenceError", "StateSlots", "chain_hashes", "make_order", "page_hash",
 ]

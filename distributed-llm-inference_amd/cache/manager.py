@@ -33,7 +33,7 @@ from typing import Hashable, Optional, Sequence
 
 from .page_identity import ROOT_PARENT, PageHash, chain_hashes, page_hash
 from .pool import PagePool
-from .reclaim import EvictionPolicy
+from .reclaim import ReclaimOrder
 from .state_slots import NoFreeSlotError, StateSlots
 
 SeqId = Hashable
@@ -140,7 +140,7 @@ class CacheManager:
         num_pages: int | Sequence[int],
         page_size: int,
         max_seqs: int = 256,
-        eviction_policy: str | EvictionPolicy = "lru",
+        eviction_policy: str | ReclaimOrder = "lru",
         enable_prefix_caching: bool = True,
         stateful: bool = False,
         watermark: float = 0.01,
@@ -271,7 +271,7 @@ class CacheManager:
                 # revive hits before taking new pages, so that no reused page can be reclaimed
                 for page in hits:
                     pool.incref(page)
-                    pool.policy.on_hit(page)
+                    pool.order.found(page)
                 table = list(hits)
             else:
                 table = []

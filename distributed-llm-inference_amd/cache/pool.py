@@ -12,7 +12,7 @@ from collections import Counter, deque
 from dataclasses import dataclass
 from typing import Optional
 
-from .reclaim import EvictionPolicy, make_policy
+from .reclaim import ReclaimOrder, make_order
 from .page_identity import PageHash
 
 
@@ -25,12 +25,12 @@ class _CachedPage:
 
 
 class PagePool:
-    def __init__(self, num_pages: int, eviction_policy: str | EvictionPolicy = "lru") -> None:
+    def __init__(self, num_pages: int, eviction_policy: str | ReclaimOrder = "lru") -> None:
         if num_pages <= 0:
             raise ValueError("num_pages must be positive")
         self.num_pages = num_pages
-        self.policy: EvictionPolicy = (
-            make_policy(eviction_policy) if isinstance(eviction_policy, str) else eviction_policy
+        self.order: ReclaimOrder = (
+            make_order(eviction_policy) if isinstance(eviction_policy, str) else eviction_policy
         )
         self.ref = [0] * num_pages
         self.free: deque[int] = deque(range(num_pages))
@@ -46,7 +46,7 @@ class PagePool:
 
     def take(self) -> int:
         """A page for a new holder. Callers check :attr:`num_available` first."""
-        page = self.free.popleft() if self.free else self._evict(self.policy.pop_victim())
+        page = self.free.popleft() if self.free else self._evict(self.order.take())
         self.ref[page] = 1
         return page
 
@@ -57,7 +57,7 @@ class PagePool:
                 raise AssertionError(f"page {page} is free and cannot gain a holder")
             self.num_idle -= 1
             if entry.children == 0:
-                self.policy.remove_candidate(page)
+                self.order.withdraw(page)
         self.ref[page] += 1
 
     def decref(self, page: int) -> None:
@@ -72,25 +72,25 @@ class PagePool:
             return
         self.num_idle += 1
         if entry.children == 0:
-            self.policy.add_candidate(page)
+            self.order.offer(page)
 
     def _evict(self, page: int) -> int:
         entry = self.cached.pop(page)
         del self.by_identity[entry.identity]
         self.num_idle -= 1
-        self.policy.on_evicted(page)
+        self.order.dropped(page)
         self.evictions += 1
         if entry.parent is not None:
             parent = self.cached[entry.parent]
             parent.children -= 1
             if parent.children == 0 and self.ref[entry.parent] == 0:
-                self.policy.add_candidate(entry.parent)
+                self.order.offer(entry.parent)
         return page
 
     def evict_all_idle(self) -> int:
         n = 0
-        while len(self.policy):
-            self.free.append(self._evict(self.policy.pop_victim()))
+        while len(self.order):
+            self.free.append(self._evict(self.order.take()))
             n += 1
         return n
 
@@ -114,11 +114,11 @@ class PagePool:
                 return "orphan"
             pentry = self.cached[parent]
             if pentry.children == 0 and self.ref[parent] == 0:
-                self.policy.remove_candidate(parent)
+                self.order.withdraw(parent)
             pentry.children += 1
         self.cached[page] = _CachedPage(identity, parent, depth)
         self.by_identity[identity] = page
-        self.policy.on_cached(page, depth)
+        self.order.cached(page, depth)
         return "cached"
 
     def check(self, expected_ref: Counter) -> None:
@@ -148,5 +148,5 @@ class PagePool:
             parent = self.cached[p].parent
             assert parent is None or self.ref[parent] > 0, f"held page {p} has an idle parent"
         candidates = {p for p in idle if self.cached[p].children == 0}
-        assert len(self.policy) == len(candidates), (
-            f"policy holds {len(self.policy)} candidates, expected {len(candidates)}")
+        assert len(self.order) == len(candidates), (
+            f"the reclaim order holds {len(self.order)} candidates, expected {len(candidates)}")

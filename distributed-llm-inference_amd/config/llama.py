@@ -2,7 +2,8 @@
 
 Every size and constant of the model is a field here, read from the architecture's own
 ``config.json`` keys; nothing below this module carries a literal size.
-Parsing rules follow the reference's ``ModelConfig.from_hf_dict`` (src/dli/model/config.py:80-150).
+What is read, defaulted and refused is what the reference's ``ModelConfig.from_hf_dict`` reads,
+defaults and refuses (src/dli/model/config.py:80-150).
 """
 
 from __future__ import annotations
@@ -101,54 +102,27 @@ class LlamaConfig:
 
     @classmethod
     def from_hf_dict(cls, cfg: Mapping[str, Any]) -> "LlamaConfig":
-        """Parse a ``config.json`` dictionary.
-
-        Accepts the hub spelling (``rope_theta`` + ``rope_scaling``) and the newer
-        ``rope_parameters`` one (which wins where both are present).
+        """Parse a ``config.json`` dictionary: refusals first (:data:`_REFUSALS`), then every
+        field from its key by :data:`_FIELDS`, then the rotary constants from whichever of the two
+        spellings the file uses (``rope_theta`` + ``rope_scaling``, or ``rope_parameters``).
 
         Raises:
             UnsupportedModelError: another architecture, or an option that is not implemented.
             MissingConfigKeyError: a key without default is absent.
         """
-        model_type = cfg.get("model_type")
-        if model_type != "llama":
-            raise UnsupportedModelError(f"model_type={model_type!r} is not supported")
-        act = cfg.get("hidden_act", "silu")
-        if act != "silu":
-            raise UnsupportedModelError(f"hidden_act={act!r} (only 'silu' / SwiGLU is supported)")
-        if cfg.get("use_sliding_window") or any(
-            t != "full_attention" for t in cfg.get("layer_types") or []
-        ):
-            raise UnsupportedModelError("sliding-window attention is not supported")
-        if cfg.get("pretraining_tp", 1) not in (1, None):
-            raise UnsupportedModelError("pretraining_tp > 1 changes numerics and is not supported")
-
-        def need(key: str) -> Any:
-            if cfg.get(key) is None:
-                raise MissingConfigKeyError(key)
-            return cfg[key]
-
-        num_heads = int(need("num_attention_heads"))
-        hidden = int(need("hidden_size"))
-        attention_bias = bool(cfg.get("attention_bias", False))
-        return cls(
-            model_type=model_type,
-            vocab_size=int(need("vocab_size")),
-            hidden_size=hidden,
-            intermediate_size=int(need("intermediate_size")),
-            num_layers=int(need("num_hidden_layers")),
-            num_heads=num_heads,
-            num_kv_heads=int(cfg.get("num_key_value_heads") or num_heads),
-            head_dim=int(cfg.get("head_dim") or hidden // num_heads),
-            rms_norm_eps=float(need("rms_norm_eps")),
-            max_position_embeddings=int(cfg.get("max_position_embeddings", 4096)),
-            rope=_parse_rope(cfg),
-            tie_word_embeddings=bool(cfg.get("tie_word_embeddings", False)),
-            hidden_act=act,
-            qkv_bias=attention_bias,
-            o_bias=attention_bias,
-            mlp_bias=bool(cfg.get("mlp_bias", False)),
-        )
+        for refused, why in _REFUSALS:
+            if refused(cfg):
+                raise UnsupportedModelError(why(cfg))
+        values: dict[str, Any] = {}
+        for name, key, cast, default in _FIELDS:
+            raw = cfg.get(key)
+            if raw is None:
+                if default is _REQUIRED:
+                    raise MissingConfigKeyError(key)
+                raw = default(values) if callable(default) else default
+            values[name] = cast(raw)
+        bias = values.pop("attention_bias")  # one flag in the file, two places in the model
+        return cls(rope=_read_rope(cfg), qkv_bias=bias, o_bias=bias, **values)
 
     def to_hf_dict(self) -> dict[str, Any]:
         """The ``config.json`` dictionary that parses back to this configuration."""
@@ -185,32 +159,67 @@ class LlamaConfig:
         return out
 
 
-def _parse_rope(cfg: Mapping[str, Any]) -> RopeConfig:
-    """Rotary constants from either spelling (reference: src/dli/model/config.py:130-150)."""
-    merged: dict[str, Any] = {**dict(cfg.get("rope_scaling") or {}),
-                              **dict(cfg.get("rope_parameters") or {})}
-    theta = merged.get("rope_theta")
-    if theta is None:
-        theta = cfg.get("rope_theta")
-    if theta is None:
-        theta = 10000.0
-    rope_type = merged.get("rope_type", merged.get("type", "default"))
-    if rope_type not in SUPPORTED_ROPE_TYPES:
-        raise UnsupportedModelError(f"rope_type={rope_type!r} is not supported")
-    if rope_type == "default":
-        return RopeConfig(theta=float(theta))
-    if merged.get("factor") is None:
+_REQUIRED = object()
+
+# What is refused before anything is read: (test on the dictionary, message).
+_REFUSALS = (
+    (lambda c: c.get("model_type") != "llama",
+     lambda c: f"model_type {c.get('model_type')!r}: this configuration reads 'llama' only"),
+    (lambda c: c.get("hidden_act", "silu") != "silu",
+     lambda c: f"hidden_act {c.get('hidden_act')!r}: the feed-forward is gated with SiLU and nothing else"),
+    (lambda c: bool(c.get("use_sliding_window")) or any(t != "full_attention" for t in c.get("layer_types") or ()),
+     lambda c: "layers with a sliding window are not part of this architecture here"),
+    (lambda c: (c.get("pretraining_tp") or 1) != 1,
+     lambda c: f"pretraining_tp {c.get('pretraining_tp')}: products cut in slices round differently; only 1 is taken"),
+)
+
+# field, config.json key, type, default (a value, a function of the fields read so far, or required)
+_FIELDS = (
+    ("model_type", "model_type", str, _REQUIRED),
+    ("vocab_size", "vocab_size", int, _REQUIRED),
+    ("hidden_size", "hidden_size", int, _REQUIRED),
+    ("intermediate_size", "intermediate_size", int, _REQUIRED),
+    ("num_layers", "num_hidden_layers", int, _REQUIRED),
+    ("num_heads", "num_attention_heads", int, _REQUIRED),
+    ("num_kv_heads", "num_key_value_heads", int, lambda v: v["num_heads"]),
+    ("head_dim", "head_dim", int, lambda v: v["hidden_size"] // v["num_heads"]),
+    ("rms_norm_eps", "rms_norm_eps", float, _REQUIRED),
+    ("max_position_embeddings", "max_position_embeddings", int, 4096),
+    ("tie_word_embeddings", "tie_word_embeddings", bool, False),
+    ("hidden_act", "hidden_act", str, "silu"),
+    ("attention_bias", "attention_bias", bool, False),
+    ("mlp_bias", "mlp_bias", bool, False),
+)
+
+
+def _read_rope(cfg: Mapping[str, Any]) -> RopeConfig:
+    """Rotary constants (reference: src/dli/model/config.py:130-150). A constant is looked up in
+    ``rope_parameters`` first, then in ``rope_scaling``, then (theta only) at the top level; old
+    files call the type ``type``."""
+    places = [cfg.get("rope_parameters") or {}, cfg.get("rope_scaling") or {}]
+
+    def find(*keys: str, top_level: bool = False, default: Any = None) -> Any:
+        for place in places + ([cfg] if top_level else []):
+            for key in keys:
+                if place.get(key) is not None:
+                    return place[key]
+        return default
+
+    theta = float(find("rope_theta", top_level=True, default=10000.0))
+    kind = find("rope_type", "type", default="default")
+    if kind == "default":
+        return RopeConfig(theta=theta)
+    if kind not in SUPPORTED_ROPE_TYPES:
+        raise UnsupportedModelError(f"rope_type {kind!r}: one of {SUPPORTED_ROPE_TYPES} is needed")
+    factor = find("factor")
+    if factor is None:
         raise MissingConfigKeyError("rope_scaling.factor")
     return RopeConfig(
-        theta=float(theta),
-        rope_type=rope_type,
-        factor=float(merged["factor"]),
-        low_freq_factor=float(merged.get("low_freq_factor", 1.0)),
-        high_freq_factor=float(merged.get("high_freq_factor", 4.0)),
-        original_max_position_embeddings=int(
-            merged.get("original_max_position_embeddings", cfg.get("max_position_embeddings", 8192))
-        ),
-    )
+        theta=theta, rope_type=kind, factor=float(factor),
+        low_freq_factor=float(find("low_freq_factor", default=1.0)),
+        high_freq_factor=float(find("high_freq_factor", default=4.0)),
+        original_max_position_embeddings=int(find(
+            "original_max_position_embeddings", default=cfg.get("max_position_embeddings") or 8192)))
 
 
 def config_field_names() -> tuple[str, ...]:

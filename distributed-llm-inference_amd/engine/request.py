@@ -10,23 +10,30 @@ from ..sampling.params import SamplingParams
 
 
 class RequestStatus(Enum):
-    WAITING = "waiting"    # queued, or preempted and waiting to be recomputed
-    RUNNING = "running"    # holds cache and is scheduled every step
+    """Where a request is: in the waiting queue (new, or put back there after it lost its pages),
+    among the running ones (it owns pages and a state slot and gets tokens every step), or done."""
+
+    WAITING = "waiting"
+    RUNNING = "running"
     FINISHED = "finished"
 
 
 class FinishReason(str, Enum):
-    STOP = "stop"          # emitted an end-of-sequence or stop token
-    LENGTH = "length"      # reached max_tokens
-    ABORTED = "aborted"    # cancelled by the caller
-    CAPACITY = "capacity"  # can never fit the cache pool: rejected, never runs
+    """Why a request is done: its last token was a stop or end-of-sequence id (``stop``), it has
+    ``max_tokens`` outputs (``length``), the caller cancelled it (``aborted``), or its prompt plus
+    ``max_tokens`` exceeds the whole pool, so it was turned away on arrival (``capacity``)."""
+
+    STOP = "stop"
+    LENGTH = "length"
+    ABORTED = "aborted"
+    CAPACITY = "capacity"
 
     def __str__(self) -> str:
         return self.value
 
 
 class Priority(IntEnum):
-    """Scheduling class; the lower value is served first."""
+    """Class of service: a smaller number goes first, in admission and when victims are chosen."""
 
     INTERACTIVE = 0
     BATCH = 1
@@ -34,9 +41,12 @@ class Priority(IntEnum):
 
 @dataclass(eq=False)
 class Request:
-    """``num_computed_tokens`` counts tokens whose keys are in the cache; after a preemption it
-    drops to 0 and the request recomputes ``prompt + outputs`` when it is admitted again.
-    ``seed`` keys the request's random stream; draw ``n`` of it samples output token ``n``."""
+    """What the caller gave (id, prompt, sampling parameters, class, tenant, seed) and how far the
+    engine has come. ``num_computed_tokens`` of ``prompt + outputs`` are in the cache; a request
+    that loses its pages starts again from 0 and runs its outputs so far as part of the prompt.
+    Draw ``n`` of the random stream keyed by ``seed`` chooses output token ``n``, whatever else
+    runs. ``arrival_seq`` orders requests of one class; ``arrival_step`` is the scheduler's step
+    count when the request came, for aging."""
 
     request_id: str
     prompt_ids: list[int]
@@ -45,10 +55,11 @@ class Request:
     priority: Priority = Priority.INTERACTIVE
     tenant: str = "default"
     seed: Optional[int] = None
-    output_ids: list[int] = field(default_factory=list)
+    # progress
     status: RequestStatus = RequestStatus.WAITING
-    finish_reason: Optional[FinishReason] = None
+    output_ids: list[int] = field(default_factory=list)
     num_computed_tokens: int = 0
+    finish_reason: Optional[FinishReason] = None
     num_preemptions: int = 0
     arrival_step: int = 0
 

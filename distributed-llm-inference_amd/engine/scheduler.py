@@ -22,7 +22,7 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Mapping, Optional
+from typing import Iterable, Mapping, Optional
 
 from ..cache.manager import CacheManager, CopyOp, NoFreePagesError
 from .request import FinishReason, Priority, Request, RequestStatus
@@ -30,14 +30,14 @@ from .request import FinishReason, Priority, Request, RequestStatus
 
 @dataclass(frozen=True)
 class SchedulerConfig:
-    """Limits of a step (reference: src/dli/engine/scheduler.py:32-58).
+    """Limits of a step; names and defaults as in src/dli/engine/scheduler.py:32-58.
 
-    ``namespace`` scopes content reuse of cache pages (model and weights identity);
-    ``tenant_weights`` gives tenants a weighted fair share of admissions; after ``aging_steps``
-    steps of waiting a request counts as INTERACTIVE. ``decode_steps`` > 1 lets a step in which
-    every request decodes, nobody waits and the cache has room run up to that many tokens of each
-    request on the device before the host sees them (the reference has no counterpart; 1 keeps
-    its behaviour).
+    ``namespace`` keeps the cache pages of different models or weights apart in the content
+    index. ``tenant_weights``: share of admitted work per tenant (absent tenants weigh 1).
+    A request that has waited ``aging_steps`` steps is treated as INTERACTIVE whatever its class.
+    ``decode_steps`` > 1 lets a step in which every request decodes, nobody waits and the cache
+    has room run up to that many tokens of each request on the device before the host sees them
+    (the reference has no counterpart; 1 keeps its behaviour).
     """
 
     max_num_seqs: int = 64
@@ -48,14 +48,42 @@ class SchedulerConfig:
     decode_steps: int = 1
 
     def __post_init__(self) -> None:
-        if self.max_num_seqs < 1 or self.max_num_batched_tokens < 1:
-            raise ValueError("max_num_seqs and max_num_batched_tokens must be >= 1")
-        if self.decode_steps < 1:
-            raise ValueError("decode_steps must be >= 1")
-        if self.aging_steps < 1:
-            raise ValueError("aging_steps must be >= 1")
-        if any(w <= 0 for w in self.tenant_weights.values()):
-            raise ValueError("tenant weights must be positive")
+        for name in ("max_num_seqs", "max_num_batched_tokens", "aging_steps", "decode_steps"):
+            if getattr(self, name) < 1:
+                raise ValueError(f"{name} must be at least 1, got {getattr(self, name)}")
+        bad = {t: w for t, w in self.tenant_weights.items() if not w > 0}
+        if bad:
+            raise ValueError(f"a tenant's weight must be positive: {bad}")
+
+
+class TenantLedger:
+    """Who is owed the next admission among tenants.
+
+    Every token placed into a step is charged to its request's tenant, divided by the tenant's
+    weight; the tenant with the smallest charge is served first, so over time tokens are
+    admitted in proportion to the weights. A tenant that had nothing in the system and comes
+    back is lifted to the smallest charge among the tenants present: idle time earns nothing.
+    """
+
+    def __init__(self, weights: Mapping[str, float]) -> None:
+        self._weights = dict(weights)
+        self._charge: dict[str, float] = {}
+
+    def enter(self, tenant: str, present: Iterable[str]) -> None:
+        """``tenant`` brings a request while the tenants in ``present`` have requests queued or
+        running. One that is present itself keeps its figure."""
+        present = set(present)
+        if tenant in present:
+            return
+        floor = min((self._charge[t] for t in present if t in self._charge), default=0.0)
+        self._charge[tenant] = max(self._charge.get(tenant, 0.0), floor)
+
+    def charge(self, tenant: str, tokens: int) -> None:
+        self._charge[tenant] = self._charge.get(tenant, 0.0) + tokens / self._weights.get(tenant, 1.0)
+
+    def owed(self, tenant: str) -> float:
+        """Smaller is served sooner."""
+        return self._charge.get(tenant, 0.0)
 
 
 @dataclass(frozen=True)
@@ -92,42 +120,52 @@ class Scheduler:
         self.running: list[Request] = []
         self._by_id: dict[str, Request] = {}
         self._step = 0
-        self._vtime: dict[str, float] = {}  # tokens served / weight, per tenant
+        self.ledger = TenantLedger(config.tenant_weights)
 
     # ------------------------------------------------------------------ lifecycle
 
     def add(self, req: Request) -> bool:
-        """Queue a request; False (finished with CAPACITY) if it could never fit the pool alone."""
+        """Queue a request. One whose prompt plus ``max_tokens`` needs more pages than the pool
+        has is finished at once with CAPACITY and False comes back: admitted later it could
+        block the queue for ever."""
         if req.request_id in self._by_id:
             raise ValueError(f"duplicate request id {req.request_id!r}")
-        worst_case = len(req.prompt_ids) + req.params.max_tokens
-        if -(-worst_case // self.manager.page_size) > self.manager.num_pages:
-            req.status = RequestStatus.FINISHED
-            req.finish_reason = FinishReason.CAPACITY
+        pages_at_most = -(-(len(req.prompt_ids) + req.params.max_tokens) // self.manager.page_size)
+        if pages_at_most > self.manager.num_pages:
+            req.status, req.finish_reason = RequestStatus.FINISHED, FinishReason.CAPACITY
             return False
-        self._by_id[req.request_id] = req
+        self.ledger.enter(req.tenant, [r.tenant for r in self._by_id.values()])
         req.arrival_step = self._step
-        self._activate_tenant(req.tenant)
+        self._by_id[req.request_id] = req
         self.waiting.append(req)
         return True
 
-    def finish(self, req: Request, reason: FinishReason) -> None:
-        """Give back the request's cache and take it out of scheduling."""
+    def _release(self, req: Request, becomes: RequestStatus, reason: Optional[FinishReason] = None) -> None:
+        """Take ``req`` out of the queue it is in, returning its pages and state slot if it has
+        any, and leave it ``becomes``: FINISHED (with ``reason``) or WAITING (preempted: it keeps
+        its outputs, forgets what was computed and goes to the head of the waiting queue)."""
         if req.status is RequestStatus.RUNNING:
             self.manager.free(req.request_id)
             self.running.remove(req)
         elif req.status is RequestStatus.WAITING:
             self.waiting.remove(req)
-        req.status = RequestStatus.FINISHED
-        req.finish_reason = reason
-        self._by_id.pop(req.request_id, None)
+        req.status = becomes
+        if becomes is RequestStatus.FINISHED:
+            req.finish_reason = reason
+            self._by_id.pop(req.request_id, None)
+        else:
+            req.num_computed_tokens = 0
+            req.num_preemptions += 1
+            self.waiting.appendleft(req)
+
+    def finish(self, req: Request, reason: FinishReason) -> None:
+        self._release(req, RequestStatus.FINISHED, reason)
 
     def abort(self, request_id: str) -> Optional[Request]:
-        """Cancel a queued or running request (None for unknown or finished ids)."""
+        """Cancel a request wherever it is; None if the id is unknown or already finished."""
         req = self._by_id.get(request_id)
-        if req is None:
-            return None
-        self.finish(req, FinishReason.ABORTED)
+        if req is not None:
+            self._release(req, RequestStatus.FINISHED, FinishReason.ABORTED)
         return req
 
     @property
@@ -170,7 +208,7 @@ class Scheduler:
     def _serve_running(self, plan: SchedulerOutput, budget: int) -> int:
         """Give each running request its next token or portion; returns the budget left."""
         # Victims are taken from the end of this order, so its front always progresses.
-        self.running.sort(key=lambda r: (self._effective_priority(r), r.arrival_seq))
+        self.running.sort(key=lambda r: (self._class_of(r), r.arrival_seq))
         placed: set[str] = set()
         for req in tuple(self.running):
             if budget <= 0:
@@ -219,25 +257,20 @@ class Scheduler:
     def _place(self, plan: SchedulerOutput, req: Request, take: int) -> None:
         begin = req.num_computed_tokens
         plan.chunks.append(ScheduledChunk(req, begin, take, needs_logits=begin + take == req.num_tokens))
-        self._vtime[req.tenant] += take / self.config.tenant_weights.get(req.tenant, 1.0)
+        self.ledger.charge(req.tenant, take)
 
-    # ------------------------------------------------------------------ fairness
+    # ------------------------------------------------------------------ order of service
 
-    def _effective_priority(self, req: Request) -> int:
-        if self._step - req.arrival_step >= self.config.aging_steps:
-            return int(Priority.INTERACTIVE)
-        return int(req.priority)
+    def _class_of(self, req: Request) -> int:
+        """The request's priority class now (lower first); long waiting lifts any request to
+        the first class so that a stream of urgent requests cannot starve it."""
+        waited = self._step - req.arrival_step
+        return int(Priority.INTERACTIVE) if waited >= self.config.aging_steps else int(req.priority)
 
-    def _admission_key(self, req: Request) -> tuple[int, int, float, int]:
-        resumed = 0 if req.num_preemptions else 1  # preempted requests held a place already
-        return (self._effective_priority(req), resumed, self._vtime[req.tenant], req.arrival_seq)
-
-    def _activate_tenant(self, tenant: str) -> None:
-        """A tenant that was idle starts at the current virtual clock: no credit is banked."""
-        active = {r.tenant for r in self.waiting} | {r.tenant for r in self.running}
-        active.discard(tenant)
-        clock = min((self._vtime[t] for t in active), default=0.0)
-        self._vtime[tenant] = max(self._vtime.get(tenant, 0.0), clock)
+    def _admission_key(self, req: Request) -> tuple[int, bool, float, int]:
+        """Order of admission: class, then requests that lost their cache to a preemption (they
+        were running once) before new ones, then the tenant owed most, then arrival."""
+        return (self._class_of(req), req.num_preemptions == 0, self.ledger.owed(req.tenant), req.arrival_seq)
 
     # ------------------------------------------------------------------ memory pressure
 
@@ -246,20 +279,15 @@ class Scheduler:
         return next((r for r in reversed(self.running) if r.request_id not in exclude), None)
 
     def _preempt(self, req: Request) -> None:
-        self.manager.free(req.request_id)
-        self.running.remove(req)
-        req.status = RequestStatus.WAITING
-        req.num_computed_tokens = 0
-        req.num_preemptions += 1
-        self.waiting.appendleft(req)
+        self._release(req, RequestStatus.WAITING)
 
     def _reserve(self, req: Request) -> Optional[list[CopyOp]]:
-        """Reserve cache slots for tokens the manager has not seen (the newly sampled one)."""
-        missing = req.num_tokens - self.manager.num_tokens(req.request_id)
-        if missing <= 0:
+        """Cache slots for the tokens of ``req`` that the manager has not been told of yet (the
+        token sampled last step). The page copies this asks for, or None if no page is free."""
+        known, total = self.manager.num_tokens(req.request_id), req.num_tokens
+        if known >= total:
             return []
         try:
-            total = req.num_tokens
-            return self.manager.append_slots(req.request_id, req.token_slice(total - missing, total))
+            return self.manager.append_slots(req.request_id, req.token_slice(known, total))
         except NoFreePagesError:
             return None

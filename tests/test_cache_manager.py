@@ -11,7 +11,7 @@ import random
 import pytest
 
 from dli_amd.cache import (
-    RELEASED, CacheManager, CopyOp, CostAwarePolicy, GroupSpec, LRUPolicy, NoFreePagesError, NoFreeSlotError,
+    RELEASED, CacheManager, CopyOp, GroupSpec, OldestFirst, ReusedLast, NoFreePagesError, NoFreeSlotError,
     ROOT_PARENT, SequenceError, StateSlots, chain_hashes, page_hash,
 )
 
@@ -199,35 +199,46 @@ def test_page_identities():
     assert a[0] == want
 
 
-def test_reclaim_policies():
-    p = LRUPolicy()
+def test_reclaim_orders():
+    p = OldestFirst()
     for page in (1, 2, 3):
-        p.add_candidate(page)
-    p.remove_candidate(1)
-    p.add_candidate(1)
-    assert [p.pop_victim() for _ in range(3)] == [2, 3, 1]
+        p.offer(page)
+    p.withdraw(1)
+    p.offer(1)
+    assert [p.take() for _ in range(3)] == [2, 3, 1]
     with pytest.raises(LookupError):
-        p.pop_victim()
-    c = CostAwarePolicy(depth_weight=0.0)
-    c.on_cached(1, 0)
-    for _ in range(5):
-        c.on_hit(1)
-    c.add_candidate(1)
-    c.on_cached(2, 0)
-    c.add_candidate(2)
-    assert c.pop_victim() == 2  # a page hit often outlives a recent one-off
-    d = CostAwarePolicy(depth_weight=1.0)
-    d.on_cached(1, 10)
-    d.on_cached(2, 0)
-    d.add_candidate(1)
-    d.add_candidate(2)
-    assert d.pop_victim() == 2
-    e = CostAwarePolicy()
-    e.on_cached(7, 0)
-    for _ in range(10000):
-        e.add_candidate(7)
-        e.remove_candidate(7)
-    assert e.heap_size() < 200
+        p.take()
+    # a page that a later request found again outlives one-off pages however recent ...
+    r = ReusedLast()
+    for page in (1, 2, 3):
+        r.cached(page, 0)
+        r.offer(page)
+    r.found(1)
+    r.withdraw(1)          # revived by the request that found it
+    r.offer(1)             # and released again
+    r.cached(4, 0)
+    r.offer(4)
+    assert len(r) == 4 and [r.take() for _ in range(4)] == [2, 3, 4, 1]
+    with pytest.raises(LookupError):
+        r.take()
+    # ... but only as long as it keeps being found: one stay without a match and it is ordinary again
+    r.offer(1)
+    r.offer(5)
+    assert [r.take(), r.take()] == [1, 5]
+    # in a manager: the prefix two requests shared survives pressure that the one-off prompt does not
+    for order, kept in (("reuse", True), ("lru", False)):
+        m = CacheManager(num_pages=8, page_size=4, max_seqs=4, eviction_policy=order, watermark=0.0)
+        popular, one_off = list(range(8)), list(range(100, 108))
+        for rid, prompt in (("a", popular + [50]), ("b", popular + [51]), ("c", one_off + [52])):
+            m.allocate(rid, prompt)
+            m.mark_computed(rid, 9)
+            m.free(rid)
+        m.allocate("big", list(range(200, 224)))   # 6 of 8 pages: two of the four idle pages must go
+        m.free("big")
+        assert (m.allocate("again", popular + [1]).num_cached_tokens == 8) == kept, order
+        m.check_invariants()
+    with pytest.raises(ValueError):
+        CacheManager(num_pages=8, page_size=4, max_seqs=4, eviction_policy="newest")
 
 
 # ------------------------------------------------------------------ groups, windows, state slots
@@ -275,7 +286,7 @@ def test_state_slots_are_taken_and_given_back():
 # ------------------------------------------------------------------ random orders
 
 @pytest.mark.parametrize("seed", range(6))
-@pytest.mark.parametrize("policy", ["lru", "cost"])
+@pytest.mark.parametrize("policy", ["lru", "reuse"])
 def test_random_orders_of_requests_keep_every_invariant(seed, policy):
     rng = random.Random(seed)
     page_size = rng.choice([1, 2, 4, 8])

@@ -198,6 +198,33 @@ def test_priority_aging_and_tenant_shares():
     assert 8 <= served.count("big") <= 10 and 2 <= served.count("small") <= 4
 
 
+def test_tenant_ledger_banks_no_credit_and_preempted_requests_come_back_first():
+    from dli_amd.engine.scheduler import TenantLedger
+
+    led = TenantLedger({"heavy": 4.0})
+    led.enter("a", [])
+    led.charge("a", 100)
+    led.enter("heavy", ["a"])                 # arrives late: starts level with those present
+    assert led.owed("heavy") == led.owed("a") == 100.0
+    led.charge("heavy", 100)
+    assert led.owed("heavy") == 125.0         # a quarter of the charge for the same tokens
+    led.enter("a", ["heavy", "a"])            # present all along: keeps its own figure
+    assert led.owed("a") == 100.0
+    led.enter("idle", [])                     # nobody present: nothing to be lifted to
+    assert led.owed("idle") == 0.0
+    # a request that lost its cache is admitted before a new one of the same class
+    eng, runner, _ = make(num_pages=6, page_size=4, max_seqs=4, budget=64)
+    old = eng.add_request("old", list(range(9)), SamplingParams(max_tokens=12))
+    young = eng.add_request("young", list(range(20, 29)), SamplingParams(max_tokens=12))
+    while not young.num_preemptions:
+        eng.step()
+    late = eng.add_request("late", [5], SamplingParams(max_tokens=1))
+    run(eng)
+    firsts = [c.request.request_id for s in runner.calls for c in s.chunks if c.start == 0]
+    assert firsts.index("late") > len(firsts) - 1 - firsts[::-1].index("young")
+    assert old.num_preemptions == 0 and young.output_ids == alone(list(range(20, 29)), 12)
+
+
 # ------------------------------------------------------------------ random scenarios
 
 @pytest.mark.parametrize("seed", range(12))
