@@ -82,7 +82,7 @@ def cmd_random_weights(args: argparse.Namespace) -> int:
 
     config = json.loads(Path(args.config).read_text())
     out = write_random_model(args.out, config, seed=args.seed, std=args.std, norm_jitter=args.norm_jitter,
-                             storage=args.storage)
+                             storage=args.storage, device=args.device)
     print(out)
     return 0
 
@@ -114,6 +114,7 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     r.add_argument("--std", type=float, default=0.02)
     r.add_argument("--norm-jitter", type=float, default=0.0)
     r.add_argument("--storage", default="bfloat16", choices=["bfloat16", "float32"])
+    r.add_argument("--device", default="cpu", help="where the values are drawn (cpu, or cuda for large models)")
     r.set_defaults(fn=cmd_random_weights)
 
     t = sub.add_parser("trace", help="replay a trace of token ids (see bin/trace_run)", add_help=False)

@@ -50,11 +50,29 @@ def random_tensor(name: str, shape: tuple[int, ...], init: str, seed: int, std: 
     return out.reshape(shape)
 
 
+def _drawn_on_device(name: str, shape: tuple[int, ...], init: str, seed: int, std: float, norm_jitter: float,
+                     device: torch.device) -> torch.Tensor:
+    """The same distributions as :func:`random_tensor`, drawn by the device's generator (other
+    values for the same seed): float32 on ``device``."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode("utf-8"))) & 0x7FFFFFFFFFFFFFFF)
+    if init == "zeros":
+        return torch.zeros(shape, dtype=torch.float32, device=device)
+    if init in ("ones", "norm"):
+        out = torch.ones(shape, dtype=torch.float32, device=device)
+        if init == "norm" and norm_jitter:
+            out += norm_jitter * torch.empty(shape, dtype=torch.float32, device=device).normal_(generator=gen)
+        return out
+    return torch.empty(shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+
+
 def write_random_model(out_dir: str | Path, config: Mapping[str, Any] | Any, *, seed: int = 0,
                        std: float = 0.02, norm_jitter: float = 0.0,
-                       storage: str = "bfloat16") -> Path:
+                       storage: str = "bfloat16", device: str | torch.device = "cpu") -> Path:
     """Write ``config.json`` and ``model.safetensors`` for ``config`` (a config.json dictionary,
-    or a typed configuration with ``to_hf_dict``) with weights drawn from ``seed``."""
+    or a typed configuration with ``to_hf_dict``) with weights drawn from ``seed``. With a GPU as
+    ``device`` the values are drawn there (seconds instead of minutes for a billion weights; the
+    values are that generator's, not the host generator's)."""
     raw = dict(config.to_hf_dict()) if hasattr(config, "to_hf_dict") else dict(config)
     if storage not in ("bfloat16", "float32"):
         raise ValueError("storage must be 'bfloat16' or 'float32'")
@@ -65,6 +83,13 @@ def write_random_model(out_dir: str | Path, config: Mapping[str, Any] | Any, *, 
     for name, spec in model.weight_specs().items():
         if spec.role == "int32":
             tensors[name] = ("I32", np.zeros(spec.shape, np.int32))
+            continue
+        if torch.device(device).type != "cpu":
+            t = _drawn_on_device(name, tuple(spec.shape), spec.init, seed, std, norm_jitter, torch.device(device))
+            if storage == "bfloat16":
+                tensors[name] = ("BF16", t.to(torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16))
+            else:
+                tensors[name] = ("F32", t.cpu().numpy())
             continue
         values = random_tensor(name, tuple(spec.shape), spec.init, seed, std, norm_jitter)
         if storage == "bfloat16":

@@ -177,7 +177,7 @@ def write_safetensors(
     header: dict[str, object] = {}
     if metadata:
         header["__metadata__"] = {str(k): str(v) for k, v in metadata.items()}
-    blobs: list[bytes] = []
+    blobs: list[np.ndarray] = []  # written straight from the arrays' memory, no second copy
     offset = 0
     for name in sorted(tensors):
         tag, arr = tensors[name]
@@ -187,14 +187,15 @@ def write_safetensors(
         arr = np.ascontiguousarray(arr)
         if arr.dtype.itemsize != dt.itemsize:
             raise SafetensorsFormatError(f"{name!r}: array of {arr.dtype} cannot be stored as {tag}")
-        raw = arr.astype(dt, copy=False).tobytes() if arr.dtype != dt else arr.tobytes()
-        header[name] = {"dtype": tag, "shape": list(arr.shape), "data_offsets": [offset, offset + len(raw)]}
+        raw = np.ascontiguousarray(arr.astype(dt, copy=False) if arr.dtype != dt else arr)
+        header[name] = {"dtype": tag, "shape": list(arr.shape), "data_offsets": [offset, offset + raw.nbytes]}
         blobs.append(raw)
-        offset += len(raw)
+        offset += raw.nbytes
     text = json.dumps(header, separators=(",", ":")).encode("utf-8")
     text += b" " * ((-len(text)) % 8)
     with open(path, "wb") as fh:
         fh.write(struct.pack("<Q", len(text)))
         fh.write(text)
         for b in blobs:
-            fh.write(b)
+            if b.nbytes:
+                fh.write(memoryview(b.reshape(-1)).cast("B"))

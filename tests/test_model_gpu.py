@@ -43,7 +43,10 @@ def make_core(name: str, dtype: str, num_pages: int, page_size: int):
     return core
 
 
-def check(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str) -> None:
+def check(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str, mean_rtol: float = MEAN_RTOL) -> None:
+    """Every logit within the type's bound of the plain one; in bfloat16 also the rows' errors on
+    average (``mean_rtol`` of a row's largest logit: the default suits models of a few layers, a
+    deep model brings a bound measured for its depth)."""
     atol, rtol = TOL[dtype]
     got, ref = got.double().cpu(), ref.double()
     bound = atol + rtol * ref.abs().max(dim=-1, keepdim=True).values
@@ -53,8 +56,8 @@ def check(got: torch.Tensor, ref: torch.Tensor, dtype: str, what: str) -> None:
     assert worst <= 1.0, f"{what}: error {err.max().item():.3e} exceeds the bound by x{worst:.2f}"
     if rtol and got.shape[0] >= 8:
         mean = (err.max(dim=-1).values / ref.abs().max(dim=-1).values).mean().item()
-        WORST[dtype + " mean"] = max(WORST.get(dtype + " mean", 0.0), mean / MEAN_RTOL)
-        assert mean <= MEAN_RTOL, f"{what}: rows differ by {mean:.3f} of their largest logit on average"
+        WORST[dtype + " mean"] = max(WORST.get(dtype + " mean", 0.0), mean / mean_rtol)
+        assert mean <= mean_rtol, f"{what}: rows differ by {mean:.3f} of their largest logit on average"
 
 
 _plain_cache: dict = {}
@@ -75,7 +78,8 @@ def prompts_for(name: str, lengths, seed=5):
 
 
 CASES = [("A", 16, "float32"), ("A", 16, "bfloat16"), ("B", 8, "float32"), ("B", 8, "bfloat16"),
-         ("C", 4, "float32"), ("C", 32, "bfloat16"), ("D", 16, "bfloat16")]
+         ("C", 4, "float32"), ("C", 32, "bfloat16"), ("D", 16, "bfloat16"), ("H", 16, "float32"),
+         ("H", 16, "bfloat16")]
 
 
 @pytest.mark.parametrize("name,page,dtype", CASES)
@@ -271,7 +275,7 @@ def test_long_context_in_portions_then_decoding(name, page, dtype):
         check(got, ref[i:i + 1], dtype, f"{name} decode at {i}")
 
 
-@pytest.mark.parametrize("name,page", [("A", 16), ("B", 16), ("D", 16)])
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 16), ("D", 16), ("H", 16)])
 def test_the_same_traces_with_decode_graphs_on(name, page, monkeypatch):
     """Serving replays decode-only steps as HIP graphs of a padded, fixed shape. The traces above
     once more with that switched on (as bin/trace_run has it): the logits must still be the plain

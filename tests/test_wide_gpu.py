@@ -87,3 +87,41 @@ def test_eight_requests_decode_together_at_serving_widths():
         for r in range(8):
             fed[r] += 1
     assert core.step.graphs.replays >= 10
+
+
+def test_llama_3_2_1b_at_full_depth_and_vocabulary():
+    """All 16 layers and all 128,256 vocabulary rows of Llama-3.2-1B (random weights written to a
+    folder and loaded by name like a checkpoint), 32-bit and bfloat16 against the plain
+    implementation in 64-bit: the prompt whole, then its last tokens one by one (the reference's
+    parity bound is tests/unit/model/test_reference_parity.py:20; here the bounds are those of
+    every other whole-model test)."""
+    from dli_amd.engine.core import build_core
+    from dli_amd.trace import TraceSession
+
+    folder = model_folder("1B", device="cuda")  # a billion weights: drawn on the GPU
+    rng = random.Random(8)
+    toks = [rng.randrange(128256) for _ in range(64)]
+    cfg, w = P.load_folder(folder)
+    assert cfg["num_hidden_layers"] == 16 and w["model.embed_tokens.weight"].shape == (128256, 2048)
+    ref = P.forward_logits(w, cfg, toks)
+    # Rounding adds up over 16 layers: how far bfloat16 may drift on average is measured, not
+    # guessed, by evaluating the plain implementation itself in bfloat16. The engine accumulates
+    # in 32-bit where that evaluation rounds, so it must not be further from the 64-bit logits.
+    rounded = P.forward_logits(w, cfg, toks, dtype=torch.bfloat16).double()
+    drift = ((rounded - ref).abs().max(dim=-1).values / ref.abs().max(dim=-1).values).mean().item()
+    assert 0.01 < drift < 0.08, drift
+    del w, rounded
+    for dtype in ("float32", "bfloat16"):
+        core = build_core(folder, num_pages=8, page_size=16, max_seqs=2, dtype=dtype,
+                          enable_prefix_caching=False, watermark=0.0)
+        core.step.enable_decode_graphs(1, 128)
+        s = TraceSession(core)
+        got = s.step([{"id": "p", "tokens": toks, "want": list(range(64))}], end=["p"])
+        check(got, ref, dtype, f"1B whole {dtype}", mean_rtol=drift)
+        got = s.step([{"id": "d", "tokens": toks[:56], "want": [55]}])
+        check(got, ref[55:56], dtype, f"1B prefix {dtype}")
+        for i in range(56, 64):
+            got = s.step([{"id": "d", "tokens": [toks[i]], "want": [0]}])
+            check(got, ref[i:i + 1], dtype, f"1B decode at {i} {dtype}")
+        del core, s
+        torch.cuda.empty_cache()

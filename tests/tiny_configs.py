@@ -52,7 +52,19 @@ TINY_D = {
                      "original_max_position_embeddings": 128},
     "attention_bias": True, "tie_word_embeddings": True, "hidden_act": "silu",
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "W": WIDE}
+# heads of 128 (the head size of Llama-3.2-3B) in groups of three on one and two kv heads' worth of
+# width: the projections are wider than the model (6 x 128 on a width of 384), vocabulary odd
+TINY_H = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 331, "hidden_size": 384,
+    "intermediate_size": 640, "num_hidden_layers": 2, "num_attention_heads": 6, "num_key_value_heads": 2,
+    "head_dim": 128, "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 256},
+    "tie_word_embeddings": True, "hidden_act": "silu",
+}
+# Llama-3.2-1B as config.json has it: every layer and the whole vocabulary
+LLAMA_3_2_1B = dict(WIDE, vocab_size=128256, num_hidden_layers=16)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "H": TINY_H, "W": WIDE, "1B": LLAMA_3_2_1B}
 
 _made: dict = {}
 _tmp = None
@@ -62,20 +74,21 @@ _tmp = None
 # have a spread of about one, so attention is far from uniform (a key in the wrong place, a wrong
 # rotation or a wrong mask changes the logits) without being so sharp that bfloat16's rounding of a
 # score is blown up into a different distribution.
-STD = {"A": 0.15, "B": 0.085, "C": 0.085, "D": 0.075, "W": 0.0265}
+STD = {"A": 0.15, "B": 0.085, "C": 0.085, "D": 0.075, "H": 0.06, "W": 0.0265, "1B": 0.0265}
 
 
-def model_folder(name: str, seed: int = 11, std: float | None = None, norm_jitter: float = 0.1) -> Path:
+def model_folder(name: str, seed: int = 11, std: float | None = None, norm_jitter: float = 0.1,
+                 device: str = "cpu") -> Path:
     """A temporary folder with config.json and model.safetensors of configuration ``name``."""
     from dli_amd.weights import write_random_model
 
     global _tmp
     std = STD[name] if std is None else std
-    key = (name, seed, std, norm_jitter)
+    key = (name, seed, std, norm_jitter, device)
     if key not in _made:
         if _tmp is None:
             _tmp = tempfile.TemporaryDirectory(prefix="dli_amd_tiny_")
-        out = Path(_tmp.name) / f"{name}_{seed}_{std}_{norm_jitter}"
-        write_random_model(out, CONFIGS[name], seed=seed, std=std, norm_jitter=norm_jitter)
+        out = Path(_tmp.name) / f"{name}_{seed}_{std}_{norm_jitter}_{device}"
+        write_random_model(out, CONFIGS[name], seed=seed, std=std, norm_jitter=norm_jitter, device=device)
         _made[key] = out
     return _made[key]
