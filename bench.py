@@ -289,9 +289,21 @@ def main() -> int:
         line["prefill"] = {"value": round(2048 / t, 1), "tokens": 2048, "ms": round(t * 1e3, 3),
                            "frac": round(prefill_flops(cfg, 2048) / t / PEAK_FLOPS[short], 4)}
         points = {}
-        for b in (1, 64):
-            steps = min(args.steps, 32)
-            points[f"decode_b{b}"] = round(decode_run(engine, cfg, b, args.context, steps, min(args.warmup, 4), args.decode_steps)[0], 1)
+        steps, warm = min(args.steps, 32), min(args.warmup, 4)
+
+        def point(key, b, context, per_call):
+            tok_s, ms, _ = decode_run(engine, cfg, b, context, steps, warm, per_call)
+            points[key] = round(tok_s, 1)
+            points[key + "_ms"] = round(ms, 4)
+            points[key + "_frac"] = round(decode_bytes(cfg, b, context, itemsize) / (ms * 1e-3) / 1e9 / HBM_GBPS, 4)
+
+        for b in (1, 64):   # the headline's context, other batch sizes
+            point(f"decode_b{b}", b, args.context, args.decode_steps)
+        for b in (1, 8, 64):
+            # one token per engine step, the default of generate() and of the command line
+            point(f"decode_b{b}_one_token_per_call", b, args.context, 1)
+            # prompts of 2,048 tokens with 256 generated: the context grows from 2,048 to 2,304
+            point(f"decode_b{b}_context2304", b, 2304, args.decode_steps)
         line["points"] = points
     print(json.dumps(line))
     return 0
