@@ -174,6 +174,41 @@ class DecodeGraphs:
                 gc.enable()
         return _Captured(graph, ctx, host, dev, logits, views, width, TableRows(b, width, self.n_groups), tokens_host)
 
+    def _shape_key(self, requests: int, max_kv: int, sampled: bool, steps: int) -> tuple[int, int, int, bool, int]:
+        """The captured shape that serves ``requests`` requests of which the longest will hold
+        ``max_kv`` keys: (padded batch, key splits, block-table width, sampled, steps)."""
+        b = _bucket(requests)
+        width = max(16, _bucket(-(-max_kv // self.step_fn.manager.page_size)))
+        splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv,
+                                       ops.compute_units(self.step_fn.rt.device)))
+        return (b, splits, width, sampled, steps)
+
+    def warm_up(self, batches: Sequence[int], max_len: int, *, sampled: bool = True,
+                steps: Sequence[int] = (1,)) -> int:
+        """Capture now every graph that decode steps of ``batches`` requests with up to ``max_len``
+        keys can ask for, so that no capture (two eager forwards and a recording) falls between
+        two tokens of a live request later. Returns the number of graphs captured by this call."""
+        if not self.enabled:
+            return 0
+        ps = self.step_fn.manager.page_size
+        max_len = min(int(max_len), self.max_width * ps)
+        keys = set()
+        for n in batches:
+            if not 0 < n <= self.max_batch:
+                raise ValueError(f"batch {n} outside 1..{self.max_batch}")
+            for k in steps:
+                # the shape changes only just after the page count passes a power of two and where the
+                # key count reaches a multiple of 128 (the unit of the split rule)
+                edges = {*range(128, max_len + 1, 128), *(ps * 2 ** i for i in range(32) if ps * 2 ** i <= max_len)}
+                for kv in sorted({1, max_len, *edges, *(e + 1 for e in edges if e < max_len)}):
+                    keys.add(self._shape_key(n, kv, sampled, k))
+        made = 0
+        for key in sorted(keys):
+            if key not in self.captured:
+                self.captured[key] = self._capture(*key)
+                made += 1
+        return made
+
     # ------------------------------------------------------------------ replay
 
     def run(self, entries: Sequence[StepEntry], sampling: Optional[Sequence[tuple]] = None, steps: int = 1):
@@ -184,18 +219,15 @@ class DecodeGraphs:
         steps in a row and one list per step comes back (the block tables must already hold the
         pages of all positions that will be written)."""
         mgr = self.step_fn.manager
-        ps, n = mgr.page_size, len(entries)
-        b = _bucket(n)
-        max_kv = max(e.start + steps for e in entries)
-        width = max(16, _bucket(-(-max_kv // ps)))
-        splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv, ops.compute_units(self.step_fn.rt.device)))
+        n = len(entries)
         sampled = sampling is not None
         if steps > 1 and not sampled:
             raise ValueError("several steps in a row need the sampling parameters")
-        key = (b, splits, width, sampled, steps)
+        key = self._shape_key(n, max(e.start + steps for e in entries), sampled, steps)
+        b = key[0]
         cap = self.captured.get(key)
         if cap is None:
-            cap = self.captured[key] = self._capture(b, splits, width, sampled, steps)
+            cap = self.captured[key] = self._capture(*key)
         v = cap.views
         limit = self.step_fn.store.num_pages
         token_ids, positions, kv_len, state_slots = v["token_ids"], v["positions"], v["kv_len"], v["state_slots"]

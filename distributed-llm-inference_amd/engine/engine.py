@@ -170,6 +170,17 @@ class LLMEngine:
 
     # ------------------------------------------------------------------ API
 
+    def warm_up(self, batches: Sequence[int], max_len: int) -> int:
+        """Capture the decode graphs that steps of ``batches`` running requests with contexts up to
+        ``max_len`` tokens will replay (for every number of tokens per step that the scheduler may
+        choose), before the first request arrives. Returns how many graphs were captured; 0 for an
+        engine without graph replay."""
+        graphs = getattr(getattr(getattr(self, "core", None), "step", None), "graphs", None)
+        if graphs is None:
+            return 0
+        k = self.scheduler.config.decode_steps
+        return graphs.warm_up(batches, max_len, sampled=True, steps=tuple(range(1, k + 1)))
+
     def add_request(self, request_id: str, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None, *,
                     priority: Priority = Priority.INTERACTIVE, tenant: str = "default") -> Request:
         """Queue a request. One that can never fit finishes at once with CAPACITY."""

@@ -382,6 +382,32 @@ def test_trace_run_program(tmp_path):
     assert proc.returncode != 0 and "NoFreePagesError" in proc.stderr
 
 
+def test_warm_up_captures_every_graph_that_serving_then_replays():
+    """After ``warm_up`` no decode step captures a graph: requests of several lengths and batch
+    sizes, one and several tokens per step, only replay what exists, and the tokens are the plain
+    implementation's."""
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    name = "D"
+    for k in (1, 4):
+        eng = LLMEngine.for_model(str(model_folder(name)), dtype="bfloat16", num_blocks=96, block_size=16,
+                                  enable_prefix_caching=False,
+                                  config=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=256, decode_steps=k))
+        graphs = eng.core.step.graphs
+        made = eng.warm_up([1, 2, 3, 4], 420)
+        assert made == len(graphs.captured) > 0 and eng.warm_up([1, 2, 3, 4], 420) == 0
+        before = set(graphs.captured)
+        ps = prompts(name, [5, 250, 300, 130], seed=61)
+        reqs = [eng.add_request(f"r{i}", p, SamplingParams(max_tokens=70 + 9 * i)) for i, p in enumerate(ps)]
+        while eng.has_unfinished():
+            eng.step()
+        assert set(graphs.captured) == before, set(graphs.captured) - before
+        assert graphs.replays > 20
+        for r, p in zip(reqs, ps):
+            assert_same_or_near_tie(name, p, r.output_ids, plain_greedy(name, p, len(r.output_ids)), margin=0.25)
+
+
 def test_generate_command_line(tmp_path):
     """``python -m dli_amd random-weights`` then ``... generate`` as a user runs them (the reference's
     flag names, src/dli/server/__main__.py:65-124): the printed ids are the plain implementation's."""
