@@ -1,0 +1,466 @@
+// Matrix product for a decode step of 17 to 64 rows (it takes 1 to 64):
+//   y[m][n] = sum_k xhat[m][k] * w[n][k]
+// With this many rows the activations are no longer small beside the weights: a workgroup that
+// owns few features and reads every row for them moves more activation bytes than weight bytes.
+// So the activations of a block of 128 k are brought into LDS once per workgroup (normalised on
+// the way, if a norm is asked for) and shared by its waves, each of which owns 16 features (two
+// sets of 16 for the gated product), and k is split over workgroups (grid.y) until the launch
+// fills the chip. A split launch leaves its 32-bit partial products in [split][m][n]; the
+// elementwise kernel that has to run after the product anyway (residual sum, or rotation and
+// cache write) adds them up in the order of the splits, so the result does not depend on timing.
+//
+// Products run on the matrix cores as in the kernel for few rows:
+//   acc[16 n x 16 m] += W[16 n x 32 k] * xhat^T[32 k x 16 m]      (v_mfma_f32_16x16x32_bf16)
+// lane l supplies feature/row l%16 and eight k values; inside a block of 128 k lane group g = l/16
+// takes the run [32g, 32g+32) and product q of the block its q-th run of eight (the same
+// permutation for both operands). Weights come either row by row or in the tile order
+//   t[tile][block][q][g][c][8] = w[16*tile + c][128*block + 32*g + 8*q + (0..7)]
+// (every load of a wave is then 1 KB of consecutive memory); both are a base and two strides here.
+// Weight loads go straight to registers, two blocks ahead of their use.
+//
+//   norm        xhat = cast(norm_w[k] * cast(x[m][k] * rs[m])), rs[m] = rsqrt(sum_k x^2 / K + eps)
+//               from the parts of the row's sum of squares that the producer of x left
+//               (RMSNorm: src/dli/model/llama.py:40-44); otherwise xhat = x
+//   MID_PARTIAL float32 [split][m][n], no bias
+//   MID_STORE   cast(y + bias)                                  (one split only)
+//   MID_SWIGLU  cast(silu(cast(gate))) * cast(up), rows n and n + up_offset of w
+//               (src/dli/model/llama.py:190)                    (one split only)
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+enum { MID_PARTIAL = 0, MID_SWIGLU = 1, MID_STORE = 2 };
+
+namespace {
+
+__device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+constexpr int XPAD = 8;                // elements: rows of the staged block start 16 bytes apart in the banks
+constexpr int XROW = 128 + XPAD;
+
+struct MidArgs {
+  const bf16_t* x; int64_t ldx;
+  const float* ssq_in; int ssq_parts; const float* norm_w; float eps;
+  const bf16_t* w; int tiled;
+  const bf16_t* bias; void* out; int64_t ldo;
+  int M, N, K, up_offset, splits;
+};
+
+// MT row tiles of 16; NW x KW waves: wave (nw, kw) owns 16 features (NW tiles a workgroup) and
+// every KW-th block of the workgroup's range of k, so that a compute unit has many waves, each
+// with its next blocks of weights in flight, from the first cycle on: these launches last only a
+// few trips to memory, and what bounds them is how many bytes are under way. The NW waves of one
+// kw share that block's activations through LDS; the KW partial tiles of a feature tile meet in
+// LDS at the end and are added in the order of kw. grid (ceil(tiles / NW), splits).
+template <int MT, int NW, int KW, int EPI>
+__global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
+  constexpr int NA = EPI == MID_SWIGLU ? 2 : 1;
+  constexpr int NG = NW * 64;          // threads that stage one kw's blocks
+  constexpr int ROWS = 16 * MT;
+  constexpr int PP = ROWS * 16 / NG;   // 16-byte pieces of a block that one thread stages
+  static_assert(ROWS * 16 % NG == 0, "the block's pieces divide among the threads");
+  constexpr int XS_BYTES = 2 * KW * ROWS * XROW * 2;
+  constexpr int RED_BYTES = (KW - 1) * NW * NA * MT * 4 * 64 * 4;
+  __shared__ __attribute__((aligned(16))) char smem[XS_BYTES > RED_BYTES ? XS_BYTES : RED_BYTES];
+  __shared__ float rs_s[ROWS];
+  typedef bf16_t XBuf[KW][ROWS][XROW];
+  XBuf* xs = reinterpret_cast<XBuf*>(smem);                     // xs[buffer][kw][row][k]
+
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int nw = wave % NW, kw = wave / NW;
+  const int gtid = threadIdx.x % NG;   // thread within the kw group (its waves are consecutive)
+  const int col = lane % 16, grp = lane / 16;
+  const int M = p.M, N = p.N, K = p.K;
+  const int tiles = (N + 15) / 16;
+  const int tile = blockIdx.x * NW + nw;
+  const bool owns = tile < tiles;
+  const int split = blockIdx.y;
+  const int nblk = K / 128;
+  const int b0 = (int)((int64_t)nblk * split / p.splits), b1 = (int)((int64_t)nblk * (split + 1) / p.splits);
+  const int cnt = b1 - b0;
+  const int steps = (cnt + KW - 1) / KW;       // the same for every wave: all keep the barriers
+  // Workgroups start at different blocks of their range and wrap around: launched together and
+  // running in step, they would otherwise all ask for the same offsets inside their weights'
+  // 64 KB regions (and for the same activations) at the same time, which lands on few memory
+  // channels. The order of a feature's sum thus depends on its tile, never on the rows.
+  const int rot = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)cnt);
+  auto block_of = [&](int step) {
+    const int j = step * KW + kw;
+    if (j >= cnt) return b1;                   // beyond the range: nothing to do in this step
+    const int r = j + rot;
+    return b0 + (r >= cnt ? r - cnt : r);
+  };
+
+  // this lane's first weight fragment and the steps to the next block and product
+  const bf16_t* wbase[NA];
+  const int blk_stride = p.tiled ? 2048 : 128, q_stride = p.tiled ? 512 : 8;
+#pragma unroll
+  for (int a = 0; a < NA; ++a) {
+    const int tl = min(tile, tiles - 1);
+    if (p.tiled) {
+      wbase[a] = p.w + (int64_t)(tl + a * (p.up_offset / 16)) * 16 * K + lane * 8;
+    } else {
+      const int n = min(tl * 16 + col, N - 1) + a * p.up_offset;
+      wbase[a] = p.w + (int64_t)n * K + grp * 32;
+    }
+  }
+  bf16x8 wf[3][NA][4];
+  auto load_w = [&](bf16x8 (&dst)[NA][4], int b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        dst[a][q] = *reinterpret_cast<const bf16x8*>(wbase[a] + (int64_t)b * blk_stride + q * q_stride);
+  };
+  const bool norm = p.norm_w != nullptr;
+
+  // staging: piece i of this thread is eight k of one row of its kw's block
+  int prow[PP], pk[PP];
+#pragma unroll
+  for (int i = 0; i < PP; ++i) {
+    const int piece = gtid + i * NG;
+    prow[i] = piece / 16;
+    pk[i] = (piece % 16) * 8;
+  }
+  // every piece of a thread covers the same eight columns of the block (the group's thread
+  // count is a multiple of 16), so one pair of norm-weight vectors serves them all
+  struct Staged {
+    bf16x8 v[PP];
+    float4v nw0, nw1;
+  };
+  auto fetch_x = [&](Staged& st, int b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < PP; ++i) {
+      st.v[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (prow[i] < M) st.v[i] = *reinterpret_cast<const bf16x8*>(p.x + (int64_t)prow[i] * p.ldx + b * 128 + pk[i]);
+    }
+    if (norm) {
+      st.nw0 = *reinterpret_cast<const float4v*>(p.norm_w + b * 128 + pk[0]);
+      st.nw1 = *reinterpret_cast<const float4v*>(p.norm_w + b * 128 + pk[0] + 4);
+    }
+  };
+  auto stash_x = [&](const Staged& st, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < PP; ++i) {
+      bf16x8 v = st.v[i];
+      if (norm) {
+        const float r = rs_s[prow[i]];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float normed = (float)(bf16_t)((float)st.v[i][e] * r);
+          v[e] = (bf16_t)((e < 4 ? st.nw0[e] : st.nw1[e - 4]) * normed);
+        }
+      }
+      *reinterpret_cast<bf16x8*>(&xs[buf][kw][prow[i]][pk[i]]) = v;
+    }
+  };
+
+  float4v acc[NA][MT];
+#pragma unroll
+  for (int a = 0; a < NA; ++a)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[a][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // Memory answers in the order of the requests, so a wait for one load is a wait for all older
+  // ones: the activations of a block are therefore requested before the weights of the same
+  // step, two steps ahead like them, and what a step waits for is always the oldest request.
+  // A wave whose block lies beyond the range (the last step of an uneven split) stages and
+  // multiplies nothing but keeps every barrier.
+  Staged sx[2];
+  if (block_of(0) < b1) {
+    fetch_x(sx[0], block_of(0));
+    load_w(wf[0], block_of(0));
+  }
+  if (block_of(1) < b1) {
+    fetch_x(sx[1], block_of(1));
+    load_w(wf[1], block_of(1));
+  }
+  // rs[m] from the parts of sum x^2, added in the order of the parts
+  if (norm) {
+    for (int m = threadIdx.x; m < ROWS; m += NW * KW * 64) {
+      float sum = 0.f;
+      if (m < M)
+        for (int part = 0; part < p.ssq_parts; ++part) sum += p.ssq_in[(int64_t)part * M + m];
+      rs_s[m] = rsqrtf(sum / (float)K + p.eps);
+    }
+    __syncthreads();
+  }
+  if (block_of(0) < b1) stash_x(sx[0], 0);
+  __syncthreads();
+  for (int s0 = 0; s0 < steps; s0 += 6) {
+#pragma unroll
+    for (int r = 0; r < 6; ++r) {
+      const int step = s0 + r;
+      if (step >= steps) break;
+      const int buf = r & 1;
+      if (block_of(step + 2) < b1) {
+        fetch_x(sx[r & 1], block_of(step + 2));   // the slot of this step's block, which lies in LDS by now
+        load_w(wf[(r + 2) % 3], block_of(step + 2));
+      }
+      if (block_of(step) < b1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][kw][16 * t + col][32 * grp + 8 * q]);
+#pragma unroll
+            for (int a = 0; a < NA; ++a) acc[a][t] = mfma32(wf[r % 3][a][q], xf, acc[a][t]);
+          }
+      }
+      if (block_of(step + 1) < b1) stash_x(sx[(r + 1) & 1], buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // the kw waves of a feature tile hand their partial tiles to wave kw == 0, which adds them in
+  // the order of kw (the staged activations are done with: their memory is reused)
+  if constexpr (KW > 1) {
+    typedef float Red[NW][NA][MT][4][64];
+    Red* red = reinterpret_cast<Red*>(smem);
+    if (kw != 0) {
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) red[kw - 1][nw][a][t][i][lane] = acc[a][t][i];
+    }
+    __syncthreads();
+    if (kw != 0) return;
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          for (int k2 = 0; k2 < KW - 1; ++k2) acc[a][t][i] += red[k2][nw][a][t][i][lane];
+  }
+
+  // lane holds y[m = 16t + col][n = 16*tile + 4*grp + i]
+  if (!owns) return;
+  const int nb = tile * 16 + 4 * grp;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = 16 * t + col;
+    if (m >= M || nb >= N) continue;
+    if constexpr (EPI == MID_PARTIAL) {
+      float* dst = reinterpret_cast<float*>(p.out) + ((int64_t)split * M + m) * p.ldo + nb;
+      if (nb + 3 < N) {
+        *reinterpret_cast<float4v*>(dst) = acc[0][t];
+      } else {
+        for (int i = 0; i < 4 && nb + i < N; ++i) dst[i] = acc[0][t][i];
+      }
+    } else {
+      bf16_t* dst = reinterpret_cast<bf16_t*>(p.out) + (int64_t)m * p.ldo + nb;
+      bf16_t r[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = min(nb + i, N - 1);
+        float y0 = acc[0][t][i];
+        if (p.bias != nullptr) y0 += (float)p.bias[n];
+        if constexpr (EPI == MID_SWIGLU) {
+          float y1 = acc[NA - 1][t][i];
+          if (p.bias != nullptr) y1 += (float)p.bias[n + p.up_offset];
+          const float g = (float)(bf16_t)y0, u = (float)(bf16_t)y1;
+          r[i] = (bf16_t)((float)(bf16_t)silu<bf16_t>(g) * u);
+        } else {
+          r[i] = (bf16_t)y0;
+        }
+      }
+      if (nb + 3 < N) {
+        *reinterpret_cast<bf16x4*>(dst) = bf16x4{r[0], r[1], r[2], r[3]};
+      } else {
+        for (int i = 0; i < 4 && nb + i < N; ++i) dst[i] = r[i];
+      }
+    }
+  }
+}
+
+// The splits' values of four neighbouring features, added in the order of the splits; the loads
+// are issued eight at a time so that they share one trip to memory.
+__device__ __forceinline__ float4v sum_splits(const float* __restrict__ src, int splits, int64_t split_stride) {
+  float4v y = float4v{0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float4v v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      v[u] = s0 + u < splits ? *reinterpret_cast<const float4v*>(src + (s0 + u) * split_stride) : float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < splits) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i] = s0 + u == 0 ? v[u][i] : y[i] + v[u][i];
+      }
+  }
+  return y;
+}
+
+// stream[m][n] = cast(stream[m][n] + cast(sum_s partial[s][m][n] + bias[n])), the splits added in
+// their order, and ssq_out[part][m] = the sum of stream[m][n]^2 over the part's 1024 features, for
+// the norm that follows. One workgroup per row and part.
+__global__ __launch_bounds__(256) void mid_finish_residual_kernel(
+    const float* __restrict__ partial, int splits, const bf16_t* __restrict__ bias,
+    bf16_t* __restrict__ stream, int64_t lds_, float* __restrict__ ssq_out, int M, int N) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x, part = blockIdx.y;   // a part of a row: 1024 features
+  const int64_t split_stride = (int64_t)M * N;
+  const int n = part * 1024 + threadIdx.x * 4;
+  float sq = 0.f;
+  if (n < N) {
+    bf16_t* sp = stream + (int64_t)m * lds_ + n;
+    const bf16x4 old = *reinterpret_cast<const bf16x4*>(sp);
+    const float4v y = sum_splits(partial + (int64_t)m * N + n, splits, split_stride);
+    bf16x4 res;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float b = bias != nullptr ? (float)bias[n + i] : 0.f;
+      res[i] = (bf16_t)((float)old[i] + (float)(bf16_t)(y[i] + b));
+      sq += (float)res[i] * (float)res[i];
+    }
+    *reinterpret_cast<bf16x4*>(sp) = res;
+  }
+  const float total = block_sum(sq, scratch);
+  if (threadIdx.x == 0) ssq_out[(int64_t)part * M + m] = total;
+}
+
+// The fused q/k/v projection's partial products [split][m][n], n in the feature order of the
+// product that rotates (tile t of a q or k head holds the head's dimensions 8t..8t+7 and
+// half+8t..half+8t+7; v heads in their own order): the splits are added in their order, the bias
+// (same order) joins, q and k are rotated (src/dli/model/rope.py:50-70: pairs (i, i + half), cos
+// and sin of the row's position from `angles` [M][2][half]), q goes to out[m][head*d + dim] and
+// rotated k and v to the cache pages at slots[m] (negative: not cached). grid (rows, workgroups
+// that share a row's items); an item is four rotary pairs of a head, or four dimensions of a v head.
+__global__ __launch_bounds__(256) void mid_finish_qkv_kernel(
+    const float* __restrict__ partial, int splits, const bf16_t* __restrict__ bias,
+    const float* __restrict__ angles, const int* __restrict__ slots, bf16_t* __restrict__ out,
+    int64_t ldo, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int M, int q_heads,
+    int kv_heads, int d, int page_size) {
+  const int m = blockIdx.x;
+  const int half = d / 2, N = (q_heads + 2 * kv_heads) * d;
+  const int64_t split_stride = (int64_t)M * N;
+  const int rot_items = (q_heads + kv_heads) * (half / 4), v_items = kv_heads * (d / 4);
+  const int slot = slots[m];
+  const int64_t page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot - (int)page * page_size : 0;
+  auto summed = [&](int n) __attribute__((always_inline)) {
+    float4v y = sum_splits(partial + (int64_t)m * N + n, splits, split_stride);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) y[i] = (float)(bf16_t)(y[i] + (bias != nullptr ? (float)bias[n + i] : 0.f));
+    return y;
+  };
+  for (int item = blockIdx.y * 256 + threadIdx.x; item < rot_items + v_items; item += 256 * gridDim.y) {
+    if (item < rot_items) {
+      const int head = item / (half / 4), j = (item % (half / 4)) * 4;   // pairs j..j+3 of the head
+      const int pos = head * d + 16 * (j / 8) + j % 8;                   // where pair j's first member lies
+      const float4v a = summed(pos), b = summed(pos + 8);
+      const float4v cs = *reinterpret_cast<const float4v*>(angles + ((int64_t)m * 2 + 0) * half + j);
+      const float4v sn = *reinterpret_cast<const float4v*>(angles + ((int64_t)m * 2 + 1) * half + j);
+      bf16x4 lo, hi;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lo[i] = (bf16_t)(a[i] * cs[i] - b[i] * sn[i]);
+        hi[i] = (bf16_t)(b[i] * cs[i] + a[i] * sn[i]);
+      }
+      bf16_t* dst = nullptr;
+      if (head < q_heads) dst = out + (int64_t)m * ldo + head * d + j;
+      else if (slot >= 0) dst = k_pages + ((page * kv_heads + (head - q_heads)) * page_size + off) * d + j;
+      if (dst != nullptr) {
+        *reinterpret_cast<bf16x4*>(dst) = lo;
+        *reinterpret_cast<bf16x4*>(dst + half) = hi;
+      }
+    } else if (slot >= 0) {
+      const int vi = item - rot_items, hv = vi / (d / 4), dim = (vi % (d / 4)) * 4;
+      const float4v v = summed((q_heads + kv_heads + hv) * d + dim);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        v_pages[((page * kv_heads + hv) * d + dim + i) * page_size + off] = (bf16_t)v[i];
+    }
+  }
+}
+
+// `shape` = 16 * NW + KW for the shapes that are built.
+template <int MT, int EPI>
+int launch_mid(int nw, int kw, const MidArgs& a, hipStream_t stream) {
+  const int tiles = (a.N + 15) / 16;
+  const dim3 grid((tiles + nw - 1) / nw, a.splits);
+#define MID_CASE(NW_, KW_)                                                              \
+  if (nw == NW_ && kw == KW_) {                                                         \
+    mid_gemm_kernel<MT, NW_, KW_, EPI><<<grid, NW_ * KW_ * 64, 0, stream>>>(a);         \
+    return dli_launch_status();                                                         \
+  }
+  MID_CASE(4, 1) MID_CASE(2, 1) MID_CASE(4, 2) MID_CASE(2, 2) MID_CASE(2, 4) MID_CASE(4, 4)
+#undef MID_CASE
+  return DLI_ERR_ARGUMENT;
+}
+
+template <int EPI>
+int launch_mid_rows(int nw, int kw, const MidArgs& a, hipStream_t stream) {
+  if (a.M <= 16) return launch_mid<1, EPI>(nw, kw, a, stream);
+  if (a.M <= 32) return launch_mid<2, EPI>(nw, kw, a, stream);
+  if (a.M <= 48) return launch_mid<3, EPI>(nw, kw, a, stream);
+  return launch_mid<4, EPI>(nw, kw, a, stream);
+}
+
+}  // namespace
+
+// x [M, K] bfloat16 (row stride ldx), M <= 64, K % 128 == 0. w: [N (+ up part), K] row by row, or
+// in tile order if `tiled` (then N % 16 == 0 and up_offset % 16 == 0). norm_w == nullptr: no norm.
+// epilogue 0: out is float32 [splits][M][N] (ldo == N); 1 (gated) and 2 (store): out is bfloat16
+// [M][N] with row stride ldo, one split. waves: feature tiles per workgroup; kwaves: waves that
+// share a feature tile and split the workgroup's k (the built pairs are listed in launch_mid).
+extern "C" int dli_mid_gemm(const void* x, int64_t ldx, const float* ssq_in, int ssq_parts,
+                            const float* norm_w, float eps, const void* w, int tiled, const void* bias,
+                            void* out, int64_t ldo, int M, int N, int K, int up_offset, int epilogue,
+                            int splits, int waves, int kwaves, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return DLI_OK;
+  if (M > 64 || K <= 0 || K % 128 != 0 || ldx % 8 != 0 || ldx < K || out == nullptr || epilogue < 0 ||
+      epilogue > 2 || splits < 1 || splits > K / 128 || waves < 1 || kwaves < 1 ||
+      (epilogue != MID_PARTIAL && splits != 1) || (epilogue == MID_PARTIAL && (ldo != N || bias != nullptr)) ||
+      (epilogue != MID_PARTIAL && (ldo < N || ldo % 4 != 0)) ||
+      (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)) ||
+      (tiled && (N % 16 != 0 || up_offset % 16 != 0)) || (epilogue == MID_SWIGLU && up_offset <= 0) ||
+      (epilogue == MID_PARTIAL && N % 4 != 0))
+    return DLI_ERR_ARGUMENT;
+  const MidArgs a{(const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, tiled,
+                  (const bf16_t*)bias, out, ldo, M, N, K, up_offset, splits};
+  if (epilogue == MID_PARTIAL) return launch_mid_rows<MID_PARTIAL>(waves, kwaves, a, stream);
+  if (epilogue == MID_SWIGLU) return launch_mid_rows<MID_SWIGLU>(waves, kwaves, a, stream);
+  return launch_mid_rows<MID_STORE>(waves, kwaves, a, stream);
+}
+
+// partial: float32 [splits][M][N]; stream: bfloat16 [M][N] (row stride lds, a multiple of 4),
+// updated in place; ssq_out: float32 [ceil(N / 1024)][M]. N % 4 == 0.
+extern "C" int dli_mid_finish_residual(const float* partial, int splits, const void* bias, void* stream_buf,
+                                       int64_t lds_, float* ssq_out, int M, int N, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return DLI_OK;
+  if (partial == nullptr || stream_buf == nullptr || ssq_out == nullptr || splits < 1 || N % 4 != 0 ||
+      lds_ < N || lds_ % 4 != 0)
+    return DLI_ERR_ARGUMENT;
+  mid_finish_residual_kernel<<<dim3(M, (N + 1023) / 1024), 256, 0, stream>>>(
+      partial, splits, (const bf16_t*)bias, (bf16_t*)stream_buf, lds_, ssq_out, M, N);
+  return dli_launch_status();
+}
+
+// partial: float32 [splits][M][(q_heads + 2*kv_heads) * head_dim] in the feature order of the
+// product that rotates; bias (optional) in the same order; angles float32 [M][2][head_dim/2];
+// slots int32 [M]; out bfloat16 [M][>= q_heads*head_dim] (row stride ldo); pages as the attention
+// kernels read them. head_dim % 16 == 0.
+extern "C" int dli_mid_finish_qkv(const float* partial, int splits, const void* bias, const float* angles,
+                                  const int* slots, void* out, int64_t ldo, void* k_pages, void* v_pages,
+                                  int M, int q_heads, int kv_heads, int head_dim, int page_size,
+                                  hipStream_t stream) {
+  if (M <= 0) return DLI_OK;
+  if (partial == nullptr || angles == nullptr || slots == nullptr || out == nullptr || k_pages == nullptr ||
+      v_pages == nullptr || splits < 1 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 ||
+      head_dim % 16 != 0 || page_size <= 0 || ldo < (int64_t)q_heads * head_dim || ldo % 4 != 0)
+    return DLI_ERR_ARGUMENT;
+  const int items = (q_heads + kv_heads) * (head_dim / 8) + kv_heads * (head_dim / 4);
+  mid_finish_qkv_kernel<<<dim3(M, (items + 255) / 256), 256, 0, stream>>>(partial, splits, (const bf16_t*)bias, angles, slots, (bf16_t*)out,
+                                               ldo, (bf16_t*)k_pages, (bf16_t*)v_pages, M, q_heads, kv_heads,
+                                               head_dim, page_size);
+  return dli_launch_status();
+}

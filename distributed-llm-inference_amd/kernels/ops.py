@@ -53,6 +53,11 @@ _SIGNATURES = {
     "dli_skinny_gemm_qkv_rope": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64,
                                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_ptr],
+    "dli_mid_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_int,
+                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_mid_finish_residual": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_ptr],
+    "dli_mid_finish_qkv": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int,
+                           _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_bf16": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64,
                       _c_int, _c_ptr],
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
@@ -477,6 +482,161 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
 
 _GEMM_WORKSPACE_BYTES = 64 << 20
 _gemm_workspaces: dict[int, torch.Tensor] = {}
+
+
+MID_PARTIAL, MID_SWIGLU, MID_STORE = 0, 1, 2
+MID_ROWS = 64
+
+
+def mid_gemm_supports(rows: int, k: int, dtype: torch.dtype) -> bool:
+    """Whether the product kernel for decode steps of up to 64 rows takes this shape."""
+    return dtype == torch.bfloat16 and 0 < rows <= MID_ROWS and k > 0 and k % 128 == 0
+
+
+MID_SHAPES = ((4, 1), (2, 1), (4, 2), (2, 2), (2, 4), (4, 4))  # (waves, kwaves) that are built
+
+
+def mid_gemm_plan(n: int, k: int, epilogue: int, units: int) -> tuple[int, int, int]:
+    """``(waves, kwaves, splits)`` for a product of ``n`` output features of depth ``k``.
+
+    A workgroup has ``waves`` feature tiles of 16 and ``kwaves`` waves on each, which split its
+    range of k; ``splits`` workgroups share a feature tile's whole k (a gated product is never
+    split: its epilogue needs whole sums). These launches last a few trips to memory, so the plan
+    aims at one workgroup on every compute unit with eight to sixteen waves, each with few blocks
+    of 128 k to fetch."""
+    tiles, blocks = -(-n // 16), k // 128
+    if epilogue != MID_PARTIAL:
+        waves = 2 if tiles >= 2 * units or epilogue == MID_SWIGLU else 4
+        return waves, 4 if blocks >= 8 else (2 if blocks >= 2 else 1), 1
+    waves = 4
+    groups = -(-tiles // waves)
+    splits = max(1, min(blocks, round(units / groups)))
+    kwaves = 2 if blocks // splits >= 2 else 1
+    return waves, kwaves, splits
+
+
+def mid_tiles_help(w_rows: int, k: int, epilogue: int) -> bool:
+    """Whether decode steps of 17 to 64 rows would read a copy of a ``[w_rows, k]`` weight in tile
+    order (:func:`tile_weights`): the layer products do, where the sizes tile."""
+    n = w_rows // 2 if epilogue == SKINNY_SWIGLU else w_rows
+    return epilogue in (SKINNY_STORE, SKINNY_SWIGLU, SKINNY_RESIDUAL) and k % 128 == 0 and n % 16 == 0 and n > 0
+
+
+def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = False, n: Optional[int] = None,
+             out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+             norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None,
+             splits: Optional[int] = None, waves: Optional[int] = None,
+             kwaves: Optional[int] = None) -> torch.Tensor:
+    """``y = xhat @ w.T`` for at most 64 rows of bfloat16 ``x [rows, k]``, k a multiple of 128.
+
+    ``w`` is ``[n, k]`` (``[2n, k]``, gate rows then up rows, for ``MID_SWIGLU``), or the same in
+    tile order (:func:`tile_weights`, flat) with ``tiled`` and ``n`` given. ``norm_w``/``eps``/
+    ``ssq_in [parts, rows]``: xhat is the RMSNorm of x. ``MID_PARTIAL`` returns float32
+    ``[splits, rows, n]`` whose sum over the splits, in their order, is the product (no bias; the
+    finishing kernels add them up); ``MID_STORE`` and ``MID_SWIGLU`` return bfloat16 ``[rows, n]``.
+    """
+    _rows(x, "x", torch.bfloat16)
+    m, k = x.shape
+    _require(mid_gemm_supports(m, k, x.dtype), f"this product takes 1..64 rows and k % 128 == 0, not {m} x {k}")
+    _require(x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+    sets = 2 if epilogue == MID_SWIGLU else 1
+    if tiled:
+        _dense(w, "w", torch.bfloat16, 1)
+        _require(n is not None and n % 16 == 0 and w.numel() == sets * n * k, "tiled weights need n % 16 == 0 features of depth k")
+    else:
+        _dense(w, "w", torch.bfloat16, 2)
+        _require(w.shape[1] == k and w.shape[0] % sets == 0, "x and w differ in inner size")
+        n = w.shape[0] // sets
+    _require(epilogue in (MID_PARTIAL, MID_SWIGLU, MID_STORE), "unknown epilogue")
+    plan_waves, plan_kwaves, plan_splits = mid_gemm_plan(n, k, epilogue, _units(x.device))
+    waves = plan_waves if waves is None else waves
+    kwaves = plan_kwaves if kwaves is None else kwaves
+    splits = plan_splits if splits is None else splits
+    _require((waves, kwaves) in MID_SHAPES and 1 <= splits <= k // 128,
+             f"(waves, kwaves) must be one of {MID_SHAPES}, splits 1..k/128")
+    if epilogue == MID_PARTIAL:
+        _require(bias is None and n % 4 == 0, "partial products take no bias, n % 4 == 0")
+        if out is None:
+            out = torch.empty(splits, m, n, device=x.device, dtype=torch.float32)
+        _dense(out, "out", torch.float32, 3)
+        _require(out.shape == (splits, m, n), "out must be [splits, rows, n]")
+        ldo = n
+    else:
+        _require(splits == 1, "only partial products are split")
+        if out is None:
+            out = torch.empty(m, n, device=x.device, dtype=torch.bfloat16)
+        _rows(out, "out", torch.bfloat16)
+        _require(out.shape == (m, n) and out.stride(0) % 4 == 0 and out.data_ptr() % 8 == 0, "out must be [rows, n], rows 8-byte aligned")
+        ldo = out.stride(0)
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == sets * n, "bias length differs from rows of w")
+    parts = 0
+    if norm_w is not None:
+        _dense(norm_w, "norm_w", torch.float32, 1)
+        _require(norm_w.shape[0] == k and norm_w.data_ptr() % 16 == 0, "norm weight must have k aligned values")
+        _require(ssq_in is not None, "a fused norm needs the sums of squares")
+        _dense(ssq_in, "ssq_in", torch.float32, 2)
+        _require(ssq_in.shape[1] == m and ssq_in.shape[0] >= 1, "ssq_in must be [parts, rows]")
+        parts = ssq_in.shape[0]
+    _check(library().dli_mid_gemm(
+        _ptr(x), x.stride(0), _ptr(ssq_in) if norm_w is not None else None, parts, _ptr(norm_w), float(eps), _ptr(w),
+        int(tiled), _ptr(bias), _ptr(out), ldo, m, n, k, n if epilogue == MID_SWIGLU else 0, epilogue, splits, waves,
+        kwaves, _stream()), "mid_gemm")
+    return out
+
+
+def mid_finish_residual(partial: torch.Tensor, stream: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                        ssq_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``stream += sum over splits of partial (+ bias)`` in place (32-bit sum, the product rounded
+    to bfloat16 first, as the fused epilogue of the few-row product does), and each row's sum of
+    squares of the new stream, in parts of 1024 features, as float32 ``[parts, rows]`` for the norm
+    that follows."""
+    _dense(partial, "partial", torch.float32, 3)
+    _rows(stream, "stream", torch.bfloat16)
+    splits, m, n = partial.shape
+    _require(stream.shape == (m, n) and n % 4 == 0 and stream.stride(0) % 4 == 0 and stream.data_ptr() % 8 == 0,
+             "stream must be [rows, n] with n % 4 == 0")
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == n, "bias length differs from n")
+    parts = -(-n // 1024)
+    if ssq_out is None:
+        ssq_out = torch.empty(parts, m, device=stream.device, dtype=torch.float32)
+    _dense(ssq_out, "ssq_out", torch.float32, 2)
+    _require(ssq_out.shape == (parts, m), "ssq_out must be [ceil(n / 1024), rows]")
+    _check(library().dli_mid_finish_residual(_ptr(partial), splits, _ptr(bias), _ptr(stream), stream.stride(0),
+                                             _ptr(ssq_out), m, n, _stream()), "mid_finish_residual")
+    return ssq_out
+
+
+def mid_finish_qkv(partial: torch.Tensor, out: torch.Tensor, angles: torch.Tensor, slots: torch.Tensor,
+                   k_pages: torch.Tensor, v_pages: torch.Tensor, q_heads: int,
+                   bias: Optional[torch.Tensor] = None) -> None:
+    """The fused q/k/v projection's partial products ``[splits, rows, (q + 2 kv) * head_dim]``, in
+    the feature order of :func:`tile_weights_qkv_rope` (``bias`` too): summed over the splits,
+    rotated, q written to ``out[:, :q_heads * head_dim]`` in the usual order, rotated k and v into
+    the cache pages at ``slots`` (negative: not cached). ``angles``: :func:`rope_angles`."""
+    _dense(partial, "partial", torch.float32, 3)
+    _rows(out, "out", torch.bfloat16)
+    splits, m, n = partial.shape
+    _dense(k_pages, "k_pages", torch.bfloat16, 4)
+    _dense(v_pages, "v_pages", torch.bfloat16, 4)
+    _, kv_heads, page_size, head_dim = k_pages.shape
+    _require(v_pages.shape == (k_pages.shape[0], kv_heads, head_dim, page_size), "v_pages must be [pages, kv_heads, head_dim, page_size]")
+    _require(head_dim % 16 == 0 and n == (q_heads + 2 * kv_heads) * head_dim, "partial width differs from (q + 2 kv) * head_dim")
+    _require(out.shape[0] == m and out.shape[1] >= q_heads * head_dim and out.stride(0) % 4 == 0 and out.data_ptr() % 8 == 0,
+             "out must hold the q heads of every row")
+    _dense(angles, "angles", torch.float32, 3)
+    _require(angles.shape == (m, 2, head_dim // 2), "angles must be [rows, 2, head_dim / 2]")
+    _dense(slots, "slots", torch.int32, 1)
+    _require(slots.shape[0] == m, "slots differ from partial in rows")
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == n, "bias length differs from the features")
+    _check(library().dli_mid_finish_qkv(_ptr(partial), splits, _ptr(bias), _ptr(angles), _ptr(slots), _ptr(out),
+                                        out.stride(0), _ptr(k_pages), _ptr(v_pages), m, q_heads, kv_heads, head_dim,
+                                        page_size, _stream()), "mid_finish_qkv")
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> bool:

@@ -31,6 +31,7 @@ from .spec import PartSpec, WeightSpec
 # kernel runs. (A variant that rotated inside the attention kernel instead, repeating the rotation
 # in every split of the keys, was slower from four rows on and no faster below.)
 ROPE_IN_PRODUCT_ROWS = range(1, 17)
+FEW_ROWS = 16  # up to here the few-row product kernels run; from 17 to 64 rows the one that shares activations
 
 
 @register_part("mixer", "gqa_attention")
@@ -135,11 +136,18 @@ class GQAttention(Mixer):
     # -- decode steps with few rows: the norm before and the residual sum after are fused into
     #    the two projections' kernels
     def streams(self, ctx: Any) -> bool:
-        nh, d = self.num_heads, self.head_dim
-        return (self.rt.is_bf16 and ctx.num_decode == ctx.num_entries and self.hidden_size % 8 == 0
-                and ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype)
-                and ops.skinny_gemm_supports(ctx.num_tokens, nh * d, self.rt.dtype)
-                and ops.attention_mfma_supports(d, ctx.page_size, self.rt.dtype))
+        nh, d, n = self.num_heads, self.head_dim, ctx.num_tokens
+        if not (self.rt.is_bf16 and ctx.num_decode == ctx.num_entries and self.hidden_size % 8 == 0
+                and ops.attention_mfma_supports(d, ctx.page_size, self.rt.dtype)):
+            return False
+        if n > FEW_ROWS:
+            # 17 to 64 rows: the product kernel that shares the activations through LDS; it reads
+            # the tile-ordered copies and leaves rotation and cache write to its finishing kernel
+            return (self.w_qkv_rope is not None and self.w_o_tiled is not None
+                    and ops.mid_gemm_supports(n, self.hidden_size, self.rt.dtype)
+                    and ops.mid_gemm_supports(n, nh * d, self.rt.dtype))
+        return (ops.skinny_gemm_supports(n, self.hidden_size, self.rt.dtype)
+                and ops.skinny_gemm_supports(n, nh * d, self.rt.dtype))
 
     def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any, cache: Any) -> None:
         """``stream.x += attention(norm(stream.x))``, the norm inside the first product's kernel and
@@ -149,6 +157,9 @@ class GQAttention(Mixer):
         grp = ctx.groups[cache.group]
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
+        if n > FEW_ROWS:
+            self._forward_stream_mid(stream, norm_w, eps, ctx, cache, grp)
+            return
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
         if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS:
             # product, rotation and cache write in one kernel; only q comes back
@@ -172,3 +183,20 @@ class GQAttention(Mixer):
         paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
                                      stream=stream.x, bias=self.b_o)
+
+    def _forward_stream_mid(self, stream: DecodeStream, norm_w: torch.Tensor, eps: float, ctx: Any, cache: Any,
+                            grp: Any) -> None:
+        """The same for 17 to 64 rows: both products split k over workgroups and leave 32-bit
+        partial sums; the kernel that rotates and writes the cache, and the one that makes the
+        residual sum, add them up."""
+        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        n = stream.x.shape[0]
+        partial = ops.mid_gemm(stream.x, self.w_qkv_rope, tiled=True, n=(nh + 2 * nkv) * d, epilogue=ops.MID_PARTIAL,
+                               norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        q = self.rt.empty(n, nh * d)
+        angles = ctx.rope_angles(self.position.rotary_table().inv_freq, q.dtype)
+        ops.mid_finish_qkv(partial, q, angles, grp.slots, cache.k_pages, cache.v_pages, nh, bias=self.b_qkv_rope)
+        out = self.rt.empty(n, nh * d)
+        paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        partial = ops.mid_gemm(out, self.w_o_tiled, tiled=True, n=self.hidden_size, epilogue=ops.MID_PARTIAL)
+        stream.ssq = ops.mid_finish_residual(partial, stream.x, self.b_o)

@@ -52,16 +52,29 @@ class GatedMLP(FeedForward):
         ops.silu_mul(gate_up, act)
         return linear(self.rt, act, self.w_down, self.b_down)
 
+    FEW_ROWS = 16  # the few-row product kernels; 17 to 64 rows take the one that shares activations
+
     def streams(self, ctx: Any) -> bool:
         n = ctx.num_tokens
-        return (self.rt.is_bf16 and self.hidden_size % 8 == 0
-                and ops.skinny_gemm_supports(n, self.hidden_size, self.rt.dtype)
+        if not (self.rt.is_bf16 and self.hidden_size % 8 == 0):
+            return False
+        if n > self.FEW_ROWS:
+            return (self.w_gate_up_tiled is not None and self.w_down_tiled is not None
+                    and ops.mid_gemm_supports(n, self.hidden_size, self.rt.dtype)
+                    and ops.mid_gemm_supports(n, self.intermediate_size, self.rt.dtype))
+        return (ops.skinny_gemm_supports(n, self.hidden_size, self.rt.dtype)
                 and ops.skinny_gemm_supports(n, self.intermediate_size, self.rt.dtype))
 
     def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any) -> None:
         """``stream.x += mlp(norm(stream.x))``, norm and sum inside the two products' kernels."""
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
+        if n > self.FEW_ROWS:
+            act = ops.mid_gemm(stream.x, self.w_gate_up_tiled, tiled=True, n=self.intermediate_size,
+                               epilogue=ops.MID_SWIGLU, bias=self.b_gate_up, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+            partial = ops.mid_gemm(act, self.w_down_tiled, tiled=True, n=self.hidden_size, epilogue=ops.MID_PARTIAL)
+            stream.ssq = ops.mid_finish_residual(partial, stream.x, self.b_down)
+            return
         act = self.rt.empty(n, self.intermediate_size)
         ops.skinny_gemm(stream.x, self.w_gate_up, w_tiled=self.w_gate_up_tiled, epilogue=ops.SKINNY_SWIGLU, out=act,
                         bias=self.b_gate_up, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)

@@ -54,10 +54,14 @@ class LinearHead(Head):
         return out
 
     def streams(self, ctx) -> bool:
-        return self.rt.is_bf16 and ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype)
+        return self.rt.is_bf16 and (ctx.num_tokens > self.FEW_ROWS
+                                    or ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype))
 
     def forward_stream(self, stream: DecodeStream, norm: Norm) -> torch.Tensor:
-        """Logits of every row of the stream, the final norm computed inside the product."""
+        """Logits of every row of the stream, the final norm computed inside the product (with
+        more than a few rows: the norm kernel, then the library product)."""
+        if stream.x.shape[0] > self.FEW_ROWS:
+            return self.forward(norm.forward(stream.x))
         norm_w, eps = norm.fused_params()
         out = torch.empty(stream.x.shape[0], self.vocab_size, device=self.rt.device, dtype=torch.float32)
         ops.skinny_gemm(stream.x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out,

@@ -42,10 +42,12 @@ def linear(rt: Runtime, x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
 def decode_copy(rt: Runtime, weight: Optional[torch.Tensor], epilogue: int) -> Optional[torch.Tensor]:
     """The matrix once more in the tile order of the decode product (``ops.tile_weights``), or
     ``None`` where that would not be used: another type, sizes that do not tile, a product that
-    the 4x4-block kernel serves at every number of rows, or a runtime that does not want it."""
+    neither the few-row tile kernel nor the kernel for 17 to 64 rows reads in that order, or a
+    runtime that does not want it."""
     if (weight is None or not rt.is_bf16 or not rt.decode_weight_copy or weight.dtype != torch.bfloat16
             or weight.dim() != 2 or not weight.is_cuda):
         return None
-    if not ops.tiled_weights_help(weight.shape[0], weight.shape[1], epilogue, weight.device):
+    if not (ops.tiled_weights_help(weight.shape[0], weight.shape[1], epilogue, weight.device)
+            or ops.mid_tiles_help(weight.shape[0], weight.shape[1], epilogue)):
         return None
     return ops.tile_weights(weight)

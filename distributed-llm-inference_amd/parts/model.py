@@ -121,7 +121,7 @@ class Model:
 
     # ------------------------------------------------------------------ step
 
-    STREAM_ROWS = 16  # steps with at most this many rows, all decoding, take the fused kernels
+    STREAM_ROWS = 64  # steps with at most this many rows, all decoding, take the fused kernels
 
     def _streams(self, ctx: Any) -> bool:
         if not 0 < ctx.num_tokens <= self.STREAM_ROWS or ctx.num_decode != ctx.num_entries:

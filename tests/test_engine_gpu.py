@@ -382,6 +382,28 @@ def test_trace_run_program(tmp_path):
     assert proc.returncode != 0 and "NoFreePagesError" in proc.stderr
 
 
+@pytest.mark.parametrize("name,count", [("D", 20), ("D", 40), ("A", 20)])
+def test_many_requests_decode_together_through_the_engine(name, count):
+    """More than sixteen requests at once: configuration D's sizes tile, so its decode steps take
+    the product kernel for 17 to 64 rows inside the graphs (A's do not and take the plain path);
+    tokens are the plain implementation's either way."""
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    eng = LLMEngine.for_model(str(model_folder(name)), dtype="bfloat16", num_blocks=4 * count + 8, block_size=16,
+                              enable_prefix_caching=False,
+                              config=SchedulerConfig(max_num_seqs=count, max_num_batched_tokens=1024))
+    ps = prompts(name, [5 + (7 * i) % 23 for i in range(count)], seed=67)
+    reqs = [eng.add_request(f"r{i}", p, SamplingParams(max_tokens=12)) for i, p in enumerate(ps)]
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.core.step.graphs.replays >= 10
+    assert max(s.num_seqs for s in eng.stats.steps) == count
+    for r, p in zip(reqs, ps):
+        assert len(r.output_ids) == 12
+        assert_same_or_near_tie(name, p, r.output_ids, plain_greedy(name, p, 12), margin=0.25)
+
+
 def test_warm_up_captures_every_graph_that_serving_then_replays():
     """After ``warm_up`` no decode step captures a graph: requests of several lengths and batch
     sizes, one and several tokens per step, only replay what exists, and the tokens are the plain

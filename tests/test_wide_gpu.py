@@ -19,18 +19,23 @@ pytestmark = pytest.mark.gpu
 _plain: dict = {}
 
 
+_weights: list = []
+
+
 def plain(tokens):
     key = tuple(tokens)
     if key not in _plain:
-        cfg, w = P.load_folder(model_folder("W"))
-        _plain[key] = P.forward_logits(w, cfg, tokens)
+        if not _weights:  # converted to 64-bit once, not in every call
+            cfg, w = P.load_folder(model_folder("W"))
+            _weights.extend([cfg, {k: t.double() for k, t in w.items()}])
+        _plain[key] = P.forward_logits(_weights[1], _weights[0], tokens)
     return _plain[key]
 
 
 def make_core(dtype, pages, page=16, graphs=0):
     from dli_amd.engine.core import build_core
 
-    core = build_core(model_folder("W"), num_pages=pages, page_size=page, max_seqs=8, dtype=dtype,
+    core = build_core(model_folder("W"), num_pages=pages, page_size=page, max_seqs=max(8, graphs), dtype=dtype,
                       enable_prefix_caching=False, watermark=0.0)
     if graphs:
         core.step.enable_decode_graphs(graphs, pages * page)
@@ -58,35 +63,39 @@ def test_whole_prompt_then_decoding_at_serving_widths(dtype):
         assert core.step.graphs is not None and core.step.graphs.replays >= 24
 
 
-def test_eight_requests_decode_together_at_serving_widths():
-    """Prompts of different lengths go in as a mixed batch of portions, then all eight decode side
-    by side (the 16x16-tile products with their fused norm, SwiGLU and residual epilogues)."""
+@pytest.mark.parametrize("count", [8, 24, 64])
+def test_requests_decode_together_at_serving_widths(count):
+    """Prompts of different lengths go in as mixed batches of portions, then all decode side by
+    side: eight through the 16x16-tile products with their fused norm, SwiGLU and residual
+    epilogues, 24 and 64 through the product kernel that shares the activations through LDS and
+    its finishing kernels (two and four row tiles)."""
     from dli_amd.trace import TraceSession
 
-    rng = random.Random(4)
-    lens = [37, 64, 50, 33, 71, 48, 40, 59]
-    toks = [[rng.randrange(32003) for _ in range(n + 10)] for n in lens]
-    core = make_core("bfloat16", pages=48, graphs=8)
+    rng = random.Random(4 + count)
+    lens = [rng.randrange(18, 44) for _ in range(count)]
+    steps = 10 if count == 8 else 4
+    toks = [[rng.randrange(32003) for _ in range(n + steps)] for n in lens]
+    core = make_core("bfloat16", pages=4 * count + 8, graphs=count)
     s = TraceSession(core)
-    fed = [0] * 8
+    fed = [0] * count
     # prompts in two mixed steps of portions
     for part in (0, 1):
         entries = []
-        for r in range(8):
+        for r in range(count):
             n = lens[r] // 2 if part == 0 else lens[r] - lens[r] // 2
             entries.append({"id": r, "tokens": toks[r][fed[r]:fed[r] + n], "want": [n - 1] if part else []})
             fed[r] += n
         out = s.step(entries)
-    rows = torch.stack([plain(toks[r])[lens[r] - 1] for r in range(8)])
+    rows = torch.stack([plain(toks[r])[lens[r] - 1] for r in range(count)])
     check(out, rows, "bfloat16", "wide mixed prompts")
-    for stepno in range(10):
-        entries = [{"id": r, "tokens": [toks[r][fed[r]]], "want": [0]} for r in range(8)]
+    for stepno in range(steps):
+        entries = [{"id": r, "tokens": [toks[r][fed[r]]], "want": [0]} for r in range(count)]
         out = s.step(entries)
-        rows = torch.stack([plain(toks[r])[fed[r]] for r in range(8)])
-        check(out, rows, "bfloat16", f"wide decode step {stepno}")
-        for r in range(8):
+        rows = torch.stack([plain(toks[r])[fed[r]] for r in range(count)])
+        check(out, rows, "bfloat16", f"wide decode step {stepno} of {count}")
+        for r in range(count):
             fed[r] += 1
-    assert core.step.graphs.replays >= 10
+    assert core.step.graphs.replays >= steps
 
 
 def test_llama_3_2_1b_at_full_depth_and_vocabulary():
