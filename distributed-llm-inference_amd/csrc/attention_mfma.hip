@@ -41,6 +41,22 @@ __device__ __forceinline__ short bf16_bits(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Maximum as one instruction. fmaxf() asks for a quieted NaN, which costs a second instruction per
+// operand that the compiler cannot prove canonical (every matrix-core result); scores are never
+// NaN here (masked ones are -inf), and the instruction itself orders -inf and finite values as
+// fmaxf does. The prefill kernel is bound by the vector unit's instruction count: 65 -> 59 us a
+// layer at 2,048 tokens of the 1B sizes.
+__device__ __forceinline__ float max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // Reductions over the four lanes l, l^16, l^32, l^48 (the lane groups that share a column) with
 // the gfx950 lane-swap instructions: after v_permlane32_swap of two copies of v, one copy holds
 // the lower half's values in both halves and the other the upper half's; v_permlane16_swap does
@@ -48,10 +64,10 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float column_max(float v) {
   const unsigned u = __float_as_uint(v);
   const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const float m = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
   const unsigned um = __float_as_uint(m);
   const auto b = __builtin_amdgcn_permlane16_swap(um, um, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float column_sum(float v) {
   const unsigned u = __float_as_uint(v);
@@ -96,8 +112,8 @@ __device__ __forceinline__ void attend_tile(ColumnTile<DCH>& st, const short4v (
       if (key > last_visible || key < first_visible) sv[i] = -INFINITY;
     }
   }
-  const float tile_max = column_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
-  const float m_new = fmaxf(st.m, tile_max);
+  const float tile_max = column_max(max2(max3(sv[0], sv[1], sv[2]), sv[3]));
+  const float m_new = max2(st.m, tile_max);
   const float m_safe = m_new == -INFINITY ? 0.f : m_new;
   const float alpha = fast_exp2(st.m - m_safe);
   float p[4];
@@ -661,10 +677,10 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
       bf16x8 pb[2];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        float tile_max = fmaxf(fmaxf(fmaxf(sv[j][0], sv[j][1]), fmaxf(sv[j][2], sv[j][3])),
-                               fmaxf(fmaxf(sv[j][4], sv[j][5]), fmaxf(sv[j][6], sv[j][7])));
+        float tile_max = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]),
+                              max2(sv[j][6], sv[j][7]));
         tile_max = column_max(tile_max) * scale_log2e;  // the scale is positive
-        const float m_new = fmaxf(st[j].m, tile_max);
+        const float m_new = max2(st[j].m, tile_max);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
         alpha[j] = fast_exp2(st[j].m - m_safe);
         float tile_sum = 0.f;
@@ -675,7 +691,11 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
           pb[j][i] = (bf16_t)p;
         }
         // l stays a per-lane partial sum (the lanes of a column share m, hence alpha): the
-        // four partial sums of a column are added once, after the last tile
+        // four partial sums of a column are added once, after the last tile. (Taking the sum
+        // from the matrix cores instead, as the product of P^T with a row of ones, saves sixteen
+        // additions a lane and tile and was slower, 62 against 59 us; so was computing S^T of the
+        // next tile before the softmax of this one inside a wave, 68 us: two waves a SIMD already
+        // cover each other's waits.)
         st[j].l = st[j].l * alpha[j] + tile_sum;
         st[j].m = m_new;
       }
