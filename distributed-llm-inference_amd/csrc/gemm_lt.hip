@@ -104,3 +104,17 @@ extern "C" int dli_gemm_bf16(const void* x, int64_t ldx, const void* w, int64_t 
                                              &p.algo, workspace, (size_t)workspace_bytes, stream);
   return st == HIPBLAS_STATUS_SUCCESS ? DLI_OK : DLI_ERR_LAUNCH;
 }
+
+// Whether the library has a kernel for this product (the plan is made and cached as for a call).
+extern "C" int dli_gemm_bf16_usable(int64_t rows, int64_t feats, int64_t k, int64_t ldx, int64_t ldw, int64_t ldo,
+                                    int bias, int64_t workspace_bytes, int device) {
+  if (rows <= 0 || feats <= 0 || k <= 0 || ldx < k || ldw < k || ldo < feats || workspace_bytes < 0) return 0;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  hipblasLtHandle_t handle = handle_for(device);
+  if (handle == nullptr) return 0;
+  const Key key{device, rows, feats, k, ldx, ldw, ldo, bias ? 1 : 0, workspace_bytes};
+  auto it = g_plans.find(key);
+  if (it == g_plans.end())
+    it = g_plans.emplace(key, make_plan(handle, rows, feats, k, ldx, ldw, ldo, bias != 0, (size_t)workspace_bytes)).first;
+  return it->second.usable ? 1 : 0;
+}

@@ -60,6 +60,8 @@ _SIGNATURES = {
                            _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_bf16": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64,
                       _c_int, _c_ptr],
+    "dli_gemm_bf16_usable": [_c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_i64, _c_int],
+    "dli_prenorm_blocks_bf16": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
@@ -637,6 +639,29 @@ def mid_finish_qkv(partial: torch.Tensor, out: torch.Tensor, angles: torch.Tenso
     _check(library().dli_mid_finish_qkv(_ptr(partial), splits, _ptr(bias), _ptr(angles), _ptr(slots), _ptr(out),
                                         out.stride(0), _ptr(k_pages), _ptr(v_pages), m, q_heads, kv_heads, head_dim,
                                         page_size, _stream()), "mid_finish_qkv")
+
+
+def gemm_workspace(device: torch.device) -> tuple[torch.Tensor, int]:
+    """The device buffer that the vendor library's products may use, and its size in bytes."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    workspace = _gemm_workspaces.get(index)
+    if workspace is None:
+        workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return workspace, _GEMM_WORKSPACE_BYTES
+
+
+def prenorm_blocks(x: torch.Tensor, blocks, count: int, step) -> bool:
+    """Run ``count`` pre-norm blocks (ctypes array of ``parts.native.BlockArgs``) on the residual
+    stream ``x`` for the step described by ``step`` (``parts.native.StepArgs``), all launches
+    issued from C. Whoever fills the structures has checked shapes and sizes. False, with nothing
+    launched, where an argument or a product's shape is refused."""
+    _rows(x, "x", torch.bfloat16)
+    status = library().dli_prenorm_blocks_bf16(_ptr(x), ctypes.cast(blocks, ctypes.c_void_p), int(count),
+                                               ctypes.cast(ctypes.pointer(step), ctypes.c_void_p), _stream())
+    if status == -1:
+        return False
+    _check(status, "prenorm_blocks")
+    return True
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> bool:

@@ -100,6 +100,20 @@ class GQAttention(Mixer):
     def sub_parts(self) -> dict[str, Part]:
         return {"position": self.position}
 
+    def native_fields(self) -> Optional[dict]:
+        from .native import _bf16_matrix, _bf16_vector
+
+        nh, nkv, d, h = self.num_heads, self.num_kv_heads, self.head_dim, self.hidden_size
+        table = self.position.rotary_table()
+        if not self.rt.is_bf16 or self.shares_kv or table is None or table.pairing != "half":
+            return None
+        if not (_bf16_matrix(self.w_qkv, (nh + 2 * nkv) * d, h) and _bf16_matrix(self.w_o, h, nh * d)
+                and _bf16_vector(self.b_qkv, (nh + 2 * nkv) * d) and _bf16_vector(self.b_o, h)):
+            return None
+        return {"w_qkv": self.w_qkv, "b_qkv": self.b_qkv, "w_o": self.w_o, "b_o": self.b_o,
+                "inv_freq": table.inv_freq, "rotary_dim": table.dim, "hidden": h, "q_heads": nh, "kv_heads": nkv,
+                "head_dim": d, "scale": self.scale, "window": self.window}
+
     def cache_spec(self) -> Optional[PagedKVSpec]:
         return None if self.shares_kv else PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
 

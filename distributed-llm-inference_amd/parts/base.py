@@ -86,6 +86,13 @@ class Part:
         """Tensors of this part by local name (the checkpoint name is ``prefix + name``)."""
         return {}
 
+    def native_fields(self) -> Optional[dict]:
+        """What the loop in C that issues a whole step's launches (:mod:`dli_amd.parts.native`)
+        needs to know of this part: tensors and constants by the names of its argument structure,
+        or ``None`` (the default) for a part that this route does not cover; the step then runs
+        part by part."""
+        return None
+
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """Receive the tensors of :meth:`weight_specs`, already on the device and typed by role."""
 

@@ -27,6 +27,19 @@ class PreNormBlock(Block):
         f = parts["feed_forward"].forward(h, ctx)
         return x, f
 
+    def native_fields(self, parts: Mapping[str, Part]) -> Optional[dict]:
+        """This arrangement with its parts' tensors and constants, for the loop in C that issues a
+        step's launches; ``None`` unless all four parts describe themselves and agree on the width."""
+        n1, n2 = parts["mixer_norm"].native_fields(), parts["feed_forward_norm"].native_fields()
+        mix, ff = parts["mixer"].native_fields(), parts["feed_forward"].native_fields()
+        if n1 is None or n2 is None or mix is None or ff is None:
+            return None
+        if not ({"w_qkv", "w_o", "inv_freq"} <= mix.keys() and {"w_gate_up", "w_down"} <= ff.keys()):
+            return None  # parts of another kind that describe themselves for another route
+        if not n1["width"] == n2["width"] == mix["hidden"] == ff["hidden"]:
+            return None
+        return {**mix, **ff, "norm1_w": n1["w"], "eps1": n1["eps"], "norm2_w": n2["w"], "eps2": n2["eps"]}
+
     def streams(self, ctx: Any, parts: Mapping[str, Part]) -> bool:
         fused_norms = all(hasattr(parts[r], "fused_params") for r in ("mixer_norm", "feed_forward_norm"))
         return fused_norms and parts["mixer"].streams(ctx) and parts["feed_forward"].streams(ctx)

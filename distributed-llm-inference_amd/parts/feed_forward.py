@@ -46,6 +46,16 @@ class GatedMLP(FeedForward):
         self.w_gate_up_tiled = decode_copy(self.rt, self.w_gate_up, ops.SKINNY_SWIGLU)
         self.w_down_tiled = decode_copy(self.rt, self.w_down, ops.SKINNY_RESIDUAL)
 
+    def native_fields(self):
+        from .native import _bf16_matrix, _bf16_vector
+
+        h, i = self.hidden_size, self.intermediate_size
+        if not (self.rt.is_bf16 and _bf16_matrix(self.w_gate_up, 2 * i, h) and _bf16_matrix(self.w_down, h, i)
+                and _bf16_vector(self.b_gate_up, 2 * i) and _bf16_vector(self.b_down, h)):
+            return None
+        return {"w_gate_up": self.w_gate_up, "b_gate_up": self.b_gate_up, "w_down": self.w_down, "b_down": self.b_down,
+                "hidden": h, "intermediate": i}
+
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         gate_up = linear(self.rt, x, self.w_gate_up, self.b_gate_up)
         act = self.rt.empty(x.shape[0], self.intermediate_size)

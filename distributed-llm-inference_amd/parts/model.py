@@ -49,6 +49,9 @@ class Model:
             self.layers.append(BuiltLayer(blk, parts))
         self.final_norm = build_part("norm", spec.final_norm, runtime)
         self.head = build_part("head", spec.head, runtime)
+        self._native: dict = {}
+        self.native_steps = True   # steps with portions: all layers' launches from one call where the blocks allow
+        self.native_runs = 0       # how many steps went that way
 
     # ------------------------------------------------------------------ weights
 
@@ -124,6 +127,9 @@ class Model:
     STREAM_ROWS = 64  # steps with at most this many rows, all decoding, take the fused kernels
 
     def _streams(self, ctx: Any) -> bool:
+        # Steps that hold a portion run eagerly, where the host's time per launch decides: the fused
+        # kernels would be fewer launches, but issued one by one from Python they take longer than
+        # the plain kernels issued from the loop in C (2.1 against 1.7 ms for 64 tokens at the 1B sizes).
         if not 0 < ctx.num_tokens <= self.STREAM_ROWS or ctx.num_decode != ctx.num_entries:
             return False
         if not (self.embedding.streams(ctx) and self.head.streams(ctx) and hasattr(self.final_norm, "fused_params")):
@@ -144,6 +150,16 @@ class Model:
             ops.gather_rows(logits, ctx.logit_rows, out)
         return out
 
+    def _native_blocks(self, caches: Sequence[Any]):
+        """The schedule as one array of block descriptions for the loop in C, made once per list
+        of layer caches; ``None`` if some block or cache is not of the kind that route covers."""
+        hit = self._native.get(id(caches))
+        if hit is None or hit[0] is not caches:
+            from .native import NativeBlocks
+
+            hit = self._native[id(caches)] = (caches, NativeBlocks.build(self, caches))
+        return hit[1]
+
     def forward(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
         """Run the step's tokens through the schedule; float32 logits ``[wanted rows, vocab]``."""
         ctx.begin_forward()
@@ -151,9 +167,14 @@ class Model:
             return self._forward_stream(ctx, caches)
         x = self.embedding.forward(ctx.token_ids)
         delta: Optional[torch.Tensor] = None
-        for entry, cache in zip(self.spec.schedule, caches):
-            layer = self.layers[entry.layer]
-            x, delta = layer.block.forward(x, delta, ctx, cache, layer.parts)
+        native = self._native_blocks(caches) if self.rt.is_bf16 and self.native_steps and ctx.num_tokens > 0 else None
+        if native is not None:
+            delta = native.run(x, ctx)      # every layer's launches from one call; None: nothing ran
+            self.native_runs += delta is not None
+        if delta is None:
+            for entry, cache in zip(self.spec.schedule, caches):
+                layer = self.layers[entry.layer]
+                x, delta = layer.block.forward(x, delta, ctx, cache, layer.parts)
         k = ctx.logit_rows.shape[0]
         if k == 0:
             return torch.empty(0, self.spec.vocab_size, device=self.rt.device, dtype=torch.float32)

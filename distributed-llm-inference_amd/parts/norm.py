@@ -30,6 +30,12 @@ class RMSNorm(Norm):
         """Weight and eps, for a consumer that computes this norm inside its own kernel."""
         return self.weight, self.eps
 
+    def native_fields(self) -> Optional[dict]:
+        w = self.weight
+        if w is None or w.dtype != torch.float32 or not w.is_cuda or not w.is_contiguous() or w.data_ptr() % 32:
+            return None
+        return {"w": w, "eps": self.eps, "width": self.width}
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         out = torch.empty_like(x)
         if delta is None:

@@ -296,3 +296,39 @@ def test_the_same_traces_with_decode_graphs_on(name, page, monkeypatch):
     test_most_in_one_step_then_last_32_one_by_one(name, page, "bfloat16")
     assert all(core.step.graphs is not None for core in cores)
     assert sum(core.step.graphs.replays for core in cores) > 60
+
+
+@pytest.mark.parametrize("name,page", [("A", 16), ("B", 16), ("C", 32), ("D", 16), ("H", 16)])
+def test_layers_issued_from_one_call_equal_the_parts_one_by_one(name, page):
+    """Steps that hold portions run every layer's launches from one call into the library where
+    the model's blocks allow it (bfloat16, the architecture's own parts). The kernels and their
+    order are the same as when every part is called by itself, so the logits are equal bit for
+    bit: mixed steps of portions and single tokens, with pages used again."""
+    from dli_amd.trace import TraceSession
+
+    a, b, c = prompts_for(name, [161, 95, 83], seed=17)
+    # steps of more than 64 rows (fewer take the fused kernels of the decode path where the sizes allow)
+    plans = [
+        [("a", 90, True)], [("a", 2, False), ("b", 71, True)], [("a", 1, True), ("b", 24, True), ("c", 80, True)],
+        [("c", 1, True), ("a", 1, True)], [("a", 67, True), ("c", 1, True)],
+    ]
+    outs = {}
+    for native in (True, False):
+        core = make_core(name, "bfloat16", 24, page)
+        core.model.native_steps = native
+        s = TraceSession(core)
+        fed = {"a": 0, "b": 0, "c": 0}
+        toks = {"a": a, "b": b, "c": c}
+        got = []
+        for step in plans:
+            entries = []
+            for rid, n, want in step:
+                entries.append({"id": rid, "tokens": toks[rid][fed[rid]:fed[rid] + n],
+                                "want": list(range(n)) if want else []})
+                fed[rid] += n
+            got.append(s.step(entries).clone())
+        outs[native] = got
+        assert (core.model.native_runs > 0) == native, (name, native, core.model.native_runs)
+    for x, y in zip(outs[True], outs[False]):
+        assert torch.equal(x, y)
+    check(outs[True][0], plain_logits(name, a)[:90], "bfloat16", f"{name} native first portion")
