@@ -382,7 +382,9 @@ __global__ __launch_bounds__(256) void mid_finish_qkv_kernel(
   }
 }
 
-// `shape` = 16 * NW + KW for the shapes that are built.
+// The workgroup shapes that are built: four feature tiles a workgroup with one or two waves on
+// each for the plain products, two tiles with one, two or four waves on each for the gated one
+// (whose waves hold two sets of weights). Others are refused.
 template <int MT, int EPI>
 int launch_mid(int nw, int kw, const MidArgs& a, hipStream_t stream) {
   const int tiles = (a.N + 15) / 16;
@@ -392,7 +394,11 @@ int launch_mid(int nw, int kw, const MidArgs& a, hipStream_t stream) {
     mid_gemm_kernel<MT, NW_, KW_, EPI><<<grid, NW_ * KW_ * 64, 0, stream>>>(a);         \
     return dli_launch_status();                                                         \
   }
-  MID_CASE(4, 1) MID_CASE(2, 1) MID_CASE(4, 2) MID_CASE(2, 2) MID_CASE(2, 4) MID_CASE(4, 4)
+  if constexpr (EPI == MID_SWIGLU) {
+    MID_CASE(2, 1) MID_CASE(2, 2) MID_CASE(2, 4)
+  } else {
+    MID_CASE(4, 1) MID_CASE(4, 2)
+  }
 #undef MID_CASE
   return DLI_ERR_ARGUMENT;
 }

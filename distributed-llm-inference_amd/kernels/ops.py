@@ -495,7 +495,8 @@ def mid_gemm_supports(rows: int, k: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and 0 < rows <= MID_ROWS and k > 0 and k % 128 == 0
 
 
-MID_SHAPES = ((4, 1), (2, 1), (4, 2), (2, 2), (2, 4), (4, 4))  # (waves, kwaves) that are built
+MID_SHAPES = ((4, 1), (4, 2))              # (waves, kwaves) that are built for the plain products
+MID_SHAPES_GATED = ((2, 1), (2, 2), (2, 4))  # and for the gated one
 
 
 def mid_gemm_plan(n: int, k: int, epilogue: int, units: int) -> tuple[int, int, int]:
@@ -507,9 +508,10 @@ def mid_gemm_plan(n: int, k: int, epilogue: int, units: int) -> tuple[int, int, 
     aims at one workgroup on every compute unit with eight to sixteen waves, each with few blocks
     of 128 k to fetch."""
     tiles, blocks = -(-n // 16), k // 128
-    if epilogue != MID_PARTIAL:
-        waves = 2 if tiles >= 2 * units or epilogue == MID_SWIGLU else 4
-        return waves, 4 if blocks >= 8 else (2 if blocks >= 2 else 1), 1
+    if epilogue == MID_SWIGLU:
+        return 2, 4 if blocks >= 8 else (2 if blocks >= 2 else 1), 1
+    if epilogue == MID_STORE:
+        return 4, 2 if blocks >= 2 else 1, 1
     waves = 4
     groups = -(-tiles // waves)
     splits = max(1, min(blocks, round(units / groups)))
@@ -554,8 +556,9 @@ def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = F
     waves = plan_waves if waves is None else waves
     kwaves = plan_kwaves if kwaves is None else kwaves
     splits = plan_splits if splits is None else splits
-    _require((waves, kwaves) in MID_SHAPES and 1 <= splits <= k // 128,
-             f"(waves, kwaves) must be one of {MID_SHAPES}, splits 1..k/128")
+    built = MID_SHAPES_GATED if epilogue == MID_SWIGLU else MID_SHAPES
+    _require((waves, kwaves) in built and 1 <= splits <= k // 128,
+             f"(waves, kwaves) must be one of {built}, splits 1..k/128")
     if epilogue == MID_PARTIAL:
         _require(bias is None and n % 4 == 0, "partial products take no bias, n % 4 == 0")
         if out is None:
