@@ -231,7 +231,9 @@ def main() -> int:
                          "128 generated tokens each, with reuse of cached pages")
     ap.add_argument("--budget", type=int, default=2048, help="tokens a step for --serving")
     ap.add_argument("--only-prefill", action="store_true",
-                    help="run only the 2,048-token prefill steps (for profiling) and print their time")
+                    help="run only prefill steps of --prefill-tokens tokens (for profiling) and print their time")
+    ap.add_argument("--prefill-tokens", type=int, default=2048,
+                    help="prompt length of --only-prefill (the line of the default run always has 2,048)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
@@ -257,12 +259,17 @@ def main() -> int:
                        "decode_steps_per_engine_step": min(args.decode_steps, 8)}, **got}))
         return 0
     max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
-    engine, cfg = make_engine(raw, args.dtype, max_batch, args.context, args.block_size, budget=8192,
+    context = max(args.context, args.prefill_tokens + 64) if args.only_prefill else args.context
+    engine, cfg = make_engine(raw, args.dtype, max_batch, context, args.block_size,
+                              budget=max(8192, args.prefill_tokens if args.only_prefill else 0),
                               decode_steps=args.decode_steps)
 
     if args.only_prefill:
-        t = prefill_run(engine, cfg, 2048, repeats=args.steps)
-        print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": 2048, "tok_s": round(2048 / t, 1)}))
+        n = args.prefill_tokens
+        t = prefill_run(engine, cfg, n, repeats=args.steps)
+        print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": n, "tok_s": round(n / t, 1),
+                          "frac": round(prefill_flops(cfg, n) / t / PEAK_FLOPS[short], 4),
+                          "attention_gflop_per_layer": round(2 * cfg.num_heads * cfg.head_dim * n * (n + 1) / 1e9, 2)}))
         return 0
     tok_s, ms, per_engine_step = decode_run(engine, cfg, args.batch, args.context, args.steps, args.warmup,
                                             args.decode_steps)
