@@ -330,14 +330,14 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float keep = fast_exp2(m_run - m_safe);  // rescales what earlier rounds left
     const float weight = lane < n ? fast_exp2(m_s - m_safe) : 0.f;
-    l_run = l_run * keep + wave_sum(l_s * weight);
+    l_run = __fmaf_rn(l_run, keep, wave_sum(__fmul_rn(l_s, weight)));
 #pragma unroll
     for (int v = 0; v < DV; ++v) acc[v] *= keep;
 #pragma unroll
     for (int j = 0; j < SMAX; ++j) {
       const float wj = __shfl(weight, j, DLI_WAVE);
 #pragma unroll
-      for (int v = 0; v < DV; ++v) acc[v] += po[j][v] * wj;
+      for (int v = 0; v < DV; ++v) acc[v] = __fmaf_rn(po[j][v], wj, acc[v]);
     }
     m_run = m_new;
   }
@@ -756,12 +756,13 @@ extern "C" int dli_attention_prefill_tile_rows(int head_dim, int q_heads, int kv
   return hw == 0 ? PF_TILE_ROWS : (4 / hw) * 32;
 }
 
-extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pages,
-                                         const void* v_pages, void* out, int64_t out_stride,
-                                         float* part_o, float* part_ml, const int* kv_len,
-                                         const int* block_tables, int table_stride, int requests,
-                                         int q_heads, int kv_heads, int head_dim, int page_size,
-                                         float scale, int window, int splits, hipStream_t stream) {
+// merge: whether the partial results of more than one run of keys are merged into `out` here, or
+// left in part_o / part_ml for the kernel that reads them next.
+static int attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                            void* out, int64_t out_stride, float* part_o, float* part_ml,
+                            const int* kv_len, const int* block_tables, int table_stride, int requests,
+                            int q_heads, int kv_heads, int head_dim, int page_size, float scale,
+                            int window, int splits, bool merge, hipStream_t stream) {
   if (requests <= 0) return DLI_OK;
   if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || splits < 1 || splits > 65535 || requests > 65535 ||
@@ -784,7 +785,7 @@ extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const 
   }
 #undef DECODE_CASE
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
-  if (splits > 1) {
+  if (splits > 1 && merge) {
     const int pairs = requests * q_heads;
 #define MERGE(S, V)                                                             \
   attention_merge_kernel<S, V><<<(pairs + 3) / 4, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, \
@@ -800,6 +801,32 @@ extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const 
 #undef MERGE
   }
   return dli_launch_status();
+}
+
+extern "C" int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pages,
+                                         const void* v_pages, void* out, int64_t out_stride,
+                                         float* part_o, float* part_ml, const int* kv_len,
+                                         const int* block_tables, int table_stride, int requests,
+                                         int q_heads, int kv_heads, int head_dim, int page_size,
+                                         float scale, int window, int splits, hipStream_t stream) {
+  return attention_decode(q, q_stride, k_pages, v_pages, out, out_stride, part_o, part_ml, kv_len, block_tables,
+                          table_stride, requests, q_heads, kv_heads, head_dim, page_size, scale, window, splits,
+                          true, stream);
+}
+
+// The same without the merge: with two or more runs of keys the partial results stay in part_o
+// [requests][q_heads][splits][head_dim] and part_ml [requests][q_heads][splits][2] and `out` is not
+// written (dli_skinny_gemm_merged reads them).
+extern "C" int dli_attention_decode_partial_bf16(const void* q, int64_t q_stride, const void* k_pages,
+                                                 const void* v_pages, float* part_o, float* part_ml,
+                                                 const int* kv_len, const int* block_tables,
+                                                 int table_stride, int requests, int q_heads, int kv_heads,
+                                                 int head_dim, int page_size, float scale, int window,
+                                                 int splits, hipStream_t stream) {
+  if (splits < 2) return DLI_ERR_ARGUMENT;
+  return attention_decode(q, q_stride, k_pages, v_pages, nullptr, 0, part_o, part_ml, kv_len, block_tables,
+                          table_stride, requests, q_heads, kv_heads, head_dim, page_size, scale, window, splits,
+                          false, stream);
 }
 
 // ---------------------------------------------------------------- decode without an allocation

@@ -33,10 +33,18 @@
 //                 t of a head holds its dimensions 8t..8t+7 and half+8t..half+8t+7, i.e. eight
 //                 rotary pairs, whose partners sit 32 lanes apart in the product's result. q is
 //                 stored to out in the usual order; k and v go to the pages only.
+//   MERGED   the activations are not read from x but made in the kernel from the split-key partial
+//            results of the decode attention (o_s, m_s, l_s per request, head and run of keys):
+//            x[m][head*D + d] = cast(sum_s o_s[d] 2^(m_s - M) / sum_s l_s 2^(m_s - M)), the same
+//            arithmetic in the same order as attention_merge_kernel, so that the o projection of a
+//            step of one to four rows needs no merge kernel before it. Each wave merges the run of
+//            k that it multiplies (all loads of a lane in flight at once) and hands it to its
+//            lanes through LDS. TILED, EPI_RESIDUAL, at most 16 runs.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2, EPI_F32 = 3, EPI_QKV = 4 };
 
@@ -50,6 +58,17 @@ struct QkvRope {
   bf16_t* v_pages;
   int q_heads, kv_heads, head_dim, page_size;
 };
+
+// What MERGED reads instead of x: part_o [rows][heads][splits][head_dim] and part_ml
+// [rows][heads][splits][2] (running maximum in units of log2, sum) float32.
+struct MergedIn {
+  const float* part_o;
+  const float* part_ml;
+  int splits, heads, head_dim;
+};
+#define MERGE_ROWS 4     // rows of a step whose o projection merges by itself
+#define MERGE_RANGE 512  // the longest run of k of one wave
+#define MERGE_SPLITS 16
 
 __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -98,14 +117,17 @@ __device__ __forceinline__ bf16x8 finish_x(const XFrag<NORM>& f, float rs) {
 // KS waves split k, NS groups of waves split the workgroup's tiles, each wave owns NT tiles:
 // a workgroup computes NS*NT tiles of 16 features with KS*NS waves. The activation fragments are
 // loaded once per block of k and reused for the wave's NT tiles.
-template <int KS, int NS, int NT, int MT, int EPI, bool NORM, bool TILED>
+template <int KS, int NS, int NT, int MT, int EPI, bool NORM, bool TILED, bool MERGED = false>
 __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
     const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
     const bf16_t* __restrict__ bias, void* __restrict__ out, int64_t ldo,
     bf16_t* __restrict__ stream, int64_t lds_, float* __restrict__ ssq_out, int M, int N, int K,
-    int up_offset, QkvRope qr) {
+    int up_offset, QkvRope qr, MergedIn mi) {
   static_assert(EPI != EPI_QKV || (TILED && MT == 1), "the q/k/v epilogue reads tiled weights, at most 16 rows");
+  static_assert(!MERGED || (TILED && MT == 1 && NS == 1 && !NORM), "merged activations: tiled weights, one row tile");
+  // MERGED: each wave's run of k for up to MERGE_ROWS rows
+  __shared__ __align__(16) bf16_t xs[MERGED ? KS : 1][MERGED ? MERGE_ROWS : 1][MERGED ? MERGE_RANGE : 8];
   constexpr int NA = EPI == EPI_SWIGLU ? 2 : 1;  // weight row sets per tile (gate and up)
   constexpr int KR = KS > 1 ? KS - 1 : 1;
   __shared__ float red[KR][NS][NT][NA][MT][4][64];  // k-split waves 1.. hand their tiles to wave 0
@@ -223,6 +245,58 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           af[j][a][q] = *w_at(wrow[j][a], s, q);
+  }
+  if constexpr (MERGED) {
+    // The wave's run of k, four values a lane and turn: the statistics and partial outputs of all
+    // runs of keys are asked for before the first is used. Sums in the order of
+    // attention_merge_kernel: the denominators pairwise as its butterfly adds them (lanes 8
+    // apart, then 4, 2, 1), the outputs run by run.
+    const int kb0 = s_begin * 32, quads = (s_end - s_begin) * 8;
+    const int D = mi.head_dim, S = mi.splits;
+    for (int item = lane; item < M * quads; item += 64) {
+      const int row = item / quads, idx = (item - row * quads) * 4;
+      const int k = kb0 + idx, head = k / D, d = k - head * D;
+      const int64_t base = ((int64_t)row * mi.heads + head) * S;
+      float2v ml[MERGE_SPLITS];
+      float4v po[MERGE_SPLITS];
+#pragma unroll
+      for (int j = 0; j < MERGE_SPLITS; ++j) {
+        ml[j] = float2v{-INFINITY, 0.f};
+        po[j] = float4v{0.f, 0.f, 0.f, 0.f};
+        if (j < S) {
+          ml[j] = *reinterpret_cast<const float2v*>(mi.part_ml + (base + j) * 2);
+          po[j] = *reinterpret_cast<const float4v*>(mi.part_o + (base + j) * D + d);
+        }
+      }
+      float m_all = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < MERGE_SPLITS; ++j) m_all = fmaxf(m_all, ml[j][0]);
+      const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+      float wgt[MERGE_SPLITS], t[MERGE_SPLITS];
+#pragma unroll
+      for (int j = 0; j < MERGE_SPLITS; ++j) {
+        wgt[j] = j < S ? __builtin_amdgcn_exp2f(ml[j][0] - m_safe) : 0.f;
+        t[j] = __fmul_rn(ml[j][1], wgt[j]);
+      }
+#pragma unroll
+      for (int h = MERGE_SPLITS / 2; h > 0; h >>= 1)
+#pragma unroll
+        for (int j = 0; j < h; ++j) t[j] = __fadd_rn(t[j], t[j + h]);
+      const float inv = t[0] > 0.f ? 1.f / t[0] : 0.f;
+      float4v acc4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < MERGE_SPLITS; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc4[i] = __fmaf_rn(po[j][i], wgt[j], acc4[i]);
+      bf16_t* dst = &xs[ks][row][idx];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)__fmul_rn(acc4[i], inv);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xrow[t] = &xs[ks][min(t * 16 + col, M - 1)][0] - kb0;
+  }
+  if (s + 4 <= s_end) {
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -435,7 +509,7 @@ static void launch_skinny(SK_PARAMS) {
   const int groups = (tiles + NS * NT - 1) / (NS * NT);
   skinny_gemm_kernel<KS, NS, NT, MT, EPI, NORM, TILED><<<groups, KS * NS * 64, 0, stream>>>(
       (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
-      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset, qr);
+      out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset, qr, MergedIn{});
 }
 
 // shapes of the workgroup: 0: 4 k-waves x 1 tile (few tiles, short k); 1: 8 k-waves x 1 tile (few
@@ -520,6 +594,39 @@ extern "C" int dli_skinny_gemm_qkv_rope(const void* x, int64_t ldx, const float*
   if (norm_w != nullptr) dispatch_shape<1, EPI_QKV, true, true>(shape, SK_ARGS);
   else dispatch_shape<1, EPI_QKV, false, true>(shape, SK_ARGS);
   return dli_launch_status();
+}
+
+// The o projection of a decode step of at most MERGE_ROWS rows, fed with the split-key partial
+// results of the attention instead of its merged output (MERGED above): stream += merge(...) @ w^T
+// (+ bias), and the parts of the rows' sums of squares. w_tiled [N, K] in tile order with
+// K = heads * head_dim; splits 2..MERGE_SPLITS; shape 0 or 1 (4 or 8 waves split k).
+extern "C" int dli_skinny_gemm_merged(const float* part_o, const float* part_ml, int splits, int heads,
+                                      int head_dim, const void* w_tiled, const void* bias, void* stream_buf,
+                                      int64_t lds_, float* ssq_out, int M, int N, int shape, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return DLI_OK;
+  const int64_t K64 = (int64_t)heads * head_dim;
+  if (M > MERGE_ROWS || splits < 2 || splits > MERGE_SPLITS || heads <= 0 || head_dim <= 0 || head_dim % 4 != 0 ||
+      K64 % 128 != 0 || K64 > (1 << 20) || N % 16 != 0 || (shape != 0 && shape != 1) || part_o == nullptr ||
+      part_ml == nullptr || w_tiled == nullptr || stream_buf == nullptr || ssq_out == nullptr)
+    return DLI_ERR_ARGUMENT;
+  const int K = (int)K64, ks = shape == 0 ? 4 : 8;
+  if (((K / 128 + ks - 1) / ks) * 128 > MERGE_RANGE) return DLI_ERR_ARGUMENT;
+  const MergedIn mi{part_o, part_ml, splits, heads, head_dim};
+  const int groups = N / 16;
+#define MERGED_LAUNCH(KS)                                                                          \
+  skinny_gemm_kernel<KS, 1, 1, 1, EPI_RESIDUAL, false, true, true><<<groups, KS * 64, 0, stream>>>( \
+      nullptr, 0, nullptr, 0, nullptr, 0.f, (const bf16_t*)w_tiled, (const bf16_t*)bias, nullptr, 0, \
+      (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, 0, QkvRope{}, mi)
+  if (shape == 0) MERGED_LAUNCH(4);
+  else MERGED_LAUNCH(8);
+#undef MERGED_LAUNCH
+  return dli_launch_status();
+}
+
+extern "C" int dli_skinny_gemm_merged_limits(int* rows, int* splits) {
+  *rows = MERGE_ROWS;
+  *splits = MERGE_SPLITS;
+  return DLI_OK;
 }
 
 extern "C" int dli_embedding_ssq(const void* table, const int* ids, void* out, float* ssq, int rows,

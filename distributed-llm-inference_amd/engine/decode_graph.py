@@ -49,6 +49,7 @@ class _Captured:
     width: int              # block-table entries per row
     rows: TableRows         # what the block-table rows hold, so that a replay patches them
     tokens_host: Optional[torch.Tensor] = None  # pinned int32 [steps * b]: sampled tokens (sampling graphs)
+    staged: Optional[torch.cuda.Event] = None   # the last copy of host to dev: host is not refilled before it
 
 
 class DecodeGraphs:
@@ -229,6 +230,10 @@ class DecodeGraphs:
         if cap is None:
             cap = self.captured[key] = self._capture(*key)
         v = cap.views
+        if cap.staged is not None:
+            # a caller that used the last logits without waiting for them (a copy on the stream,
+            # say) comes back while the copy of the staging buffer may still be queued
+            cap.staged.synchronize()
         limit = self.step_fn.store.num_pages
         token_ids, positions, kv_len, state_slots = v["token_ids"], v["positions"], v["kv_len"], v["state_slots"]
         # The step's arrays are filled in bulk (one conversion per array instead of one per number):
@@ -260,6 +265,10 @@ class DecodeGraphs:
             ts, ks, pp, sd, dr = zip(*sampling)
             temp[:n], v["top_k"][:n], top_p[:n], seeds[:n], counters[:n] = ts, ks, pp, sd, dr
         cap.dev.copy_(cap.host, non_blocking=True)
+        if not sampled:  # the sampling path waits for the whole replay below
+            if cap.staged is None:
+                cap.staged = torch.cuda.Event()
+            cap.staged.record()
         cap.graph.replay()
         self.replays += 1
         if sampled:

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "dli_skinny_gemm_qkv_rope": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64,
                                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_ptr],
+    "dli_skinny_gemm_merged": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int,
+                               _c_int, _c_int, _c_ptr],
     "dli_mid_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_int,
                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_mid_finish_residual": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_ptr],
@@ -68,6 +70,8 @@ _SIGNATURES = {
     "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "dli_attention_decode_partial_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_decode_bf16_static": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int,
                                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_rope_angles": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -482,6 +486,57 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
     return ssq_out if epilogue == SKINNY_RESIDUAL else None
 
 
+MERGED_ROWS, MERGED_SPLITS, _MERGED_RANGE = 4, 16, 512  # csrc/skinny_gemm.hip: MERGE_ROWS, MERGE_SPLITS, MERGE_RANGE
+
+
+def skinny_gemm_merged_supports(rows: int, n: int, heads: int, head_dim: int, splits: int,
+                                device: torch.device) -> bool:
+    """Whether :func:`skinny_gemm_merged` takes this o projection: few rows, few runs of keys, a
+    product that the 16x16-tile kernel runs with k split over the waves of a workgroup."""
+    k = heads * head_dim
+    if not (0 < rows <= MERGED_ROWS and 2 <= splits <= MERGED_SPLITS and head_dim % 4 == 0 and k % 128 == 0
+            and n % 16 == 0):
+        return False
+    kernel, shape, _ = skinny_gemm_plan(rows, n, k, SKINNY_RESIDUAL, device, tiled=True)
+    return kernel == "tiles16" and shape in (0, 1) and -(-(k // 128) // (4 if shape == 0 else 8)) * 128 <= _MERGED_RANGE
+
+
+def skinny_gemm_merged(part_o: torch.Tensor, part_ml: torch.Tensor, splits: int, heads: int, head_dim: int,
+                       w_tiled: torch.Tensor, stream: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                       ssq_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``stream += merge(part_o, part_ml) @ w.T (+ bias)`` for at most four rows: the o projection
+    of a decode step fed with the partial results that :func:`attention_decode` leaves with
+    ``merge=False`` (``part_o [rows, heads, splits, head_dim]``, ``part_ml [rows, heads, splits, 2]``),
+    merged inside the product's kernel with the arithmetic of the merge kernel. Returns the parts
+    of the rows' sums of squares like the residual epilogue of :func:`skinny_gemm`."""
+    _rows(stream, "stream", torch.bfloat16)
+    m, n = stream.shape
+    k = heads * head_dim
+    _require(skinny_gemm_merged_supports(m, n, heads, head_dim, splits, stream.device),
+             f"the merging o projection takes 1..{MERGED_ROWS} rows and 2..{MERGED_SPLITS} runs of keys, "
+             f"not {m} rows, {splits} runs, {heads} heads of {head_dim}")
+    _dense(part_o, "part_o", torch.float32)
+    _dense(part_ml, "part_ml", torch.float32)
+    _require(part_o.numel() >= m * heads * splits * head_dim and part_ml.numel() >= m * heads * splits * 2,
+             "partial-result buffers are too small")
+    _require(part_o.data_ptr() % 16 == 0 and part_ml.data_ptr() % 8 == 0, "partial results must be 16-byte aligned")
+    _dense(w_tiled, "w_tiled", torch.bfloat16, 1)
+    _require(w_tiled.numel() == n * k and w_tiled.data_ptr() % 16 == 0, "w_tiled must hold [n, heads*head_dim] in tile order")
+    if bias is not None:
+        _dense(bias, "bias", torch.bfloat16, 1)
+        _require(bias.shape[0] == n, "bias length differs from rows of w")
+    _, shape, n_parts = skinny_gemm_plan(m, n, k, SKINNY_RESIDUAL, stream.device, tiled=True)
+    if ssq_out is None:
+        ssq_out = torch.empty(n_parts, m, device=stream.device, dtype=torch.float32)
+    _dense(ssq_out, "ssq_out", torch.float32, 2)
+    _require(ssq_out.shape == (n_parts, m), f"ssq_out must be [{n_parts}, rows] for this product")
+    _require(stream.data_ptr() % 8 == 0, "stream must be 8-byte aligned")
+    _check(library().dli_skinny_gemm_merged(
+        _ptr(part_o), _ptr(part_ml), int(splits), int(heads), int(head_dim), _ptr(w_tiled), _ptr(bias), _ptr(stream),
+        stream.stride(0), _ptr(ssq_out), m, n, shape, _stream()), "skinny_gemm_merged")
+    return ssq_out
+
+
 _GEMM_WORKSPACE_BYTES = 64 << 20
 _gemm_workspaces: dict[int, torch.Tensor] = {}
 
@@ -852,17 +907,20 @@ def _check_paged(q, k_pages, v_pages, out, q_heads):
     return kv_heads, page_size, head_dim
 
 
-def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: Optional[torch.Tensor],
                      kv_len: torch.Tensor, block_tables: torch.Tensor, q_heads: int, scale: float,
                      window: int = 0, splits: int = 1, part_o: Optional[torch.Tensor] = None,
-                     part_ml: Optional[torch.Tensor] = None) -> None:
+                     part_ml: Optional[torch.Tensor] = None, merge: bool = True) -> None:
     """Decode attention: row ``e`` of ``q`` is request ``e``'s single query over its ``kv_len[e]`` keys.
 
     With ``splits > 1`` each request's keys are cut into that many runs whose partial results go
     through ``part_o [rows, q_heads, splits, head_dim]`` and ``part_ml [rows, q_heads, splits, 2]``
-    (float32) and are merged by a second kernel.
+    (float32) and are merged by a second kernel; with ``merge=False`` (``splits > 1`` only) they
+    are left there for :func:`skinny_gemm_merged` and ``out`` is not written (it may be None).
     """
-    kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
+    _require(merge or splits > 1, "without a merge there must be two or more runs of keys")
+    kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out if out is not None else q, q_heads)
+    _require(merge is False or out is not None, "out is needed unless the partial results are left unmerged")
     rows = q.shape[0]
     _dense(kv_len, "kv_len", torch.int32, 1)
     _dense(block_tables, "block_tables", torch.int32, 2)
@@ -874,6 +932,12 @@ def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
         _dense(part_ml, "part_ml", torch.float32)
         _require(part_o.numel() >= rows * q_heads * splits * head_dim and part_ml.numel() >= rows * q_heads * splits * 2,
                  "partial-result buffers are too small")
+    if not merge:
+        _check(library().dli_attention_decode_partial_bf16(
+            _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(part_o), _ptr(part_ml), _ptr(kv_len),
+            _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size, float(scale),
+            int(window), int(splits), _stream()), "attention_decode")
+        return
     _check(library().dli_attention_decode_bf16(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml),
         _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size,

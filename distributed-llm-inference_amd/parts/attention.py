@@ -20,7 +20,7 @@ from typing import Any, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .attention_kernels import paged_attention
+from .attention_kernels import decode_attention_unmerged, paged_attention
 from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
 from .linear import decode_copy, linear
 from .registry import build_part, register_part
@@ -31,6 +31,12 @@ from .spec import PartSpec, WeightSpec
 # kernel runs. (A variant that rotated inside the attention kernel instead, repeating the rotation
 # in every split of the keys, was slower from four rows on and no faster below.)
 ROPE_IN_PRODUCT_ROWS = range(1, 17)
+# Decode steps with this many rows leave the merge of the runs of keys to the o projection, whose
+# waves merge the k that they multiply while their first weights are on their way. Every workgroup
+# of that product repeats the merge of all rows, so it pays for one or two rows only (a batch-1
+# step at the 1B sizes: 9.7 -> 7.3 us for merge plus product, 2% of the step; nothing gained at
+# two rows; at three and four rows the step was 6% slower than with the merge kernel).
+MERGE_IN_PRODUCT_ROWS = 2
 FEW_ROWS = 16  # up to here the few-row product kernels run; from 17 to 64 rows the one that shares activations
 
 
@@ -193,6 +199,17 @@ class GQAttention(Mixer):
                 inv_freq, rotary_dim = table.inv_freq, table.dim
             ops.rope_kv_write(qkv, ctx.positions, inv_freq, rotary_dim, grp.slots if nkv else None,
                               cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
+        if n <= MERGE_IN_PRODUCT_ROWS and self.w_o_tiled is not None:
+            # the o projection merges the runs of keys itself while its first
+            # weights are on their way, and no merge kernel runs between the two
+            left = decode_attention_unmerged(
+                qkv[:, :nh * d], cache.k_pages, cache.v_pages, ctx, grp, nh, self.scale, self.window,
+                lambda splits: ops.skinny_gemm_merged_supports(n, self.hidden_size, nh, d, splits, qkv.device))
+            if left is not None:
+                splits, part_o, part_ml = left
+                stream.ssq = ops.skinny_gemm_merged(part_o, part_ml, splits, nh, d, self.w_o_tiled, stream.x,
+                                                    bias=self.b_o)
+                return
         out = self.rt.empty(n, nh * d)
         paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,

@@ -57,6 +57,24 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
                               tile_entry, tile_q0, q_heads, scale, window)
 
 
+def decode_attention_unmerged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, ctx: Any, grp: Any,
+                              q_heads: int, scale: float, window: int, wanted) -> Any:
+    """Attention of a step in which every row is one request's single token, without the kernel
+    that merges the runs of keys: ``(splits, part_o, part_ml)`` for the product that merges while
+    it loads (``ops.skinny_gemm_merged``), or None (nothing has run) where the step's keys are
+    not split or ``wanted(splits)`` says that this product does not take them."""
+    _, kv_heads, page_size, head_dim = k_pages.shape
+    nd = ctx.num_decode
+    if nd != ctx.num_tokens or not ops.attention_mfma_supports(head_dim, page_size, k_pages.dtype):
+        return None
+    splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device)
+    if splits < 2 or not wanted(splits):
+        return None
+    ops.attention_decode(q[:nd], k_pages, v_pages, None, ctx.kv_len, grp.block_tables, q_heads, scale, window,
+                         splits, part_o, part_ml, merge=False)
+    return splits, part_o, part_ml
+
+
 def _decode_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, head_dim: int, device: torch.device):
     group = q_heads // kv_heads
     splits = getattr(ctx, "forced_splits", None) or choose_splits(

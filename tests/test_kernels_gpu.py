@@ -224,6 +224,67 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
     assert err < tol(torch.bfloat16), err
 
 
+@pytest.mark.parametrize("rows", [1, 2, 3, 4])
+@pytest.mark.parametrize("qh,kvh,d,n,splits", [(32, 8, 64, 2048, 16), (32, 8, 64, 2048, 8), (8, 2, 48, 304, 3),
+                                               (24, 8, 128, 3072, 16), (2, 1, 64, 48, 2), (16, 16, 16, 512, 5)])
+def test_o_projection_that_merges_the_split_key_results_itself(ops, rows, qh, kvh, d, n, splits):
+    """Attention without its merge kernel, then the o projection that merges while it loads,
+    against attention with the merge kernel and the plain residual product: the same bits, since
+    both add in the same order. Lengths make some runs of keys empty; a bias; rows of the stream
+    wider than the product."""
+    bs = 16
+    lens = [(1, kv) for kv in [700, 33, 1, 255][:rows]]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=rows + d + splits)
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    q, kp, vp, kv_len, tables = q.cuda(), kp.cuda(), vp.cuda(), dev(kv_len), dev(tables)
+    scale = 1.0 / math.sqrt(d)
+    k = qh * d
+    gen = torch.Generator().manual_seed(n + rows)
+    w = (torch.randn(n, k, generator=gen) / math.sqrt(k)).bfloat16().cuda()
+    bias = torch.randn(n, generator=gen).bfloat16().cuda()
+    wt = ops.tile_weights(w)
+    base = torch.randn(rows, n + 8, generator=gen).bfloat16().cuda()
+    assert ops.skinny_gemm_merged_supports(rows, n, qh, d, splits, q.device)
+
+    def partials():
+        return (torch.full((rows * qh * splits * d,), float("nan"), device="cuda"),
+                torch.full((rows * qh * splits * 2,), float("nan"), device="cuda"))
+
+    po, pm = partials()
+    out = torch.empty_like(q)
+    ops.attention_decode(q, kp, vp, out, kv_len, tables, qh, scale, 0, splits, po, pm)
+    want = base.clone()
+    ssq_want = ops.skinny_gemm(out, w, w_tiled=wt, epilogue=ops.SKINNY_RESIDUAL, stream=want[:, :n], bias=bias)
+
+    po, pm = partials()
+    ops.attention_decode(q, kp, vp, None, kv_len, tables, qh, scale, 0, splits, po, pm, merge=False)
+    got = base.clone()
+    ssq_got = ops.skinny_gemm_merged(po, pm, splits, qh, d, wt, got[:, :n], bias=bias)
+    assert torch.equal(got, want)
+    assert torch.equal(ssq_got, ssq_want)
+    # and both are the product of the attention's output (64-bit reference)
+    ref = base[:, :n].cpu().double() + (out.cpu().double() @ w.cpu().double().T + bias.cpu().double())
+    assert (got[:, :n].cpu().double() - ref).abs().max() < 3e-2 * max(1.0, ref.abs().max().item())
+
+
+def test_the_merging_o_projection_refuses_what_it_does_not_take(ops):
+    dev = torch.device("cuda")
+    assert not ops.skinny_gemm_merged_supports(5, 2048, 32, 64, 8, dev)       # rows
+    assert not ops.skinny_gemm_merged_supports(1, 2048, 32, 64, 17, dev)      # runs of keys
+    assert not ops.skinny_gemm_merged_supports(1, 2048, 32, 64, 1, dev)       # nothing to merge
+    assert not ops.skinny_gemm_merged_supports(1, 2048, 6, 32, 4, dev)        # k % 128
+    assert not ops.skinny_gemm_merged_supports(1, 2048, 64, 128, 4, dev)      # a wave's run of k too long
+    stream = torch.zeros(1, 2048, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelArgumentError):
+        ops.skinny_gemm_merged(torch.zeros(8, device="cuda"), torch.zeros(8, device="cuda"), 17, 32, 64,
+                               torch.zeros(2048 * 2048, device="cuda", dtype=torch.bfloat16), stream)
+    q = torch.zeros(1, 2048, device="cuda", dtype=torch.bfloat16)
+    pages = torch.zeros(2, 8, 16, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelArgumentError):
+        ops.attention_decode(q, pages, pages.view(2, 8, 64, 16), None, torch.ones(1, dtype=torch.int32, device="cuda"),
+                             torch.zeros(1, 1, dtype=torch.int32, device="cuda"), 32, 1.0, 0, 1, merge=False)
+
+
 @pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37])
 @pytest.mark.parametrize("pair", [False, True])

@@ -98,6 +98,47 @@ def test_requests_decode_together_at_serving_widths(count):
     assert core.step.graphs.replays >= steps
 
 
+@pytest.mark.parametrize("count", [1, 2])
+def test_one_and_two_requests_decode_without_a_merge_kernel(count, monkeypatch):
+    """With one or two rows and keys enough for two runs, the o projection merges the runs of
+    keys itself: the path is taken (counted), agrees with the plain implementation, and gives the
+    bits of the path with the merge kernel. The steps' logits are copied on the stream and looked
+    at only after the last step: a replay must not refill its staging buffer while the copy of the
+    step before is still queued."""
+    from dli_amd.kernels import ops
+    from dli_amd.parts import attention
+    from dli_amd.trace import TraceSession
+
+    rng = random.Random(11 + count)
+    lens = [300, 270][:count]
+    steps = 6
+    toks = [[rng.randrange(32003) for _ in range(n + steps)] for n in lens]
+    calls = []
+    real = ops.skinny_gemm_merged
+    monkeypatch.setattr(ops, "skinny_gemm_merged", lambda *a, **k: (calls.append(a[2]), real(*a, **k))[1])
+
+    def run(limit):
+        monkeypatch.setattr(attention, "MERGE_IN_PRODUCT_ROWS", limit)
+        core = make_core("bfloat16", pages=48, graphs=count)
+        s = TraceSession(core)
+        s.step([{"id": r, "tokens": toks[r][:lens[r]], "want": []} for r in range(count)])
+        outs = []
+        for i in range(steps):
+            outs.append(s.step([{"id": r, "tokens": [toks[r][lens[r] + i]], "want": [0]} for r in range(count)]).clone())
+        return outs
+
+    merged = run(2)
+    assert calls and all(splits >= 2 for splits in calls)
+    for i, out in enumerate(merged):
+        rows = torch.stack([plain(toks[r])[lens[r] + i] for r in range(count)])
+        check(out, rows, "bfloat16", f"decode step {i} of {count} without a merge kernel")
+    seen = len(calls)
+    separate = run(0)
+    assert len(calls) == seen
+    for a, b in zip(merged, separate):
+        assert torch.equal(a, b)
+
+
 def test_llama_3_2_1b_at_full_depth_and_vocabulary():
     """All 16 layers and all 128,256 vocabulary rows of Llama-3.2-1B (random weights written to a
     folder and loaded by name like a checkpoint), 32-bit and bfloat16 against the plain
