@@ -51,15 +51,17 @@ def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, 
                 prefix_caching=False):
     import torch
 
-    from dli_amd.engine import LLMEngine, SchedulerConfig
-    from dli_amd.parts.base import Runtime
-    from dli_amd.weights.loader import build_model, parse_dtype
-    from dli_amd.weights.random_init import fill_random_on_device
+    import tempfile
 
-    rt = Runtime(torch.device("cuda:0"), parse_dtype(dtype))
-    model, cfg = build_model(raw, rt)
-    model.config = cfg
-    fill_random_on_device(model, seed=0, std=0.02)
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.weights import load_model, write_random_model
+
+    # The weights take the road that generation takes: a folder with config.json and
+    # model.safetensors (drawn on the GPU, a few seconds for a billion), read by the loader.
+    with tempfile.TemporaryDirectory(prefix="dli_amd_bench_") as folder:
+        write_random_model(folder, raw, seed=0, std=0.02, device="cuda:0")
+        model = load_model(folder, dtype=dtype, device="cuda:0")
+    cfg = model.config
     pages = num_pages or batch * (-(-(context + SLACK) // block_size) + 1) + 8
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=prefix_caching,

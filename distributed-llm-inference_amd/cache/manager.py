@@ -27,6 +27,8 @@ written.
 
 from __future__ import annotations
 
+import functools
+import threading
 from collections import Counter
 from dataclasses import dataclass, field
 from typing import Hashable, Optional, Sequence
@@ -46,6 +48,28 @@ class NoFreePagesError(RuntimeError):
 
 class SequenceError(KeyError):
     """Unknown or duplicate request id."""
+
+
+class WrongThreadError(RuntimeError):
+    """A manager that is confined to one thread was changed from another."""
+
+
+def _confined(method):
+    """The manager has no lock: one thread (the engine's loop) makes every change. With
+    ``confine_to_thread`` a change from any other thread fails at once instead of corrupting the
+    tables some steps later (the reference's block manager checks the same:
+    src/dli/kv/block_manager.py:447-449)."""
+
+    @functools.wraps(method)
+    def checked(self, *args, **kwargs):
+        home = self._home_thread
+        if home is not None and threading.get_ident() != home:
+            raise WrongThreadError(
+                f"CacheManager.{method.__name__} called from thread {threading.get_ident()}, but the manager "
+                f"belongs to thread {home} (hand it over with adopt())")
+        return method(self, *args, **kwargs)
+
+    return checked
 
     def __str__(self) -> str:
         return str(self.args[0]) if self.args else ""
@@ -131,6 +155,8 @@ class CacheManager:
         stateful: the model keeps per-request state outside the pages (disables content reuse).
         watermark: fraction of each group's pages kept back when *admitting* prompts, so running
             requests can still grow (block_manager.py:138-139).
+        confine_to_thread: every call that changes the manager must come from the thread that
+            made it (or that last called :meth:`adopt`); any other raises :class:`WrongThreadError`.
     """
 
     def __init__(
@@ -144,7 +170,9 @@ class CacheManager:
         enable_prefix_caching: bool = True,
         stateful: bool = False,
         watermark: float = 0.01,
+        confine_to_thread: bool = False,
     ) -> None:
+        self._home_thread: Optional[int] = threading.get_ident() if confine_to_thread else None
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if not groups:
@@ -164,6 +192,11 @@ class CacheManager:
         self._reserve = [int(watermark * c) for c in counts]
         self._seqs: dict[SeqId, _Seq] = {}
         self._stats = CacheStats()
+
+    def adopt(self) -> None:
+        """The calling thread becomes the one that may change a confined manager."""
+        if self._home_thread is not None:
+            self._home_thread = threading.get_ident()
 
     # ------------------------------------------------------------------ queries
 
@@ -243,6 +276,7 @@ class CacheManager:
 
     # ------------------------------------------------------------------ lifecycle
 
+    @_confined
     def allocate(self, seq_id: SeqId, token_ids: Sequence[int], *, namespace: bytes = b"",
                  respect_watermark: bool = True) -> Allocation:
         """Admit a prompt: reuse cached leading pages, take the rest, take a state slot.
@@ -290,6 +324,7 @@ class CacheManager:
         self._seqs[seq_id] = seq
         return Allocation(tuple(tuple(t) for t in tables), n_cached, seq.state_slot)
 
+    @_confined
     def append_slots(self, seq_id: SeqId, token_ids: Sequence[int]) -> list[CopyOp]:
         """Reserve slots for tokens appended to the request; returns the page copies that must be
         done on the device before the next write (copy-on-write of a shared partial page)."""
@@ -325,6 +360,7 @@ class CacheManager:
             seq.tail_tokens.extend(token_ids)
         return ops
 
+    @_confined
     def reserve_ahead(self, seq_id: SeqId, extra_tokens: int) -> None:
         """Make room for ``extra_tokens`` more tokens than the request has, without naming them:
         the pages they will need are taken now, :meth:`append_slots` uses them later. For steps
@@ -348,6 +384,7 @@ class CacheManager:
                     seq.tables[g].append(pool.take())
         seq.reserved = max(seq.reserved, target)
 
+    @_confined
     def mark_computed(self, seq_id: SeqId, num_computed_tokens: int) -> None:
         """Record that the keys of the first ``num_computed_tokens`` tokens are written.
 
@@ -364,6 +401,7 @@ class CacheManager:
             if spec.kind == "window":
                 self._release_passed(seq, g, spec.window)
 
+    @_confined
     def fork(self, parent_id: SeqId, child_id: SeqId) -> int:
         """Create ``child_id`` sharing every page of the parent; returns the child's state slot
         (copying the parent's state into it is the caller's business)."""
@@ -383,6 +421,7 @@ class CacheManager:
             tail_tokens=list(parent.tail_tokens), num_registered=parent.num_registered)
         return slot
 
+    @_confined
     def free(self, seq_id: SeqId) -> None:
         """Give back everything a finished, aborted or preempted request holds. Cached pages stay
         revivable; the others return to the free list."""
@@ -395,6 +434,7 @@ class CacheManager:
                     pool.decref(page)
         self.slots.give_back(seq.state_slot)
 
+    @_confined
     def reset_prefix_cache(self) -> int:
         """Reclaim every idle cached page; returns how many."""
         return sum(p.evict_all_idle() for p in self.pools)

@@ -44,7 +44,9 @@ def pages_for_budget(model: Model, page_size: int, budget_bytes: int) -> int:
 def build_core(model: Model | str | Path, *, num_pages: int, page_size: int = 16, max_seqs: int = 64,
                dtype: str | torch.dtype = "bfloat16", device: str = "cuda",
                enable_prefix_caching: bool = True, eviction_policy: str = "lru",
-               watermark: float = 0.01) -> EngineCore:
+               watermark: float = 0.01, confine_to_thread: bool = True) -> EngineCore:
+    """``confine_to_thread``: the cache manager refuses changes from any thread but the one that
+    built the core (``core.manager.adopt()`` hands it to another)."""
     if not isinstance(model, Model):
         model = load_model(model, dtype=dtype, device=device)
     specs = model.cache_specs()
@@ -52,5 +54,5 @@ def build_core(model: Model | str | Path, *, num_pages: int, page_size: int = 16
     manager = CacheManager(
         group_specs(store.groups), num_pages=num_pages, page_size=page_size, max_seqs=max_seqs,
         eviction_policy=eviction_policy, enable_prefix_caching=enable_prefix_caching,
-        stateful=store.stateful, watermark=watermark)
+        stateful=store.stateful, watermark=watermark, confine_to_thread=confine_to_thread)
     return EngineCore(model, manager, store, StepFunction(model, manager, store))

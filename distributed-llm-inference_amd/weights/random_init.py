@@ -101,25 +101,3 @@ def write_random_model(out_dir: str | Path, config: Mapping[str, Any] | Any, *, 
     (out / "config.json").write_text(json.dumps(raw, indent=2) + "\n")
     write_safetensors(out / "model.safetensors", tensors, metadata={"format": "pt"})
     return out
-
-
-def fill_random_on_device(model: Model, *, seed: int = 0, std: float = 0.02) -> Model:
-    """Give ``model`` random weights drawn on its device, without a folder (for measurements on
-    large shapes). Matrices ``N(0, std)`` rounded to the activation type, norm weights 1."""
-    rt = model.rt
-    gen = torch.Generator(device=rt.device)
-    tensors = {}
-    for i, (name, spec) in enumerate(sorted(model.weight_specs().items())):
-        gen.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode("utf-8"))) & 0x7FFFFFFFFFFFFFFF)
-        if spec.role == "int32":
-            tensors[name] = torch.zeros(spec.shape, dtype=torch.int32, device=rt.device)
-        elif spec.init in ("norm", "ones"):
-            tensors[name] = torch.ones(spec.shape, dtype=torch.float32 if spec.role == "float32" else rt.dtype,
-                                       device=rt.device)
-        elif spec.init == "zeros":
-            tensors[name] = torch.zeros(spec.shape, dtype=rt.dtype, device=rt.device)
-        else:
-            t = torch.empty(spec.shape, dtype=torch.float32, device=rt.device).normal_(0.0, std, generator=gen)
-            tensors[name] = t.to(torch.float32 if spec.role == "float32" else rt.dtype)
-    model.load_weights(tensors)
-    return model

@@ -417,3 +417,55 @@ def test_reserving_ahead_takes_pages_now_and_appends_use_them():
     m.reset_prefix_cache()
     m.check_invariants()
     assert m.stats().free_pages == 8
+
+
+def test_a_confined_manager_refuses_other_threads():
+    """The owner-thread check of the reference's block manager (src/dli/kv/block_manager.py:447-449):
+    changes from a thread that does not own the manager fail at once and change nothing; reading
+    is allowed; adopt() hands the manager over."""
+    import threading
+
+    from dli_amd.cache import WrongThreadError
+
+    m = CacheManager(num_pages=8, page_size=4, confine_to_thread=True)
+    m.allocate("a", [1, 2, 3, 4, 5])
+    seen = {}
+
+    def elsewhere():
+        for name, call in (("allocate", lambda: m.allocate("b", [1, 2, 3])), ("append", lambda: m.append_slots("a", [6])),
+                           ("free", lambda: m.free("a")), ("fork", lambda: m.fork("a", "c")),
+                           ("computed", lambda: m.mark_computed("a", 5)), ("reset", m.reset_prefix_cache)):
+            try:
+                call()
+                seen[name] = "went through"
+            except WrongThreadError as e:
+                seen[name] = str(e)
+        seen["read"] = (m.block_table("a"), m.num_tokens("a"))
+
+    t = threading.Thread(target=elsewhere)
+    t.start()
+    t.join()
+    assert all("belongs to thread" in seen[k] for k in ("allocate", "append", "free", "fork", "computed", "reset")), seen
+    assert seen["read"] == (m.block_table("a"), 5)
+    m.check_invariants()
+    assert m.sequences() == ["a"]
+
+    def adopted():
+        m.adopt()
+        m.append_slots("a", [6])
+        seen["adopted"] = m.num_tokens("a")
+
+    t = threading.Thread(target=adopted)
+    t.start()
+    t.join()
+    assert seen["adopted"] == 6
+    with pytest.raises(WrongThreadError):
+        m.free("a")          # the first thread gave it away
+    m.adopt()
+    m.free("a")
+    # not confined: any thread may call
+    free_for_all = CacheManager(num_pages=4, page_size=4)
+    t = threading.Thread(target=lambda: free_for_all.allocate("x", [1]))
+    t.start()
+    t.join()
+    assert free_for_all.sequences() == ["x"]
