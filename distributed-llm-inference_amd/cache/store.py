@@ -2,9 +2,11 @@
 
 Layers are grouped by what their mixers declare (:class:`PagedKVSpec`): equal specs share one
 group, one block table per request and one pool tensor
-``[layers of the group, 2 (keys, values), pages, kv_heads * page_size * head_dim]``.
+``[layers of the group, 2 (keys, values), pages, kv_heads * page_size * head_dim]``
+(where a value's size differs from a key's: one tensor ``[layers, 1, pages, ...]`` for the keys
+and one for the values, or none if the mixer keeps no values).
 Inside a page, keys lie as ``[kv_heads][page_size][head_dim]`` and values as
-``[kv_heads][head_dim][page_size]`` (the order in which the attention kernels consume them).
+``[kv_heads][value_dim][page_size]`` (the order in which the attention kernels consume them).
 A mixer that declares a :class:`StateSpec` gets an array ``[state slots, *shape]`` instead.
 Everything is allocated once and zero-filled (reference: src/dli/kv/paged_store.py:50-52).
 """
@@ -28,7 +30,7 @@ class LayerCache:
     kind: str  # "paged" or "state"
     group: int = -1
     k_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, page_size, head_dim]
-    v_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, head_dim, page_size]
+    v_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, value_dim, page_size]; None: keys only
     state: Optional[torch.Tensor] = None    # [slots, *shape]
     writable: bool = True
     window: int = 0
@@ -59,7 +61,7 @@ def bytes_per_page(groups: Sequence[PagedKVSpec], layers_per_group: Sequence[int
                    dtype: torch.dtype) -> int:
     """Bytes that one page id costs across all groups and layers, keys and values."""
     item = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * n * page_size * g.kv_heads * g.head_dim * item for g, n in zip(groups, layers_per_group))
+    return sum(n * page_size * g.kv_heads * (g.head_dim + g.v_dim) * item for g, n in zip(groups, layers_per_group))
 
 
 class CacheStore:
@@ -70,21 +72,28 @@ class CacheStore:
         self.num_pages = num_pages
         self.groups, self._group_of = plan_groups(specs)
         self.layers_per_group = [self._group_of.count(g) for g in range(len(self.groups))]
-        self.pools: list[torch.Tensor] = []
+        # per group: the tensors [layers, 1 or 2, pages, elements] that hold its pages
+        self.pools: list[list[torch.Tensor]] = []
         for g, n_layers in zip(self.groups, self.layers_per_group):
-            page_elems = g.kv_heads * page_size * g.head_dim
-            self.pools.append(torch.zeros(n_layers, 2, num_pages, page_elems, device=rt.device, dtype=rt.dtype))
+            sizes = [g.kv_heads * page_size * g.head_dim, g.kv_heads * page_size * g.v_dim]
+            if sizes[0] == sizes[1]:
+                shapes = [(n_layers, 2, num_pages, sizes[0])]
+            else:
+                shapes = [(n_layers, 1, num_pages, n) for n in sizes if n > 0]
+            self.pools.append([torch.zeros(shape, device=rt.device, dtype=rt.dtype) for shape in shapes])
         self.layers: list[Optional[LayerCache]] = []
         seen = [0] * len(self.groups)
         for spec, g in zip(specs, self._group_of):
             if isinstance(spec, PagedKVSpec):
                 i = seen[g]
                 seen[g] += 1
-                pool = self.pools[g]
+                pools = self.pools[g]
+                keys = pools[0][i, 0]
+                values = pools[0][i, 1] if pools[0].shape[1] == 2 else (pools[1][i, 0] if len(pools) > 1 else None)
                 self.layers.append(LayerCache(
                     "paged", g,
-                    pool[i, 0].view(num_pages, spec.kv_heads, page_size, spec.head_dim),
-                    pool[i, 1].view(num_pages, spec.kv_heads, spec.head_dim, page_size),
+                    keys.view(num_pages, spec.kv_heads, page_size, spec.head_dim),
+                    None if values is None else values.view(num_pages, spec.kv_heads, spec.v_dim, page_size),
                     window=spec.window))
             elif isinstance(spec, StateSpec):
                 self.layers.append(LayerCache(
@@ -106,7 +115,7 @@ class CacheStore:
             return
         from ..kernels import ops
 
-        for g, pool in enumerate(self.pools):
+        for g, pools in enumerate(self.pools):
             mine = [o for o in ops_list if o.group == g]
             if not mine:
                 continue
@@ -115,4 +124,5 @@ class CacheStore:
                     raise ValueError(f"page copy {o} names a page outside the pool")
             src = torch.tensor([o.src for o in mine], dtype=torch.int32, device=self.rt.device)
             dst = torch.tensor([o.dst for o in mine], dtype=torch.int32, device=self.rt.device)
-            ops.copy_pages(pool, src, dst)
+            for pool in pools:
+                ops.copy_pages(pool, src, dst)

@@ -238,16 +238,17 @@ def fill(x: torch.Tensor, value: float) -> None:
 def copy_pages(pool: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
     """Copy page ``src[i]`` onto page ``dst[i]`` in every layer, keys and values.
 
-    ``pool`` is ``[layers, 2, pages, ...]``; the page ids are int32 and already range-checked.
+    ``pool`` is ``[layers, 2, pages, ...]`` (or ``[layers, 1, pages, ...]`` where keys and values
+    live in tensors of their own); the page ids are int32 and already range-checked.
     """
     _dense(pool, "pool")
-    _require(pool.dim() >= 4 and pool.shape[1] == 2, "pool must be [layers, 2, pages, ...]")
+    _require(pool.dim() >= 4 and pool.shape[1] in (1, 2), "pool must be [layers, 1 or 2, pages, ...]")
     _dense(src, "src", torch.int32, 1)
     _dense(dst, "dst", torch.int32, 1)
     _require(src.shape == dst.shape, "src and dst differ in length")
     pages = pool.shape[2]
     page_elems = pool[0, 0, 0].numel()
-    _check(library().dli_copy_pages(_ptr(pool), _ptr(src), _ptr(dst), src.shape[0], pool.shape[0] * 2, pages,
+    _check(library().dli_copy_pages(_ptr(pool), _ptr(src), _ptr(dst), src.shape[0], pool.shape[0] * pool.shape[1], pages,
                                     page_elems, _is_bf16(pool.dtype), _stream()), "copy_pages")
 
 

@@ -44,13 +44,24 @@ class PagedKVSpec:
     """A mixer that keeps keys and values of ``kv_heads x head_dim`` per token in pages.
 
     ``window`` > 0: only the last ``window`` keys are ever read, so pages that lie wholly before
-    the window may be given back while the request still runs. Layers with equal specs share one
+    the window may be given back while the request still runs. ``value_dim``: the size of a
+    value where it differs from a key's (``None``: the same; 0: the mixer keeps keys only, a
+    compressed cache for instance, and gets no value pages). Layers with equal specs share one
     group of pages and one block table.
     """
 
     kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: Optional[int] = None
+
+    def __post_init__(self) -> None:
+        if self.kv_heads <= 0 or self.head_dim <= 0 or self.window < 0 or (self.value_dim or 0) < 0:
+            raise ValueError(f"{self}: heads and sizes must be positive, window and value_dim not negative")
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

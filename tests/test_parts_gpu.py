@@ -119,7 +119,7 @@ def test_page_copies_cover_every_layer():
     from dli_amd.engine.core import build_core
 
     core = build_core(model_folder("A"), num_pages=8, page_size=16, max_seqs=2, dtype="bfloat16")
-    pool = core.store.pools[0]
+    (pool,) = core.store.pools[0]
     pool.copy_(torch.randn(pool.shape, device="cuda").to(pool.dtype))
     before = pool.clone()
     core.store.copy_pages([CopyOp(src=2, dst=5), CopyOp(src=7, dst=0)])
@@ -415,3 +415,138 @@ def test_a_toy_routed_feed_forward_and_a_toy_position_encoding_are_registered_bu
         unregister_architecture("ToyRoutedForCausalLM")
         unregister_part("feed_forward", "toy_routed")
         unregister_part("position", "toy_decay")
+
+
+# ------------------------------------------------------------------ toy mixers whose cache is not keys and values of one size
+
+def test_toy_mixers_with_smaller_values_and_with_keys_only_get_their_pages_and_step():
+    """A mixer declares the size of its values beside that of its keys (``PagedKVSpec.value_dim``):
+    a toy attention with keys of 16 and values of 8 numbers, and a toy that keeps one compressed
+    vector per token and no values at all, defined here, get pages of their own sizes, step in
+    portions and mixed batches as each request does whole, and their pages are copied on a fork."""
+    from typing import Any, Mapping
+
+    from dli_amd.cache.manager import CopyOp
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import (LayerSpec, Mixer, ModelSpec, PagedKVSpec, PartSpec, ScheduleEntry, WeightSpec,
+                               register_part, unregister_part)
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    class ToyPaged(Mixer):
+        """Single-head attention in plain torch over the request's pages; ``vd`` 0: the cached
+        vector serves as key and as value."""
+
+        def __init__(self, runtime, *, hidden_size: int, kd: int, vd: int) -> None:
+            super().__init__(runtime)
+            self.h, self.kd, self.vd = hidden_size, kd, vd
+            self.t = {}
+
+        def weight_specs(self):
+            specs = {"q.weight": WeightSpec((self.kd, self.h)), "k.weight": WeightSpec((self.kd, self.h)),
+                     "o.weight": WeightSpec((self.h, self.vd or self.kd))}
+            if self.vd:
+                specs["v.weight"] = WeightSpec((self.vd, self.h))
+            return specs
+
+        def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+            self.t = {k: v.float() for k, v in tensors.items()}
+
+        def cache_spec(self):
+            return PagedKVSpec(1, self.kd, value_dim=self.vd)
+
+        def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+            grp = ctx.groups[cache.group]
+            bs = cache.k_pages.shape[2]
+            assert (cache.v_pages is None) == (self.vd == 0)
+            assert self.vd == 0 or cache.v_pages.shape[1:] == (1, self.vd, bs)
+            xf = x.float()
+            q, k = xf @ self.t["q.weight"].T, xf @ self.t["k.weight"].T
+            slots = grp.slots.tolist()
+            for r, slot in enumerate(slots):
+                cache.k_pages[slot // bs, 0, slot % bs] = k[r].to(x.dtype)
+                if self.vd:
+                    cache.v_pages[slot // bs, 0, :, slot % bs] = (xf[r] @ self.t["v.weight"].T).to(x.dtype)
+            out = torch.empty_like(x)
+            tables = grp.block_tables.tolist()
+            kv_len, q_start = ctx.kv_len.tolist(), ctx.q_start.tolist()
+            for e in range(ctx.num_entries):
+                r0, r1 = q_start[e], q_start[e + 1]
+                pages = tables[e][:-(-kv_len[e] // bs)]
+                keys = cache.k_pages[pages, 0].reshape(-1, self.kd)[:kv_len[e]].float()
+                vals = (cache.v_pages[pages, 0].permute(0, 2, 1).reshape(-1, self.vd)[:kv_len[e]].float()
+                        if self.vd else keys)
+                for r in range(r0, r1):
+                    seen = kv_len[e] - (r1 - 1 - r)
+                    w = torch.softmax(keys[:seen] @ q[r] / self.kd ** 0.5, dim=0)
+                    out[r] = ((w @ vals[:seen]) @ self.t["o.weight"].T).to(x.dtype)
+            return out
+
+    def build(cfg):
+        h = cfg["hidden_size"]
+        norm = dict(width=h, eps=cfg["eps"])
+        mixers = [PartSpec("toy_paged", dict(hidden_size=h, kd=16, vd=8), "layers.0.mix."),
+                  PartSpec("toy_paged", dict(hidden_size=h, kd=12, vd=0), "layers.1.mix."),
+                  PartSpec("gqa_attention", dict(hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=16,
+                                                 position=PartSpec("rotary", dict(dim=16, theta=100.0))), "layers.2.attn.")]
+        layers = [LayerSpec(PartSpec("pre_norm"), {
+            "mixer_norm": ("norm", PartSpec("rms_norm", norm, f"layers.{i}.n1.")), "mixer": ("mixer", mixers[i]),
+            "feed_forward_norm": ("norm", PartSpec("rms_norm", norm, f"layers.{i}.n2.")),
+            "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=40),
+                                                      f"layers.{i}.mlp."))}) for i in range(3)]
+        return ModelSpec(
+            architecture="ToyPagedForCausalLM", vocab_size=cfg["vocab_size"], hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=cfg["vocab_size"], hidden_size=h), "embed."),
+            layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(3)),
+            final_norm=PartSpec("rms_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=cfg["vocab_size"], hidden_size=h, tied=True), "head."))
+
+    register_part("mixer", "toy_paged")(ToyPaged)
+    register_architecture("ToyPagedForCausalLM", dict, build)
+    try:
+        import tempfile
+
+        raw = {"architectures": ["ToyPagedForCausalLM"], "vocab_size": 53, "hidden_size": 32, "eps": 1e-6}
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, raw, seed=5, std=0.3, norm_jitter=0.1)
+            make = lambda: build_core(load_model(folder, dtype="float32"), num_pages=14, page_size=4, max_seqs=4,
+                                      enable_prefix_caching=False, watermark=0.0)
+            core = make()
+            store = core.store
+            assert len(store.groups) == 3                      # three different needs, three block tables
+            assert [[tuple(t.shape[1:]) for t in pools] for pools in store.pools] == [
+                [(1, 14, 4 * 16), (1, 14, 4 * 8)], [(1, 14, 4 * 12)], [(2, 14, 4 * 16)]]
+            assert store.bytes_per_page() == 4 * 4 * (16 + 8 + 12 + 16 + 16)
+            toks = {"a": [5, 9, 2, 40, 33, 7, 7, 12, 46, 1, 18, 25, 3, 3, 44, 21, 9, 30, 2, 11, 17],
+                    "b": [8, 8, 1, 30, 23, 4, 19, 36, 2, 45, 13, 27]}
+            whole = {rid: TraceSession(make()).step([{"id": rid, "tokens": t, "want": list(range(len(t)))}]).cpu()
+                     for rid, t in toks.items()}
+            assert (whole["a"][5] - whole["a"][6]).abs().max() > 1e-3    # the same token twice: the context counts
+            s = TraceSession(core)
+            got, fed = {"a": [], "b": []}, {"a": 0, "b": 0}
+            for stepplan in [{"a": 5}, {"a": 2, "b": 3}, {"a": 1, "b": 1}, {"b": 6}, {"a": 9, "b": 1}, {"a": 1, "b": 1}, {"a": 3}]:
+                entries = [{"id": rid, "tokens": toks[rid][fed[rid]:fed[rid] + n], "want": list(range(n))}
+                           for rid, n in stepplan.items()]
+                out = s.step(entries).cpu()
+                row = 0
+                for rid, n in stepplan.items():
+                    got[rid].append(out[row:row + n])
+                    row += n
+                    fed[rid] += n
+            for rid in toks:
+                assert (torch.cat(got[rid]) - whole[rid]).abs().max() < 1e-4, rid
+            # a fork inside a partly filled page copies the keys-only pages and the small values too
+            s.fork("a", "c")
+            tail = [31, 6, 50]
+            out_c = s.step([{"id": "c", "tokens": tail, "want": [0, 1, 2]}]).cpu()
+            alone = TraceSession(make()).step([{"id": "x", "tokens": toks["a"] + tail,
+                                                "want": list(range(len(toks["a"]), len(toks["a"]) + 3))}]).cpu()
+            assert (out_c - alone).abs().max() < 1e-4
+            before = [t.clone() for pools in store.pools for t in pools]
+            store.copy_pages([CopyOp(src=1, dst=13, group=g) for g in range(3)])
+            for t, b in zip([t for pools in store.pools for t in pools], before):
+                assert torch.equal(t[:, :, 13], b[:, :, 1]) and torch.equal(t[:, :, :13], b[:, :, :13])
+    finally:
+        unregister_architecture("ToyPagedForCausalLM")
+        unregister_part("mixer", "toy_paged")
