@@ -7,7 +7,9 @@ group, one block table per request and one pool tensor
 and one for the values, or none if the mixer keeps no values).
 Inside a page, keys lie as ``[kv_heads][page_size][head_dim]`` and values as
 ``[kv_heads][value_dim][page_size]`` (the order in which the attention kernels consume them).
-A mixer that declares a :class:`StateSpec` gets an array ``[state slots, *shape]`` instead.
+A mixer that declares a :class:`StateSpec` gets an array ``[state slots + 1, *shape]`` instead: one
+row per slot that a request can hold, and a last row (``scratch_slot``) that no request holds, for
+the padding rows of a replayed graph to write to.
 Everything is allocated once and zero-filled (reference: src/dli/kv/paged_store.py:50-52).
 """
 
@@ -70,6 +72,7 @@ class CacheStore:
         self.rt = rt
         self.page_size = page_size
         self.num_pages = num_pages
+        self.scratch_slot = max_seqs
         self.groups, self._group_of = plan_groups(specs)
         self.layers_per_group = [self._group_of.count(g) for g in range(len(self.groups))]
         # per group: the tensors [layers, 1 or 2, pages, elements] that hold its pages
@@ -97,7 +100,7 @@ class CacheStore:
                     window=spec.window))
             elif isinstance(spec, StateSpec):
                 self.layers.append(LayerCache(
-                    "state", state=torch.zeros(max_seqs, *spec.shape, device=rt.device, dtype=spec.dtype)))
+                    "state", state=torch.zeros(max_seqs + 1, *spec.shape, device=rt.device, dtype=spec.dtype)))
             else:
                 self.layers.append(None)
 

@@ -64,16 +64,10 @@ class DecodeGraphs:
         self.enabled = self._supported()
 
     def _supported(self) -> bool:
-        """Only the matrix-core decode path is captured: every paged layer must take it."""
-        if self.rt.dtype != torch.bfloat16 or self.step_fn.store.stateful:
+        """Graphs are recorded in bfloat16, for models all of whose mixers can be recorded."""
+        if self.rt.dtype != torch.bfloat16:
             return False
-        ps = self.step_fn.store.page_size
-        for cache in self.step_fn.store.layers:
-            if cache is None or cache.kind != "paged":
-                return False
-            if not ops.attention_mfma_supports(cache.k_pages.shape[3], ps, cache.k_pages.dtype):
-                return False
-        return True
+        return self.step_fn.model.graph_capturable(self.step_fn.store.page_size)
 
     def can_run(self, entries: Sequence[StepEntry], steps: int = 1) -> bool:
         if not self.enabled or not entries or len(entries) > self.max_batch:
@@ -108,6 +102,7 @@ class DecodeGraphs:
         views["logit_rows"][:] = np.arange(b)
         for g in range(self.n_groups):
             views[f"slots{g}"][:] = -1
+        views["state_slots"][:] = self.step_fn.store.scratch_slot
         dev.copy_(host)
         groups = [GroupView(dv[f"slots{g}"], dv[f"tables{g}"].view(b, width), width)
                   for g in range(self.n_groups)]
@@ -250,6 +245,7 @@ class DecodeGraphs:
         token_ids[n:] = 0
         positions[n:] = 0
         state_slots[:n] = [mgr.state_slot(e.seq_id) for e in entries]
+        state_slots[n:] = self.step_fn.store.scratch_slot
         rows = []
         for i, e in enumerate(entries):
             if e.want:

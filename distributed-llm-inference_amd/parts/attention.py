@@ -123,6 +123,11 @@ class GQAttention(Mixer):
     def cache_spec(self) -> Optional[PagedKVSpec]:
         return None if self.shares_kv else PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    def graph_capturable(self, page_size: int) -> bool:
+        # the matrix-core decode path is all kernels on the step's device arrays
+        return (self.rt.is_bf16 and ops.attention_mfma_supports(self.head_dim, page_size, self.rt.dtype)
+                and self.position.graph_capturable(page_size))
+
     def decode_head_tiles(self) -> int:
         # the decode kernel gives a workgroup up to 16 query heads of one kv head
         return self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 16)

@@ -114,6 +114,17 @@ class Part:
     def finalize(self) -> None:
         """Called once after the weights are loaded: build device tables, fuse tensors."""
 
+    def graph_capturable(self, page_size: int) -> bool:
+        """Whether this part's work on a step in which every request brings one token may be
+        recorded into a device graph and replayed. True promises that it reads such a step only
+        through the context's device arrays (``positions``, ``kv_len``, ``state_slots``, the
+        groups' slots and block tables: the host copies are stale in a replay), never waits for
+        the device, and tolerates padding rows: rows beyond the live requests have no keys, cache
+        slot -1 and the state slot that no request holds (``CacheStore.scratch_slot``), which they
+        may overwrite. The default is False, and a model is replayed from graphs only if all its
+        parts say True (``Model.graph_capturable``); otherwise its decode steps run eagerly."""
+        return False
+
     def streams(self, ctx: Any) -> bool:
         """Whether this part can run ``ctx``'s step on a :class:`DecodeStream` (its
         ``forward_stream``). Parts that do not implement the fused form return False, and the

@@ -19,6 +19,9 @@ class PreNormBlock(Block):
     def __init__(self, runtime: Runtime) -> None:
         super().__init__(runtime)
 
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
                 parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
         h = parts["mixer_norm"].forward(x, delta)          # x <- x + delta

@@ -19,6 +19,9 @@ class TokenEmbedding(Embedding):
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.weight: torch.Tensor | None = None
 
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
 

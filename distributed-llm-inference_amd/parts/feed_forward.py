@@ -26,6 +26,9 @@ class GatedMLP(FeedForward):
         self.w_gate_up = self.b_gate_up = self.w_down = self.b_down = None
         self.w_gate_up_tiled = self.w_down_tiled = None
 
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         h, i = self.hidden_size, self.intermediate_size
         specs = {"gate_proj.weight": WeightSpec((i, h)), "up_proj.weight": WeightSpec((i, h)),

@@ -22,6 +22,9 @@ class LinearHead(Head):
         self.weight: Optional[torch.Tensor] = None
         self.weight_tiled: Optional[torch.Tensor] = None
 
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {} if self.tied else {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
 

@@ -111,6 +111,15 @@ class Model:
             out.append(owners[0][1] if owners else None)
         return out
 
+    def graph_capturable(self, page_size: int) -> bool:
+        """Whether decode steps of this model may be recorded into device graphs: every part of it
+        says so (``Part.graph_capturable``; a mixer answers for the parts it owns)."""
+        parts = [self.embedding, self.final_norm, self.head]
+        for layer in self.layers:
+            parts.append(layer.block)
+            parts.extend(layer.parts.values())
+        return all(p.graph_capturable(page_size) for p in parts)
+
     def bind_caches(self, layer_caches: Sequence[Any]) -> list[Any]:
         """Per schedule entry, the cache it uses: its own, or a read-only view of another's."""
         out = []

@@ -20,6 +20,9 @@ class RMSNorm(Norm):
         self.width, self.eps = width, float(eps)
         self.weight: torch.Tensor | None = None
 
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {"weight": WeightSpec((self.width,), role="float32", init="norm")}
 

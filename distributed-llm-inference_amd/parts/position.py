@@ -60,6 +60,9 @@ class Rotary(PositionEncoding):
             original_max_position_embeddings)
         self._table: Optional[torch.Tensor] = None
 
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
     def finalize(self) -> None:
         # equal tables share one device tensor, so that what a step derives from a table (the cos
         # and sin of its positions) is derived once for all layers
@@ -81,3 +84,6 @@ class NoPosition(PositionEncoding):
 
     def __init__(self, runtime: Runtime) -> None:
         super().__init__(runtime)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only

@@ -550,3 +550,118 @@ def test_toy_mixers_with_smaller_values_and_with_keys_only_get_their_pages_and_s
     finally:
         unregister_architecture("ToyPagedForCausalLM")
         unregister_part("mixer", "toy_paged")
+
+
+# ------------------------------------------------------------------ a stateful toy mixer replayed from graphs
+
+@pytest.mark.parametrize("capturable", [True, False])
+def test_a_stateful_toy_mixer_that_says_it_can_be_recorded_is_replayed_from_graphs(capturable):
+    """Decode graphs are not tied to attention: a model whose parts all answer
+    ``graph_capturable`` with True is recorded and replayed, state slots included (padding rows of
+    a replay write the slot that no request holds). The toy's decode form works on the step's
+    device arrays only; with the answer False the same model decodes eagerly. Both equal each
+    request run whole."""
+    from typing import Any, Mapping
+
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import (LayerSpec, Mixer, ModelSpec, PartSpec, ScheduleEntry, StateSpec, WeightSpec,
+                               register_part, unregister_part)
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    @register_part("mixer", "toy_ema_device")
+    class ToyEMADevice(Mixer):
+        def __init__(self, runtime, *, hidden_size: int, decay: float) -> None:
+            super().__init__(runtime)
+            self.hidden_size, self.decay = hidden_size, decay
+            self.w = None
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.hidden_size, self.hidden_size))}
+
+        def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+            self.w = tensors["mix.weight"].float()
+
+        def cache_spec(self):
+            return StateSpec((self.hidden_size,), torch.float32)
+
+        def graph_capturable(self, page_size: int) -> bool:
+            return capturable
+
+        def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+            if ctx.num_decode == ctx.num_tokens:  # one token a request: device arrays only, no waiting
+                slots = ctx.state_slots.long()
+                before = cache.state[slots]
+                before = torch.where((ctx.positions == 0)[:, None], torch.zeros_like(before), before)
+                state = self.decay * before + x.float()
+                cache.state.index_copy_(0, slots, state)
+                return (state @ self.w.T).to(x.dtype)
+            out = torch.empty_like(x)
+            for e in range(ctx.num_entries):
+                r0, r1 = ctx.entry_rows(e)
+                slot = int(ctx.state_slots_host[e])
+                state = torch.zeros_like(cache.state[slot]) if ctx.is_fresh(e) else cache.state[slot].clone()
+                for r in range(r0, r1):
+                    state = self.decay * state + x[r].float()
+                    out[r] = (state @ self.w.T).to(x.dtype)
+                cache.state[slot] = state
+            return out
+
+    def build(cfg):
+        h = cfg["hidden_size"]
+        norm = dict(width=h, eps=cfg["eps"])
+        mixers = [PartSpec("gqa_attention", dict(hidden_size=h, num_heads=4, num_kv_heads=2, head_dim=16,
+                                                 position=PartSpec("rotary", dict(dim=16, theta=1e4))), "layers.0.attn."),
+                  PartSpec("toy_ema_device", dict(hidden_size=h, decay=0.6), "layers.1.ema.")]
+        layers = [LayerSpec(PartSpec("pre_norm"), {
+            "mixer_norm": ("norm", PartSpec("rms_norm", norm, f"layers.{i}.n1.")), "mixer": ("mixer", mixers[i]),
+            "feed_forward_norm": ("norm", PartSpec("rms_norm", norm, f"layers.{i}.n2.")),
+            "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=96),
+                                                      f"layers.{i}.mlp."))}) for i in range(2)]
+        return ModelSpec(
+            architecture="ToyStatefulForCausalLM", vocab_size=cfg["vocab_size"], hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=cfg["vocab_size"], hidden_size=h), "embed."),
+            layers=tuple(layers), schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+            final_norm=PartSpec("rms_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=cfg["vocab_size"], hidden_size=h, tied=True), "head."))
+
+    register_architecture("ToyStatefulForCausalLM", dict, build)
+    try:
+        import tempfile
+
+        raw = {"architectures": ["ToyStatefulForCausalLM"], "vocab_size": 96, "hidden_size": 64, "eps": 1e-5}
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, raw, seed=21, std=0.12, norm_jitter=0.1)
+
+            def make(graphs):
+                core = build_core(load_model(folder, dtype="bfloat16"), num_pages=12, page_size=16, max_seqs=4,
+                                  enable_prefix_caching=False, watermark=0.0)
+                if graphs:
+                    core.step.enable_decode_graphs(4, 12 * 16)
+                return core
+
+            toks = {"a": [5, 9, 2, 40, 33, 7, 7, 12, 60, 1, 18, 25, 3, 3, 44, 51, 9, 30, 2, 11, 17],
+                    "b": [8, 8, 1, 50, 23, 4, 19, 36, 2, 45, 13, 27, 90, 6], "c": [70, 3, 3, 15, 81, 22, 9]}
+            whole = {rid: TraceSession(make(False)).step([{"id": rid, "tokens": t, "want": list(range(len(t)))}]).float().cpu()
+                     for rid, t in toks.items()}
+            core = make(True)
+            assert (core.step.graphs is not None) == capturable
+            s = TraceSession(core)
+            heads = {"a": 15, "b": 8, "c": 1}     # c decodes from its first token on: its state starts in a replay
+            s.step([{"id": rid, "tokens": toks[rid][:n], "want": []} for rid, n in heads.items() if n > 1])
+            s.step([{"id": "c", "tokens": toks["c"][:1], "want": [0]}])
+            fed = dict(heads)
+            worst = 0.0
+            for stepno in range(6):
+                live = [rid for rid in toks if fed[rid] < len(toks[rid])]
+                out = s.step([{"id": rid, "tokens": [toks[rid][fed[rid]]], "want": [0]} for rid in live]).float().cpu()
+                for row, rid in enumerate(live):
+                    ref = whole[rid][fed[rid]]
+                    worst = max(worst, ((out[row] - ref).abs().max() / max(1.0, ref.abs().max().item())).item())
+                    fed[rid] += 1
+            assert worst < 4e-2, worst
+            assert not capturable or core.step.graphs.replays >= 6
+    finally:
+        unregister_architecture("ToyStatefulForCausalLM")
+        unregister_part("mixer", "toy_ema_device")
