@@ -63,6 +63,7 @@ def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, 
         model = load_model(folder, dtype=dtype, device="cuda:0")
     cfg = model.config
     pages = num_pages or batch * (-(-(context + SLACK) // block_size) + 1) + 8
+    pages += pages // 64  # room for the share of the pool that admission keeps back (1%)
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=prefix_caching,
         config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
