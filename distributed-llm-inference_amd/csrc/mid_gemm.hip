@@ -327,6 +327,83 @@ __global__ __launch_bounds__(256) void mid_finish_residual_kernel(
   if (threadIdx.x == 0) ssq_out[(int64_t)part * M + m] = total;
 }
 
+// The same, and the row normalised for the product that reads it next, so that none of that
+// product's 256 workgroups has to normalise all rows again: one workgroup per row holds the row's
+// new values in registers (PER x 1024 features at most), adds up its squares and writes
+// normed[m][n] = cast(norm_w[n] * cast(stream[m][n] * rs)), rs = rsqrt(sum / N + eps)
+// (src/dli/model/llama.py:40-44). ssq_out[m] gets the row's whole sum.
+template <int PER>
+__global__ __launch_bounds__(256) void mid_finish_residual_normed_kernel(
+    const float* __restrict__ partial, int splits, const bf16_t* __restrict__ bias,
+    bf16_t* __restrict__ stream, int64_t lds_, float* __restrict__ ssq_out,
+    const float* __restrict__ norm_w, float eps, bf16_t* __restrict__ normed, int64_t ldn, int M, int N) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const int64_t split_stride = (int64_t)M * N;
+  bf16x4 res[PER], old[PER];
+  float4v nw[PER], y[PER];
+  // every load of the row is asked for before the first is used: the stream's old values, the
+  // norm's weights, and the splits CH at a time for all of the thread's features
+  constexpr int CH = PER <= 2 ? 8 : (PER <= 4 ? 4 : 2);
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int n = (j * 256 + threadIdx.x) * 4;
+    old[j] = bf16x4{0, 0, 0, 0};
+    nw[j] = y[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (n < N) {
+      old[j] = *reinterpret_cast<const bf16x4*>(stream + (int64_t)m * lds_ + n);
+      nw[j] = *reinterpret_cast<const float4v*>(norm_w + n);
+    }
+  }
+  for (int s0 = 0; s0 < splits; s0 += CH) {
+    float4v v[PER][CH];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int n = (j * 256 + threadIdx.x) * 4;
+#pragma unroll
+      for (int u = 0; u < CH; ++u)
+        v[j][u] = n < N && s0 + u < splits
+                      ? *reinterpret_cast<const float4v*>(partial + (s0 + u) * split_stride + (int64_t)m * N + n)
+                      : float4v{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+#pragma unroll
+      for (int u = 0; u < CH; ++u)
+        if (s0 + u < splits) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) y[j][i] = s0 + u == 0 ? v[j][u][i] : y[j][i] + v[j][u][i];
+        }
+  }
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int n = (j * 256 + threadIdx.x) * 4;
+    if (n < N) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float b = bias != nullptr ? (float)bias[n + i] : 0.f;
+        res[j][i] = (bf16_t)((float)old[j][i] + (float)(bf16_t)(y[j][i] + b));
+        sq += (float)res[j][i] * (float)res[j][i];
+      }
+      *reinterpret_cast<bf16x4*>(stream + (int64_t)m * lds_ + n) = res[j];
+    }
+  }
+  const float total = block_sum(sq, scratch);
+  if (threadIdx.x == 0) ssq_out[m] = total;
+  const float rs = rsqrtf(total / (float)N + eps);
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int n = (j * 256 + threadIdx.x) * 4;
+    if (n < N) {
+      bf16x4 out;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[i] = (bf16_t)(nw[j][i] * (float)(bf16_t)((float)res[j][i] * rs));
+      *reinterpret_cast<bf16x4*>(normed + (int64_t)m * ldn + n) = out;
+    }
+  }
+}
+
 // The fused q/k/v projection's partial products [split][m][n], n in the feature order of the
 // product that rotates (tile t of a q or k head holds the head's dimensions 8t..8t+7 and
 // half+8t..half+8t+7; v heads in their own order): the splits are added in their order, the bias
@@ -448,6 +525,29 @@ extern "C" int dli_mid_finish_residual(const float* partial, int splits, const v
     return DLI_ERR_ARGUMENT;
   mid_finish_residual_kernel<<<dim3(M, (N + 1023) / 1024), 256, 0, stream>>>(
       partial, splits, (const bf16_t*)bias, (bf16_t*)stream_buf, lds_, ssq_out, M, N);
+  return dli_launch_status();
+}
+
+// The same with the normalised rows beside the stream: normed bfloat16 [M][N] (row stride ldn, a
+// multiple of 4), norm_w float32 [N]; ssq_out float32 [1][M]. N at most 8192.
+extern "C" int dli_mid_finish_residual_normed(const float* partial, int splits, const void* bias,
+                                              void* stream_buf, int64_t lds_, float* ssq_out,
+                                              const float* norm_w, float eps, void* normed, int64_t ldn,
+                                              int M, int N, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return DLI_OK;
+  if (partial == nullptr || stream_buf == nullptr || ssq_out == nullptr || norm_w == nullptr || normed == nullptr ||
+      splits < 1 || N % 4 != 0 || N > 8192 || lds_ < N || lds_ % 4 != 0 || ldn < N || ldn % 4 != 0)
+    return DLI_ERR_ARGUMENT;
+#define FINISH_NORMED(PER)                                                                              \
+  mid_finish_residual_normed_kernel<PER><<<M, 256, 0, stream>>>(partial, splits, (const bf16_t*)bias,   \
+                                                                (bf16_t*)stream_buf, lds_, ssq_out, norm_w, \
+                                                                eps, (bf16_t*)normed, ldn, M, N)
+  const int per = (N + 1023) / 1024;
+  if (per <= 1) FINISH_NORMED(1);
+  else if (per <= 2) FINISH_NORMED(2);
+  else if (per <= 4) FINISH_NORMED(4);
+  else FINISH_NORMED(8);
+#undef FINISH_NORMED
   return dli_launch_status();
 }
 

@@ -58,6 +58,8 @@ _SIGNATURES = {
     "dli_mid_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_int,
                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "dli_mid_finish_residual": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_ptr],
+    "dli_mid_finish_residual_normed": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64,
+                                       _c_int, _c_int, _c_ptr],
     "dli_mid_finish_qkv": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int,
                            _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_bf16": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64,
@@ -647,12 +649,21 @@ def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = F
     return out
 
 
+MID_NORMED_WIDTH = 8192  # the widest row that the normalising finish holds in one workgroup
+
+
 def mid_finish_residual(partial: torch.Tensor, stream: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                        ssq_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        ssq_out: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None,
+                        eps: float = 0.0, normed_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``stream += sum over splits of partial (+ bias)`` in place (32-bit sum, the product rounded
     to bfloat16 first, as the fused epilogue of the few-row product does), and each row's sum of
     squares of the new stream, in parts of 1024 features, as float32 ``[parts, rows]`` for the norm
-    that follows."""
+    that follows.
+
+    With ``norm_w`` (float32 ``[n]``, ``n <= MID_NORMED_WIDTH``), ``eps`` and ``normed_out``
+    (bfloat16 ``[rows, n]``) that norm is applied here as well: ``normed_out`` gets the RMSNorm of
+    the new stream with the two roundings of the fused norm prologues, for a product that then
+    reads it as it is; the sums of squares come back whole, as ``[1, rows]``."""
     _dense(partial, "partial", torch.float32, 3)
     _rows(stream, "stream", torch.bfloat16)
     splits, m, n = partial.shape
@@ -661,11 +672,23 @@ def mid_finish_residual(partial: torch.Tensor, stream: torch.Tensor, bias: Optio
     if bias is not None:
         _dense(bias, "bias", torch.bfloat16, 1)
         _require(bias.shape[0] == n, "bias length differs from n")
-    parts = -(-n // 1024)
+    parts = 1 if norm_w is not None else -(-n // 1024)
     if ssq_out is None:
         ssq_out = torch.empty(parts, m, device=stream.device, dtype=torch.float32)
     _dense(ssq_out, "ssq_out", torch.float32, 2)
-    _require(ssq_out.shape == (parts, m), "ssq_out must be [ceil(n / 1024), rows]")
+    _require(ssq_out.shape == (parts, m), f"ssq_out must be [{parts}, rows]")
+    if norm_w is not None:
+        _dense(norm_w, "norm_w", torch.float32, 1)
+        _require(norm_w.shape[0] == n and norm_w.data_ptr() % 16 == 0, "norm weight must have n aligned values")
+        _require(n <= MID_NORMED_WIDTH, f"rows wider than {MID_NORMED_WIDTH} are normalised by the product that reads them")
+        _require(normed_out is not None, "the normalised rows need normed_out")
+        _rows(normed_out, "normed_out", torch.bfloat16)
+        _require(normed_out.shape == (m, n) and normed_out.stride(0) % 4 == 0 and normed_out.data_ptr() % 8 == 0,
+                 "normed_out must be [rows, n]")
+        _check(library().dli_mid_finish_residual_normed(
+            _ptr(partial), splits, _ptr(bias), _ptr(stream), stream.stride(0), _ptr(ssq_out), _ptr(norm_w), float(eps),
+            _ptr(normed_out), normed_out.stride(0), m, n, _stream()), "mid_finish_residual")
+        return ssq_out
     _check(library().dli_mid_finish_residual(_ptr(partial), splits, _ptr(bias), _ptr(stream), stream.stride(0),
                                              _ptr(ssq_out), m, n, _stream()), "mid_finish_residual")
     return ssq_out

@@ -22,7 +22,7 @@ import torch
 from ..kernels import ops
 from .attention_kernels import decode_attention_unmerged, paged_attention
 from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
-from .linear import decode_copy, linear
+from .linear import decode_copy, finish_residual, linear
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
 
@@ -174,16 +174,17 @@ class GQAttention(Mixer):
         return (ops.skinny_gemm_supports(n, self.hidden_size, self.rt.dtype)
                 and ops.skinny_gemm_supports(n, nh * d, self.rt.dtype))
 
-    def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any, cache: Any) -> None:
+    def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any, cache: Any,
+                       following: Optional[Norm] = None) -> None:
         """``stream.x += attention(norm(stream.x))``, the norm inside the first product's kernel and
-        the sum inside the last one's."""
+        the sum inside the last one's. ``following``: the norm that the stream meets next."""
         nh, d = self.num_heads, self.head_dim
         nkv = 0 if self.shares_kv else self.num_kv_heads
         grp = ctx.groups[cache.group]
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
         if n > FEW_ROWS:
-            self._forward_stream_mid(stream, norm_w, eps, ctx, cache, grp)
+            self._forward_stream_mid(stream, norm, ctx, cache, grp, following)
             return
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
         if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS:
@@ -212,27 +213,32 @@ class GQAttention(Mixer):
                 lambda splits: ops.skinny_gemm_merged_supports(n, self.hidden_size, nh, d, splits, qkv.device))
             if left is not None:
                 splits, part_o, part_ml = left
-                stream.ssq = ops.skinny_gemm_merged(part_o, part_ml, splits, nh, d, self.w_o_tiled, stream.x,
-                                                    bias=self.b_o)
+                stream.wrote(ops.skinny_gemm_merged(part_o, part_ml, splits, nh, d, self.w_o_tiled, stream.x,
+                                                    bias=self.b_o))
                 return
         out = self.rt.empty(n, nh * d)
         paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
-        stream.ssq = ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
-                                     stream=stream.x, bias=self.b_o)
+        stream.wrote(ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
+                                     stream=stream.x, bias=self.b_o))
 
-    def _forward_stream_mid(self, stream: DecodeStream, norm_w: torch.Tensor, eps: float, ctx: Any, cache: Any,
-                            grp: Any) -> None:
+    def _forward_stream_mid(self, stream: DecodeStream, norm: Norm, ctx: Any, cache: Any, grp: Any,
+                            following: Optional[Norm]) -> None:
         """The same for 17 to 64 rows: both products split k over workgroups and leave 32-bit
         partial sums; the kernel that rotates and writes the cache, and the one that makes the
-        residual sum, add them up."""
+        residual sum (and applies the norm that follows), add them up."""
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         n = stream.x.shape[0]
-        partial = ops.mid_gemm(stream.x, self.w_qkv_rope, tiled=True, n=(nh + 2 * nkv) * d, epilogue=ops.MID_PARTIAL,
-                               norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        ready = stream.normed_by(norm)
+        if ready is not None:
+            partial = ops.mid_gemm(ready, self.w_qkv_rope, tiled=True, n=(nh + 2 * nkv) * d, epilogue=ops.MID_PARTIAL)
+        else:
+            norm_w, eps = norm.fused_params()
+            partial = ops.mid_gemm(stream.x, self.w_qkv_rope, tiled=True, n=(nh + 2 * nkv) * d,
+                                   epilogue=ops.MID_PARTIAL, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         q = self.rt.empty(n, nh * d)
         angles = ctx.rope_angles(self.position.rotary_table().inv_freq, q.dtype)
         ops.mid_finish_qkv(partial, q, angles, grp.slots, cache.k_pages, cache.v_pages, nh, bias=self.b_qkv_rope)
         out = self.rt.empty(n, nh * d)
         paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
         partial = ops.mid_gemm(out, self.w_o_tiled, tiled=True, n=self.hidden_size, epilogue=ops.MID_PARTIAL)
-        stream.ssq = ops.mid_finish_residual(partial, stream.x, self.b_o)
+        finish_residual(self.rt, stream, partial, self.b_o, following)

@@ -83,6 +83,29 @@ class DecodeStream:
 
     x: torch.Tensor
     ssq: torch.Tensor
+    # The rows of ``x`` already normalised by ``normed_for`` (a norm's weight address and eps),
+    # where the kernel that last wrote ``x`` was told which norm follows and applied it too.
+    normed: Optional[torch.Tensor] = None
+    normed_for: Optional[tuple] = None
+
+    def wrote(self, ssq: torch.Tensor, normed: Optional[torch.Tensor] = None, norm: Any = None) -> None:
+        """``x`` has new values: their sums of squares, and their normalised rows if ``norm`` was
+        applied as well. Every part that changes ``x`` says so through this call."""
+        self.ssq = ssq
+        self.normed = normed
+        self.normed_for = norm_key(norm) if normed is not None else None
+
+    def normed_by(self, norm: Any) -> Optional[torch.Tensor]:
+        """The rows normalised by this very norm, if the last writer left them."""
+        return self.normed if self.normed is not None and self.normed_for == norm_key(norm) else None
+
+
+def norm_key(norm: Any) -> Optional[tuple]:
+    """What identifies a norm for :class:`DecodeStream`: its weight's address and its eps."""
+    if norm is None or not hasattr(norm, "fused_params"):
+        return None
+    w, eps = norm.fused_params()
+    return (w.data_ptr(), float(eps))
 
 
 class Part:
@@ -222,6 +245,12 @@ class Block(Part):
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
                 parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
         raise NotImplementedError
+
+    def first_norm(self, parts: Mapping[str, Part]) -> Optional["Norm"]:
+        """The norm that this arrangement applies to the stream before anything else, if there is
+        one: the block before it may apply it in the kernel that writes the stream (the fused
+        decode path passes it on as ``following``)."""
+        return None
 
 
 class Head(Part):

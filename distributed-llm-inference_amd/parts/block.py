@@ -47,6 +47,12 @@ class PreNormBlock(Block):
         fused_norms = all(hasattr(parts[r], "fused_params") for r in ("mixer_norm", "feed_forward_norm"))
         return fused_norms and parts["mixer"].streams(ctx) and parts["feed_forward"].streams(ctx)
 
-    def forward_stream(self, stream: DecodeStream, ctx: Any, cache: Any, parts: Mapping[str, Part]) -> None:
-        parts["mixer"].forward_stream(stream, parts["mixer_norm"], ctx, cache)
-        parts["feed_forward"].forward_stream(stream, parts["feed_forward_norm"], ctx)
+    def first_norm(self, parts: Mapping[str, Part]) -> Optional[Part]:
+        return parts["mixer_norm"]
+
+    def forward_stream(self, stream: DecodeStream, ctx: Any, cache: Any, parts: Mapping[str, Part],
+                       following: Optional[Part] = None) -> None:
+        """``following``: the norm that whatever comes after this block applies first (the last
+        kernel of the block may apply it while it writes the stream)."""
+        parts["mixer"].forward_stream(stream, parts["mixer_norm"], ctx, cache, following=parts["feed_forward_norm"])
+        parts["feed_forward"].forward_stream(stream, parts["feed_forward_norm"], ctx, following=following)

@@ -4,13 +4,13 @@ both halves; the activation kernel reads them side by side."""
 
 from __future__ import annotations
 
-from typing import Any, Mapping
+from typing import Any, Mapping, Optional
 
 import torch
 
 from ..kernels import ops
 from .base import DecodeStream, FeedForward, Norm, Runtime
-from .linear import decode_copy, linear
+from .linear import decode_copy, finish_residual, linear
 from .registry import register_part
 from .spec import WeightSpec
 
@@ -78,18 +78,26 @@ class GatedMLP(FeedForward):
         return (ops.skinny_gemm_supports(n, self.hidden_size, self.rt.dtype)
                 and ops.skinny_gemm_supports(n, self.intermediate_size, self.rt.dtype))
 
-    def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any) -> None:
-        """``stream.x += mlp(norm(stream.x))``, norm and sum inside the two products' kernels."""
+    def forward_stream(self, stream: DecodeStream, norm: Norm, ctx: Any, following: Optional[Norm] = None) -> None:
+        """``stream.x += mlp(norm(stream.x))``, norm and sum inside the two products' kernels.
+        ``following``: the norm that the stream meets next; with 17 to 64 rows the kernel that makes
+        the residual sum applies it as well, so that the next product reads normalised rows."""
         n = stream.x.shape[0]
         norm_w, eps = norm.fused_params()
         if n > self.FEW_ROWS:
-            act = ops.mid_gemm(stream.x, self.w_gate_up_tiled, tiled=True, n=self.intermediate_size,
-                               epilogue=ops.MID_SWIGLU, bias=self.b_gate_up, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+            ready = stream.normed_by(norm)
+            if ready is not None:
+                act = ops.mid_gemm(ready, self.w_gate_up_tiled, tiled=True, n=self.intermediate_size,
+                                   epilogue=ops.MID_SWIGLU, bias=self.b_gate_up)
+            else:
+                act = ops.mid_gemm(stream.x, self.w_gate_up_tiled, tiled=True, n=self.intermediate_size,
+                                   epilogue=ops.MID_SWIGLU, bias=self.b_gate_up, norm_w=norm_w, eps=eps,
+                                   ssq_in=stream.ssq)
             partial = ops.mid_gemm(act, self.w_down_tiled, tiled=True, n=self.hidden_size, epilogue=ops.MID_PARTIAL)
-            stream.ssq = ops.mid_finish_residual(partial, stream.x, self.b_down)
+            finish_residual(self.rt, stream, partial, self.b_down, following)
             return
         act = self.rt.empty(n, self.intermediate_size)
         ops.skinny_gemm(stream.x, self.w_gate_up, w_tiled=self.w_gate_up_tiled, epilogue=ops.SKINNY_SWIGLU, out=act,
                         bias=self.b_gate_up, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
-        stream.ssq = ops.skinny_gemm(act, self.w_down, w_tiled=self.w_down_tiled, epilogue=ops.SKINNY_RESIDUAL,
-                                     stream=stream.x, bias=self.b_down)
+        stream.wrote(ops.skinny_gemm(act, self.w_down, w_tiled=self.w_down_tiled, epilogue=ops.SKINNY_RESIDUAL,
+                                     stream=stream.x, bias=self.b_down))

@@ -64,7 +64,8 @@ class LinearHead(Head):
         """Logits of every row of the stream, the final norm computed inside the product (with
         more than a few rows: the norm kernel, then the library product)."""
         if stream.x.shape[0] > self.FEW_ROWS:
-            return self.forward(norm.forward(stream.x))
+            ready = stream.normed_by(norm)  # the last residual sum's kernel may have normalised already
+            return self.forward(ready if ready is not None else norm.forward(stream.x))
         norm_w, eps = norm.fused_params()
         out = torch.empty(stream.x.shape[0], self.vocab_size, device=self.rt.device, dtype=torch.float32)
         ops.skinny_gemm(stream.x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out,

@@ -147,9 +147,11 @@ class Model:
 
     def _forward_stream(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
         stream = self.embedding.forward_stream(ctx.token_ids)
-        for entry, cache in zip(self.spec.schedule, caches):
-            layer = self.layers[entry.layer]
-            layer.block.forward_stream(stream, ctx, cache, layer.parts)
+        order = [self.layers[entry.layer] for entry in self.spec.schedule]
+        for i, (layer, cache) in enumerate(zip(order, caches)):
+            # the norm that the stream meets next: the following entry's first, or the final one
+            after = order[i + 1].block.first_norm(order[i + 1].parts) if i + 1 < len(order) else self.final_norm
+            layer.block.forward_stream(stream, ctx, cache, layer.parts, following=after)
         logits = self.head.forward_stream(stream, self.final_norm)
         k = ctx.logit_rows.shape[0]
         if getattr(ctx, "all_rows_wanted", False):

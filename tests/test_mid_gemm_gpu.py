@@ -136,6 +136,39 @@ def test_finish_of_a_residual_product(ops, m, n, splits, with_bias):
     assert (ssq.sum(0).cpu().double() - ref_ssq.cpu()).abs().max() < 1e-4 * ref_ssq.max().item()
 
 
+@pytest.mark.parametrize("m,n,splits", [(1, 64, 1), (24, 200, 3), (64, 2048, 8), (33, 3076, 11), (17, 8192, 2), (5, 5000, 4)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_finish_of_a_residual_product_that_also_normalises(ops, m, n, splits, with_bias):
+    """The same stream as the plain finish leaves, bit for bit, its whole sums of squares, and
+    beside it the rows normalised as the fused norm prologues normalise (two roundings)."""
+    torch.manual_seed(m + n + 1)
+    partial = torch.randn(splits, m, n, device="cuda")
+    base = (torch.randn(m, n + 4, device="cuda") * 3).bfloat16()
+    bias = torch.randn(n, device="cuda").bfloat16() if with_bias else None
+    nw = (1 + 0.1 * torch.randn(n, device="cuda")).float()
+    plain = base.clone()
+    parts = ops.mid_finish_residual(partial, plain[:, :n], bias)
+    got = base.clone()
+    wide = torch.full((m, n + 8), 7.0, device="cuda", dtype=torch.bfloat16)
+    ssq = ops.mid_finish_residual(partial, got[:, :n], bias, norm_w=nw, eps=1e-5, normed_out=wide[:, :n])
+    assert torch.equal(got, plain)
+    assert ssq.shape == (1, m)
+    ref_ssq = got[:, :n].double().pow(2).sum(-1)
+    assert (ssq[0].double() - ref_ssq).abs().max() < 1e-4 * ref_ssq.max().item()
+    assert (parts.sum(0).double() - ref_ssq).abs().max() < 1e-4 * ref_ssq.max().item()
+    want = ref_norm_bf16(got[:, :n], nw, 1e-5)
+    # rs from sums added in another order may move the inner rounding by one step of bfloat16,
+    # which the outer rounding can double
+    diff = (wide[:, :n].float() - want.float()).abs()
+    assert (diff <= 2.0 ** -6 * want.float().abs() + 1e-6).all()
+    assert (diff > 0).float().mean() < 0.02
+    assert (wide[:, n:] == 7.0).all()
+    with pytest.raises(ops.KernelArgumentError):
+        ops.mid_finish_residual(torch.zeros(1, 2, 8196, device="cuda"), torch.zeros(2, 8196, device="cuda").bfloat16(),
+                                norm_w=torch.ones(8196, device="cuda"), eps=1e-5,
+                                normed_out=torch.zeros(2, 8196, device="cuda").bfloat16())
+
+
 @pytest.mark.parametrize("m", [1, 17, 64])
 @pytest.mark.parametrize("qh,kvh,d,k,bs", [(4, 4, 16, 128, 16), (6, 2, 32, 384, 8), (5, 1, 48, 256, 4),
                                            (32, 8, 64, 2048, 16), (3, 3, 128, 640, 16)])
