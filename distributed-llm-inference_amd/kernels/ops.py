@@ -64,6 +64,8 @@ _SIGNATURES = {
                            _c_int, _c_int, _c_int, _c_ptr],
     "dli_gemm_bf16": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64,
                       _c_int, _c_ptr],
+    "dli_gemm_bf16_f32": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64,
+                      _c_int, _c_ptr],
     "dli_gemm_bf16_usable": [_c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_i64, _c_int],
     "dli_prenorm_blocks_bf16": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
     "dli_embedding_ssq": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
@@ -748,12 +750,14 @@ def prenorm_blocks(x: torch.Tensor, blocks, count: int, step) -> bool:
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> bool:
     """``out = x @ w.T (+ bias)`` for bfloat16 matrices with contiguous rows through the vendor
-    library, 32-bit accumulation, the bias added before the one rounding. The library's choice
+    library, 32-bit accumulation, the bias added before the one rounding (``out`` float32: the
+    sums as they are, unrounded). The library's choice
     of kernel is looked up once per shape. Returns False where the library has no kernel for the
     shape (nothing was computed then)."""
     _rows(x, "x", torch.bfloat16)
     _rows(w, "w", torch.bfloat16)
-    _rows(out, "out", torch.bfloat16)
+    _require(out.dtype in (torch.bfloat16, torch.float32), "out must be bfloat16 or float32")
+    _rows(out, "out", out.dtype)
     rows, k = x.shape
     feats = w.shape[0]
     _require(w.shape[1] == k and out.shape == (rows, feats), "x [n, k], w [m, k] and out [n, m] do not fit")
@@ -764,8 +768,9 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optiona
     workspace = _gemm_workspaces.get(index)
     if workspace is None:
         workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
-    status = library().dli_gemm_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(bias), _ptr(out), out.stride(0),
-                                     rows, feats, k, _ptr(workspace), _GEMM_WORKSPACE_BYTES, index, _stream())
+    call = library().dli_gemm_bf16 if out.dtype == torch.bfloat16 else library().dli_gemm_bf16_f32
+    status = call(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(bias), _ptr(out), out.stride(0),
+                  rows, feats, k, _ptr(workspace), _GEMM_WORKSPACE_BYTES, index, _stream())
     if status == -1:
         return False
     _check(status, "gemm_bf16")

@@ -49,6 +49,11 @@ class LinearHead(Head):
             out = torch.empty(rows, self.vocab_size, device=self.rt.device, dtype=torch.float32)
             ops.skinny_gemm(x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out)
             return out
+        if self.rt.is_bf16 and rows > 0 and x.dtype == torch.bfloat16:
+            # many rows: the library's product, leaving the 32-bit sums as the logits
+            out = torch.empty(rows, self.vocab_size, device=self.rt.device, dtype=torch.float32)
+            if ops.gemm_bf16(x, self.weight, out):
+                return out
         logits = linear(self.rt, x, self.weight)
         if logits.dtype == torch.float32:
             return logits

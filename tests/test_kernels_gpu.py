@@ -359,6 +359,13 @@ def test_library_product_called_directly(ops, m, n, k, with_bias):
     again = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
     assert ops.gemm_bf16(x, w, again, bias)
     assert torch.equal(again, out)
+    # the 32-bit sums themselves (the logits of many rows): far closer to the 64-bit product, and
+    # rounding them gives the bfloat16 result
+    wide = torch.full((m, n + 4), 7.0, device="cuda", dtype=torch.float32)
+    if ops.gemm_bf16(x, w, wide[:, :n], bias):
+        assert (wide[:, :n].cpu().double() - ref).abs().max() < 1e-4 * max(1.0, ref.abs().max().item())
+        assert (wide[:, n:] == 7.0).all()
+        assert ((wide[:, :n].bfloat16().float() - out.float()).abs() <= 2.0 ** -7 * out.float().abs() + 1e-6).all()
 
 
 @pytest.mark.parametrize("with_bias", [False, True])
