@@ -612,13 +612,24 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
     if (T < 2) stash(T, begin + T * 32, stage[T % RD]);
   }
   __syncthreads();
-  for (int it0 = 0; it0 < n_tiles; it0 += RD) {
-#pragma unroll
-   for (int r = 0; r < RD; ++r) {
-    const int it = it0 + r;
-    if (it >= n_tiles) break;
+  typedef short short4a __attribute__((ext_vector_type(4)));
+  union VFrag {
+    bf16x8 v;
+    short4a h[2];
+  };
+  // A tile's work in two halves. The first reads the tile's fragments from LDS, makes S^T and the
+  // softmax (vector unit, mostly); the second makes P*V (matrix cores) and moves tile it+2 on its
+  // way (memory and LDS). What a wave carries from one to the other:
+  VFrag vf[DCH];
+  bf16x8 pb[2];
+  bool active = false;
+  auto sees = [&](int it) __attribute__((always_inline)) {  // whether any of the wave's queries sees a key of the tile
+    const int t = begin + it * 32;
+    return wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1);
+  };
+  auto scores = [&](int it) __attribute__((always_inline)) {
     const int t = begin + it * 32, buf = it % 3;
-    if (wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1)) {
+    {
       const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
       const bf16_t* ks = &lds[buf][0];
       const bf16_t* vs = &lds[buf][K_ELEMS];
@@ -630,11 +641,6 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
         kf0[c] = *reinterpret_cast<const bf16x8*>(ks + col * KPAD + c * 32 + grp * 8);
         kf1[c] = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KPAD + c * 32 + grp * 8);
       }
-      typedef short short4a __attribute__((ext_vector_type(4)));
-      union VFrag {
-        bf16x8 v;
-        short4a h[2];
-      } vf[DCH];
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
         vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 4 * grp);
@@ -674,7 +680,6 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
         }
       }
       float alpha[2];
-      bf16x8 pb[2];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         float tile_max = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]),
@@ -694,8 +699,7 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
         // four partial sums of a column are added once, after the last tile. (Taking the sum
         // from the matrix cores instead, as the product of P^T with a row of ones, saves sixteen
         // additions a lane and tile and was slower, 62 against 59 us; so was computing S^T of the
-        // next tile before the softmax of this one inside a wave, 68 us: two waves a SIMD already
-        // cover each other's waits.)
+        // next tile before the softmax of this one inside a wave, 68 us.)
         st[j].l = st[j].l * alpha[j] + tile_sum;
         st[j].m = m_new;
       }
@@ -706,17 +710,50 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
 #pragma unroll
           for (int c = 0; c < DCH; ++c) st[j].o[c] *= alpha[j];
       }
-#pragma unroll
-      for (int c = 0; c < DCH; ++c)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
     }
+  };
+  auto values = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < DCH; ++c)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
+  };
+  auto move_on = [&](int it, int slot) __attribute__((always_inline)) {
     // tile it+2 leaves its register slot for LDS; the slot then receives tile it+2+RD
-    const int slot = (r + 2) % RD;
     stash((it + 2) % 3, begin + (it + 2) * 32, stage[slot]);
     fetch(begin + (it + 2 + RD) * 32, stage[slot]);
-    __syncthreads();
-   }
+  };
+  auto scores_half = [&](int it) __attribute__((always_inline)) {
+    active = sees(it);
+    if (active) scores(it);
+  };
+  auto values_half = [&](int it, int slot) __attribute__((always_inline)) {
+    if (active) values();
+    move_on(it, slot);
+  };
+  // The paired kernel tests once per tile whether the wave has work, the single one before each
+  // half: the same work either way, but the compiler orders the two forms differently, and each
+  // kernel is 5 to 15% faster in its form (timed at 2,048 to 16,384 tokens, heads of 64 and 128).
+  // Tried and slower by 10 to 15%: the second set half a tile behind the first (two barriers a
+  // tile), so that one set's products run beside the other's softmax; and the pair's key tiles
+  // dealt out evenly to the two sets with a merge of their states at the end.
+  for (int it0 = 0; it0 < n_tiles; it0 += RD) {
+#pragma unroll
+    for (int r = 0; r < RD; ++r) {
+      const int it = it0 + r;
+      if (it >= n_tiles) break;
+      if constexpr (PAIR) {
+        if (sees(it)) {
+          scores(it);
+          values();
+        }
+        move_on(it, (r + 2) % RD);
+      } else {
+        scores_half(it);
+        values_half(it, (r + 2) % RD);
+      }
+      __syncthreads();
+    }
   }
 
 #pragma unroll
@@ -896,12 +933,17 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (hw > 0) {
     const dim3 sgrid(tiles, q_heads / hw);
-    // Mirror tiles are paired (pair_tiles 1, or -1 and a launch of one to eight workgroups per
-    // compute unit: with fewer, pairing leaves units idle; with more, the queue of workgroups
-    // evens the causal triangle out by itself and single tiles were faster, measured at 16K
-    // tokens). The tile list has to hold all tiles of a request.
+    // Mirror tiles are paired (pair_tiles 1, or -1 and a launch in the range where it was faster:
+    // with too few workgroups pairing leaves compute units idle; with many, the queue of
+    // workgroups evens the causal triangle out by itself. Heads of up to 64: from two to under
+    // four workgroups per unit (2,048 tokens at the 1B sizes: 58 against 70 us; 4,096: 192 against
+    // 179; 8,192: 697 against 550); larger heads, whose single-tile kernel holds one wave a SIMD:
+    // from one a unit on (heads of 128, 2,048 tokens: 84 against 129 us; 16,384: 2.9 against 4.0 ms).
+    // The tile list has to hold all tiles of a request.
     const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
-    const bool pair = pair_tiles >= 0 ? pair_tiles != 0 : (launch >= units && launch <= 8 * units);
+    const bool in_range = head_dim <= 64 ? (launch >= 2 * units && launch < 4 * units)
+                                         : launch >= units;
+    const bool pair = pair_tiles >= 0 ? pair_tiles != 0 : in_range;
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \
     if (pair)                                                                                     \
