@@ -620,14 +620,14 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   // A tile's work in two halves. The first reads the tile's fragments from LDS, makes S^T and the
   // softmax (vector unit, mostly); the second makes P*V (matrix cores) and moves tile it+2 on its
   // way (memory and LDS). What a wave carries from one to the other:
-  VFrag vf[DCH];
-  bf16x8 pb[2];
+  VFrag vf_kept[DCH];
+  bf16x8 pb_kept[2];
   bool active = false;
   auto sees = [&](int it) __attribute__((always_inline)) {  // whether any of the wave's queries sees a key of the tile
     const int t = begin + it * 32;
     return wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1);
   };
-  auto scores = [&](int it) __attribute__((always_inline)) {
+  auto scores = [&](int it, VFrag (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
     const int t = begin + it * 32, buf = it % 3;
     {
       const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
@@ -712,7 +712,7 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
       }
     }
   };
-  auto values = [&]() __attribute__((always_inline)) {
+  auto values = [&](VFrag (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
 #pragma unroll
     for (int c = 0; c < DCH; ++c)
 #pragma unroll
@@ -725,10 +725,10 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   };
   auto scores_half = [&](int it) __attribute__((always_inline)) {
     active = sees(it);
-    if (active) scores(it);
+    if (active) scores(it, vf_kept, pb_kept);
   };
   auto values_half = [&](int it, int slot) __attribute__((always_inline)) {
-    if (active) values();
+    if (active) values(vf_kept, pb_kept);
     move_on(it, slot);
   };
   // The paired kernel tests once per tile whether the wave has work, the single one before each
@@ -744,8 +744,10 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
       if (it >= n_tiles) break;
       if constexpr (PAIR) {
         if (sees(it)) {
-          scores(it);
-          values();
+          VFrag vf[DCH];
+          bf16x8 pb[2];
+          scores(it, vf, pb);
+          values(vf, pb);
         }
         move_on(it, (r + 2) % RD);
       } else {
