@@ -53,6 +53,9 @@ _SIGNATURES = {
     "dli_skinny_gemm_qkv_rope": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_i64,
                                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_ptr],
+    "dli_head_gemm_supports": [_c_int, _c_int, _c_int],
+    "dli_head_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int,
+                      _c_int, _c_ptr],
     "dli_skinny_gemm_merged": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int,
                                _c_int, _c_int, _c_ptr],
     "dli_mid_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_int,
@@ -489,6 +492,43 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
             _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w), _ptr(bias), _ptr(out), ldo,
             _ptr(stream), lds, _ptr(ssq_out), m, n, k, up_offset, epilogue, a, _stream()), "skinny4_gemm")
     return ssq_out if epilogue == SKINNY_RESIDUAL else None
+
+
+def head_gemm_supports(rows: int, n: int, k: int, dtype: torch.dtype) -> bool:
+    """Whether :func:`head_gemm` takes this product (at most 16 rows, ``n % 16 == 0``, ``k`` one
+    of 1024, 2048, 3072, 4096)."""
+    return dtype == torch.bfloat16 and bool(library().dli_head_gemm_supports(int(rows), int(n), int(k)))
+
+
+def head_gemm(x: torch.Tensor, w_tiled: torch.Tensor, out: torch.Tensor, norm_w: Optional[torch.Tensor] = None,
+              eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None, workgroups: int = 0) -> None:
+    """``out = xhat @ w.T`` as float32 for at most 16 rows and the many rows of a vocabulary:
+    workgroups that stay for the whole launch walk the tiles of ``w_tiled`` (:func:`tile_weights`
+    of ``w [n, k]``) in turn, each wave keeping its normalised activations in registers. ``norm_w``,
+    ``eps``, ``ssq_in [parts, rows]``: the RMSNorm of ``x`` as in :func:`skinny_gemm`. The sums are
+    those of :func:`skinny_gemm` with ``shape=4``, to the bit. ``workgroups``: how many (0: two per
+    compute unit)."""
+    _rows(x, "x", torch.bfloat16)
+    m, k = x.shape
+    _rows(out, "out", torch.float32)
+    n = out.shape[1]
+    _require(out.shape[0] == m, "out must be [rows, n]")
+    _require(head_gemm_supports(m, n, k, x.dtype), f"the logits kernel takes 1..16 rows, n % 16 == 0 and k of 1024 to "
+             f"4096 in steps of 1024, not {m} x {k} -> {n}")
+    _dense(w_tiled, "w_tiled", torch.bfloat16, 1)
+    _require(w_tiled.numel() == n * k and w_tiled.data_ptr() % 16 == 0, "w_tiled must hold [n, k] in tile order")
+    _require(x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and out.stride(0) % 4 == 0 and out.data_ptr() % 16 == 0,
+             "operands must be 16-byte aligned")
+    parts = 0
+    if norm_w is not None:
+        _dense(norm_w, "norm_w", torch.float32, 1)
+        _require(norm_w.shape[0] == k and norm_w.data_ptr() % 16 == 0, "norm weight must have k aligned values")
+        _require(ssq_in is not None, "a fused norm needs the sums of squares")
+        _dense(ssq_in, "ssq_in", torch.float32, 2)
+        _require(ssq_in.shape[1] == m and ssq_in.shape[0] >= 1, "ssq_in must be [parts, rows]")
+        parts = ssq_in.shape[0]
+    _check(library().dli_head_gemm(_ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w_tiled),
+                                   _ptr(out), out.stride(0), m, n, k, int(workgroups), _stream()), "head_gemm")
 
 
 MERGED_ROWS, MERGED_SPLITS, _MERGED_RANGE = 4, 16, 512  # csrc/skinny_gemm.hip: MERGE_ROWS, MERGE_SPLITS, MERGE_RANGE

@@ -47,7 +47,7 @@ class LinearHead(Head):
                 and ops.skinny_gemm_supports(rows, self.hidden_size, self.rt.dtype)):
             # the usual case of a prompt's step: logits for its last row only
             out = torch.empty(rows, self.vocab_size, device=self.rt.device, dtype=torch.float32)
-            ops.skinny_gemm(x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out)
+            self._few_rows(x, out)
             return out
         if self.rt.is_bf16 and rows > 0 and x.dtype == torch.bfloat16:
             # many rows: the library's product, leaving the 32-bit sums as the logits
@@ -73,6 +73,14 @@ class LinearHead(Head):
             return self.forward(ready if ready is not None else norm.forward(stream.x))
         norm_w, eps = norm.fused_params()
         out = torch.empty(stream.x.shape[0], self.vocab_size, device=self.rt.device, dtype=torch.float32)
-        ops.skinny_gemm(stream.x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out,
-                        norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        self._few_rows(stream.x, out, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         return out
+
+    def _few_rows(self, x: torch.Tensor, out: torch.Tensor, **norm) -> None:
+        """At most 16 rows: the kernel whose workgroups stay and walk the table (a long stream:
+        at the 1B sizes 89 to 100 us for 1 to 16 rows against 92 to 112 with a workgroup per pair
+        of tiles), where it takes the sizes; else the few-row product."""
+        if self.weight_tiled is not None and ops.head_gemm_supports(x.shape[0], self.vocab_size, self.hidden_size, x.dtype):
+            ops.head_gemm(x, self.weight_tiled, out, **norm)
+        else:
+            ops.skinny_gemm(x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out, **norm)

@@ -337,6 +337,44 @@ def test_attention_finds_one_far_key_among_hundreds(ops):
                 assert (got[h] - want).abs().max() < 0.05, (e, row, h)
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("n,k", [(48, 1024), (3088, 2048), (1008, 3072), (272, 4096)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_logits_kernel_whose_workgroups_stay(ops, m, n, k, norm):
+    """The product for a vocabulary of rows (workgroups that walk the tiles in turn, activations
+    kept in registers): the same bits as the tile-by-tile kernel with 4 k-waves on two tiles,
+    whatever the number of workgroups (fewer than pairs of tiles, one, an odd number of tiles at
+    the end); against a 64-bit product; rows of the output wider than the product."""
+    torch.manual_seed(m + n + k)
+    x = (torch.randn(m, k, device="cuda") * 2).bfloat16()
+    w = (torch.randn(n, k, device="cuda") / math.sqrt(k)).bfloat16()
+    wt = ops.tile_weights(w)
+    kw = {}
+    xhat = x
+    if norm:
+        nw = (1 + 0.1 * torch.randn(k, device="cuda")).float()
+        ssq = x.float().pow(2)
+        parts = torch.stack([ssq[:, :k // 3].sum(-1), ssq[:, k // 3:].sum(-1)]).contiguous()
+        kw = dict(norm_w=nw, eps=1e-5, ssq_in=parts)
+        xf = x.float()
+        r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)
+        xhat = (nw * (xf * r).bfloat16().float()).bfloat16()
+    assert ops.head_gemm_supports(m, n, k, torch.bfloat16)
+    want = torch.empty(m, n, device="cuda", dtype=torch.float32)
+    ops.skinny_gemm(x, w, w_tiled=wt, epilogue=ops.SKINNY_F32, out=want, shape=4, **kw)
+    for workgroups in (0, 1, 5, n // 32 + 3):
+        wide = torch.full((m, n + 4), 7.0, device="cuda", dtype=torch.float32)
+        ops.head_gemm(x, wt, wide[:, :n], workgroups=workgroups, **kw)
+        assert torch.equal(wide[:, :n], want), workgroups
+        assert (wide[:, n:] == 7.0).all()
+    ref = xhat.cpu().double() @ w.cpu().double().T
+    assert (want.cpu().double() - ref).abs().max() < 2e-3 * max(1.0, ref.abs().max().item())
+    assert not ops.head_gemm_supports(17, n, k, torch.bfloat16) and not ops.head_gemm_supports(m, n, 1536, torch.bfloat16)
+    assert not ops.head_gemm_supports(m, n + 8, k, torch.bfloat16) and not ops.head_gemm_supports(m, n, k, torch.float32)
+    with pytest.raises(ops.KernelArgumentError):
+        ops.head_gemm(x[:, :512].contiguous(), wt, wide[:, :n])
+
+
 @pytest.mark.parametrize("m,n,k", [(17, 48, 64), (100, 301, 160), (512, 2048, 2048), (70, 1000, 96), (2048, 96, 4104)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_library_product_called_directly(ops, m, n, k, with_bias):
