@@ -227,11 +227,12 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
 @pytest.mark.parametrize("rows", [1, 2, 3, 4])
 @pytest.mark.parametrize("qh,kvh,d,n,splits", [(32, 8, 64, 2048, 16), (32, 8, 64, 2048, 8), (8, 2, 48, 304, 3),
                                                (24, 8, 128, 3072, 16), (2, 1, 64, 48, 2), (16, 16, 16, 512, 5)])
-def test_o_projection_that_merges_the_split_key_results_itself(ops, rows, qh, kvh, d, n, splits):
+@pytest.mark.parametrize("window", [0, 45])
+def test_o_projection_that_merges_the_split_key_results_itself(ops, rows, qh, kvh, d, n, splits, window):
     """Attention without its merge kernel, then the o projection that merges while it loads,
     against attention with the merge kernel and the plain residual product: the same bits, since
-    both add in the same order. Lengths make some runs of keys empty; a bias; rows of the stream
-    wider than the product."""
+    both add in the same order. Lengths (and a window) make some runs of keys empty; a bias; rows
+    of the stream wider than the product."""
     bs = 16
     lens = [(1, kv) for kv in [700, 33, 1, 255][:rows]]
     q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=rows + d + splits)
@@ -252,12 +253,12 @@ def test_o_projection_that_merges_the_split_key_results_itself(ops, rows, qh, kv
 
     po, pm = partials()
     out = torch.empty_like(q)
-    ops.attention_decode(q, kp, vp, out, kv_len, tables, qh, scale, 0, splits, po, pm)
+    ops.attention_decode(q, kp, vp, out, kv_len, tables, qh, scale, window, splits, po, pm)
     want = base.clone()
     ssq_want = ops.skinny_gemm(out, w, w_tiled=wt, epilogue=ops.SKINNY_RESIDUAL, stream=want[:, :n], bias=bias)
 
     po, pm = partials()
-    ops.attention_decode(q, kp, vp, None, kv_len, tables, qh, scale, 0, splits, po, pm, merge=False)
+    ops.attention_decode(q, kp, vp, None, kv_len, tables, qh, scale, window, splits, po, pm, merge=False)
     got = base.clone()
     ssq_got = ops.skinny_gemm_merged(po, pm, splits, qh, d, wt, got[:, :n], bias=bias)
     assert torch.equal(got, want)
