@@ -736,7 +736,8 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   // kernel is 5 to 15% faster in its form (timed at 2,048 to 16,384 tokens, heads of 64 and 128).
   // Tried and slower by 10 to 15%: the second set half a tile behind the first (two barriers a
   // tile), so that one set's products run beside the other's softmax; and the pair's key tiles
-  // dealt out evenly to the two sets with a merge of their states at the end.
+  // dealt out evenly to the two sets with a merge of their states at the end. Slower by 45% in the
+  // single-tile kernel: S^T of tile it+1 sent to the matrix cores before the softmax of tile it.
   for (int it0 = 0; it0 < n_tiles; it0 += RD) {
 #pragma unroll
     for (int r = 0; r < RD; ++r) {
