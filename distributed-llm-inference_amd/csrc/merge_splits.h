@@ -1,0 +1,71 @@
+// The merge of the partial results that decode attention leaves when a request's keys are cut into
+// runs: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M) with M = max_s m_s, for four
+// consecutive dims of one (request, head). Used by the kernels that merge on their own way (the
+// o projection of very few rows, the last workgroup of a decode attention launch); sums in the
+// order of attention_merge_kernel, so that all three give the same bits: the denominators pairwise
+// as its butterfly adds them (lanes 8 apart, then 4, 2, 1), the outputs run by run.
+#pragma once
+#include "common.h"
+
+#define MERGE_SPLITS 16  // the most runs of keys that merged_quad takes
+
+typedef float merge_float2 __attribute__((ext_vector_type(2)));
+typedef float merge_float4 __attribute__((ext_vector_type(4)));
+
+// A float that another workgroup of the same launch may have stored (with device_store): read at
+// the device's scope, past the caches that are private to a part of the chip.
+__device__ __forceinline__ float device_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void device_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// part_o [.. slots][head_dim], part_ml [.. slots][2]; `base`: the first of the S slots of this
+// (request, head); d: the first of the four dims. All loads are asked for before the first is used.
+// SAME_LAUNCH: the partial results were stored by other workgroups of this launch.
+template <bool SAME_LAUNCH = false>
+__device__ __forceinline__ merge_float4 merged_quad(const float* part_o, const float* part_ml, int64_t base, int S,
+                                                    int head_dim, int d) {
+  merge_float2 ml[MERGE_SPLITS];
+  merge_float4 po[MERGE_SPLITS];
+#pragma unroll
+  for (int j = 0; j < MERGE_SPLITS; ++j) {
+    ml[j] = merge_float2{-INFINITY, 0.f};
+    po[j] = merge_float4{0.f, 0.f, 0.f, 0.f};
+    if (j < S) {
+      const float* ml_at = part_ml + (base + j) * 2;
+      const float* po_at = part_o + (base + j) * head_dim + d;
+      if constexpr (SAME_LAUNCH) {
+        ml[j] = merge_float2{device_load(ml_at), device_load(ml_at + 1)};
+        po[j] = merge_float4{device_load(po_at), device_load(po_at + 1), device_load(po_at + 2), device_load(po_at + 3)};
+      } else {
+        ml[j] = *reinterpret_cast<const merge_float2*>(ml_at);
+        po[j] = *reinterpret_cast<const merge_float4*>(po_at);
+      }
+    }
+  }
+  float m_all = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < MERGE_SPLITS; ++j) m_all = fmaxf(m_all, ml[j][0]);
+  const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+  float wgt[MERGE_SPLITS], t[MERGE_SPLITS];
+#pragma unroll
+  for (int j = 0; j < MERGE_SPLITS; ++j) {
+    wgt[j] = j < S ? __builtin_amdgcn_exp2f(ml[j][0] - m_safe) : 0.f;
+    t[j] = __fmul_rn(ml[j][1], wgt[j]);
+  }
+#pragma unroll
+  for (int h = MERGE_SPLITS / 2; h > 0; h >>= 1)
+#pragma unroll
+    for (int j = 0; j < h; ++j) t[j] = __fadd_rn(t[j], t[j + h]);
+  const float inv = t[0] > 0.f ? 1.f / t[0] : 0.f;
+  merge_float4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < MERGE_SPLITS; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __fmaf_rn(po[j][i], wgt[j], acc[i]);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = __fmul_rn(acc[i], inv);
+  return acc;
+}

@@ -41,6 +41,7 @@
 //            k that it multiplies (all loads of a lane in flight at once) and hands it to its
 //            lanes through LDS. TILED, EPI_RESIDUAL, at most 16 runs.
 #include "common.h"
+#include "merge_splits.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
@@ -68,7 +69,6 @@ struct MergedIn {
 };
 #define MERGE_ROWS 4     // rows of a step whose o projection merges by itself
 #define MERGE_RANGE 512  // the longest run of k of one wave
-#define MERGE_SPLITS 16
 
 __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -247,50 +247,17 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
           af[j][a][q] = *w_at(wrow[j][a], s, q);
   }
   if constexpr (MERGED) {
-    // The wave's run of k, four values a lane and turn: the statistics and partial outputs of all
-    // runs of keys are asked for before the first is used. Sums in the order of
-    // attention_merge_kernel: the denominators pairwise as its butterfly adds them (lanes 8
-    // apart, then 4, 2, 1), the outputs run by run.
+    // The wave's run of k, four values a lane and turn, merged as attention_merge_kernel does.
     const int kb0 = s_begin * 32, quads = (s_end - s_begin) * 8;
     const int D = mi.head_dim, S = mi.splits;
     for (int item = lane; item < M * quads; item += 64) {
       const int row = item / quads, idx = (item - row * quads) * 4;
       const int k = kb0 + idx, head = k / D, d = k - head * D;
       const int64_t base = ((int64_t)row * mi.heads + head) * S;
-      float2v ml[MERGE_SPLITS];
-      float4v po[MERGE_SPLITS];
-#pragma unroll
-      for (int j = 0; j < MERGE_SPLITS; ++j) {
-        ml[j] = float2v{-INFINITY, 0.f};
-        po[j] = float4v{0.f, 0.f, 0.f, 0.f};
-        if (j < S) {
-          ml[j] = *reinterpret_cast<const float2v*>(mi.part_ml + (base + j) * 2);
-          po[j] = *reinterpret_cast<const float4v*>(mi.part_o + (base + j) * D + d);
-        }
-      }
-      float m_all = -INFINITY;
-#pragma unroll
-      for (int j = 0; j < MERGE_SPLITS; ++j) m_all = fmaxf(m_all, ml[j][0]);
-      const float m_safe = m_all == -INFINITY ? 0.f : m_all;
-      float wgt[MERGE_SPLITS], t[MERGE_SPLITS];
-#pragma unroll
-      for (int j = 0; j < MERGE_SPLITS; ++j) {
-        wgt[j] = j < S ? __builtin_amdgcn_exp2f(ml[j][0] - m_safe) : 0.f;
-        t[j] = __fmul_rn(ml[j][1], wgt[j]);
-      }
-#pragma unroll
-      for (int h = MERGE_SPLITS / 2; h > 0; h >>= 1)
-#pragma unroll
-        for (int j = 0; j < h; ++j) t[j] = __fadd_rn(t[j], t[j + h]);
-      const float inv = t[0] > 0.f ? 1.f / t[0] : 0.f;
-      float4v acc4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < MERGE_SPLITS; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc4[i] = __fmaf_rn(po[j][i], wgt[j], acc4[i]);
+      const float4v merged = merged_quad(mi.part_o, mi.part_ml, base, S, D, d);
       bf16_t* dst = &xs[ks][row][idx];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)__fmul_rn(acc4[i], inv);
+      for (int i = 0; i < 4; ++i) dst[i] = (bf16_t)merged[i];
     }
     __syncthreads();
 #pragma unroll

@@ -77,6 +77,9 @@ _SIGNATURES = {
     "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "dli_attention_decode_self_merging_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
+                                               _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                               _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_decode_partial_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_decode_bf16_static": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int,
@@ -979,13 +982,18 @@ def _check_paged(q, k_pages, v_pages, out, q_heads):
 def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: Optional[torch.Tensor],
                      kv_len: torch.Tensor, block_tables: torch.Tensor, q_heads: int, scale: float,
                      window: int = 0, splits: int = 1, part_o: Optional[torch.Tensor] = None,
-                     part_ml: Optional[torch.Tensor] = None, merge: bool = True) -> None:
+                     part_ml: Optional[torch.Tensor] = None, merge: bool = True,
+                     arrivals: Optional[torch.Tensor] = None) -> None:
     """Decode attention: row ``e`` of ``q`` is request ``e``'s single query over its ``kv_len[e]`` keys.
 
     With ``splits > 1`` each request's keys are cut into that many runs whose partial results go
     through ``part_o [rows, q_heads, splits, head_dim]`` and ``part_ml [rows, q_heads, splits, 2]``
     (float32) and are merged by a second kernel; with ``merge=False`` (``splits > 1`` only) they
     are left there for :func:`skinny_gemm_merged` and ``out`` is not written (it may be None).
+    ``arrivals``: int32 counters (one per request, kv head and 16 query heads of its group; zero before
+    the first launch, and every launch leaves them zero) with which the launch merges by itself, the
+    workgroup that finishes last doing the second kernel's work with the same result to the bit
+    (up to :data:`SELF_MERGING_SPLITS` runs; beyond that the second kernel runs as without them).
     """
     _require(merge or splits > 1, "without a merge there must be two or more runs of keys")
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out if out is not None else q, q_heads)
@@ -1007,11 +1015,22 @@ def attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
             _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size, float(scale),
             int(window), int(splits), _stream()), "attention_decode")
         return
+    if arrivals is not None and splits > 1:
+        _dense(arrivals, "arrivals", torch.int32, 1)
+        _require(arrivals.numel() >= rows * kv_heads * ((q_heads // kv_heads + 15) // 16),
+                 "one arrival counter per request, kv head and tile of 16 heads")
+        _check(library().dli_attention_decode_self_merging_bf16(
+            _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml),
+            _ptr(arrivals), _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads,
+            head_dim, page_size, float(scale), int(window), int(splits), _stream()), "attention_decode")
+        return
     _check(library().dli_attention_decode_bf16(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml),
         _ptr(kv_len), _ptr(block_tables), block_tables.stride(0), rows, q_heads, kv_heads, head_dim, page_size,
         float(scale), int(window), int(splits), _stream()), "attention_decode")
 
+
+SELF_MERGING_SPLITS = 16  # csrc/merge_splits.h: MERGE_SPLITS
 
 STATIC_SCRATCH_FLOATS = 2 * 1024 * 1024  # csrc/no_alloc.h: DLI_STATIC_SCRATCH_FLOATS
 

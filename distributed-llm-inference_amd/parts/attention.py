@@ -33,10 +33,11 @@ from .spec import PartSpec, WeightSpec
 ROPE_IN_PRODUCT_ROWS = range(1, 17)
 # Decode steps with this many rows leave the merge of the runs of keys to the o projection, whose
 # waves merge the k that they multiply while their first weights are on their way. Every workgroup
-# of that product repeats the merge of all rows, so it pays for one or two rows only (a batch-1
-# step at the 1B sizes: 9.7 -> 7.3 us for merge plus product, 2% of the step; nothing gained at
-# two rows; at three and four rows the step was 6% slower than with the merge kernel).
-MERGE_IN_PRODUCT_ROWS = 2
+# of that product repeats the merge of all rows, so it pays for one row only (a batch-1 step at
+# the 1B sizes: 0.902 ms against 0.935 with the attention launch that merges in its last
+# workgroups; at two rows 1.002 against 0.994; at three and four rows 6% slower than even a
+# separate merge kernel).
+MERGE_IN_PRODUCT_ROWS = 1
 FEW_ROWS = 16  # up to here the few-row product kernels run; from 17 to 64 rows the one that shares activations
 
 
@@ -60,6 +61,24 @@ class GQAttention(Mixer):
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self.w_qkv_tiled = self.w_o_tiled = None
         self.w_qkv_rope = self.b_qkv_rope = None  # tile order with rotary pairs, for the product that rotates
+        self._arrivals: Optional[torch.Tensor] = None
+
+    ARRIVAL_COUNTERS = 4096  # keys are cut into runs only when requests x kv heads are few
+
+    def arrival_counters(self, needed: int) -> Optional[torch.Tensor]:
+        """``needed`` counters with which a decode attention launch merges its runs of keys by
+        itself (``ops.attention_decode``): zero when made, and every launch leaves them zero. They
+        are this layer's own, since launches that share counters must not overlap, and they are
+        made once and kept, since captured graphs hold their address. None (then the merge
+        kernel runs) if more are needed than there are, or if they would have to be made while
+        the stream is being captured into a graph: their memory would belong to that graph."""
+        if needed > self.ARRIVAL_COUNTERS:
+            return None
+        if self._arrivals is None:
+            if torch.cuda.is_current_stream_capturing():
+                return None
+            self._arrivals = torch.zeros(self.ARRIVAL_COUNTERS, device=self.rt.device, dtype=torch.int32)
+        return self._arrivals
 
     # -- weights
     def weight_specs(self) -> dict[str, WeightSpec]:
@@ -155,7 +174,8 @@ class GQAttention(Mixer):
                           cache.k_pages if nkv else None, cache.v_pages if nkv else None, nh, nkv, d)
         q = qkv[:, :nh * d]
         out = self.rt.empty(x.shape[0], nh * d)
-        paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window,
+                        self.arrival_counters)
         return linear(self.rt, out, self.w_o, self.b_o)
 
     # -- decode steps with few rows: the norm before and the residual sum after are fused into
@@ -217,7 +237,8 @@ class GQAttention(Mixer):
                                                     bias=self.b_o))
                 return
         out = self.rt.empty(n, nh * d)
-        paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window,
+                        self.arrival_counters)
         stream.wrote(ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
                                      stream=stream.x, bias=self.b_o))
 
@@ -239,6 +260,7 @@ class GQAttention(Mixer):
         angles = ctx.rope_angles(self.position.rotary_table().inv_freq, q.dtype)
         ops.mid_finish_qkv(partial, q, angles, grp.slots, cache.k_pages, cache.v_pages, nh, bias=self.b_qkv_rope)
         out = self.rt.empty(n, nh * d)
-        paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window)
+        paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window,
+                        self.arrival_counters)
         partial = ops.mid_gemm(out, self.w_o_tiled, tiled=True, n=self.hidden_size, epilogue=ops.MID_PARTIAL)
         finish_residual(self.rt, stream, partial, self.b_o, following)

@@ -7,7 +7,7 @@ decode kernel and portions to the tiled prefill kernel.
 
 from __future__ import annotations
 
-from typing import Any
+from typing import Any, Callable, Optional
 
 import torch
 
@@ -35,8 +35,11 @@ def choose_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int =
 
 
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
-                    ctx: Any, grp: Any, q_heads: int, scale: float, window: int = 0) -> None:
-    """Attention of every row of the step over its request's pages, into ``out``."""
+                    ctx: Any, grp: Any, q_heads: int, scale: float, window: int = 0,
+                    arrival_counters: Optional[Callable[[int], Optional[torch.Tensor]]] = None) -> None:
+    """Attention of every row of the step over its request's pages, into ``out``.
+    ``arrival_counters(n)``: the caller's ``n`` counters with which the decode kernel merges its
+    runs of keys by itself (see ``ops.attention_decode``), or None."""
     if ctx.num_tokens == 0:
         return
     _, kv_heads, page_size, head_dim = k_pages.shape
@@ -49,8 +52,11 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
     nd = ctx.num_decode
     if nd > 0:
         splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device)
+        arrivals = None
+        if arrival_counters is not None and 1 < splits <= ops.SELF_MERGING_SPLITS:
+            arrivals = arrival_counters(nd * kv_heads * (-(-(q_heads // kv_heads) // 16)))
         ops.attention_decode(q[:nd], k_pages, v_pages, out[:nd], ctx.kv_len, grp.block_tables, q_heads,
-                             scale, window, splits, part_o, part_ml)
+                             scale, window, splits, part_o, part_ml, arrivals=arrivals)
     if ctx.num_entries > nd:
         tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads), first_entry=nd)
         ops.attention_prefill(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,

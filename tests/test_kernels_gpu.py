@@ -224,6 +224,40 @@ def test_attention_decode_mfma(ops, qh, kvh, d, bs, splits, window):
     assert err < tol(torch.bfloat16), err
 
 
+@pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
+@pytest.mark.parametrize("splits", [2, 5, 16, 17])
+@pytest.mark.parametrize("window", [0, 45])
+def test_attention_decode_that_merges_in_its_last_workgroup(ops, qh, kvh, d, bs, splits, window):
+    """With arrival counters the launch merges its runs of keys by itself: the same bits as with the
+    merge kernel, launch after launch on the same counters (each leaves them zero), also after a
+    launch with other lengths; 17 runs are more than it takes, then the merge kernel runs."""
+    rng = torch.Generator().manual_seed(d * 5 + bs + splits)
+    rand = [int(x) for x in torch.randint(1, 40 * bs, (5,), generator=rng)]
+    lens = [(1, n) for n in [1, bs, bs + 1, 3 * bs - 1, 15, 17] + rand]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + bs + splits)
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    q, kp, vp, kv_len, tables = q.cuda(), kp.cuda(), vp.cuda(), dev(kv_len), dev(tables)
+    scale = 1.0 / math.sqrt(d)
+    n = len(lens)
+    counters = torch.zeros(n * kvh * (-(-(qh // kvh) // 16)) + 3, dtype=torch.int32, device="cuda")
+
+    def run(rows, arrivals):
+        part_o = torch.full((rows * qh * splits * d,), float("nan"), device="cuda")
+        part_ml = torch.full((rows * qh * splits * 2,), float("nan"), device="cuda")
+        out = torch.full((rows, qh * d), 9.0, dtype=torch.bfloat16, device="cuda")
+        ops.attention_decode(q[:rows], kp, vp, out, kv_len, tables, qh, scale, window, splits, part_o, part_ml,
+                             arrivals=arrivals)
+        return out
+
+    want = run(n, None)
+    for rows in (n, 3, n):
+        got = run(rows, counters)
+        assert torch.equal(got, want[:rows]), rows
+        assert int(counters.abs().sum()) == 0
+    with pytest.raises(ops.KernelArgumentError):
+        run(n, counters[:2])
+
+
 @pytest.mark.parametrize("rows", [1, 2, 3, 4])
 @pytest.mark.parametrize("qh,kvh,d,n,splits", [(32, 8, 64, 2048, 16), (32, 8, 64, 2048, 8), (8, 2, 48, 304, 3),
                                                (24, 8, 128, 3072, 16), (2, 1, 64, 48, 2), (16, 16, 16, 512, 5)])

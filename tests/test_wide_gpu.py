@@ -100,8 +100,8 @@ def test_requests_decode_together_at_serving_widths(count):
 
 @pytest.mark.parametrize("count", [1, 2])
 def test_one_and_two_requests_decode_without_a_merge_kernel(count, monkeypatch):
-    """With one or two rows and keys enough for two runs, the o projection merges the runs of
-    keys itself: the path is taken (counted), agrees with the plain implementation, and gives the
+    """With one or two rows (two: where the limit is set so) and keys enough for two runs, the o
+    projection merges the runs of keys itself: the path is taken (counted), agrees with the plain implementation, and gives the
     bits of the path with the merge kernel. The steps' logits are copied on the stream and looked
     at only after the last step: a replay must not refill its staging buffer while the copy of the
     step before is still queued."""
@@ -135,6 +135,52 @@ def test_one_and_two_requests_decode_without_a_merge_kernel(count, monkeypatch):
     seen = len(calls)
     separate = run(0)
     assert len(calls) == seen
+    for a, b in zip(merged, separate):
+        assert torch.equal(a, b)
+
+
+def test_decode_attention_merges_its_runs_of_keys_in_the_launch(monkeypatch):
+    """Four requests with keys enough for several runs: the decode attention launches merge by
+    themselves (counted: arrival counters are passed), also when replayed from graphs, step after
+    step on the same counters; the result agrees with the plain implementation and has the bits of
+    the path with the merge kernel."""
+    from dli_amd.kernels import ops
+    from dli_amd.parts import attention
+    from dli_amd.trace import TraceSession
+
+    rng = random.Random(23)
+    lens = [300, 270, 140, 17]
+    steps = 6
+    toks = [[rng.randrange(32003) for _ in range(n + steps)] for n in lens]
+    seen = []
+    real = ops.attention_decode
+
+    def counted(*a, **k):
+        seen.append((a[9] if len(a) > 9 else k.get("splits", 1), k.get("arrivals") is not None))
+        return real(*a, **k)
+
+    monkeypatch.setattr(ops, "attention_decode", counted)
+
+    def run(self_merging):
+        if not self_merging:
+            monkeypatch.setattr(attention.GQAttention, "arrival_counters", lambda self, needed: None)
+        core = make_core("bfloat16", pages=64, graphs=4)
+        s = TraceSession(core)
+        s.step([{"id": r, "tokens": toks[r][:lens[r]], "want": []} for r in range(4)])
+        outs = []
+        for i in range(steps):
+            outs.append(s.step([{"id": r, "tokens": [toks[r][lens[r] + i]], "want": [0]} for r in range(4)]).clone())
+        assert core.step.graphs.replays >= steps - 1
+        return outs
+
+    merged = run(True)
+    assert seen and all(splits >= 2 and counters for splits, counters in seen)
+    for i, out in enumerate(merged):
+        rows = torch.stack([plain(toks[r])[lens[r] + i] for r in range(4)])
+        check(out, rows, "bfloat16", f"decode step {i} that merges in the attention launch")
+    del seen[:]
+    separate = run(False)
+    assert seen and not any(counters for _, counters in seen)
     for a, b in zip(merged, separate):
         assert torch.equal(a, b)
 
