@@ -107,7 +107,7 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
 #pragma unroll
   for (int g = 0; g < MG; ++g) {
     const int m = 4 * g + r;
-    xrow[g] = m < M ? (int)(m * ldx * 2) : -1;
+    xrow[g] = m < M ? (int)(m * ldx * 2) : (int)x_bytes;  // past the end: what is added stays there
     rs[g] = 1.f;
   }
   float4v acc[FQ][MG];
@@ -125,27 +125,35 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     float4v g0, g1;
   };
   const int xpad = chunks * 128 + 32;  // XL: values per row of xs; rows 64 bytes apart in the banks
-  // Every turn of the loop issues the same loads (the last one reads its own chunk again), so the
-  // number of loads in flight is known at compile time and only the current chunk is waited for.
+  // Every turn of the loop issues the same loads (a turn past the wave's last chunk reads the
+  // last chunk's weights again and zeros for x), so the number of loads in flight is known at
+  // compile time and only the current chunk is waited for.
   auto fetch = [&](int c, Stage& st) __attribute__((always_inline)) {
-    const int k = c * 128 + blk * 8;
-    const bool inside = k < K;  // the last chunk may reach past k; K % 8 == 0
-    const int kc = inside ? k : 0;
+    const int k = min(c, c1 - 1) * 128 + blk * 8;
+    const bool inside = k < K && c < c1;  // the last chunk may reach past k; K % 8 == 0
+    const int kc = k < K ? k : 0;
 #pragma unroll
     for (int f = 0; f < FQ; ++f) st.wf[f].raw = *reinterpret_cast<const u32x4*>(wrow[f] + kc);
     if constexpr (!XL) {
+      const int k_at = inside ? k * 2 : (int)x_bytes;  // one offset for every case, no branch
 #pragma unroll
-      for (int g = 0; g < MG; ++g)
-        st.xf[g].raw = __builtin_amdgcn_raw_buffer_load_b128(
-            xres, inside && xrow[g] >= 0 ? xrow[g] + k * 2 : (int)x_bytes, 0, 0);
+      for (int g = 0; g < MG; ++g) st.xf[g].raw = __builtin_amdgcn_raw_buffer_load_b128(xres, xrow[g] + k_at, 0, 0);
       if constexpr (NORM) {
         st.g0 = *reinterpret_cast<const float4v*>(norm_w + kc);
         st.g1 = *reinterpret_cast<const float4v*>(norm_w + kc + 4);
       }
     }
   };
-  Stage cur;
-  if (XL && c0 < c1) fetch(c0, cur);  // the first weights are on their way while x is staged
+  // DEPTH chunks are on their way at a time, each in registers of its own: the loop is written
+  // out for all of them, so that no chunk is copied (a copy waits for its loads) and each is
+  // waited for only when its turn has come.
+  constexpr int DEPTH = 4;
+  Stage st[DEPTH];
+  auto fetch_first = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) fetch(c0 + d, st[d]);
+  };
+  if (XL && c0 < c1) fetch_first();  // the first weights are on their way while x is staged
   if constexpr (NORM) {
     // rs[m] from the parts of sum x^2. The parts are dealt out to all blocks of all waves (block
     // q of 16*KS takes the parts q, q + 16*KS, ...), eight loads at a time so that they share one
@@ -182,7 +190,7 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     }
   }
 
-  if (!XL && c0 < c1) fetch(c0, cur);
+  if (!XL && c0 < c1) fetch_first();
   if constexpr (XL) {
     // thread t stages the 8 values at k = 8*(t % (chunks*16)) of row t / (chunks*16), and so on
     __shared__ float rs_row[4 * MG];
@@ -215,34 +223,42 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     }
     __syncthreads();
   }
-  if (c0 < c1) {
-    for (int c = c0; c < c1; ++c) {
-      Stage nxt;
-      fetch(min(c + 1, c1 - 1), nxt);
-      if constexpr (XL) {
+  auto multiply = [&](Stage& cur, int c) __attribute__((always_inline)) {
+    if constexpr (XL) {
 #pragma unroll
-        for (int g = 0; g < MG; ++g) {
-          const int m = 4 * g + r;
-          cur.xf[g].raw = u32x4{0, 0, 0, 0};
-          if (m < M) cur.xf[g].raw = *reinterpret_cast<const u32x4*>(xs + (int64_t)m * xpad + c * 128 + blk * 8);
-        }
-      } else if constexpr (NORM) {
-#pragma unroll
-        for (int g = 0; g < MG; ++g)
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const float normed = (float)(bf16_t)((float)cur.xf[g].e[i] * rs[g]);
-            cur.xf[g].e[i] = (bf16_t)((i < 4 ? cur.g0[i] : cur.g1[i - 4]) * normed);
-          }
+      for (int g = 0; g < MG; ++g) {
+        const int m = 4 * g + r;
+        cur.xf[g].raw = u32x4{0, 0, 0, 0};
+        if (m < M && c < c1)
+          cur.xf[g].raw = *reinterpret_cast<const u32x4*>(xs + (int64_t)m * xpad + c * 128 + blk * 8);
       }
+    } else if constexpr (NORM) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
+      for (int g = 0; g < MG; ++g)
 #pragma unroll
-        for (int f = 0; f < FQ; ++f)
-#pragma unroll
-          for (int g = 0; g < MG; ++g) acc[f][g] = mfma4(cur.wf[f].h[h], cur.xf[g].h[h], acc[f][g]);
-      cur = nxt;
+        for (int i = 0; i < 8; ++i) {
+          const float normed = (float)(bf16_t)((float)cur.xf[g].e[i] * rs[g]);
+          cur.xf[g].e[i] = (bf16_t)((i < 4 ? cur.g0[i] : cur.g1[i - 4]) * normed);
+        }
     }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int f = 0; f < FQ; ++f)
+#pragma unroll
+        for (int g = 0; g < MG; ++g) acc[f][g] = mfma4(cur.wf[f].h[h], cur.xf[g].h[h], acc[f][g]);
+  };
+  if (c0 < c1) {
+    int c = c0;
+    for (; c + DEPTH < c1; c += DEPTH) {  // groups that have a chunk behind them
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        multiply(st[d], c + d);
+        fetch(c + d + DEPTH, st[d]);
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) multiply(st[d], c + d);  // the last group (turns past the end add zeros)
   }
 
   // blocks l/4 that differ in their upper two bits are added by lane swaps, the remaining four

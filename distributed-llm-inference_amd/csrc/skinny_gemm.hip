@@ -88,10 +88,9 @@ struct XFrag<false> {
 
 template <bool NORM>
 __device__ __forceinline__ XFrag<NORM> fetch_x(const bf16_t* __restrict__ xrow,
-                                               const float* __restrict__ norm_w, int k, bool live) {
+                                               const float* __restrict__ norm_w, int k) {
   XFrag<NORM> f;
-  f.v = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-  if (live) f.v = *reinterpret_cast<const bf16x8*>(xrow + k);
+  f.v = *reinterpret_cast<const bf16x8*>(xrow + k);
   if constexpr (NORM) {
     f.w0 = *reinterpret_cast<const float4v*>(norm_w + k);
     f.w1 = *reinterpret_cast<const float4v*>(norm_w + k + 4);
@@ -160,43 +159,119 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
   // EPI_RESIDUAL: the stream values that this lane will add to at the end (lane holds
   // y[m = 16t + col][n = 16*tile + 4*grp + i]) are asked for now, so that the epilogue does not
   // wait for a trip to memory of its own
-  float old_s[EPI == EPI_RESIDUAL ? NT : 1][EPI == EPI_RESIDUAL ? MT : 1][4];
+  bf16_t old_s[EPI == EPI_RESIDUAL ? NT : 1][EPI == EPI_RESIDUAL ? MT : 1][4];
   if constexpr (EPI == EPI_RESIDUAL) {
-    if (ks == 0) {
+    // In every wave and for every element (only the first k-split wave uses them; an element past
+    // the edge reads the edge's and is not stored): a load under a condition is waited for on
+    // the spot, one trip to memory after the other, and leaves the count of loads on their way
+    // unknown to everything behind it.
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int t = 0; t < MT; ++t)
+      for (int t = 0; t < MT; ++t)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int n = (tile0 + j) * 16 + 4 * grp + i, m = t * 16 + col;
-            old_s[j][t][i] = m < M && n < N ? (float)stream[(int64_t)m * lds_ + n] : 0.f;
-          }
-    }
+        for (int i = 0; i < 4; ++i) {
+          const int n = (tile0 + j) * 16 + 4 * grp + i, m = t * 16 + col;
+          old_s[j][t][i] = stream[(int64_t)min(m, M - 1) * lds_ + min(n, N - 1)];
+        }
   }
 
   const bf16_t* xrow[MT];
-  bool live[MT];
   float rs[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + col;
-    live[t] = m < M;
     xrow[t] = x + (int64_t)min(m, M - 1) * ldx;
     rs[t] = 1.f;
   }
+  float4v acc[NT][NA][MT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[j][a][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // this wave's share of the k steps of 32
+  const int steps = K / 32;
+  const int s_begin = TILED ? 4 * (int)((int64_t)(steps / 4) * ks / KS) : (int)((int64_t)steps * ks / KS);
+  const int s_end = TILED ? 4 * (int)((int64_t)(steps / 4) * (ks + 1) / KS) : (int)((int64_t)steps * (ks + 1) / KS);
+  int s = s_begin;
+  // Blocks of 128: lane group g reads k in [32g, 32g + 32). The weights and activations of the
+  // next block are asked for before the products of the current one. The two sets of registers
+  // take turns in a loop that is written out for both, with the last block's products apart, so
+  // that at every product the number of younger loads is known and the wait is for the block's
+  // own loads alone (with one body for every turn, the turn without younger loads decides the
+  // wait of all: each block was then waited for right after it had been asked for). Rows past
+  // the last read the last row again (their results are dropped), so no load is conditional.
+  struct Block {
+    bf16x8 a[NT][NA][4];
+    XFrag<NORM> x[MT][4];
+  };
+  auto fetch_weights = [&](Block& b, int at) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b.a[j][a][q] = *w_at(wrow[j][a], at, q);
+  };
+  auto fetch_rows = [&](Block& b, int at) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) b.x[t][q] = fetch_x<NORM>(xrow[t], norm_w, at * 32 + grp * 32 + q * 8);
+  };
+  auto multiply = [&](const Block& b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bf16x8 bf = finish_x<NORM>(b.x[t][q], rs[t]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int a = 0; a < NA; ++a) acc[j][a][t] = mfma32(b.a[j][a][q], bf, acc[j][a][t]);
+      }
+    }
+  };
+  int blocks = (s_end - s) / 4;
+  Block b0, b1;
   if constexpr (NORM) {
     // rs[m] from the parts of sum x^2 that the producer of x left. The parts are dealt out to
     // all lane groups of all waves (group q of W*4 takes the parts q, q + 4W, ...), eight loads
     // at a time so that they share one trip to memory; a wave adds its four groups, the waves'
-    // sums meet in LDS and are added in wave order.
+    // sums meet in LDS and are added in wave order. The first block of weights and rows is asked
+    // for right behind the first eight parts and before anything waits for them, so that it is
+    // on its way while the sums are made.
     constexpr int W = KS * NS;
     __shared__ float rsum[W][MT][16];
+    float first[MT][8];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = min(t * 16 + col, M - 1);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        // no load is conditional (a part past the last reads the last and counts as zero), so
+        // that the number of loads on their way is known where the first is waited for
+        const int p = wave * 4 + grp + u * 4 * W;
+        const float part = ssq_in[(int64_t)min(p, ssq_parts - 1) * M + m];
+        first[t][u] = p < ssq_parts ? part : 0.f;
+      }
+    }
+    // (a wave without a block of its own, k being short, reads the matrix's first block)
+    if (TILED || blocks > 0) {
+      fetch_rows(b0, blocks > 0 ? s : 0);
+      fetch_weights(b0, blocks > 0 ? s : 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const int m = min(t * 16 + col, M - 1);
       float sum = 0.f;
-      for (int p0 = wave * 4 + grp; p0 < ssq_parts; p0 += 32 * W) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sum += first[t][u];
+      for (int p0 = wave * 4 + grp + 32 * W; p0 < ssq_parts; p0 += 32 * W) {
         float v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -218,33 +293,8 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
       for (int wv = 0; wv < W; ++wv) sum += rsum[wv][t][col];
       rs[t] = rsqrtf(sum / (float)K + eps);
     }
-  }
-
-  float4v acc[NT][NA][MT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j)
-#pragma unroll
-    for (int a = 0; a < NA; ++a)
-#pragma unroll
-      for (int t = 0; t < MT; ++t) acc[j][a][t] = float4v{0.f, 0.f, 0.f, 0.f};
-
-  // this wave's share of the k steps of 32
-  const int steps = K / 32;
-  const int s_begin = TILED ? 4 * (int)((int64_t)(steps / 4) * ks / KS) : (int)((int64_t)steps * ks / KS);
-  const int s_end = TILED ? 4 * (int)((int64_t)(steps / 4) * (ks + 1) / KS) : (int)((int64_t)steps * (ks + 1) / KS);
-  int s = s_begin;
-  // blocks of 128: lane group g reads k in [32g, 32g + 32). The weights of the next block are
-  // requested before the products of the current one, so two blocks are in flight per wave.
-  bf16x8 af[NT][NA][4];
-  XFrag<NORM> xf[MT][4];
-  if (s + 4 <= s_end) {
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int a = 0; a < NA; ++a)
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          af[j][a][q] = *w_at(wrow[j][a], s, q);
+  } else {
+    if (blocks > 0) fetch_weights(b0, s);
   }
   if constexpr (MERGED) {
     // The wave's run of k, four values a lane and turn, merged as attention_merge_kernel does.
@@ -263,59 +313,49 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) xrow[t] = &xs[ks][min(t * 16 + col, M - 1)][0] - kb0;
   }
-  if (s + 4 <= s_end) {
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) xf[t][q] = fetch_x<NORM>(xrow[t], norm_w, s * 32 + grp * 32 + q * 8, live[t]);
+  if constexpr (!NORM) {
+    if (blocks > 0) fetch_rows(b0, s);
   }
-  for (; s + 4 <= s_end; s += 4) {
-    const int kb = s * 32 + grp * 32;
-    bf16x8 nf[NT][NA][4];
-    XFrag<NORM> nx[MT][4];
-    const bool more = s + 8 <= s_end;
-    if (more) {
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int a = 0; a < NA; ++a)
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            nf[j][a][q] = *w_at(wrow[j][a], s + 4, q);
-#pragma unroll
-      for (int t = 0; t < MT; ++t)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) nx[t][q] = fetch_x<NORM>(xrow[t], norm_w, kb + 128 + q * 8, live[t]);
-    }
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const bf16x8 bf = finish_x<NORM>(xf[t][q], rs[t]);
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int a = 0; a < NA; ++a) acc[j][a][t] = mfma32(af[j][a][q], bf, acc[j][a][t]);
+  if constexpr (MT > 1) {
+    // several row tiles: one body for every turn (the registers do not hold two whole blocks)
+    for (; s + 4 <= s_end; s += 4) {
+      const bool more = s + 8 <= s_end;
+      if (more) {
+        fetch_weights(b1, s + 4);
+        fetch_rows(b1, s + 4);
       }
+      multiply(b0);
+      if (more) b0 = b1;
     }
-    if (more) {
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int a = 0; a < NA; ++a)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) af[j][a][q] = nf[j][a][q];
-#pragma unroll
-      for (int t = 0; t < MT; ++t)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) xf[t][q] = nx[t][q];
+  } else if (blocks > 0) {
+    while (blocks >= 3) {
+      fetch_rows(b1, s + 4);
+      fetch_weights(b1, s + 4);
+      __builtin_amdgcn_sched_barrier(0);  // all of the next block's loads leave before the products
+      multiply(b0);
+      fetch_rows(b0, s + 8);
+      fetch_weights(b0, s + 8);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(b1);
+      s += 8;
+      blocks -= 2;
     }
+    if (blocks == 2) {
+      fetch_rows(b1, s + 4);
+      fetch_weights(b1, s + 4);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(b0);
+      multiply(b1);
+    } else {
+      multiply(b0);
+    }
+    s = s_begin + (s_end - s_begin) / 4 * 4;
   }
   for (; !TILED && s < s_end; ++s) {  // single steps: lane group g reads k in [8g, 8g + 8)
     const int kb = s * 32 + grp * 8;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const bf16x8 bf = finish_x<NORM>(fetch_x<NORM>(xrow[t], norm_w, kb, live[t]), rs[t]);
+      const bf16x8 bf = finish_x<NORM>(fetch_x<NORM>(xrow[t], norm_w, kb), rs[t]);
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -431,7 +471,7 @@ __global__ __launch_bounds__(KS * NS * 64) void skinny_gemm_kernel(
             reinterpret_cast<bf16_t*>(out)[(int64_t)m * ldo + n] = (bf16_t)(sg * u);
           } else {  // EPI_RESIDUAL
             bf16_t* sp = stream + (int64_t)m * lds_ + n;
-            const bf16_t summed = (bf16_t)(old_s[EPI == EPI_RESIDUAL ? j : 0][EPI == EPI_RESIDUAL ? t : 0][i] + (float)(bf16_t)y[0][i]);
+            const bf16_t summed = (bf16_t)((float)old_s[EPI == EPI_RESIDUAL ? j : 0][EPI == EPI_RESIDUAL ? t : 0][i] + (float)(bf16_t)y[0][i]);
             *sp = summed;
             sq += (float)summed * (float)summed;
           }
