@@ -146,16 +146,21 @@ __device__ __forceinline__ void load_k(short4v (&kreg)[DCH], const bf16_t* __res
   for (int c = 0; c < DCH; ++c) kreg[c] = *reinterpret_cast<const short4v*>(p + c * 4);
 }
 
-// Keys at or beyond `end_key` are replaced by zero so that a zero probability never multiplies
-// whatever a not yet written slot holds.
 template <int DCH>
 __device__ __forceinline__ void load_v(short4v (&vreg)[DCH], const bf16_t* __restrict__ v_pages,
                                        int64_t page, int kv_heads, int kvh, int page_size, int off,
-                                       int col, int grp, int t, int end_key) {
+                                       int col, int grp) {
   constexpr int D = DCH * 16;
   const bf16_t* p = v_pages + ((page * kv_heads + kvh) * D + col) * page_size + off + 4 * grp;
 #pragma unroll
   for (int c = 0; c < DCH; ++c) vreg[c] = *reinterpret_cast<const short4v*>(p + (int64_t)c * 16 * page_size);
+}
+
+// Values of keys at or beyond `end_key` are replaced by zero so that a zero probability never
+// multiplies whatever a not yet written slot holds. Apart from the loads: what looks at loaded
+// values waits for them.
+template <int DCH>
+__device__ __forceinline__ void blank_v(short4v (&vreg)[DCH], int grp, int t, int end_key) {
   if (t + 16 > end_key) {
 #pragma unroll
     for (int c = 0; c < DCH; ++c)
@@ -184,7 +189,8 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   const int group = q_heads / kv_heads;
   const int head_tiles = (group + 15) / 16;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y % head_tiles;
-  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int lane = threadIdx.x % DLI_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / DLI_WAVE);  // known to be the same in all lanes
   const int col = lane % 16, grp = lane / 16;
   const int head_in_group = ht * 16 + col;
   const bool valid = head_in_group < group;
@@ -209,37 +215,77 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
 
   ColumnTile<DCH> st;
   st.init();
-  // A wave takes every fourth tile of 16 keys. The step is as long as its chain of dependent
-  // memory accesses, so the tiles are taken UN at a time: first all their block-table entries,
-  // then all their keys and values, then the arithmetic. Tiles past the end read page 0 and are
-  // skipped.
-  constexpr int UN = DCH <= 4 ? 4 : 2;
-  int tp = (k0 + wave * 16) / page_size, toff = (k0 + wave * 16) % page_size;
-  for (int t0 = k0 + wave * 16; t0 < k1; t0 += 64 * UN) {
+  // A wave takes every fourth tile of 16 keys, UN tiles (a group) at a time. A group costs a chain
+  // of two trips to memory (its block-table entries, then its keys and values), so the chain is
+  // taken apart: while group g is multiplied, the keys and values of group g+1 are on their way
+  // (two sets of registers take turns) and the table entries of group g+2 have been asked for.
+  // No load hangs on a condition (a tile past the run's end reads the run's last tile again and
+  // is skipped by the arithmetic; values of keys past the end are blanked when they are used),
+  // so at every wait the number of younger loads is known and only the group's own are waited for.
+  constexpr int UN = 1, NG = 4;  // tiles of a group, groups on their way
+  constexpr int STEP = 64 * UN;  // keys between a wave's groups
+  struct Group {
+    short4v k[UN][DCH], v[UN][DCH];
+  };
+  struct Where {
     int64_t page[UN];
     int off[UN];
+  };
+  const int t_first = k0 + wave * 16;
+  if (t_first < k1) {
+    const int t_last = (k1 - 1) / 16 * 16;  // the run's last tile
+    auto look_up = [&](Where& w, int tg) __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int t = t0 + 64 * u;
-      page[u] = t < k1 ? table[tp] : 0;
-      off[u] = toff;
-      toff += 64;
-      while (toff >= page_size) { toff -= page_size; ++tp; }
+      for (int u = 0; u < UN; ++u) {
+        const int t = min(tg + 64 * u, t_last);
+        w.page[u] = table[t / page_size];
+        w.off[u] = t % page_size;
+      }
+    };
+    auto fetch = [&](Group& g, const Where& w) __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        load_k<DCH>(g.k[u], k_pages, w.page[u], kv_heads, kvh, page_size, w.off[u], col, grp);
+        load_v<DCH>(g.v[u], v_pages, w.page[u], kv_heads, kvh, page_size, w.off[u], col, grp);
+      }
+    };
+    auto attend = [&](const Group& g, int tg) __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int t = tg + 64 * u;
+        if (t < k1) {
+          const bool need_mask = t + 16 > k1 || t < first_visible;
+          short4v v[DCH];  // a copy: the group's registers are written by loads only
+#pragma unroll
+          for (int c = 0; c < DCH; ++c) v[c] = g.v[u][c];
+          blank_v<DCH>(v, grp, t, k1);
+          attend_tile<DCH>(st, g.k[u], qreg, v, t, grp, k1 - 1, first_visible, scale_log2e, need_mask);
+        }
+      }
+    };
+    // NG sets of registers take turns; set d holds group g = d (mod NG), and where[d] the place of
+    // the group that it loads next
+    Group sets[NG];
+    Where where[NG];
+#pragma unroll
+    for (int d = 0; d < NG; ++d) look_up(where[d], t_first + d * STEP);
+#pragma unroll
+    for (int d = 0; d < NG; ++d) {
+      fetch(sets[d], where[d]);
+      look_up(where[d], t_first + (d + NG) * STEP);
     }
-    short4v kreg[UN][DCH], vreg[UN][DCH];
+    int tg = t_first;
+    for (; tg + NG * STEP < k1; tg += NG * STEP) {  // rounds that have a group behind them
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      load_k<DCH>(kreg[u], k_pages, page[u], kv_heads, kvh, page_size, off[u], col, grp);
-      load_v<DCH>(vreg[u], v_pages, page[u], kv_heads, kvh, page_size, off[u], col, grp, t0 + 64 * u, k1);
-    }
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int t = t0 + 64 * u;
-      if (t < k1) {
-        const bool need_mask = t + 16 > k1 || t < first_visible;
-        attend_tile<DCH>(st, kreg[u], qreg, vreg[u], t, grp, k1 - 1, first_visible, scale_log2e, need_mask);
+      for (int d = 0; d < NG; ++d) {
+        attend(sets[d], tg + d * STEP);
+        fetch(sets[d], where[d]);
+        look_up(where[d], tg + (d + 2 * NG) * STEP);
+        __builtin_amdgcn_sched_barrier(0);  // the loads leave before the next group's arithmetic
       }
     }
+#pragma unroll
+    for (int d = 0; d < NG; ++d) attend(sets[d], tg + d * STEP);  // the last round
   }
 
   // merge the four waves' states in wave 0
@@ -449,7 +495,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int off = t % page_size;
     short4v kreg[DCH], vreg[DCH];
     load_k<DCH>(kreg, k_pages, page, kv_heads, kvh, page_size, off, col, grp);
-    load_v<DCH>(vreg, v_pages, page, kv_heads, kvh, page_size, off, col, grp, t, end);
+    load_v<DCH>(vreg, v_pages, page, kv_heads, kvh, page_size, off, col, grp);
+    blank_v<DCH>(vreg, grp, t, end);
     // a tile needs masking if it reaches beyond the first query's position or before the window
     const bool need_mask = t + 15 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
     const int low0 = window > 0 ? pos[0] - window + 1 : 0;
