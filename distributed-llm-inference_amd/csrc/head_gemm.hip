@@ -51,7 +51,8 @@ __global__ __launch_bounds__(HEAD_KS * 64) void head_gemm_kernel(
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int p = p0 + u * 4 * KS;
-        v[u] = p < ssq_parts ? ssq_in[(int64_t)p * M + m] : 0.f;
+        const float part = ssq_in[(int64_t)min(p, ssq_parts - 1) * M + m];
+        v[u] = p < ssq_parts ? part : 0.f;
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) sum += v[u];
@@ -70,15 +71,13 @@ __global__ __launch_bounds__(HEAD_KS * 64) void head_gemm_kernel(
   // 32*grp + 8*q + (0..7) for block b and product q
   bf16x8 xn[KB][4];
   {
-    const bool live = col < M;
     const bf16_t* xrow = x + (int64_t)min(col, M - 1) * ldx;
 #pragma unroll
     for (int b = 0; b < KB; ++b)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int k = (kb0 + b) * 128 + grp * 32 + q * 8;
-        bf16x8 v = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (live) v = *reinterpret_cast<const bf16x8*>(xrow + k);
+        bf16x8 v = *reinterpret_cast<const bf16x8*>(xrow + k);  // rows past the last: the last again, not stored
         if constexpr (NORM) {
           const float4v w0 = *reinterpret_cast<const float4v*>(norm_w + k);
           const float4v w1 = *reinterpret_cast<const float4v*>(norm_w + k + 4);
@@ -117,8 +116,10 @@ __global__ __launch_bounds__(HEAD_KS * 64) void head_gemm_kernel(
 #pragma unroll
     for (int b = 0; b < KB; ++b) {
       // the block after this one: of this pair, or the first of the workgroup's next pair
+      // (past the last pair the last one's first block again: a load under a condition would leave
+      // the number of loads on their way unknown, and every block would be waited for at once)
       if (b + 1 < KB) load_block(wf[(b + 1) % 2], pair, b + 1);
-      else if (next_pair < pairs) load_block(wf[0], next_pair, 0);
+      else load_block(wf[0], min(next_pair, pairs - 1), 0);
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll

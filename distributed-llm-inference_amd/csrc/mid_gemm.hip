@@ -39,13 +39,23 @@ __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 raw) {
+  union {
+    u32x4 r;
+    bf16x8 v;
+  } u;
+  u.r = raw;
+  return u.v;
+}
+
 constexpr int XPAD = 8;                // elements: rows of the staged block start 16 bytes apart in the banks
 constexpr int XROW = 128 + XPAD;
 
 struct MidArgs {
   const bf16_t* x; int64_t ldx;
   const float* ssq_in; int ssq_parts; const float* norm_w; float eps;
-  const bf16_t* w; int tiled;
+  const bf16_t* w; int tiled; int w_rows;
   const bf16_t* bias; void* out; int64_t ldo;
   int M, N, K, up_offset, splits;
 };
@@ -88,33 +98,44 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   // 64 KB regions (and for the same activations) at the same time, which lands on few memory
   // channels. The order of a feature's sum thus depends on its tile, never on the rows.
   const int rot = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)cnt);
-  auto block_of = [&](int step) {
-    const int j = step * KW + kw;
-    if (j >= cnt) return b1;                   // beyond the range: nothing to do in this step
-    const int r = j + rot;
+  // whether this wave has a block in this step (the last step of an uneven split may have none)
+  auto live = [&](int step) { return step * KW + kw < cnt; };
+  auto block_of = [&](int step) {  // always a block of the range: where there is none, the last
+    const int r = min(step * KW + kw, cnt - 1) + rot;
     return b0 + (r >= cnt ? r - cnt : r);
   };
 
-  // this lane's first weight fragment and the steps to the next block and product
-  const bf16_t* wbase[NA];
-  const int blk_stride = p.tiled ? 2048 : 128, q_stride = p.tiled ? 512 : 8;
+  // Weights and activations are read through buffer resources that end with the matrix and with
+  // the last row: a load that is not wanted (a step without a block, a row that does not exist)
+  // is sent past the end, where it returns zeros and costs no memory traffic. So every step
+  // issues the same loads, the number of loads on their way is known at every wait, and a step
+  // waits for its own block only.
+  const unsigned w_bytes = (unsigned)((int64_t)p.w_rows * K * 2);
+  const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, w_bytes, 0x00020000);
+  const unsigned x_bytes = (unsigned)(((int64_t)(M - 1) * p.ldx + K) * 2);
+  const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, x_bytes, 0x00020000);
+  // this lane's first weight fragment (byte offset) and the steps to the next block and product
+  unsigned wbase[NA];
+  const int blk_stride = p.tiled ? 4096 : 256, q_stride = p.tiled ? 1024 : 16;
 #pragma unroll
   for (int a = 0; a < NA; ++a) {
     const int tl = min(tile, tiles - 1);
     if (p.tiled) {
-      wbase[a] = p.w + (int64_t)(tl + a * (p.up_offset / 16)) * 16 * K + lane * 8;
+      wbase[a] = (unsigned)(((int64_t)(tl + a * (p.up_offset / 16)) * 16 * K + lane * 8) * 2);
     } else {
       const int n = min(tl * 16 + col, N - 1) + a * p.up_offset;
-      wbase[a] = p.w + (int64_t)n * K + grp * 32;
+      wbase[a] = (unsigned)(((int64_t)n * K + grp * 32) * 2);
     }
   }
   bf16x8 wf[3][NA][4];
-  auto load_w = [&](bf16x8 (&dst)[NA][4], int b) __attribute__((always_inline)) {
+  auto load_w = [&](bf16x8 (&dst)[NA][4], int b, bool wanted) __attribute__((always_inline)) {
 #pragma unroll
     for (int a = 0; a < NA; ++a)
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        dst[a][q] = *reinterpret_cast<const bf16x8*>(wbase[a] + (int64_t)b * blk_stride + q * q_stride);
+      for (int q = 0; q < 4; ++q) {
+        const unsigned at = wanted ? wbase[a] + (unsigned)(b * blk_stride + q * q_stride) : w_bytes;
+        dst[a][q] = as_bf16x8(__builtin_amdgcn_raw_buffer_load_b128(wres, (int)at, 0, 0));
+      }
   };
   const bool norm = p.norm_w != nullptr;
 
@@ -132,16 +153,16 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
     bf16x8 v[PP];
     float4v nw0, nw1;
   };
-  auto fetch_x = [&](Staged& st, int b) __attribute__((always_inline)) {
+  const float* nw_at = norm ? p.norm_w : reinterpret_cast<const float*>(p.w);  // always readable
+  auto fetch_x = [&](Staged& st, int b, bool wanted) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < PP; ++i) {
-      st.v[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (prow[i] < M) st.v[i] = *reinterpret_cast<const bf16x8*>(p.x + (int64_t)prow[i] * p.ldx + b * 128 + pk[i]);
+      const unsigned at = wanted && prow[i] < M ? (unsigned)(((int64_t)prow[i] * p.ldx + b * 128 + pk[i]) * 2) : x_bytes;
+      st.v[i] = as_bf16x8(__builtin_amdgcn_raw_buffer_load_b128(xres, (int)at, 0, 0));
     }
-    if (norm) {
-      st.nw0 = *reinterpret_cast<const float4v*>(p.norm_w + b * 128 + pk[0]);
-      st.nw1 = *reinterpret_cast<const float4v*>(p.norm_w + b * 128 + pk[0] + 4);
-    }
+    // (without a norm the same two loads, of anything: no load hangs on a condition)
+    st.nw0 = *reinterpret_cast<const float4v*>(nw_at + b * 128 + pk[0]);
+    st.nw1 = *reinterpret_cast<const float4v*>(nw_at + b * 128 + pk[0] + 4);
   };
   auto stash_x = [&](const Staged& st, int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -171,14 +192,10 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   // A wave whose block lies beyond the range (the last step of an uneven split) stages and
   // multiplies nothing but keeps every barrier.
   Staged sx[2];
-  if (block_of(0) < b1) {
-    fetch_x(sx[0], block_of(0));
-    load_w(wf[0], block_of(0));
-  }
-  if (block_of(1) < b1) {
-    fetch_x(sx[1], block_of(1));
-    load_w(wf[1], block_of(1));
-  }
+  fetch_x(sx[0], block_of(0), live(0));
+  load_w(wf[0], block_of(0), live(0));
+  fetch_x(sx[1], block_of(1), live(1));
+  load_w(wf[1], block_of(1), live(1));
   // rs[m] from the parts of sum x^2, added in the order of the parts
   if (norm) {
     for (int m = threadIdx.x; m < ROWS; m += NW * KW * 64) {
@@ -189,7 +206,7 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
     }
     __syncthreads();
   }
-  if (block_of(0) < b1) stash_x(sx[0], 0);
+  if (live(0)) stash_x(sx[0], 0);
   __syncthreads();
   for (int s0 = 0; s0 < steps; s0 += 6) {
 #pragma unroll
@@ -197,11 +214,9 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
       const int step = s0 + r;
       if (step >= steps) break;
       const int buf = r & 1;
-      if (block_of(step + 2) < b1) {
-        fetch_x(sx[r & 1], block_of(step + 2));   // the slot of this step's block, which lies in LDS by now
-        load_w(wf[(r + 2) % 3], block_of(step + 2));
-      }
-      if (block_of(step) < b1) {
+      fetch_x(sx[r & 1], block_of(step + 2), live(step + 2));   // the slot of this step's block, which lies in LDS by now
+      load_w(wf[(r + 2) % 3], block_of(step + 2), live(step + 2));
+      if (live(step)) {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -211,7 +226,7 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
             for (int a = 0; a < NA; ++a) acc[a][t] = mfma32(wf[r % 3][a][q], xf, acc[a][t]);
           }
       }
-      if (block_of(step + 1) < b1) stash_x(sx[(r + 1) & 1], buf ^ 1);
+      if (live(step + 1)) stash_x(sx[(r + 1) & 1], buf ^ 1);
       __syncthreads();
     }
   }
@@ -508,7 +523,11 @@ extern "C" int dli_mid_gemm(const void* x, int64_t ldx, const float* ssq_in, int
       (tiled && (N % 16 != 0 || up_offset % 16 != 0)) || (epilogue == MID_SWIGLU && up_offset <= 0) ||
       (epilogue == MID_PARTIAL && N % 4 != 0))
     return DLI_ERR_ARGUMENT;
-  const MidArgs a{(const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, tiled,
+  // the kernel addresses the matrix and the rows with 32-bit byte offsets
+  const int64_t w_rows = epilogue == MID_SWIGLU ? (int64_t)up_offset + N : N;
+  if (w_rows * K * 2 >= ((int64_t)1 << 32) - 4096 || ((int64_t)(M - 1) * ldx + K) * 2 >= ((int64_t)1 << 31))
+    return DLI_ERR_ARGUMENT;
+  const MidArgs a{(const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, tiled, (int)w_rows,
                   (const bf16_t*)bias, out, ldo, M, N, K, up_offset, splits};
   if (epilogue == MID_PARTIAL) return launch_mid_rows<MID_PARTIAL>(waves, kwaves, a, stream);
   if (epilogue == MID_SWIGLU) return launch_mid_rows<MID_SWIGLU>(waves, kwaves, a, stream);
