@@ -332,16 +332,22 @@ def skinny_gemm_supports(rows: int, k: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and 0 < rows <= 64 and k > 0 and k % 32 == 0
 
 
-def skinny_gemm_shape(n: int, k: int, tiled: bool = False) -> int:
+def skinny_gemm_shape(n: int, k: int, tiled: bool = False, units: int = 256) -> int:
     """Workgroup shape for ``n`` output features of depth ``k``: with few tiles of 16 features the
-    waves of a workgroup split k (8 ways when k is long, or when there are fewer tiles than
-    compute units and the weights are tiled), with many they split the tiles so that the
-    activations are read once per 8 tiles. From cold-cache timings on MI355X."""
+    waves of a workgroup split k, with many they split the tiles so that the activations are read
+    once per 8 tiles. From cold-cache timings on MI355X (``units`` compute units); with tiled
+    weights at the 1B, 1.7B and 3B sizes: four k-waves on one tile each where the tiles are no
+    more than the compute units or fill them evenly with short rows (6.5 us against 6.8 and 7.4
+    for q/k/v at the 1B sizes, 16.2 against 16.8 for gate and up), else on two tiles each, which
+    halves the workgroups and with them the uneven last round (11.5 us against 13.9 for q/k/v
+    at the 3B sizes, 8.6 against 10.1 at the 1.7B sizes)."""
     tiles = -(-n // 16)
-    if tiled:          # fewer tiles than compute units: 8 k-waves; else 4 k-waves on two tiles each
+    if tiled:
         if tiles >= 2048 and k >= 3072:
             return 2   # a vocabulary with long rows: no split of k
-        return 1 if tiles <= 256 else 4
+        if tiles <= units or (tiles % units == 0 and k <= 2048):
+            return 0
+        return 4
     if tiles >= 768:   # a vocabulary
         return 3
     return 1 if k >= 4096 else 0
@@ -394,26 +400,25 @@ def skinny_gemm_plan(rows: int, n: int, k: int, epilogue: int, device: torch.dev
     activations that exist, which wins for one to four rows; with more rows the activations'
     traffic grows and the tile kernel, which reads them once per 16 features, is ahead.
     ``tiled``: a copy of the weights in tile order is at hand (at most 16 rows); the tile kernel
-    then reads whole lines too and takes over from three rows on, and below that where the
+    then reads whole lines too and takes over from two rows on, and below that where the
     product has few features.
     """
     if blocks4 is None and rows <= 16 and k % 8 == 0:
         # long rows and so few features that tiles of 16 would leave half the compute units idle
         # (2048 at the 1B sizes; not 3072 at the 3B sizes, where the tile kernel is ahead from 4 rows on)
         deep = k >= 4096 and -(-n // 16) * 2 <= _units(device)
-        if rows <= 4:
+        if deep:
+            blocks4 = 1   # (the shape of 16 k-waves was ahead for one to four rows until the loads of
+            #               a wave's chunks overlapped: now 9.8 against 10.8 us for down at the 1B sizes)
+        elif rows <= 4:
             out_feats = n * (2 if epilogue == SKINNY_SWIGLU else 1)
             few = out_feats <= 16 * _units(device)
-            if deep:
-                blocks4 = 2
-            elif not (tiled and (rows >= 3 or few)):
+            if not (tiled and (rows >= 2 or few)):
                 blocks4 = 1 if few else 0
-        elif deep:
-            blocks4 = 1
     if blocks4 is not None:
         feats = int(library().dli_skinny4_tile_features(blocks4, epilogue))
         return "blocks4", blocks4, -(-n // feats)
-    return "tiles16", skinny_gemm_shape(n, k, tiled and rows <= 16), -(-n // 16)
+    return "tiles16", skinny_gemm_shape(n, k, tiled and rows <= 16, _units(device)), -(-n // 16)
 
 
 def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optional[torch.Tensor] = None,
@@ -545,8 +550,19 @@ def skinny_gemm_merged_supports(rows: int, n: int, heads: int, head_dim: int, sp
     if not (0 < rows <= MERGED_ROWS and 2 <= splits <= MERGED_SPLITS and head_dim % 4 == 0 and k % 128 == 0
             and n % 16 == 0):
         return False
+    return _merged_shape(rows, n, k, device) is not None
+
+
+def _merged_shape(rows: int, n: int, k: int, device: torch.device) -> Optional[int]:
+    """The workgroup shape (0: four k-waves, 1: eight) with which the merging o projection runs:
+    the plan's own where a wave's run of k fits the merge's buffer, else eight k-waves if that does."""
     kernel, shape, _ = skinny_gemm_plan(rows, n, k, SKINNY_RESIDUAL, device, tiled=True)
-    return kernel == "tiles16" and shape in (0, 1) and -(-(k // 128) // (4 if shape == 0 else 8)) * 128 <= _MERGED_RANGE
+    if kernel != "tiles16" or shape not in (0, 1):
+        return None
+    for candidate in (shape, 1):
+        if -(-(k // 128) // (4 if candidate == 0 else 8)) * 128 <= _MERGED_RANGE:
+            return candidate
+    return None
 
 
 def skinny_gemm_merged(part_o: torch.Tensor, part_ml: torch.Tensor, splits: int, heads: int, head_dim: int,
@@ -573,7 +589,8 @@ def skinny_gemm_merged(part_o: torch.Tensor, part_ml: torch.Tensor, splits: int,
     if bias is not None:
         _dense(bias, "bias", torch.bfloat16, 1)
         _require(bias.shape[0] == n, "bias length differs from rows of w")
-    _, shape, n_parts = skinny_gemm_plan(m, n, k, SKINNY_RESIDUAL, stream.device, tiled=True)
+    _, _, n_parts = skinny_gemm_plan(m, n, k, SKINNY_RESIDUAL, stream.device, tiled=True)
+    shape = _merged_shape(m, n, k, stream.device)
     if ssq_out is None:
         ssq_out = torch.empty(n_parts, m, device=stream.device, dtype=torch.float32)
     _dense(ssq_out, "ssq_out", torch.float32, 2)
@@ -885,7 +902,7 @@ def skinny_gemm_qkv_rope(x: torch.Tensor, w_tiled: torch.Tensor, q_out: torch.Te
         _require(ssq_in.shape[1] == m and ssq_in.shape[0] >= 1, "ssq_in must be [parts, rows]")
         parts = ssq_in.shape[0]
     if shape is None:
-        shape = skinny_gemm_shape(n, k, tiled=True)
+        shape = skinny_gemm_shape(n, k, tiled=True, units=_units(x.device))
     _require(shape in (0, 1, 2, 3, 4), "shape must be 0..4")
     _check(library().dli_skinny_gemm_qkv_rope(
         _ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w_tiled), _ptr(bias), _ptr(q_out),
