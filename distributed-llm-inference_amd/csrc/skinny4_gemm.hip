@@ -129,7 +129,7 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
   // last chunk's weights again and zeros for x), so the number of loads in flight is known at
   // compile time and only the current chunk is waited for.
   auto fetch = [&](int c, Stage& st) __attribute__((always_inline)) {
-    const int k = min(c, c1 - 1) * 128 + blk * 8;
+    const int k = max(min(c, c1 - 1), 0) * 128 + blk * 8;  // (a wave without chunks reads the first one, for nothing)
     const bool inside = k < K && c < c1;  // the last chunk may reach past k; K % 8 == 0
     const int kc = k < K ? k : 0;
 #pragma unroll
@@ -153,7 +153,40 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) fetch(c0 + d, st[d]);
   };
-  if (XL && c0 < c1) fetch_first();  // the first weights are on their way while x is staged
+  // What the prologue needs is asked for before anything is waited for, in the order of its use:
+  // the first parts of the rows' sums of squares, the first pieces of x that a thread stages (XL),
+  // the first chunks of weights. No load hangs on a condition (a part past the last reads the
+  // last and counts as zero, a piece past the end its row's first), so that the sums wait for the
+  // parts alone and the staging for the pieces alone, the weights on their way meanwhile.
+  constexpr int WG = KS * 64;
+  const int per_row = chunks * 16;          // XL: 16-byte pieces of a staged row
+  const int pieces = XL ? M * per_row : 0;  // thread t stages pieces t, t + WG, ...
+  float first[NORM ? MG : 1][8];
+  if constexpr (NORM) {
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+      const int m = min(4 * g + r, M - 1);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int p = ks * 16 + blk + u * 16 * KS;
+        const float part = ssq_in[(int64_t)min(p, ssq_parts - 1) * M + m];
+        first[g][u] = p < ssq_parts ? part : 0.f;
+      }
+    }
+  }
+  Frag16 piece;
+  float4v piece_g0, piece_g1;
+  if constexpr (XL) {
+    const int idx = min((int)threadIdx.x, pieces - 1);
+    const int m = idx / per_row, k = (idx - m * per_row) * 8, kc = k < K ? k : 0;
+    piece.raw = *reinterpret_cast<const u32x4*>(x + (int64_t)m * ldx + kc);
+    if constexpr (NORM) {
+      piece_g0 = *reinterpret_cast<const float4v*>(norm_w + kc);
+      piece_g1 = *reinterpret_cast<const float4v*>(norm_w + kc + 4);
+    }
+  }
+  fetch_first();
+  __builtin_amdgcn_sched_barrier(0);
   if constexpr (NORM) {
     // rs[m] from the parts of sum x^2. The parts are dealt out to all blocks of all waves (block
     // q of 16*KS takes the parts q, q + 16*KS, ...), eight loads at a time so that they share one
@@ -164,7 +197,9 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     for (int g = 0; g < MG; ++g) {
       const int m = min(4 * g + r, M - 1);
       float sum = 0.f;
-      for (int p0 = ks * 16 + blk; p0 < ssq_parts; p0 += 128 * KS) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sum += first[g][u];
+      for (int p0 = ks * 16 + blk + 128 * KS; p0 < ssq_parts; p0 += 128 * KS) {
         float v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -190,7 +225,6 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     }
   }
 
-  if (!XL && c0 < c1) fetch_first();
   if constexpr (XL) {
     // thread t stages the 8 values at k = 8*(t % (chunks*16)) of row t / (chunks*16), and so on
     __shared__ float rs_row[4 * MG];
@@ -201,16 +235,10 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
       }
       __syncthreads();
     }
-    const int per_row = chunks * 16;
-    for (int idx = threadIdx.x; idx < M * per_row; idx += KS * 64) {
+    auto stage = [&](int idx, Frag16 v, float4v g0, float4v g1) __attribute__((always_inline)) {
       const int m = idx / per_row, k = (idx - m * per_row) * 8;
-      Frag16 v;
-      v.raw = u32x4{0, 0, 0, 0};
       if (k < K) {
-        v.raw = *reinterpret_cast<const u32x4*>(x + (int64_t)m * ldx + k);
         if constexpr (NORM) {
-          const float4v g0 = *reinterpret_cast<const float4v*>(norm_w + k);
-          const float4v g1 = *reinterpret_cast<const float4v*>(norm_w + k + 4);
           const float rsm = rs_row[m];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
@@ -218,8 +246,22 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
             v.e[i] = (bf16_t)((i < 4 ? g0[i] : g1[i - 4]) * normed);
           }
         }
+      } else {
+        v.raw = u32x4{0, 0, 0, 0};
       }
       *reinterpret_cast<u32x4*>(xs + (int64_t)m * xpad + k) = v.raw;
+    };
+    if ((int)threadIdx.x < pieces) stage(threadIdx.x, piece, piece_g0, piece_g1);
+    for (int idx = threadIdx.x + WG; idx < pieces; idx += WG) {
+      const int m = idx / per_row, k = (idx - m * per_row) * 8, kc = k < K ? k : 0;
+      Frag16 v;
+      float4v g0 = {0.f, 0.f, 0.f, 0.f}, g1 = g0;
+      v.raw = *reinterpret_cast<const u32x4*>(x + (int64_t)m * ldx + kc);
+      if constexpr (NORM) {
+        g0 = *reinterpret_cast<const float4v*>(norm_w + kc);
+        g1 = *reinterpret_cast<const float4v*>(norm_w + kc + 4);
+      }
+      stage(idx, v, g0, g1);
     }
     __syncthreads();
   }

@@ -418,7 +418,14 @@ def skinny_gemm_plan(rows: int, n: int, k: int, epilogue: int, device: torch.dev
     if blocks4 is not None:
         feats = int(library().dli_skinny4_tile_features(blocks4, epilogue))
         return "blocks4", blocks4, -(-n // feats)
-    return "tiles16", skinny_gemm_shape(n, k, tiled and rows <= 16, _units(device)), -(-n // 16)
+    shape = skinny_gemm_shape(n, k, tiled and rows <= 16, _units(device))
+    if tiled and rows <= MERGED_ROWS and shape == 0 and -(-n // 16) <= _units(device):
+        # Few tiles and very few rows: eight k-waves are as fast as four (4.3 against 4.4 us for o at
+        # the 1B sizes), and the o projection that merges the attention's runs of keys itself, whose
+        # waves each merge the k they multiply, is faster with them; it has to add in the same order
+        # as this one to give the same bits.
+        shape = 1
+    return "tiles16", shape, -(-n // 16)
 
 
 def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optional[torch.Tensor] = None,
@@ -554,17 +561,13 @@ def skinny_gemm_merged_supports(rows: int, n: int, heads: int, head_dim: int, sp
 
 
 def _merged_shape(rows: int, n: int, k: int, device: torch.device) -> Optional[int]:
-    """The workgroup shape (0: four k-waves, 1: eight) with which the merging o projection runs, or
-    None if the plan has the product on another kernel: eight k-waves where a wave's run of k then
-    fits the merge's buffer (each wave merges half as much as with four: 7.3 against 7.9 us at the
-    1B sizes), else four."""
+    """The workgroup shape (0: four k-waves, 1: eight) with which the merging o projection runs:
+    that of the plain product with the residual sum, so that both add in the same order, or None
+    if that one runs on another kernel or a wave's run of k does not fit the merge's buffer."""
     kernel, shape, _ = skinny_gemm_plan(rows, n, k, SKINNY_RESIDUAL, device, tiled=True)
     if kernel != "tiles16" or shape not in (0, 1):
         return None
-    for candidate in (1, 0):
-        if -(-(k // 128) // (4 if candidate == 0 else 8)) * 128 <= _MERGED_RANGE:
-            return candidate
-    return None
+    return shape if -(-(k // 128) // (4 if shape == 0 else 8)) * 128 <= _MERGED_RANGE else None
 
 
 def skinny_gemm_merged(part_o: torch.Tensor, part_ml: torch.Tensor, splits: int, heads: int, head_dim: int,
