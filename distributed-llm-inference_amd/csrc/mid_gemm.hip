@@ -295,20 +295,37 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   }
 }
 
-// The splits' values of four neighbouring features, added in the order of the splits; the loads
-// are issued eight at a time so that they share one trip to memory.
-__device__ __forceinline__ float4v sum_splits(const float* __restrict__ src, int splits, int64_t split_stride) {
-  float4v y = float4v{0.f, 0.f, 0.f, 0.f};
-  for (int s0 = 0; s0 < splits; s0 += 8) {
+// The splits' values of four neighbouring features, added in the order of the splits. The first
+// eight are asked for together and without conditions (a split past the last reads the last and
+// is not added), apart from their sum, so that a kernel can ask for everything it needs before it
+// waits for anything; further splits follow eight at a time.
+struct Splits8 {
+  float4v v[8];
+};
+__device__ __forceinline__ Splits8 load_splits(const float* __restrict__ src, int splits, int64_t split_stride) {
+  Splits8 s;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) s.v[u] = *reinterpret_cast<const float4v*>(src + min(u, splits - 1) * split_stride);
+  return s;
+}
+__device__ __forceinline__ float4v sum_splits(const Splits8& first, const float* __restrict__ src, int splits,
+                                              int64_t split_stride) {
+  float4v y = first.v[0];
+#pragma unroll
+  for (int u = 1; u < 8; ++u)
+    if (u < splits) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = y[i] + first.v[u][i];
+    }
+  for (int s0 = 8; s0 < splits; s0 += 8) {
     float4v v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
-      v[u] = s0 + u < splits ? *reinterpret_cast<const float4v*>(src + (s0 + u) * split_stride) : float4v{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4v*>(src + min(s0 + u, splits - 1) * split_stride);
 #pragma unroll
     for (int u = 0; u < 8; ++u)
       if (s0 + u < splits) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) y[i] = s0 + u == 0 ? v[u][i] : y[i] + v[u][i];
+        for (int i = 0; i < 4; ++i) y[i] = y[i] + v[u][i];
       }
   }
   return y;
@@ -325,10 +342,13 @@ __global__ __launch_bounds__(256) void mid_finish_residual_kernel(
   const int64_t split_stride = (int64_t)M * N;
   const int n = part * 1024 + threadIdx.x * 4;
   float sq = 0.f;
+  // (a thread past the row's end reads the row's last four features, for nothing)
+  const int nc = min(n, N - 4);
+  const bf16x4 old = *reinterpret_cast<const bf16x4*>(stream + (int64_t)m * lds_ + nc);
+  const Splits8 first = load_splits(partial + (int64_t)m * N + nc, splits, split_stride);
   if (n < N) {
     bf16_t* sp = stream + (int64_t)m * lds_ + n;
-    const bf16x4 old = *reinterpret_cast<const bf16x4*>(sp);
-    const float4v y = sum_splits(partial + (int64_t)m * N + n, splits, split_stride);
+    const float4v y = sum_splits(first, partial + (int64_t)m * N + n, splits, split_stride);
     bf16x4 res;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -363,12 +383,10 @@ __global__ __launch_bounds__(256) void mid_finish_residual_normed_kernel(
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int n = (j * 256 + threadIdx.x) * 4;
-    old[j] = bf16x4{0, 0, 0, 0};
-    nw[j] = y[j] = float4v{0.f, 0.f, 0.f, 0.f};
-    if (n < N) {
-      old[j] = *reinterpret_cast<const bf16x4*>(stream + (int64_t)m * lds_ + n);
-      nw[j] = *reinterpret_cast<const float4v*>(norm_w + n);
-    }
+    const int nc = min(n, N - 4);  // past the row's end: its last four features, for nothing
+    y[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    old[j] = *reinterpret_cast<const bf16x4*>(stream + (int64_t)m * lds_ + nc);
+    nw[j] = *reinterpret_cast<const float4v*>(norm_w + nc);
   }
   for (int s0 = 0; s0 < splits; s0 += CH) {
     float4v v[PER][CH];
@@ -376,10 +394,9 @@ __global__ __launch_bounds__(256) void mid_finish_residual_normed_kernel(
     for (int j = 0; j < PER; ++j) {
       const int n = (j * 256 + threadIdx.x) * 4;
 #pragma unroll
-      for (int u = 0; u < CH; ++u)
-        v[j][u] = n < N && s0 + u < splits
-                      ? *reinterpret_cast<const float4v*>(partial + (s0 + u) * split_stride + (int64_t)m * N + n)
-                      : float4v{0.f, 0.f, 0.f, 0.f};
+      for (int u = 0; u < CH; ++u)  // no load under a condition: a split past the last reads the last
+        v[j][u] = *reinterpret_cast<const float4v*>(partial + min(s0 + u, splits - 1) * split_stride +
+                                                    (int64_t)m * N + min(n, N - 4));
     }
 #pragma unroll
     for (int j = 0; j < PER; ++j)
@@ -438,8 +455,8 @@ __global__ __launch_bounds__(256) void mid_finish_qkv_kernel(
   const int slot = slots[m];
   const int64_t page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot - (int)page * page_size : 0;
-  auto summed = [&](int n) __attribute__((always_inline)) {
-    float4v y = sum_splits(partial + (int64_t)m * N + n, splits, split_stride);
+  auto summed = [&](const Splits8& first, int n) __attribute__((always_inline)) {
+    float4v y = sum_splits(first, partial + (int64_t)m * N + n, splits, split_stride);
 #pragma unroll
     for (int i = 0; i < 4; ++i) y[i] = (float)(bf16_t)(y[i] + (bias != nullptr ? (float)bias[n + i] : 0.f));
     return y;
@@ -448,9 +465,13 @@ __global__ __launch_bounds__(256) void mid_finish_qkv_kernel(
     if (item < rot_items) {
       const int head = item / (half / 4), j = (item % (half / 4)) * 4;   // pairs j..j+3 of the head
       const int pos = head * d + 16 * (j / 8) + j % 8;                   // where pair j's first member lies
-      const float4v a = summed(pos), b = summed(pos + 8);
+      // both members' splits and the angles are asked for before any of them is used
+      const Splits8 fa = load_splits(partial + (int64_t)m * N + pos, splits, split_stride);
+      const Splits8 fb = load_splits(partial + (int64_t)m * N + pos + 8, splits, split_stride);
       const float4v cs = *reinterpret_cast<const float4v*>(angles + ((int64_t)m * 2 + 0) * half + j);
       const float4v sn = *reinterpret_cast<const float4v*>(angles + ((int64_t)m * 2 + 1) * half + j);
+      __builtin_amdgcn_sched_barrier(0);
+      const float4v a = summed(fa, pos), b = summed(fb, pos + 8);
       bf16x4 lo, hi;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -466,7 +487,8 @@ __global__ __launch_bounds__(256) void mid_finish_qkv_kernel(
       }
     } else if (slot >= 0) {
       const int vi = item - rot_items, hv = vi / (d / 4), dim = (vi % (d / 4)) * 4;
-      const float4v v = summed((q_heads + kv_heads + hv) * d + dim);
+      const int pos = (q_heads + kv_heads + hv) * d + dim;
+      const float4v v = summed(load_splits(partial + (int64_t)m * N + pos, splits, split_stride), pos);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         v_pages[((page * kv_heads + hv) * d + dim + i) * page_size + off] = (bf16_t)v[i];
