@@ -28,3 +28,26 @@ def test_runs_shrink_as_the_batch_grows():
     got = [choose_splits(requests=b, kv_head_tiles=8, max_keys=4096) for b in (1, 2, 4, 8, 16, 32, 64)]
     assert got == sorted(got, reverse=True) and got[0] > got[-1] == 1
     assert all(1 <= s <= MAX_SPLITS for s in got)
+
+
+def test_rows_of_a_decode_graph():
+    """Powers of two up to 32 rows, then multiples of 16: a product's cost grows with its row tiles."""
+    from dli_amd.engine.decode_graph import _batch_bucket
+
+    assert [_batch_bucket(n) for n in (1, 2, 3, 5, 9, 16, 17, 32)] == [1, 2, 4, 8, 16, 16, 32, 32]
+    assert [_batch_bucket(n) for n in (33, 40, 48, 49, 64, 65)] == [48, 48, 48, 64, 64, 80]
+
+
+def test_workgroup_shape_of_the_tile_kernel_from_sizes():
+    """The rule read off timings at the 1B, 1.7B and 3B sizes (256 compute units): four k-waves on
+    one tile where tiles are few or fill the units evenly with short rows, else on two tiles; a
+    vocabulary with long rows does not split k."""
+    from dli_amd.kernels.ops import skinny_gemm_shape
+
+    tiled = lambda n, k: skinny_gemm_shape(n, k, tiled=True, units=256)
+    assert tiled(2048, 2048) == 0 and tiled(3072, 2048) == 0       # o and q/k/v at the 1B sizes
+    assert tiled(8192, 2048) == 0                                   # gate and up at the 1B sizes: 512 tiles
+    assert tiled(5120, 3072) == 4 and tiled(8192, 3072) == 4       # q/k/v and gate/up at the 3B sizes
+    assert tiled(6144, 2048) == 4                                   # q/k/v at the 1.7B sizes: 384 tiles
+    assert tiled(128256, 3072) == 2 and tiled(128256, 2048) == 4   # vocabularies
+    assert skinny_gemm_shape(2048, 8192) == 1 and skinny_gemm_shape(2048, 2048) == 0 and skinny_gemm_shape(128256, 2048) == 3
