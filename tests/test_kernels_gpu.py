@@ -500,7 +500,7 @@ def test_skinny_gemm_epilogues(ops, m, n, k, shape):
 
 @pytest.mark.parametrize("m", [1, 8, 33])
 @pytest.mark.parametrize("shape", [0, 2, 3])
-@pytest.mark.parametrize("inter,k,parts", [(160, 64, 1), (512, 192, 5), (8192, 2048, 128)])
+@pytest.mark.parametrize("inter,k,parts", [(160, 64, 1), (512, 192, 5), (8192, 2048, 128), (160, 128, 600)])
 def test_skinny_gemm_norm_and_swiglu(ops, m, inter, k, shape, parts):
     torch.manual_seed(m + inter)
     x = (torch.randn(m, k, device="cuda") * 2).bfloat16()
@@ -674,7 +674,7 @@ def test_skinny4_gemm_epilogues(ops, m, n, k, blocks4):
 
 @pytest.mark.parametrize("m", [1, 8, 13])
 @pytest.mark.parametrize("blocks4", [0, 1, 2])
-@pytest.mark.parametrize("inter,k,parts", [(160, 64, 1), (500, 192, 5), (8192, 2048, 128)])
+@pytest.mark.parametrize("inter,k,parts", [(160, 64, 1), (500, 192, 5), (8192, 2048, 128), (160, 128, 2100)])
 def test_skinny4_gemm_norm_and_swiglu(ops, m, inter, k, parts, blocks4):
     torch.manual_seed(m + inter)
     x = (torch.randn(m, k, device="cuda") * 2).bfloat16()
