@@ -352,15 +352,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   // cache under the workgroups that still stream keys: 40 us instead of 16 for the launch.)
   if (valid) {
     const int64_t slot = ((int64_t)e * q_heads + head) * splits + split;
-    float* po = part_o + slot * D + 4 * grp;
+    const __amdgpu_buffer_rsrc_t po = device_scope_buffer(part_o);
 #pragma unroll
-    for (int c = 0; c < DCH; ++c)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) device_store(po + c * 16 + i, st.o[c][i]);
-    if (grp == 0) {
-      device_store(part_ml + slot * 2, m_all);
-      device_store(part_ml + slot * 2 + 1, l_all);
-    }
+    for (int c = 0; c < DCH; ++c) device_store4(po, (unsigned)((slot * D + 4 * grp + c * 16) * 4), st.o[c]);
+    if (grp == 0) device_store2(device_scope_buffer(part_ml), (unsigned)(slot * 2 * 4), merge_float2{m_all, l_all});
   }
   // every store of this wave has been acknowledged before the count goes up ...
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");

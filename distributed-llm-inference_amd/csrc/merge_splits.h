@@ -12,18 +12,54 @@
 typedef float merge_float2 __attribute__((ext_vector_type(2)));
 typedef float merge_float4 __attribute__((ext_vector_type(4)));
 
-// A float that another workgroup of the same launch may have stored (with device_store): read at
-// the device's scope, past the caches that are private to a part of the chip.
-__device__ __forceinline__ float device_load(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// What one workgroup of a launch hands to another goes through memory at the device's scope, past
+// the caches that are private to a part of the chip: buffer loads and stores with the sc1 bit
+// (bit 4 of the builtins' cache policy on gfx940 and later), 8 or 16 bytes a lane. The resource
+// spans the whole address range behind the pointer (offsets are 32-bit byte offsets).
+typedef unsigned merge_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned merge_u32x2 __attribute__((ext_vector_type(2)));
+constexpr int DEVICE_SCOPE = 1 << 4;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t device_scope_buffer(const void* p) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, 0xffffffffu, 0x00020000);
 }
-__device__ __forceinline__ void device_store(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ merge_float4 device_load4(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
+  union {
+    merge_u32x4 raw;
+    merge_float4 f;
+  } u;
+  u.raw = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_offset, 0, DEVICE_SCOPE);
+  return u.f;
+}
+__device__ __forceinline__ merge_float2 device_load2(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {
+  union {
+    merge_u32x2 raw;
+    merge_float2 f;
+  } u;
+  u.raw = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_offset, 0, DEVICE_SCOPE);
+  return u.f;
+}
+__device__ __forceinline__ void device_store4(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, merge_float4 v) {
+  union {
+    merge_u32x4 raw;
+    merge_float4 f;
+  } u;
+  u.f = v;
+  __builtin_amdgcn_raw_buffer_store_b128(u.raw, r, (int)byte_offset, 0, DEVICE_SCOPE);
+}
+__device__ __forceinline__ void device_store2(__amdgpu_buffer_rsrc_t r, unsigned byte_offset, merge_float2 v) {
+  union {
+    merge_u32x2 raw;
+    merge_float2 f;
+  } u;
+  u.f = v;
+  __builtin_amdgcn_raw_buffer_store_b64(u.raw, r, (int)byte_offset, 0, DEVICE_SCOPE);
 }
 
 // part_o [.. slots][head_dim], part_ml [.. slots][2]; `base`: the first of the S slots of this
 // (request, head); d: the first of the four dims. All loads are asked for before the first is used.
-// SAME_LAUNCH: the partial results were stored by other workgroups of this launch.
+// SAME_LAUNCH: the partial results were stored by other workgroups of this launch (each array
+// under 4 GB).
 template <bool SAME_LAUNCH = false>
 __device__ __forceinline__ merge_float4 merged_quad(const float* part_o, const float* part_ml, int64_t base, int S,
                                                     int head_dim, int d) {
@@ -37,8 +73,8 @@ __device__ __forceinline__ merge_float4 merged_quad(const float* part_o, const f
       const float* ml_at = part_ml + (base + j) * 2;
       const float* po_at = part_o + (base + j) * head_dim + d;
       if constexpr (SAME_LAUNCH) {
-        ml[j] = merge_float2{device_load(ml_at), device_load(ml_at + 1)};
-        po[j] = merge_float4{device_load(po_at), device_load(po_at + 1), device_load(po_at + 2), device_load(po_at + 3)};
+        ml[j] = device_load2(device_scope_buffer(part_ml), (unsigned)((base + j) * 2 * 4));
+        po[j] = device_load4(device_scope_buffer(part_o), (unsigned)(((base + j) * head_dim + d) * 4));
       } else {
         ml[j] = *reinterpret_cast<const merge_float2*>(ml_at);
         po[j] = *reinterpret_cast<const merge_float4*>(po_at);
