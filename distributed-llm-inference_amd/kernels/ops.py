@@ -521,7 +521,7 @@ def head_gemm(x: torch.Tensor, w_tiled: torch.Tensor, out: torch.Tensor, norm_w:
     workgroups that stay for the whole launch walk the tiles of ``w_tiled`` (:func:`tile_weights`
     of ``w [n, k]``) in turn, each wave keeping its normalised activations in registers. ``norm_w``,
     ``eps``, ``ssq_in [parts, rows]``: the RMSNorm of ``x`` as in :func:`skinny_gemm`. The sums are
-    those of :func:`skinny_gemm` with ``shape=4``, to the bit. ``workgroups``: how many (0: two per
+    those of :func:`skinny_gemm` with ``shape=4``, to the bit. ``workgroups``: how many (0: one per
     compute unit)."""
     _rows(x, "x", torch.bfloat16)
     m, k = x.shape
