@@ -36,9 +36,9 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--decode-weight-copy", action=argparse.BooleanOptionalAction, default=True,
                    help="keep a second copy of the bfloat16 matrices in the decode kernels' order "
                         "(faster decode steps, twice the weight memory)")
-    p.add_argument("--decode-steps", type=int, default=1,
+    p.add_argument("--decode-steps", type=int, default=8,
                    help="tokens of every request that one decoding step runs on the device before the host "
-                        "looks (same tokens, fewer round trips; needs --cuda-graphs)")
+                        "looks (same tokens, fewer round trips; one without --cuda-graphs or in float32)")
 
 
 def _read_prompts(args: argparse.Namespace) -> list[list[int]]:

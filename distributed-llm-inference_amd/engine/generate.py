@@ -36,11 +36,13 @@ def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
              dtype: str = "bfloat16", num_blocks: Optional[int] = None, kv_cache_gb: Optional[float] = None,
              block_size: int = 16, max_num_seqs: int = 64, max_num_batched_tokens: int = 512,
              enable_prefix_caching: bool = True, eos_token_ids: Collection[int] = (), seed: int = 0,
-             cuda_graphs: bool = True, device: str = "cuda", decode_steps: int = 1,
+             cuda_graphs: bool = True, device: str = "cuda", decode_steps: int = 8,
              decode_weight_copy: bool = True) -> list[list[int]]:
     """Load ``model`` (a folder or a loaded model), run ``prompts`` to completion, return token ids.
-    ``decode_steps`` > 1: decoding steps run that many tokens of every request on the device
-    before the host looks (same tokens, fewer round trips)."""
+    ``decode_steps``: decoding steps run up to that many tokens of every request on the device
+    before the host looks (same tokens, fewer round trips: nobody watches tokens arrive here, so
+    the default is eight where an engine's own is one; 7.5 k against 6.8 k tokens/s at batch 8 and
+    the 1B sizes). Without decode graphs (32-bit, ``cuda_graphs=False``) a step is one token."""
     engine = LLMEngine.for_model(
         model, num_blocks=num_blocks, kv_cache_gb=kv_cache_gb, block_size=block_size, dtype=dtype,
         config=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=max_num_batched_tokens,
