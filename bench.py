@@ -232,7 +232,7 @@ def main() -> int:
                          "step. mixed: 64 requests, prompts of 128 to 2,048 tokens, 256 generated tokens each; "
                          "shared-prefix: 32 requests that share 1,024 tokens and add 64 to 512 of their own, "
                          "128 generated tokens each, with reuse of cached pages")
-    ap.add_argument("--budget", type=int, default=2048, help="tokens a step for --serving")
+    ap.add_argument("--budget", type=int, default=4096, help="tokens a step for --serving")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run only prefill steps of --prefill-tokens tokens (for profiling) and print their time")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
