@@ -25,13 +25,16 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
                    help="auto = bfloat16")
     kv = p.add_mutually_exclusive_group()
     kv.add_argument("--num-blocks", type=int, default=None)
-    kv.add_argument("--kv-cache-gb", type=float, default=None, help="cache pool size in GiB (default 1)")
+    kv.add_argument("--kv-cache-gb", type=float, default=None,
+                    help="cache pool size in GiB (with neither: as many pages as the live requests can fill, "
+                         "within four fifths of the free device memory)")
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--no-prefix-caching", action="store_true",
                    help="no reuse of cached pages across requests")
     p.add_argument("--cuda-graphs", action=argparse.BooleanOptionalAction, default=True,
                    help="replay decode steps through HIP graphs (steps that fit no captured shape run eagerly)")
-    p.add_argument("--max-num-seqs", type=int, default=64)
+    p.add_argument("--max-num-seqs", type=int, default=256,
+                   help="most requests that are live at a time (the reference's server takes 64)")
     p.add_argument("--max-num-batched-tokens", type=int, default=4096,
                    help="tokens of a step, portions of prompts and decoded tokens together (the reference's "
                         "server takes 512; prompts run at twice the rate in steps of thousands of rows)")

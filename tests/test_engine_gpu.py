@@ -503,3 +503,23 @@ def test_generation_without_the_decode_copy_of_the_weights():
         for g, w, p in zip(got, want, ps):
             assert len(g) == 20
             assert_same_or_near_tie(name, p, g, w, margin=0.25)
+
+
+def test_generate_sizes_its_pool_from_the_requests():
+    """``generate`` with no pool size: as many pages as its live requests can fill (here the 8 longest
+    of 30; the others wait), and every request's tokens are the plain implementation's; the same
+    through a pool that holds all 30 at once."""
+    from dli_amd.engine.generate import generate, pages_for_requests
+    from dli_amd.sampling import SamplingParams
+
+    name = "B"
+    lengths = [3 + (7 * i) % 45 for i in range(30)]
+    ps = prompts(name, lengths, seed=31)
+    news = [4 + i % 9 for i in range(30)]
+    want = [plain_greedy(name, p, n) for p, n in zip(ps, news)]
+    for seqs in (8, 256):
+        got = generate(str(model_folder(name)), ps, [SamplingParams(max_tokens=n) for n in news], dtype="float32",
+                       max_num_seqs=seqs, max_num_batched_tokens=64)
+        assert got == want, seqs
+    few = pages_for_requests([a + b for a, b in zip(lengths, news)], 16, 8, 10 ** 9)
+    assert few < pages_for_requests([a + b for a, b in zip(lengths, news)], 16, 256, 10 ** 9)

@@ -51,3 +51,17 @@ def test_workgroup_shape_of_the_tile_kernel_from_sizes():
     assert tiled(6144, 2048) == 4                                   # q/k/v at the 1.7B sizes: 384 tiles
     assert tiled(128256, 3072) == 2 and tiled(128256, 2048) == 4   # vocabularies
     assert skinny_gemm_shape(2048, 8192) == 1 and skinny_gemm_shape(2048, 2048) == 0 and skinny_gemm_shape(128256, 2048) == 3
+
+
+def test_pool_of_generate_from_its_requests():
+    """Pages for the requests that can be live together, a page of look ahead each and the share
+    that admission keeps back; never more than the memory holds."""
+    from dli_amd.engine.generate import pages_for_requests
+
+    assert pages_for_requests([], 16, 4, 100) == 1
+    # 100 and 33 tokens in pages of 16: 7 + 1 and 3 + 1 pages; only the two longest are live together
+    assert pages_for_requests([100, 33, 20], 16, 2, 10 ** 6) == 12 + 12 // 50 + 8
+    assert pages_for_requests([100, 33, 20], 16, 8, 10 ** 6) == 15 + 15 // 50 + 8
+    assert pages_for_requests([16] * 1000, 16, 256, 10 ** 6) == 512 + 10 + 8
+    assert pages_for_requests([16] * 1000, 16, 256, 300) == 300          # what the memory holds
+    assert pages_for_requests([1600, 16], 16, 256, 50) == 50
