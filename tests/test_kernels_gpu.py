@@ -99,9 +99,10 @@ def test_gemm_f32(ops, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("qh,kvh,d,rd,bs", [(4, 4, 16, 16, 16), (6, 2, 32, 32, 8), (3, 1, 48, 32, 4), (2, 2, 80, 80, 16)])
-# few tokens: one item per thread; many: a workgroup per 8 tokens, which writes v in runs where the
-# slots are consecutive and aligned in a page (and element by element where they are not)
-@pytest.mark.parametrize("n,slots_as", [(11, "scattered"), (70, "scattered"), (203, "consecutive"), (150, "offset")])
+# up to 512 tokens: one item per thread; more: a workgroup per 8 tokens, which writes v in runs where
+# the slots are consecutive and aligned in a page (and element by element where they are not)
+@pytest.mark.parametrize("n,slots_as", [(11, "scattered"), (70, "scattered"), (203, "consecutive"), (150, "offset"),
+                                        (512, "offset"), (530, "scattered"), (707, "consecutive"), (650, "offset")])
 def test_rope_kv_write(ops, dtype, qh, kvh, d, rd, bs, n, slots_as):
     torch.manual_seed(4)
     pages = max(9, -(-n // bs) + 3)
