@@ -624,7 +624,7 @@ MID_SHAPES = ((4, 1), (4, 2))              # (waves, kwaves) that are built for 
 MID_SHAPES_GATED = ((2, 1), (2, 2), (2, 4))  # and for the gated one
 
 
-def mid_gemm_plan(n: int, k: int, epilogue: int, units: int) -> tuple[int, int, int]:
+def mid_gemm_plan(n: int, k: int, epilogue: int, units: int, rows: int = 64) -> tuple[int, int, int]:
     """``(waves, kwaves, splits)`` for a product of ``n`` output features of depth ``k``.
 
     A workgroup has ``waves`` feature tiles of 16 and ``kwaves`` waves on each, which split its
@@ -634,9 +634,12 @@ def mid_gemm_plan(n: int, k: int, epilogue: int, units: int) -> tuple[int, int, 
     of 128 k to fetch."""
     tiles, blocks = -(-n // 16), k // 128
     if epilogue == MID_SWIGLU:
-        # (two k-waves a tile are ahead of four at 32 and 48 rows, 19.6 against 20.4 and 21.1 against
-        # 21.9 us at the 1B sizes, and level at 64)
-        return 2, 2 if blocks >= 2 else 1, 1
+        # (two against four k-waves a tile, cold weights: 21.1 and 21.4 us at 32 rows, 23.4 and 23.0
+        # at 48, 28.7 and 26.1 at 64 at the 1B sizes; with k of 3072 24.8 and 24.5, 29.9 and 27.2, 37.4
+        # and 31.9. In a decode step of 64 rows, where part of the weights is warm: 2.93 to 2.96 ms with
+        # either at the 1B sizes, 5.48 against 5.39 ms at the 3B sizes. Four tiles a workgroup, or one,
+        # were behind at every number of rows.)
+        return 2, (4 if rows > 32 and blocks >= 24 else 2) if blocks >= 2 else 1, 1
     if epilogue == MID_STORE:
         return 4, 2 if blocks >= 2 else 1, 1
     waves = 4
@@ -679,7 +682,7 @@ def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = F
         _require(w.shape[1] == k and w.shape[0] % sets == 0, "x and w differ in inner size")
         n = w.shape[0] // sets
     _require(epilogue in (MID_PARTIAL, MID_SWIGLU, MID_STORE), "unknown epilogue")
-    plan_waves, plan_kwaves, plan_splits = mid_gemm_plan(n, k, epilogue, _units(x.device))
+    plan_waves, plan_kwaves, plan_splits = mid_gemm_plan(n, k, epilogue, _units(x.device), m)
     waves = plan_waves if waves is None else waves
     kwaves = plan_kwaves if kwaves is None else kwaves
     splits = plan_splits if splits is None else splits

@@ -109,7 +109,11 @@ def test_shapes_that_the_product_refuses(ops):
         ops.mid_gemm(x[:8], w.view(-1), epilogue=ops.MID_PARTIAL, tiled=True, n=24)  # no whole tiles
     assert not ops.mid_gemm_supports(8, 96, torch.bfloat16) and not ops.mid_gemm_supports(8, 128, torch.float32)
     assert ops.mid_gemm_plan(2048, 8192, ops.MID_PARTIAL, 256) == (4, 2, 8)
-    assert ops.mid_gemm_plan(8192, 2048, ops.MID_SWIGLU, 256) == (2, 2, 1)
+    assert ops.mid_gemm_plan(8192, 2048, ops.MID_SWIGLU, 256, rows=32) == (2, 2, 1)
+    assert ops.mid_gemm_plan(8192, 2048, ops.MID_SWIGLU, 256, rows=64) == (2, 2, 1)
+    assert ops.mid_gemm_plan(8192, 3072, ops.MID_SWIGLU, 256, rows=33) == (2, 4, 1)
+    assert ops.mid_gemm_plan(8192, 3072, ops.MID_SWIGLU, 256, rows=32) == (2, 2, 1)
+    assert ops.mid_gemm_plan(8192, 256, ops.MID_SWIGLU, 256, rows=64) == (2, 2, 1)
     assert ops.mid_gemm_plan(48, 128, ops.MID_PARTIAL, 256) == (4, 1, 1)
 
 
