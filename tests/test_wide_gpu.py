@@ -63,12 +63,14 @@ def test_whole_prompt_then_decoding_at_serving_widths(dtype):
         assert core.step.graphs is not None and core.step.graphs.replays >= 24
 
 
-@pytest.mark.parametrize("count", [8, 24, 40, 64])
+@pytest.mark.parametrize("count", [8, 24, 40, 64, 130])
 def test_requests_decode_together_at_serving_widths(count):
     """Prompts of different lengths go in as mixed batches of portions, then all decode side by
     side: eight through the 16x16-tile products with their fused norm, SwiGLU and residual
     epilogues, 24, 40 and 64 through the product kernel that shares the activations through LDS and
-    its finishing kernels (two, three and four row tiles: graphs of 32, 48 and 64 rows)."""
+    its finishing kernels (two, three and four row tiles: graphs of 32, 48 and 64 rows), 130
+    through the library's products with separate norm, rotation and SwiGLU kernels (a graph of
+    144 rows)."""
     from dli_amd.trace import TraceSession
 
     rng = random.Random(4 + count)
