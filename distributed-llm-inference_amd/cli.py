@@ -31,8 +31,9 @@ def _add_engine_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--no-prefix-caching", action="store_true",
                    help="no reuse of cached pages across requests")
-    p.add_argument("--cuda-graphs", action=argparse.BooleanOptionalAction, default=True,
-                   help="replay decode steps through HIP graphs (steps that fit no captured shape run eagerly)")
+    p.add_argument("--cuda-graphs", action=argparse.BooleanOptionalAction, default=None,
+                   help="replay decode steps through HIP graphs (steps that fit no captured shape run eagerly); "
+                        "with neither form: where the call decodes enough steps for recording them to pay")
     p.add_argument("--max-num-seqs", type=int, default=256,
                    help="most requests that are live at a time (the reference's server takes 64)")
     p.add_argument("--max-num-batched-tokens", type=int, default=4096,

@@ -42,12 +42,28 @@ def pages_for_requests(lengths: Sequence[int], block_size: int, max_num_seqs: in
     return max(1, min(wanted, most)) if each else 1
 
 
+GRAPHS_PAY_FROM = 512  # decode steps of a call from which recording its decode graphs pays
+
+
+def graphs_pay(max_tokens: Sequence[int], max_num_seqs: int) -> bool:
+    """Whether a call that builds its own engine should record decode graphs: the graphs of a
+    call are recorded during it (some ten of them, 0.5 to 0.7 s at the 1B sizes) and save about a
+    millisecond a decode step afterwards, so they pay from several hundred steps on (64 requests
+    with 256 tokens each: 0.94 s without, 1.3 to 1.4 s with them; the same on an engine that has
+    them already: 0.70 s). The steps are estimated as the longest generation times the rounds
+    that the requests need at ``max_num_seqs`` a time."""
+    if not max_tokens:
+        return False
+    rounds = -(-len(max_tokens) // max(1, max_num_seqs))
+    return max(max_tokens) * rounds >= GRAPHS_PAY_FROM
+
+
 def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
              params: SamplingParams | Sequence[SamplingParams] | None = None, *,
              dtype: str = "bfloat16", num_blocks: Optional[int] = None, kv_cache_gb: Optional[float] = None,
              block_size: int = 16, max_num_seqs: int = 256, max_num_batched_tokens: int = 4096,
              enable_prefix_caching: bool = True, eos_token_ids: Collection[int] = (), seed: int = 0,
-             cuda_graphs: bool = True, device: str = "cuda", decode_steps: int = 8,
+             cuda_graphs: Optional[bool] = None, device: str = "cuda", decode_steps: int = 8,
              decode_weight_copy: bool = True) -> list[list[int]]:
     """Load ``model`` (a folder or a loaded model), run ``prompts`` to completion, return token ids.
 
@@ -65,7 +81,9 @@ def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
     tokens a second of 64 (256 such requests: 2.0 s against 2.9 s).
     The pool: with neither ``num_blocks`` nor ``kv_cache_gb``, as many pages as the live requests
     can fill (:func:`pages_for_requests`), within four fifths of the device memory that is free
-    once the weights are loaded; an engine's own default is 1 GiB."""
+    once the weights are loaded; an engine's own default is 1 GiB.
+    ``cuda_graphs``: None decides by :func:`graphs_pay` (an engine of its own records them always:
+    it lives longer than a call)."""
     import torch
 
     from ..weights.loader import load_model
@@ -80,6 +98,8 @@ def generate(model: str | Path | Any, prompts: Sequence[Sequence[int]],
             raise ValueError("one SamplingParams per prompt, or one for all")
     if isinstance(model, (str, Path)):
         model = load_model(model, dtype=dtype, device=device, decode_weight_copy=decode_weight_copy)
+    if cuda_graphs is None:
+        cuda_graphs = graphs_pay([q.max_tokens for q in per], max_num_seqs)
     max_model_len = None
     if num_blocks is None and kv_cache_gb is None and prompts:
         lengths = [len(p) + q.max_tokens for p, q in zip(prompts, per)]

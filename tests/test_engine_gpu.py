@@ -454,7 +454,7 @@ def test_generate_command_line(tmp_path):
     cfg, w = P.load_folder(folder)
     ps = [[11, 5, 300, 42, 7, 7, 129], list(range(3, 3 + 41))]
     (tmp_path / "prompts.txt").write_text(json.dumps(ps[1]) + "\n")
-    for dtype, block, extra in (("float32", 8, ["--no-prefix-caching"]), ("bfloat16", 16, ["--max-num-batched-tokens", "24"]),
+    for dtype, block, extra in (("float32", 8, ["--no-prefix-caching"]), ("bfloat16", 16, ["--max-num-batched-tokens", "24", "--cuda-graphs"]),
                                 ("auto", 16, ["--no-cuda-graphs", "--num-blocks", "12"])):
         proc = subprocess.run(
             [sys.executable, "-m", "dli_amd", "generate", "--model", str(folder), "--dtype", dtype, "--block-size",
@@ -498,7 +498,7 @@ def test_generation_without_the_decode_copy_of_the_weights():
     ps = prompts(name, [9, 40], seed=23)
     want = [plain_greedy(name, p, 20) for p in ps]
     for copy in (True, False):
-        got = generate(str(model_folder(name)), ps, SamplingParams(max_tokens=20), dtype="bfloat16", num_blocks=32,
+        got = generate(str(model_folder(name)), ps, SamplingParams(max_tokens=20), dtype="bfloat16", num_blocks=32, cuda_graphs=True,
                        enable_prefix_caching=False, decode_weight_copy=copy)
         for g, w, p in zip(got, want, ps):
             assert len(g) == 20

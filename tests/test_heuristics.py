@@ -65,3 +65,13 @@ def test_pool_of_generate_from_its_requests():
     assert pages_for_requests([16] * 1000, 16, 256, 10 ** 6) == 512 + 10 + 8
     assert pages_for_requests([16] * 1000, 16, 256, 300) == 300          # what the memory holds
     assert pages_for_requests([1600, 16], 16, 256, 50) == 50
+
+
+def test_a_call_records_graphs_where_it_decodes_long_enough():
+    from dli_amd.engine.generate import GRAPHS_PAY_FROM, graphs_pay
+
+    assert not graphs_pay([], 64)
+    assert not graphs_pay([16, 256], 256)                      # 256 decode steps
+    assert graphs_pay([16, GRAPHS_PAY_FROM], 256)
+    assert graphs_pay([256] * 600, 256)                        # three rounds of 256 steps
+    assert not graphs_pay([256] * 256, 256) and graphs_pay([256] * 257, 256)
