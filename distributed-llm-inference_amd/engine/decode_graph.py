@@ -122,12 +122,6 @@ class DecodeGraphs:
         ctx.all_rows_wanted = True  # logit_rows is the identity here
         model, caches = self.step_fn.model, self.step_fn.caches
         side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(2):  # warm up libraries and the allocator outside the capture
-                model.forward(ctx, caches)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
         views["temperature"].view(np.float32)[:] = 0.0  # padding rows are greedy
         views["top_p"].view(np.float32)[:] = 1.0
         views["top_k"][:] = -1
@@ -139,7 +133,7 @@ class DecodeGraphs:
             scratch = ops.sample_scratch(b, dev_name)
         ps = self.step_fn.manager.page_size
 
-        def body():
+        def body(steps=steps):
             # `steps` decode steps back to back: after each, the sampled tokens become the next
             # inputs and positions, lengths, slots and draw counters move on, all on the device
             for j in range(steps):
@@ -155,9 +149,12 @@ class DecodeGraphs:
                 tokens_host.copy_(tokens_all.view(-1), non_blocking=True)
             return logits
 
+        # One step outside the capture: what the parts and the libraries set up at their first call
+        # with these shapes (buffers that live on, plans of products) must not happen inside it.
         dev.copy_(host)
+        side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            body()
+            body(1)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()

@@ -188,7 +188,7 @@ class Scheduler:
         """How many tokens each request of the step may decode before the host looks again: more
         than one only if the step is all decoding, nobody waits for admission, nothing was
         preempted or has to be copied, and the pages for the extra tokens can be reserved now.
-        Never more than the request with the fewest tokens left may still produce."""
+        Never more than the request with the fewest tokens left may still produce, and a power of two."""
         k = self.config.decode_steps
         if k <= 1 or not plan.chunks or self.waiting or plan.preempted or plan.copy_ops:
             return 1
@@ -198,6 +198,7 @@ class Scheduler:
             k = min(k, ch.request.params.max_tokens - len(ch.request.output_ids))
         if k <= 1:
             return 1
+        k = 1 << (k.bit_length() - 1)  # a power of two: a runner that records a graph for each count records few
         try:
             for ch in plan.chunks:
                 self.manager.reserve_ahead(ch.request.request_id, k - 1)

@@ -307,6 +307,7 @@ def test_several_tokens_per_step_give_the_same_outputs(k):
     for s in runner.calls:  # never past a request's limit, never while somebody waits or a prompt runs
         if s.decode_steps > 1:
             assert all(c.num_tokens == 1 and c.needs_logits for c in s.chunks)
+            assert s.decode_steps & (s.decode_steps - 1) == 0   # powers of two only
     m.reset_prefix_cache()
     m.check_invariants()
     assert m.stats().free_pages == m.stats().num_pages and m.slots.num_free == m.slots.num_slots
