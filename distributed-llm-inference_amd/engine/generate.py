@@ -47,7 +47,7 @@ GRAPHS_PAY_FROM = 512  # decode steps of a call from which recording its decode 
 
 def graphs_pay(max_tokens: Sequence[int], max_num_seqs: int) -> bool:
     """Whether a call that builds its own engine should record decode graphs: the graphs of a
-    call are recorded during it (some ten of them, 0.5 to 0.7 s at the 1B sizes) and save about a
+    call are recorded during it (some ten of them, about 0.5 s at the 1B sizes) and save about a
     millisecond a decode step afterwards, so they pay from several hundred steps on (64 requests
     with 256 tokens each: 0.94 s without, 1.3 to 1.4 s with them; the same on an engine that has
     them already: 0.70 s). The steps are estimated as the longest generation times the rounds
