@@ -1,13 +1,16 @@
 // 32-bit matrix product for the true 32-bit path: out[m][n] = sum_k a[m][k] * w[n][k]
 // (+ bias[n]) (+ residual[m][n]). Plain FMA on the vector units, no matrix-core mode, so every
-// product and sum is IEEE single precision. The k loop runs in ascending order for every output
-// element whatever the tile it falls in, so a row's result does not depend on how many other rows
-// are in the batch.
+// product and sum is IEEE single precision. Every output element sums its k in the same fixed
+// order whatever the tile it falls in, so a row's result does not depend on how many other rows
+// are in the batch: runs of GF_RUN consecutive k are summed in ascending order, and the runs'
+// sums are added in ascending order (the rounding error of a long sum then grows with the
+// length of a run plus the number of runs, not with k).
 #include "common.h"
 
 #define GF_BM 64
 #define GF_BN 64
 #define GF_BK 16
+#define GF_RUN 256  // a multiple of GF_BK
 
 __global__ __launch_bounds__(256) void gemm_f32_nt_kernel(
     const float* __restrict__ a, int64_t lda, const float* __restrict__ w, int64_t ldw,
@@ -18,7 +21,8 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_kernel(
   const int tid = threadIdx.x;
   const int tx = tid % 16, ty = tid / 16;
   const int m0 = blockIdx.y * GF_BM, n0 = blockIdx.x * GF_BN;
-  float acc[4][4] = {};
+  float acc[4][4] = {};    // the run of k in progress
+  float total[4][4] = {};  // the finished runs
   const int lrow = tid / 4;          // 0..63: tile row loaded by this thread
   const int lk = (tid % 4) * 4;      // 0,4,8,12: first of its four k values
   const bool vec = (k % 4 == 0) && (lda % 4 == 0) && (ldw % 4 == 0) &&
@@ -54,6 +58,15 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
     }
+    if ((k0 + GF_BK) % GF_RUN == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          total[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -63,7 +76,7 @@ __global__ __launch_bounds__(256) void gemm_f32_nt_kernel(
     for (int j = 0; j < 4; ++j) {
       const int gn = n0 + tx * 4 + j;
       if (gn >= n) continue;
-      float v = acc[i][j];
+      float v = total[i][j] + acc[i][j];
       if (bias != nullptr) v += bias[gn];
       if (residual != nullptr) v += residual[(int64_t)gm * ldr + gn];
       out[(int64_t)gm * ldo + gn] = v;

@@ -32,6 +32,6 @@ def pytest_terminal_summary(terminalreporter, exitstatus, config) -> None:
     mod = sys.modules.get("test_model_gpu")
     worst = getattr(mod, "WORST", None)
     if worst:
-        terminalreporter.write_line(
-            "largest logit error as a fraction of its bound: "
-            + ", ".join(f"{k} {v:.3f}" for k, v in sorted(worst.items())))
+        terminalreporter.write_line("largest logit error as a fraction of its bound, and the test that saw it:")
+        for key, (ratio, test) in sorted(worst.items()):
+            terminalreporter.write_line(f"  {key} {ratio:.3f}  {test}")
