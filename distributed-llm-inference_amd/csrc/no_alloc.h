@@ -1,9 +1,7 @@
 // Entry points that allocate nothing.
 //
 // For callers that cannot allocate device memory around a call: code under HIP graph capture,
-// tight serving loops, harnesses that forbid hipMalloc. The reference has no counterpart (its
-// decode attention allocates its partial-result tensors with torch at every call,
-// src/dli/model/paged_attention.py:249-262).
+// tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

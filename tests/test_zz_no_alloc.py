@@ -1,6 +1,8 @@
 """The decode attention that allocates nothing (csrc/no_alloc.h) against the entry point that takes
-the caller's partial-result buffers: called through ctypes, twice in a row, the second call with a
-smaller input, so that what the first call left in the static array must not matter."""
+the caller's partial-result buffers (the same bits) and against the plain float64 attention of
+tests/kernel_refs.py (so that the two cannot be wrong alike): called through ctypes, twice in a
+row, the second call with a smaller input, so that what the first call left in the static array
+must not matter."""
 
 from __future__ import annotations
 
@@ -9,7 +11,11 @@ import ctypes
 import pytest
 import torch
 
+from kernel_refs import ref_paged_attention
+
 pytestmark = pytest.mark.gpu
+
+BF16_TOL = 1.6e-2  # the bound of the decode attention's own kernel test
 
 
 def _case(seed, requests, q_heads, kv_heads, head_dim, page, max_len, splits):
@@ -68,6 +74,10 @@ def test_decode_attention_without_allocation_equals_the_one_with_buffers():
         rc, got = _run(lib, c, static=True)
         assert rc_ref == 0 and rc == 0
         assert torch.equal(got, ref), (got.float() - ref.float()).abs().max()
+        plain = ref_paged_attention(c["q"].cpu(), c["k"].cpu(), c["v"].cpu(), list(range(c["requests"] + 1)),
+                                    c["kv_len"].tolist(), c["tables"].tolist(), c["q_heads"], c["head_dim"] ** -0.5)
+        err = (got.cpu().double() - plain).abs().max().item()
+        assert err < BF16_TOL, err
         assert not torch.equal(got, torch.full_like(got, 7.0))
         del got
         assert torch.cuda.memory_allocated() <= before
