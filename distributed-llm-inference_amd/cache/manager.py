@@ -49,6 +49,9 @@ class NoFreePagesError(RuntimeError):
 class SequenceError(KeyError):
     """Unknown or duplicate request id."""
 
+    def __str__(self) -> str:  # KeyError would print the message's repr, quotes and all
+        return str(self.args[0]) if self.args else ""
+
 
 class WrongThreadError(RuntimeError):
     """A manager that is confined to one thread was changed from another."""
@@ -70,9 +73,6 @@ def _confined(method):
         return method(self, *args, **kwargs)
 
     return checked
-
-    def __str__(self) -> str:
-        return str(self.args[0]) if self.args else ""
 
 
 @dataclass(frozen=True)
@@ -279,50 +279,48 @@ class CacheManager:
     @_confined
     def allocate(self, seq_id: SeqId, token_ids: Sequence[int], *, namespace: bytes = b"",
                  respect_watermark: bool = True) -> Allocation:
-        """Admit a prompt: reuse cached leading pages, take the rest, take a state slot.
+        """Admit a prompt: reuse cached leading pages, take the rest, take a state slot
+        (reference: src/dli/kv/block_manager.py:238-284, there for one group and no slots).
 
         Raises:
             SequenceError: the id is live already.
             NoFreePagesError / NoFreeSlotError: not enough pages or slots (nothing changed).
             ValueError: empty prompt.
         """
+        n = len(token_ids)
+        if n == 0:
+            raise ValueError(f"request {seq_id!r} brings an empty prompt")
         if seq_id in self._seqs:
-            raise SequenceError(f"sequence {seq_id!r} already allocated")
-        if not token_ids:
-            raise ValueError("cannot allocate an empty prompt")
+            raise SequenceError(f"request {seq_id!r} holds cache already")
         if self.slots.num_free == 0:
             raise NoFreeSlotError(f"all {self.slots.num_slots} state slots are taken")
         hits, hashes = self._lookup(token_ids, namespace)
-        if not self._admissible(len(token_ids), hits, respect_watermark=respect_watermark):
+        pages = self._ceil(n)
+        if not self._admissible(n, hits, respect_watermark=respect_watermark):
             raise NoFreePagesError(
-                f"need {self._ceil(len(token_ids)) - len(hits)} pages, "
-                f"{self.num_available_pages} available (reserve {max(self._reserve)})"
-            )
-        total = self._ceil(len(token_ids))
-        tables: list[list[int]] = []
-        for g, pool in enumerate(self.pools):
-            if g == 0:
-                # revive hits before taking new pages, so that no reused page can be reclaimed
-                for page in hits:
-                    pool.incref(page)
-                    pool.order.found(page)
-                table = list(hits)
-            else:
-                table = []
-            while len(table) < total:
-                table.append(pool.take())
-            tables.append(table)
-        n_cached = len(hits) * self.page_size
-        self._stats.prompt_tokens_queried += len(token_ids)
-        self._stats.prompt_tokens_hit += n_cached
-        seq = _Seq(tables=tables, num_tokens=len(token_ids), num_computed=n_cached, namespace=namespace,
+                f"request {seq_id!r} needs {pages - len(hits)} more pages for its {n} tokens; "
+                f"{self.num_available_pages} can be had ({max(self._reserve)} kept back)")
+        # Everything below succeeds: the checks above have counted the pages.
+        tables = [self._fill_table(pool, hits if g == 0 else (), pages) for g, pool in enumerate(self.pools)]
+        seq = _Seq(tables=tables, num_tokens=n, num_computed=len(hits) * self.page_size, namespace=namespace,
                    state_slot=self.slots.take(), released=[0] * len(self.pools))
         if self.prefix_caching:
-            seq.page_hashes = hashes
+            seq.page_hashes, seq.num_registered = hashes, len(hits)
             seq.tail_tokens = list(token_ids[len(hashes) * self.page_size:])
-            seq.num_registered = len(hits)
+        self._stats.prompt_tokens_queried += n
+        self._stats.prompt_tokens_hit += seq.num_computed
         self._seqs[seq_id] = seq
-        return Allocation(tuple(tuple(t) for t in tables), n_cached, seq.state_slot)
+        return Allocation(tuple(map(tuple, tables)), seq.num_computed, seq.state_slot)
+
+    @staticmethod
+    def _fill_table(pool: PagePool, hits: Sequence[int], pages: int) -> list[int]:
+        """A new request's table in one group: the cached pages that its prompt matched, then
+        fresh ones up to ``pages``. The matched pages are taken hold of first, so that none of
+        them can be reclaimed to make room for the fresh ones."""
+        for page in hits:
+            pool.incref(page)
+            pool.order.found(page)
+        return [*hits, *(pool.take() for _ in range(pages - len(hits)))]
 
     @_confined
     def append_slots(self, seq_id: SeqId, token_ids: Sequence[int]) -> list[CopyOp]:

@@ -469,3 +469,25 @@ def test_a_confined_manager_refuses_other_threads():
     t.start()
     t.join()
     assert free_for_all.sequences() == ["x"]
+
+
+def test_messages_of_unknown_requests_and_of_the_policy_that_is_not_built():
+    """A request id's error prints as its message, not as a quoted repr (it is a KeyError for
+    callers that catch that); and the reference's second eviction policy, which is not built, is
+    refused by name with the nearest one named, instead of silently selecting another order."""
+    from dli_amd.cache.manager import SequenceError
+    from dli_amd.cache.reclaim import make_order
+
+    assert str(SequenceError("unknown sequence 'x'")) == "unknown sequence 'x'"
+    m = CacheManager(num_pages=4, page_size=4)
+    with pytest.raises(SequenceError, match="^unknown sequence 'nobody'$"):
+        m.num_tokens("nobody")
+    with pytest.raises(KeyError):
+        m.free("nobody")
+    assert make_order("lru").name == "lru" and make_order("reuse").name == "reuse"
+    with pytest.raises(ValueError, match="'reuse' is the nearest"):
+        make_order("cost")
+    with pytest.raises(ValueError, match="'reuse' is the nearest"):
+        CacheManager(num_pages=4, page_size=4, eviction_policy="cost")
+    with pytest.raises(ValueError, match="unknown eviction policy"):
+        make_order("random")
