@@ -83,7 +83,9 @@ class RequestOutput:
 
 @dataclass(frozen=True)
 class StepStats:
-    """Shape and timing (seconds) of one step (reference: src/dli/engine/engine.py:39-54)."""
+    """Shape and timing (seconds) of one step (the fields of src/dli/engine/engine.py:39-54, and
+    ``decode_steps``: how many tokens each request of the step decoded, 1 unless the step ran
+    several on the device)."""
 
     num_seqs: int
     num_batched_tokens: int
@@ -93,10 +95,23 @@ class StepStats:
     schedule_s: float
     forward_s: float
     postprocess_s: float
+    decode_steps: int = 1
 
     @property
     def total_s(self) -> float:
         return self.schedule_s + self.forward_s + self.postprocess_s
+
+    @classmethod
+    def of(cls, plan: SchedulerOutput, marks: Sequence[float]) -> "StepStats":
+        """The record of a step that ran ``plan``; ``marks``: the clock before scheduling, after
+        it, after the forward pass, and at the end. A chunk counts as decoding if it is the one
+        token whose successor is sampled; everything else is prompt work."""
+        decoding = sum(1 for c in plan.chunks if c.num_tokens == 1 and c.needs_logits)
+        tokens = plan.num_batched_tokens
+        spans = [later - earlier for earlier, later in zip(marks, marks[1:])]
+        return cls(num_seqs=len(plan.chunks), num_batched_tokens=tokens, num_prefill_tokens=tokens - decoding,
+                   num_decode_tokens=decoding, num_preempted=len(plan.preempted), schedule_s=spans[0],
+                   forward_s=spans[1], postprocess_s=spans[2], decode_steps=plan.decode_steps)
 
 
 @dataclass
@@ -201,41 +216,39 @@ class LLMEngine:
         return self.scheduler.has_unfinished
 
     def step(self) -> list[RequestOutput]:
-        t0 = time.perf_counter()
-        sched = self.scheduler.schedule()
-        t1 = time.perf_counter()
+        """Schedule, run, sample, append; one :class:`StepStats` per call, also for a step in
+        which nothing could be scheduled."""
+        marks = [time.perf_counter()]
+        plan = self.scheduler.schedule()
+        marks.append(time.perf_counter())
         outputs: list[RequestOutput] = []
-        if sched.chunks:
-            sampling = [c for c in sched.chunks if c.needs_logits]
-            fused = getattr(self.runner, "execute_and_sample", None) if self._sample_is_default else None
-            if fused is not None:
-                tokens = fused(sched)
-            else:
-                logits = self.runner.execute(sched)
-            t2 = time.perf_counter()
-            k = sched.decode_steps
-            for ch in sched.chunks:
-                ch.request.num_computed_tokens += ch.num_tokens + k - 1
-            if fused is None:
-                tokens = self._sample(
-                    logits, [c.request.params for c in sampling], [c.request.seed for c in sampling],
-                    [len(c.request.output_ids) for c in sampling])
-            rounds = tokens if k > 1 else [tokens]  # one list of tokens per decoded position
-            if len(rounds) != k or any(len(r) != len(sampling) for r in rounds):
+        if plan.chunks:
+            rounds = self._run(plan, marks)
+            wanted = [c for c in plan.chunks if c.needs_logits]
+            if len(rounds) != plan.decode_steps or any(len(r) != len(wanted) for r in rounds):
                 raise RuntimeError("the sampler returned a wrong number of tokens")
-            for i, ch in enumerate(sampling):
-                outputs.append(self._append_tokens(ch.request, [int(r[i]) for r in rounds]))
+            outputs = [self._append_tokens(c.request, [int(r[i]) for r in rounds]) for i, c in enumerate(wanted)]
         else:
-            t2 = t1
-        t3 = time.perf_counter()
-        prefill = sum(c.num_tokens for c in sched.chunks if c.num_tokens > 1 or not c.needs_logits)
-        total = sched.num_batched_tokens
-        self.stats.steps.append(StepStats(
-            num_seqs=len(sched.chunks), num_batched_tokens=total, num_prefill_tokens=prefill,
-            num_decode_tokens=total - prefill, num_preempted=len(sched.preempted),
-            schedule_s=t1 - t0, forward_s=t2 - t1, postprocess_s=t3 - t2))
+            marks.append(marks[-1])
+        marks.append(time.perf_counter())
+        self.stats.steps.append(StepStats.of(plan, marks))
         self._step_no += 1
         return outputs
+
+    def _run(self, plan: SchedulerOutput, marks: list[float]) -> list[Sequence[int]]:
+        """Run the plan's chunks and choose the tokens: one sequence of token ids (in the order
+        of the chunks that need logits) per decoded position. Notes the time after the forward
+        pass in ``marks`` and moves every request's count of computed tokens on."""
+        fused = getattr(self.runner, "execute_and_sample", None) if self._sample_is_default else None
+        result = fused(plan) if fused is not None else self.runner.execute(plan)
+        marks.append(time.perf_counter())
+        for c in plan.chunks:
+            c.request.num_computed_tokens += c.num_tokens + plan.decode_steps - 1
+        if fused is None:
+            wanted = [c.request for c in plan.chunks if c.needs_logits]
+            result = self._sample(result, [r.params for r in wanted], [r.seed for r in wanted],
+                                  [len(r.output_ids) for r in wanted])
+        return result if plan.decode_steps > 1 else [result]
 
     def generate(self, prompts: Iterable[Sequence[int]],
                  params: SamplingParams | Sequence[SamplingParams] | None = None) -> list[list[int]]:
