@@ -58,4 +58,8 @@ struct DliBlockArgs {
   void* v_pages;
   float eps1, eps2, scale;
   int32_t rotary_dim, hidden, q_heads, kv_heads, head_dim, intermediate, window, group, shape;
+  int32_t kind;  // which arrangement of which parts this describes: DLI_BLOCK_PRENORM_RMS_GQA_SILU, the only one
 };
+
+// kind: x += attention(rms(x)) with rotary pairs (i, i + dim/2); x += down(silu(gate(rms(x))) * up(rms(x)))
+#define DLI_BLOCK_PRENORM_RMS_GQA_SILU 1

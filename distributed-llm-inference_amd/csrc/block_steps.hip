@@ -43,6 +43,7 @@ int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pa
 namespace {
 
 bool block_is_sane(const DliBlockArgs& b, const DliStepArgs& s) {
+  if (b.kind != DLI_BLOCK_PRENORM_RMS_GQA_SILU) return false;  // the loop below computes this arrangement only
   if (b.norm1_w == nullptr || b.norm2_w == nullptr || b.w_qkv == nullptr || b.w_o == nullptr ||
       b.w_gate_up == nullptr || b.w_down == nullptr || b.inv_freq == nullptr || b.k_pages == nullptr ||
       b.v_pages == nullptr)

@@ -13,7 +13,7 @@ metadata carriers of src/dli/model/kv_cache.py:94-210.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Hashable, Optional, Sequence
+from typing import Any, Callable, Hashable, Optional, Sequence
 
 import numpy as np
 import torch
@@ -103,8 +103,11 @@ class StepContext:
     kv_len_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     state_slots_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     seq_ids: list = field(default_factory=list)
+    # per mixer (``id(mixer)``), what it answered to ``Mixer.decode_plan`` for this step: set only
+    # on the context of a recorded step, whose host arrays say nothing about the steps it will replay
+    decode_plans: dict = field(default_factory=dict)
     _tiles: dict = field(default_factory=dict)
-    _angles: dict = field(default_factory=dict)
+    _memo: dict = field(default_factory=dict)
 
     @property
     def max_kv_len(self) -> int:
@@ -118,20 +121,17 @@ class StepContext:
         return int(self.q_start_host[e]), int(self.q_start_host[e + 1])
 
     def begin_forward(self) -> None:
-        """Called at the start of every forward pass over this context: forgets what was derived
+        """Called at the start of every forward pass over this context: forgets what parts derived
         from arrays that may have changed on the device since the last pass (positions move when a
         graph runs several decode steps on one context)."""
-        self._angles.clear()
+        self._memo.clear()
 
-    def rope_angles(self, inv_freq: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-        """cos/sin of the step's positions for the rotary table ``inv_freq``, ``[tokens, 2, half]``:
-        made at the first call of a forward pass and shared by all layers that use that table."""
-        key = (inv_freq.data_ptr(), dtype)
-        hit = self._angles.get(key)
+    def memo(self, key: Hashable, make: Callable[[], Any]) -> Any:
+        """``make()``, made at the first call with this key in a forward pass and kept until the
+        next pass begins: for what several layers derive alike from the step's device arrays."""
+        hit = self._memo.get(key)
         if hit is None:
-            from ..kernels import ops
-
-            hit = self._angles[key] = ops.rope_angles(self.positions, inv_freq, dtype)
+            hit = self._memo[key] = make()
         return hit
 
     def is_fresh(self, e: int) -> bool:

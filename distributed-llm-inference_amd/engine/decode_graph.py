@@ -26,7 +26,6 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from ..parts.attention_kernels import choose_splits
 from .batch import GroupView, StepContext, StepEntry
 from .table_rows import TableRows
 
@@ -65,7 +64,7 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self.max_width = max(1, max_blocks_per_seq)
         self.n_groups = step_fn.manager.num_groups
-        self.captured: dict[tuple[int, int, int, bool, int], _Captured] = {}
+        self.captured: dict[tuple, _Captured] = {}
         self.replays = 0
         self.enabled = self._supported()
 
@@ -95,7 +94,7 @@ class DecodeGraphs:
             at += -(-n // 4) * 4  # 16-byte aligned starts
         return offsets, at
 
-    def _capture(self, b: int, splits: int, width: int, sampled: bool, steps: int = 1) -> _Captured:
+    def _capture(self, b: int, plans: tuple, width: int, sampled: bool, steps: int = 1) -> _Captured:
         dev_name = self.rt.device
         offsets, total = self._layout(b, width)
         host = torch.zeros(total, dtype=torch.int32).pin_memory()
@@ -118,7 +117,7 @@ class DecodeGraphs:
             kv_len=dv["kv_len"], state_slots=dv["state_slots"], logit_rows=dv["logit_rows"], groups=groups,
             q_start_host=np.arange(b + 1, dtype=np.int32), kv_len_host=np.zeros(b, np.int32),
             state_slots_host=np.zeros(b, np.int32), seq_ids=[None] * b)
-        ctx.forced_splits = splits
+        ctx.decode_plans = {id(part): plan for part, plan in zip(self.step_fn.plan_owners, plans)}
         ctx.all_rows_wanted = True  # logit_rows is the identity here
         model, caches = self.step_fn.model, self.step_fn.caches
         side = torch.cuda.Stream()
@@ -173,14 +172,14 @@ class DecodeGraphs:
                 gc.enable()
         return _Captured(graph, ctx, host, dev, logits, views, width, TableRows(b, width, self.n_groups), tokens_host)
 
-    def _shape_key(self, requests: int, max_kv: int, sampled: bool, steps: int) -> tuple[int, int, int, bool, int]:
+    def _shape_key(self, requests: int, max_kv: int, sampled: bool, steps: int) -> tuple:
         """The captured shape that serves ``requests`` requests of which the longest will hold
-        ``max_kv`` keys: (padded batch, key splits, block-table width, sampled, steps)."""
+        ``max_kv`` keys: (padded batch, what each part that keeps a cache plans for such a step,
+        block-table width, sampled, steps)."""
         b = _batch_bucket(requests)
         width = max(16, _bucket(-(-max_kv // self.step_fn.manager.page_size)))
-        splits = _bucket(choose_splits(b, self.step_fn.decode_head_tiles, max_kv,
-                                       ops.compute_units(self.step_fn.rt.device)))
-        return (b, splits, width, sampled, steps)
+        plans = tuple(part.decode_plan(b, max_kv) for part in self.step_fn.plan_owners)
+        return (b, plans, width, sampled, steps)
 
     def warm_up(self, batches: Sequence[int], max_len: int, *, sampled: bool = True,
                 steps: Sequence[int] = (1,)) -> int:

@@ -43,9 +43,10 @@ class StepFunction:
         self.vocab_size = model.spec.vocab_size
         self.steps_run = 0
         self.graphs = None  # DecodeGraphs, when the engine enables graph replay of decode steps
-        # workgroups per request and key split in the decode kernels of the parts that keep pages
-        self.decode_head_tiles = max([1] + [int(part.decode_head_tiles()) for part in model.cache_owners()
-                                            if part is not None and hasattr(part, "decode_head_tiles")])
+        # the parts that keep something per request, each once: they are asked how they would lay
+        # out a decode step before one is recorded (``Mixer.decode_plan``)
+        self.plan_owners = list({id(part): part for part in model.cache_owners()
+                                 if part is not None and hasattr(part, "decode_plan")}.values())
 
     def enable_decode_graphs(self, max_batch: int, max_model_len: int) -> None:
         """Replay decode-only steps through HIP graphs (bfloat16 with the matrix-core decode path

@@ -20,7 +20,7 @@ from typing import Any, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .attention_kernels import decode_attention_unmerged, paged_attention
+from .attention_kernels import decode_attention_unmerged, head_tiles, paged_attention, planned_splits
 from .base import DecodeStream, Mixer, Norm, PagedKVSpec, Part, Runtime
 from .linear import decode_copy, finish_residual, linear
 from .registry import build_part, register_part
@@ -130,14 +130,16 @@ class GQAttention(Mixer):
 
         nh, nkv, d, h = self.num_heads, self.num_kv_heads, self.head_dim, self.hidden_size
         table = self.position.rotary_table()
+        if type(self) is not GQAttention:
+            return None  # a subclass computes something else: it must describe itself
         if not self.rt.is_bf16 or self.shares_kv or table is None or table.pairing != "half":
             return None
         if not (_bf16_matrix(self.w_qkv, (nh + 2 * nkv) * d, h) and _bf16_matrix(self.w_o, h, nh * d)
                 and _bf16_vector(self.b_qkv, (nh + 2 * nkv) * d) and _bf16_vector(self.b_o, h)):
             return None
-        return {"w_qkv": self.w_qkv, "b_qkv": self.b_qkv, "w_o": self.w_o, "b_o": self.b_o,
+        return {"kind": "gqa_rotary_half", "w_qkv": self.w_qkv, "b_qkv": self.b_qkv, "w_o": self.w_o, "b_o": self.b_o,
                 "inv_freq": table.inv_freq, "rotary_dim": table.dim, "hidden": h, "q_heads": nh, "kv_heads": nkv,
-                "head_dim": d, "scale": self.scale, "window": self.window}
+                "head_dim": d, "scale": self.scale, "window": self.window, "plan_owner": id(self)}
 
     def cache_spec(self) -> Optional[PagedKVSpec]:
         return None if self.shares_kv else PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
@@ -147,9 +149,10 @@ class GQAttention(Mixer):
         return (self.rt.is_bf16 and ops.attention_mfma_supports(self.head_dim, page_size, self.rt.dtype)
                 and self.position.graph_capturable(page_size))
 
-    def decode_head_tiles(self) -> int:
-        # the decode kernel gives a workgroup up to 16 query heads of one kv head
-        return self.num_kv_heads * -(-(self.num_heads // self.num_kv_heads) // 16)
+    def decode_plan(self, requests: int, max_keys: int) -> Optional[int]:
+        """Into how many runs the decode kernel cuts each request's keys in a recorded step."""
+        return planned_splits(requests, head_tiles(self.num_heads, self.num_kv_heads), max_keys,
+                              ops.compute_units(self.rt.device))
 
     # -- step
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
@@ -175,7 +178,7 @@ class GQAttention(Mixer):
         q = qkv[:, :nh * d]
         out = self.rt.empty(x.shape[0], nh * d)
         paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window,
-                        self.arrival_counters)
+                        self.arrival_counters, planned=ctx.decode_plans.get(id(self)))
         return linear(self.rt, out, self.w_o, self.b_o)
 
     # -- decode steps with few rows: the norm before and the residual sum after are fused into
@@ -209,7 +212,7 @@ class GQAttention(Mixer):
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
         if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS:
             # product, rotation and cache write in one kernel; only q comes back
-            angles = ctx.rope_angles(self.position.rotary_table().inv_freq, qkv.dtype)
+            angles = self.position.step_angles(ctx, qkv.dtype)
             ops.skinny_gemm_qkv_rope(stream.x, self.w_qkv_rope, qkv, angles, grp.slots, cache.k_pages, cache.v_pages,
                                      nh, bias=self.b_qkv_rope, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         else:
@@ -230,7 +233,8 @@ class GQAttention(Mixer):
             # weights are on their way, and no merge kernel runs between the two
             left = decode_attention_unmerged(
                 qkv[:, :nh * d], cache.k_pages, cache.v_pages, ctx, grp, nh, self.scale, self.window,
-                lambda splits: ops.skinny_gemm_merged_supports(n, self.hidden_size, nh, d, splits, qkv.device))
+                lambda splits: ops.skinny_gemm_merged_supports(n, self.hidden_size, nh, d, splits, qkv.device),
+                planned=ctx.decode_plans.get(id(self)))
             if left is not None:
                 splits, part_o, part_ml = left
                 stream.wrote(ops.skinny_gemm_merged(part_o, part_ml, splits, nh, d, self.w_o_tiled, stream.x,
@@ -238,7 +242,7 @@ class GQAttention(Mixer):
                 return
         out = self.rt.empty(n, nh * d)
         paged_attention(qkv[:, :nh * d], cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window,
-                        self.arrival_counters)
+                        self.arrival_counters, planned=ctx.decode_plans.get(id(self)))
         stream.wrote(ops.skinny_gemm(out, self.w_o, w_tiled=self.w_o_tiled, epilogue=ops.SKINNY_RESIDUAL,
                                      stream=stream.x, bias=self.b_o))
 
@@ -257,10 +261,10 @@ class GQAttention(Mixer):
             partial = ops.mid_gemm(stream.x, self.w_qkv_rope, tiled=True, n=(nh + 2 * nkv) * d,
                                    epilogue=ops.MID_PARTIAL, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         q = self.rt.empty(n, nh * d)
-        angles = ctx.rope_angles(self.position.rotary_table().inv_freq, q.dtype)
+        angles = self.position.step_angles(ctx, q.dtype)
         ops.mid_finish_qkv(partial, q, angles, grp.slots, cache.k_pages, cache.v_pages, nh, bias=self.b_qkv_rope)
         out = self.rt.empty(n, nh * d)
         paged_attention(q, cache.k_pages, cache.v_pages, out, ctx, grp, nh, self.scale, self.window,
-                        self.arrival_counters)
+                        self.arrival_counters, planned=ctx.decode_plans.get(id(self)))
         partial = ops.mid_gemm(out, self.w_o_tiled, tiled=True, n=self.hidden_size, epilogue=ops.MID_PARTIAL)
         finish_residual(self.rt, stream, partial, self.b_o, following)

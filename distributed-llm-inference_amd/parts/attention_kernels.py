@@ -34,12 +34,24 @@ def choose_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int =
     return max(1, min(want, most, limit))
 
 
+def planned_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int = 256) -> int:
+    """:func:`choose_splits` rounded up to a power of two: the coarse form of the rule, for steps
+    that are recorded once and replayed for a range of lengths (each distinct answer is a
+    recording of its own)."""
+    splits, coarse = choose_splits(requests, kv_head_tiles, max_keys, units), 1
+    while coarse < splits:
+        coarse *= 2
+    return coarse
+
+
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                     ctx: Any, grp: Any, q_heads: int, scale: float, window: int = 0,
-                    arrival_counters: Optional[Callable[[int], Optional[torch.Tensor]]] = None) -> None:
+                    arrival_counters: Optional[Callable[[int], Optional[torch.Tensor]]] = None,
+                    planned: Optional[int] = None) -> None:
     """Attention of every row of the step over its request's pages, into ``out``.
     ``arrival_counters(n)``: the caller's ``n`` counters with which the decode kernel merges its
-    runs of keys by itself (see ``ops.attention_decode``), or None."""
+    runs of keys by itself (see ``ops.attention_decode``), or None. ``planned``: the number of
+    runs that the mixer promised for this step when it was recorded (``Mixer.decode_plan``)."""
     if ctx.num_tokens == 0:
         return
     _, kv_heads, page_size, head_dim = k_pages.shape
@@ -51,7 +63,7 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
         return
     nd = ctx.num_decode
     if nd > 0:
-        splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device)
+        splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device, planned)
         arrivals = None
         if arrival_counters is not None and 1 < splits <= ops.SELF_MERGING_SPLITS:
             arrivals = arrival_counters(nd * kv_heads * (-(-(q_heads // kv_heads) // 16)))
@@ -64,7 +76,8 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
 
 
 def decode_attention_unmerged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, ctx: Any, grp: Any,
-                              q_heads: int, scale: float, window: int, wanted) -> Any:
+                              q_heads: int, scale: float, window: int, wanted,
+                              planned: Optional[int] = None) -> Any:
     """Attention of a step in which every row is one request's single token, without the kernel
     that merges the runs of keys: ``(splits, part_o, part_ml)`` for the product that merges while
     it loads (``ops.skinny_gemm_merged``), or None (nothing has run) where the step's keys are
@@ -73,7 +86,7 @@ def decode_attention_unmerged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: t
     nd = ctx.num_decode
     if nd != ctx.num_tokens or not ops.attention_mfma_supports(head_dim, page_size, k_pages.dtype):
         return None
-    splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device)
+    splits, part_o, part_ml = _decode_splits(ctx, nd, q_heads, kv_heads, head_dim, q.device, planned)
     if splits < 2 or not wanted(splits):
         return None
     ops.attention_decode(q[:nd], k_pages, v_pages, None, ctx.kv_len, grp.block_tables, q_heads, scale, window,
@@ -81,10 +94,23 @@ def decode_attention_unmerged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: t
     return splits, part_o, part_ml
 
 
-def _decode_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, head_dim: int, device: torch.device):
-    group = q_heads // kv_heads
-    splits = getattr(ctx, "forced_splits", None) or choose_splits(
-        nd, kv_heads * (-(-group // 16)), ctx.max_decode_kv_len, ops.compute_units(device))
+def head_tiles(q_heads: int, kv_heads: int) -> int:
+    """Workgroups that one request's token gives the decode kernel per run of keys: a workgroup
+    takes up to 16 query heads of one kv head."""
+    return kv_heads * -(-(q_heads // kv_heads) // 16)
+
+
+def step_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, device: torch.device,
+                planned: Optional[int] = None) -> int:
+    """Runs of keys for the ``nd`` single-token rows of this step: what was planned when the step
+    was recorded, else the rule applied to the step's own lengths."""
+    return planned or choose_splits(nd, head_tiles(q_heads, kv_heads), ctx.max_decode_kv_len,
+                                    ops.compute_units(device))
+
+
+def _decode_splits(ctx: Any, nd: int, q_heads: int, kv_heads: int, head_dim: int, device: torch.device,
+                   planned: Optional[int] = None):
+    splits = step_splits(ctx, nd, q_heads, kv_heads, device, planned)
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty(nd * q_heads * splits * head_dim, device=device, dtype=torch.float32)

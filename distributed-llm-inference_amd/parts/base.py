@@ -12,7 +12,7 @@ of the step laid end to end; what belongs to which request is in the :class:`Ste
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Mapping, Optional, NamedTuple
+from typing import Any, Hashable, Mapping, Optional, NamedTuple
 
 import torch
 
@@ -202,6 +202,17 @@ class PositionEncoding(Part):
     def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], positions: torch.Tensor) -> None:
         """In-place change of q and k for the given absolute positions (default: nothing)."""
 
+    def step_angles(self, ctx: Any, dtype: torch.dtype) -> torch.Tensor:
+        """For an encoding with a rotary table: cos and sin of the step's positions,
+        ``[tokens, 2, dim/2]`` rounded to ``dtype``, for a product kernel that rotates in its
+        epilogue. Made by the first layer that asks in a forward pass and shared by all layers
+        whose tables are the same tensor (``StepContext.memo``)."""
+        from ..kernels import ops
+
+        table = self.rotary_table().inv_freq
+        return ctx.memo(("rotary_angles", table.data_ptr(), dtype),
+                        lambda: ops.rope_angles(ctx.positions, table, dtype))
+
 
 class Mixer(Part):
     """The part of a layer that mixes information between positions.
@@ -216,10 +227,15 @@ class Mixer(Part):
     def cache_spec(self) -> Optional[PagedKVSpec | StateSpec]:
         return None
 
-    def decode_head_tiles(self) -> int:
-        """Workgroups that one request's decoded token gives the mixer's kernel per split of its
-        keys (1 where that means nothing); the step function sizes key splits with the largest."""
-        return 1
+    def decode_plan(self, requests: int, max_keys: int) -> Hashable:
+        """How this mixer would lay out a recorded step in which ``requests`` requests bring one
+        token each and the longest holds ``max_keys`` keys: any hashable value (``None``: nothing
+        to choose). Whoever records such steps for replay asks every mixer, records one graph per
+        distinct answer and hands the answer back as ``ctx.decode_plans[id(mixer)]`` while the
+        step is recorded, when the host arrays that the mixer would otherwise choose from are
+        not there. Answers should be coarse (few distinct ones over the lengths of a request's
+        life), since each is a recording of its own."""
+        return None
 
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
         raise NotImplementedError
@@ -245,6 +261,17 @@ class Block(Part):
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
                 parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
         raise NotImplementedError
+
+    def native_fields(self, parts: Mapping[str, Part]) -> Optional[dict]:  # type: ignore[override]
+        """This arrangement with its parts' tensors and constants, for the loop in C that issues a
+        whole step's launches: a dict with the key ``"kind"`` naming an arrangement that the loop
+        implements, or ``None`` (the default) for any other; the step then runs part by part."""
+        return None
+
+    def streams(self, ctx: Any, parts: Mapping[str, Part]) -> bool:  # type: ignore[override]
+        """Whether this arrangement and its parts can run ``ctx``'s step on a
+        :class:`DecodeStream` (``forward_stream(stream, ctx, cache, parts, following=...)``)."""
+        return False
 
     def first_norm(self, parts: Mapping[str, Part]) -> Optional["Norm"]:
         """The norm that this arrangement applies to the stream before anything else, if there is

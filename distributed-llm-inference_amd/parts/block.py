@@ -30,18 +30,26 @@ class PreNormBlock(Block):
         f = parts["feed_forward"].forward(h, ctx)
         return x, f
 
+    # the arrangement of parts that the loop in C implements (``DLI_BLOCK_PRENORM_RMS_GQA_SILU``)
+    NATIVE_KIND = 1
+    NATIVE_PARTS = {"mixer_norm": "rms_norm", "mixer": "gqa_rotary_half", "feed_forward_norm": "rms_norm",
+                    "feed_forward": "gated_silu"}
+
     def native_fields(self, parts: Mapping[str, Part]) -> Optional[dict]:
         """This arrangement with its parts' tensors and constants, for the loop in C that issues a
-        step's launches; ``None`` unless all four parts describe themselves and agree on the width."""
-        n1, n2 = parts["mixer_norm"].native_fields(), parts["feed_forward_norm"].native_fields()
-        mix, ff = parts["mixer"].native_fields(), parts["feed_forward"].native_fields()
-        if n1 is None or n2 is None or mix is None or ff is None:
+        step's launches. That loop hard-codes one order of work, so the answer is ``None`` unless
+        this is exactly this class (a subclass must describe itself), each of the four parts
+        names exactly the kind that the loop computes, and all agree on the width."""
+        if type(self) is not PreNormBlock:
             return None
-        if not ({"w_qkv", "w_o", "inv_freq"} <= mix.keys() and {"w_gate_up", "w_down"} <= ff.keys()):
-            return None  # parts of another kind that describe themselves for another route
+        fields = {role: parts[role].native_fields() for role in self.NATIVE_PARTS}
+        if any(f is None or f.get("kind") != self.NATIVE_PARTS[role] for role, f in fields.items()):
+            return None
+        n1, n2, mix, ff = (fields[r] for r in ("mixer_norm", "feed_forward_norm", "mixer", "feed_forward"))
         if not n1["width"] == n2["width"] == mix["hidden"] == ff["hidden"]:
             return None
-        return {**mix, **ff, "norm1_w": n1["w"], "eps1": n1["eps"], "norm2_w": n2["w"], "eps2": n2["eps"]}
+        return {**mix, **ff, "kind": self.NATIVE_KIND, "norm1_w": n1["w"], "eps1": n1["eps"], "norm2_w": n2["w"],
+                "eps2": n2["eps"]}
 
     def streams(self, ctx: Any, parts: Mapping[str, Part]) -> bool:
         fused_norms = all(hasattr(parts[r], "fused_params") for r in ("mixer_norm", "feed_forward_norm"))

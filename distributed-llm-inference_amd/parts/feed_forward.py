@@ -53,10 +53,12 @@ class GatedMLP(FeedForward):
         from .native import _bf16_matrix, _bf16_vector
 
         h, i = self.hidden_size, self.intermediate_size
+        if type(self) is not GatedMLP:
+            return None  # a subclass computes something else: it must describe itself
         if not (self.rt.is_bf16 and _bf16_matrix(self.w_gate_up, 2 * i, h) and _bf16_matrix(self.w_down, h, i)
                 and _bf16_vector(self.b_gate_up, 2 * i) and _bf16_vector(self.b_down, h)):
             return None
-        return {"w_gate_up": self.w_gate_up, "b_gate_up": self.b_gate_up, "w_down": self.w_down, "b_down": self.b_down,
+        return {"kind": "gated_silu", "w_gate_up": self.w_gate_up, "b_gate_up": self.b_gate_up, "w_down": self.w_down, "b_down": self.b_down,
                 "hidden": h, "intermediate": i}
 
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:

@@ -29,6 +29,16 @@ class BuiltLayer:
     parts: dict[str, Part]
 
 
+class BoundCaches(list):
+    """The caches of a model's schedule entries, in schedule order (what :meth:`Model.bind_caches`
+    returns and :meth:`Model.forward` takes), with room for what the model derives from them: the
+    description of its blocks for the loop in C holds the addresses of these very pages, so it
+    lives and dies with this list and not with the model."""
+
+    derived: Any = None             # NativeBlocks, or False where that route does not apply
+    derived_for: int = -1           # the model's ``weights_version`` it was made for
+
+
 def _walk(part: Part):
     yield part
     for sub in part.sub_parts().values():
@@ -49,7 +59,7 @@ class Model:
             self.layers.append(BuiltLayer(blk, parts))
         self.final_norm = build_part("norm", spec.final_norm, runtime)
         self.head = build_part("head", spec.head, runtime)
-        self._native: dict = {}
+        self.weights_version = 0   # counts load_weights(): what was derived from older tensors is stale
         self.native_steps = True   # steps with portions: all layers' launches from one call where the blocks allow
         self.native_runs = 0       # how many steps went that way
 
@@ -89,6 +99,7 @@ class Model:
         self.head.tie(self.embedding.table())
         for part in self._all_parts():
             part.finalize()
+        self.weights_version += 1
 
     # ------------------------------------------------------------------ cache needs
 
@@ -120,9 +131,9 @@ class Model:
             parts.extend(layer.parts.values())
         return all(p.graph_capturable(page_size) for p in parts)
 
-    def bind_caches(self, layer_caches: Sequence[Any]) -> list[Any]:
+    def bind_caches(self, layer_caches: Sequence[Any]) -> BoundCaches:
         """Per schedule entry, the cache it uses: its own, or a read-only view of another's."""
-        out = []
+        out = BoundCaches()
         for i, entry in enumerate(self.spec.schedule):
             if entry.cache_of is not None:
                 src = layer_caches[entry.cache_of]
@@ -162,14 +173,17 @@ class Model:
         return out
 
     def _native_blocks(self, caches: Sequence[Any]):
-        """The schedule as one array of block descriptions for the loop in C, made once per list
-        of layer caches; ``None`` if some block or cache is not of the kind that route covers."""
-        hit = self._native.get(id(caches))
-        if hit is None or hit[0] is not caches:
+        """The schedule as one array of block descriptions for the loop in C, made once per bound
+        list of caches and set of weights and kept on that list; ``None`` if some block or cache
+        is not of the kind that route covers, or the caches are not a :class:`BoundCaches`."""
+        if not isinstance(caches, BoundCaches):
+            return None
+        if caches.derived is None or caches.derived_for != self.weights_version:
             from .native import NativeBlocks
 
-            hit = self._native[id(caches)] = (caches, NativeBlocks.build(self, caches))
-        return hit[1]
+            caches.derived = NativeBlocks.build(self, caches) or False
+            caches.derived_for = self.weights_version
+        return caches.derived or None
 
     def forward(self, ctx: Any, caches: Sequence[Any]) -> torch.Tensor:
         """Run the step's tokens through the schedule; float32 logits ``[wanted rows, vocab]``."""

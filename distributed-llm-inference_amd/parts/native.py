@@ -21,7 +21,7 @@ from typing import Any, Optional, Sequence
 import torch
 
 from ..kernels import ops
-from .attention_kernels import choose_splits
+from .attention_kernels import step_splits
 
 MAX_GROUPS, MAX_SHAPES = 4, 4
 _p, _i32, _i64, _f = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
@@ -45,7 +45,7 @@ class BlockArgs(ctypes.Structure):
                 ("w_gate_up", _p), ("b_gate_up", _p), ("w_down", _p), ("b_down", _p), ("inv_freq", _p),
                 ("k_pages", _p), ("v_pages", _p), ("eps1", _f), ("eps2", _f), ("scale", _f), ("rotary_dim", _i32),
                 ("hidden", _i32), ("q_heads", _i32), ("kv_heads", _i32), ("head_dim", _i32), ("intermediate", _i32),
-                ("window", _i32), ("group", _i32), ("shape", _i32)]
+                ("window", _i32), ("group", _i32), ("shape", _i32), ("kind", _i32)]
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -69,12 +69,14 @@ class NativeBlocks:
         self.device = device
         self.array = (BlockArgs * len(blocks))()
         self.shapes: list[tuple[int, int, int]] = []   # (head_dim, q_heads, kv_heads), by shape index
+        self.plan_owners: list[int] = []                 # per shape, the first mixer of that shape
         self.keep = []                                   # tensors whose addresses the array holds
         self.widths = dict(hidden=0, qkv=0, attn=0, gate_up=0, act=0)
         for a, f, cache in zip(self.array, blocks, caches):
             shape = (f["head_dim"], f["q_heads"], f["kv_heads"])
             if shape not in self.shapes:
                 self.shapes.append(shape)
+                self.plan_owners.append(f.get("plan_owner", 0))
             for name in ("norm1_w", "norm2_w", "w_qkv", "b_qkv", "w_o", "b_o", "w_gate_up", "b_gate_up", "w_down",
                          "b_down", "inv_freq"):
                 setattr(a, name, _ptr(f[name]))
@@ -84,7 +86,7 @@ class NativeBlocks:
             for name in ("eps1", "eps2", "scale", "rotary_dim", "hidden", "q_heads", "kv_heads", "head_dim",
                          "intermediate", "window"):
                 setattr(a, name, f[name])
-            a.group, a.shape = cache.group, self.shapes.index(shape)
+            a.group, a.shape, a.kind = cache.group, self.shapes.index(shape), f["kind"]
             d, qh, kvh = shape
             w = self.widths
             w["hidden"] = max(w["hidden"], f["hidden"])
@@ -102,9 +104,8 @@ class NativeBlocks:
         fields = []
         for entry, cache in zip(model.spec.schedule, caches):
             layer = model.layers[entry.layer]
-            describe = getattr(layer.block, "native_fields", None)
-            f = describe(layer.parts) if describe is not None else None
-            if (f is None or cache is None or cache.kind != "paged" or not cache.writable
+            f = layer.block.native_fields(layer.parts)
+            if (f is None or not isinstance(f.get("kind"), int) or cache is None or cache.kind != "paged" or not cache.writable
                     or not 0 <= cache.group < MAX_GROUPS or cache.window != f["window"]):
                 return None
             kvh, d = f["kv_heads"], f["head_dim"]
@@ -149,8 +150,8 @@ class NativeBlocks:
                 tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(d, qh, kvh), first_entry=nd)
                 sh.tile_entry, sh.tile_q0, sh.tiles = tile_entry.data_ptr(), tile_q0.data_ptr(), tile_entry.shape[0]
             if nd > 0:
-                splits = choose_splits(nd, kvh * (-(-(qh // kvh) // 16)), ctx.max_decode_kv_len,
-                                       ops.compute_units(self.device))
+                # mixers of one shape plan alike, so the first one's answer for a recorded step holds for all
+                splits = step_splits(ctx, nd, qh, kvh, self.device, ctx.decode_plans.get(self.plan_owners[i]))
                 sh.decode_splits = splits
                 if splits > 1:
                     parts_o = max(parts_o, nd * qh * splits * d)

@@ -26,17 +26,37 @@ def plain_greedy(name, prompt, n):
 
 
 def assert_same_or_near_tie(name, prompt, got, want, margin):
-    """Tokens must be the plain implementation's; a difference is allowed only where the plain
-    logits of the two candidates are within ``margin`` of each other (then the run is cut there)."""
+    """Greedy tokens of the engine against the plain implementation, the whole run: ``got`` equals
+    ``want`` (the plain implementation's own greedy run), or else every token of ``got`` is checked
+    against the plain logits of the engine's own tokens before it (teacher forcing: one plain
+    evaluation of ``prompt + got``): the token must be the plain model's best there, or lie within
+    ``margin`` of it, where rounding decides. A run that parts from the plain one at a near-tie
+    is thus still checked to its end."""
+    assert len(got) == len(want), (len(got), len(want))
+    if list(got) == list(want):
+        return
     cfg, w = P.load_folder(model_folder(name))
-    toks = list(prompt)
-    for g, x in zip(got, want):
-        if g != x:
-            logits = P.forward_logits(w, cfg, toks)[-1]
-            gap = (logits[x] - logits[g]).item()
-            assert 0 <= gap < margin, f"token {g} instead of {x}: plain logits differ by {gap}"
-            return
-        toks.append(x)
+    logits = P.forward_logits(w, cfg, list(prompt) + list(got[:-1]))
+    for j, g in enumerate(got):
+        row = logits[len(prompt) - 1 + j]
+        gap = (row.max() - row[g]).item()
+        assert gap < margin, f"token {j} is {g}: the plain logits prefer {int(row.argmax())} by {gap}"
+
+
+def assert_draws_follow_the_plain_distribution(name, prompt, got, params, seed, tol):
+    """Seeded tokens of the engine against the plain implementation, the whole run: at every
+    position the request's uniform draw (host Philox, keyed by seed and position) must lie in the
+    token's cell of the plain cumulative distribution over the engine's own tokens before it, or
+    within ``tol`` of that cell, where rounding decides."""
+    from test_sampling_gpu import philox_uniform
+
+    cfg, w = P.load_folder(model_folder(name))
+    logits = P.forward_logits(w, cfg, list(prompt) + list(got[:-1]))
+    for j, tok in enumerate(got):
+        probs = P.sampling_probabilities(logits[len(prompt) - 1 + j], params.temperature, params.top_k, params.top_p)
+        hi = float(torch.cumsum(probs, 0)[tok])
+        lo, u = hi - float(probs[tok]), philox_uniform(seed, j)
+        assert lo - tol <= u <= hi + tol, f"draw {j}: token {tok} has the cell [{lo}, {hi}], the draw is {u}"
 
 
 @pytest.mark.parametrize("name,dtype,block", [("A", "float32", 16), ("B", "float32", 8), ("A", "bfloat16", 16),
@@ -336,6 +356,104 @@ def test_graph_replay_under_preemption_bf16(name, reuse):
         assert_same_or_near_tie(name, p, r.output_ids, plain_greedy(name, p, 44), margin=0.25)
     eng.manager.reset_prefix_cache()
     assert eng.manager.stats().used_pages == 0
+
+
+@pytest.mark.parametrize("name", ["A", "D"])
+@pytest.mark.parametrize("reuse", [False, True])
+def test_eight_tokens_a_step_in_a_pool_that_runs_out_bf16(name, reuse):
+    """What ``generate()`` and the command line do by default (bfloat16, decode graphs, up to
+    eight tokens of every request per engine step), in a pool so small that requests lose their
+    pages and recompute and that reserving pages ahead fails half-way in some steps (what was
+    reserved so far then stays with its request and a single token is decoded): the reference's
+    tests/unit/engine/test_preemption.py:32-61 with tests/unit/model/test_cuda_graph_gpu.py:129-150,
+    on the real block tables, the kernel that moves positions and slots on between the tokens of
+    a step, and the graphs' rows. Greedy and seeded requests side by side; every token of every
+    request is checked against the plain implementation on the request's own tokens before it."""
+    from dli_amd.cache.manager import NoFreePagesError
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+    from dli_amd.sampling import SamplingParams
+
+    ps = prompts(name, [40, 23, 55, 31, 47, 18, 60, 12, 35, 50], seed=71)
+    eng = LLMEngine.for_model(str(model_folder(name)), dtype="bfloat16", num_blocks=16, block_size=16,
+                              enable_prefix_caching=reuse,
+                              config=SchedulerConfig(max_num_seqs=6, max_num_batched_tokens=64, decode_steps=8))
+    graphs = eng.core.step.graphs
+    assert graphs is not None and eng.scheduler.config.decode_steps == 8
+    refused = []
+    reserve = eng.manager.reserve_ahead
+
+    def counting(*a, **k):
+        try:
+            return reserve(*a, **k)
+        except NoFreePagesError:
+            refused.append(a)
+            raise
+
+    eng.manager.reserve_ahead = counting
+    seeded = {1: SamplingParams(max_tokens=44, temperature=0.8, top_k=40, seed=11),
+              4: SamplingParams(max_tokens=44, temperature=1.0, seed=12),
+              7: SamplingParams(max_tokens=44, temperature=0.9, top_p=0.95, seed=13)}
+    reqs = [eng.add_request(f"r{i}", p, seeded.get(i, SamplingParams(max_tokens=44))) for i, p in enumerate(ps)]
+    while eng.has_unfinished():
+        eng.step()
+        eng.manager.check_invariants()
+    steps = eng.stats.steps
+    assert sum(s.num_preempted for s in steps) > 0 and max(r.num_preemptions for r in reqs) > 0
+    assert sum(1 for s in steps if s.decode_steps > 1) >= 3 and max(s.decode_steps for s in steps) == 8
+    assert refused, "reserving ahead never failed: the pool was meant to be too small for that"
+    assert graphs.replays > 0
+    if reuse:
+        assert eng.manager.stats().evictions > 0
+    for i, (p, r) in enumerate(zip(ps, reqs)):
+        assert len(r.output_ids) == 44
+        if i in seeded:
+            assert_draws_follow_the_plain_distribution(name, p, r.output_ids, seeded[i], seeded[i].seed, 0.05)
+        else:
+            assert_same_or_near_tie(name, p, r.output_ids, plain_greedy(name, p, 44), margin=0.25)
+    eng.manager.reset_prefix_cache()
+    assert eng.manager.stats().used_pages == 0
+
+
+def test_a_graph_of_more_than_64_rows_cuts_the_keys_as_its_mixer_planned(monkeypatch):
+    """Decode steps of more than 64 requests are recorded through the loop in C that issues all
+    layers' launches. While a graph is recorded the context's host arrays say nothing about the
+    steps that it will replay, so the number of runs into which the keys are cut must be the one
+    that the mixer planned for the graph's shape (two kv heads: 80 rows leave compute units idle
+    unless long requests' keys are cut), not one computed from those arrays; and the logits are
+    the plain implementation's."""
+    from test_model_gpu import check, plain_logits
+    from dli_amd.engine.core import build_core
+    from dli_amd.kernels import ops
+    from dli_amd.trace import TraceSession
+
+    name, count = "B", 70
+    lens = [600 if r % 20 == 0 else 20 + r % 7 for r in range(count)]
+    toks = [prompts(name, [n + 3], seed=200 + r)[0] for r, n in enumerate(lens)]
+    core = build_core(model_folder(name), num_pages=sum(-(-(n + 3) // 16) for n in lens) + 4, page_size=16,
+                      max_seqs=count, dtype="bfloat16", enable_prefix_caching=False, watermark=0.0)
+    core.step.enable_decode_graphs(count, 640)
+    seen = []
+    real = ops.prenorm_blocks
+
+    def recording(x, blocks, n_blocks, step):
+        seen.append((step.rows, step.num_decode, step.shapes[0].decode_splits))
+        return real(x, blocks, n_blocks, step)
+
+    monkeypatch.setattr(ops, "prenorm_blocks", recording)
+    s = TraceSession(core)
+    for r in range(count):
+        s.step([{"id": r, "tokens": toks[r][:lens[r]], "want": []}])
+    del seen[:]
+    for i in range(3):
+        out = s.step([{"id": r, "tokens": [toks[r][lens[r] + i]], "want": [0]} for r in range(count)])
+        if i == 0 or i == 2:
+            rows = torch.stack([plain_logits(name, toks[r])[lens[r] + i] for r in range(count)])
+            check(out, rows, "bfloat16", f"decode step {i} of {count} requests")
+    assert core.step.graphs.replays == 3
+    (key,) = core.step.graphs.captured
+    planned = set(key[1])
+    assert len(planned) == 1 and min(planned) > 1, key
+    assert seen and all(rows == 80 and nd == 80 and splits == min(planned) for rows, nd, splits in seen), seen
 
 
 def test_trace_run_program(tmp_path):

@@ -665,3 +665,167 @@ def test_a_stateful_toy_mixer_that_says_it_can_be_recorded_is_replayed_from_grap
     finally:
         unregister_architecture("ToyStatefulForCausalLM")
         unregister_part("mixer", "toy_ema_device")
+
+
+# ------------------------------------------------------------------ a toy block arrangement
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_block_arrangement_is_registered_built_and_stepped(dtype):
+    """Another arrangement of a layer's parts, defined here and nowhere in the framework: one norm,
+    and mixer and feed-forward side by side, ``x + attention(norm(x)) + mlp(norm(x))``. It
+    implements ``forward`` only (no description for the loop in C, no fused decode form), so every
+    optional route must step aside by itself, in both precisions: the model below has such a
+    layer, a pre-norm layer, and such a layer again, and runs whole, in portions, mixed and token
+    by token (through decode graphs in bfloat16) against a plain float64 model of that
+    arrangement written with the plain implementation's parts."""
+    import tempfile
+    from typing import Any, Mapping
+
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import Block, LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part, unregister_part
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    @register_part("block", "toy_parallel")
+    class ToyParallel(Block):
+        roles = ("norm", "mixer", "feed_forward")
+
+        def __init__(self, runtime) -> None:
+            super().__init__(runtime)
+
+        def graph_capturable(self, page_size: int) -> bool:
+            return True  # nothing here reads the host's arrays
+
+        def forward(self, x, delta, ctx: Any, cache: Any, parts: Mapping[str, Any]):
+            h = parts["norm"].forward(x, delta)  # x <- x + delta
+            return x, parts["mixer"].forward(h, ctx, cache) + parts["feed_forward"].forward(h, ctx)
+
+    h, heads, kv_heads, d, inter, vocab, eps, theta = 48, 3, 1, 16, 80, 53, 1e-5, 1000.0
+
+    def build(cfg):
+        norm = dict(width=h, eps=eps)
+        pos = PartSpec("rotary", dict(dim=d, theta=theta))
+        layers = []
+        for i, kind in enumerate(("toy_parallel", "pre_norm", "toy_parallel")):
+            p = f"layers.{i}."
+            parts = {"mixer": ("mixer", PartSpec("gqa_attention", dict(hidden_size=h, num_heads=heads, num_kv_heads=kv_heads,
+                                                                      head_dim=d, position=pos), p + "attn.")),
+                     "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=inter),
+                                                               p + "mlp."))}
+            if kind == "toy_parallel":
+                parts["norm"] = ("norm", PartSpec("rms_norm", norm, p + "n."))
+            else:
+                parts["mixer_norm"] = ("norm", PartSpec("rms_norm", norm, p + "n1."))
+                parts["feed_forward_norm"] = ("norm", PartSpec("rms_norm", norm, p + "n2."))
+            layers.append(LayerSpec(PartSpec(kind), parts))
+        return ModelSpec(
+            architecture="ToyParallelForCausalLM", vocab_size=vocab, hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=vocab, hidden_size=h), "embed."),
+            layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(3)),
+            final_norm=PartSpec("rms_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=vocab, hidden_size=h, tied=True), "head."))
+
+    def plain(w, tokens):
+        """The same model in float64: the arrangement above, part by part."""
+        w = {k: v.double() for k, v in w.items()}
+        sizes = dict(num_heads=heads, num_kv_heads=kv_heads, head_dim=d)
+        inv_freq = P.inverse_frequencies({"rope_type": "default", "theta": theta}, d)
+        cos, sin = P.rope_cos_sin(inv_freq, torch.arange(len(tokens)), torch.float64)
+        x = w["embed.weight"][torch.tensor(tokens)]
+        for i, kind in enumerate(("toy_parallel", "pre_norm", "toy_parallel")):
+            p = f"layers.{i}."
+            if kind == "toy_parallel":
+                n = P.rms_norm(x, w[p + "n.weight"], eps)
+                x = x + P.attention_block(n, w, p + "attn.", sizes, cos, sin) + P.swiglu_mlp(n, w, p + "mlp.")
+            else:
+                x = x + P.attention_block(P.rms_norm(x, w[p + "n1.weight"], eps), w, p + "attn.", sizes, cos, sin)
+                x = x + P.swiglu_mlp(P.rms_norm(x, w[p + "n2.weight"], eps), w, p + "mlp.")
+        return P.linear(P.rms_norm(x, w["norm.weight"], eps), w["embed.weight"])
+
+    register_architecture("ToyParallelForCausalLM", dict, build)
+    try:
+        from test_model_gpu import check
+
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, {"architectures": ["ToyParallelForCausalLM"]}, seed=12, std=0.15,
+                                        norm_jitter=0.1)
+            _, weights = P.load_folder(folder)
+            rng = torch.Generator().manual_seed(3)
+            toks = {rid: torch.randint(0, vocab, (n,), generator=rng).tolist() for rid, n in (("a", 45), ("b", 23))}
+            ref = {rid: plain(weights, t) for rid, t in toks.items()}
+            model = load_model(folder, dtype=dtype)
+            core = build_core(model, num_pages=12, page_size=16, max_seqs=4, enable_prefix_caching=False, watermark=0.0)
+            core.step.enable_decode_graphs(4, 12 * 16)
+            assert (core.step.graphs is not None) == (dtype == "bfloat16")
+            s = TraceSession(core)
+            for rid, t in toks.items():  # whole
+                got = s.step([{"id": rid, "tokens": t, "want": list(range(len(t)))}], end=[rid])
+                check(got, ref[rid], dtype, f"toy block, {rid} whole")
+            # portions of changing size beside the other request's portions, then token by token together
+            fed = {"a": 0, "b": 0}
+            for plan in ({"a": 16}, {"a": 7, "b": 5}, {"a": 2, "b": 9}, {"a": 5, "b": 2}, {"a": 3}):
+                entries = [{"id": rid, "tokens": toks[rid][fed[rid]:fed[rid] + n], "want": list(range(n))}
+                           for rid, n in plan.items()]
+                got = s.step(entries)
+                want = torch.cat([ref[rid][fed[rid]:fed[rid] + n] for rid, n in plan.items()])
+                check(got, want, dtype, f"toy block, portions {plan} at {fed}")
+                for rid, n in plan.items():
+                    fed[rid] += n
+            assert model.native_runs == 0, "the loop in C knows the pre-norm arrangement only"
+            while fed["b"] < len(toks["b"]):
+                got = s.step([{"id": rid, "tokens": [toks[rid][fed[rid]]], "want": [0]} for rid in ("a", "b")])
+                check(got, torch.stack([ref[rid][fed[rid]] for rid in ("a", "b")]), dtype, f"toy block, decode at {fed}")
+                fed = {rid: n + 1 for rid, n in fed.items()}
+            if dtype == "bfloat16":
+                assert core.step.graphs.replays > 0
+            core.manager.check_invariants()
+    finally:
+        unregister_architecture("ToyParallelForCausalLM")
+        unregister_part("block", "toy_parallel")
+
+
+def test_a_subclass_of_a_built_in_part_is_not_taken_for_it_by_the_loop_in_c():
+    """The loop in C that issues a step's launches hard-codes what the built-in parts compute. A
+    part that inherits from one of them and changes its arithmetic (here: attention whose output is
+    halved) inherits ``native_fields`` too; it must not be run as its parent. The same weights in
+    Llama's own arrangement go through the loop, and give other logits."""
+    import dataclasses
+
+    from dli_amd.architectures.llama import build_llama_spec
+    from dli_amd.config import LlamaConfig, register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import PartSpec, register_part, unregister_part
+    from dli_amd.parts.attention import GQAttention
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model
+
+    @register_part("mixer", "toy_halved_attention")
+    class Halved(GQAttention):
+        def forward(self, x, ctx, cache):
+            return super().forward(x, ctx, cache) * 0.5
+
+    def build(cfg):
+        spec = build_llama_spec(cfg)
+        layers = []
+        for ls in spec.layers:
+            family, mixer = ls.parts["mixer"]
+            layers.append(dataclasses.replace(ls, parts={**ls.parts, "mixer": (
+                family, dataclasses.replace(mixer, kind="toy_halved_attention"))}))
+        return dataclasses.replace(spec, layers=tuple(layers))
+
+    register_architecture("LlamaForCausalLM", LlamaConfig.from_hf_dict, build, model_types=("llama",), replace=True)
+    try:
+        halved = load_model(model_folder("D"), dtype="bfloat16")
+    finally:
+        register_architecture("LlamaForCausalLM", LlamaConfig.from_hf_dict, build_llama_spec, model_types=("llama",),
+                              replace=True)
+        unregister_part("mixer", "toy_halved_attention")
+    plain_model = load_model(model_folder("D"), dtype="bfloat16")
+    toks = list(range(3, 93))
+    outs = []
+    for model in (halved, plain_model):
+        core = build_core(model, num_pages=8, page_size=16, max_seqs=2, enable_prefix_caching=False, watermark=0.0)
+        outs.append(TraceSession(core).step([{"id": "r", "tokens": toks, "want": [89]}]).clone())
+    assert halved.native_runs == 0 and plain_model.native_runs == 1
+    assert not torch.allclose(outs[0], outs[1], atol=1e-3)

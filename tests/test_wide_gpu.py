@@ -187,6 +187,34 @@ def test_decode_attention_merges_its_runs_of_keys_in_the_launch(monkeypatch):
         assert torch.equal(a, b)
 
 
+_one_b: dict = {}
+
+
+def one_b():
+    """Llama-3.2-1B with random weights, written to a folder once (a billion weights: drawn on the
+    GPU) and loaded as the plain implementation reads a checkpoint; its weights in 64-bit are
+    kept, so that every plain evaluation does not convert them again."""
+    if not _one_b:
+        folder = model_folder("1B", device="cuda")
+        cfg, w = P.load_folder(folder)
+        assert cfg["num_hidden_layers"] == 16 and w["model.embed_tokens.weight"].shape == (128256, 2048)
+        _one_b.update(folder=folder, cfg=cfg, w=w, w64={k: t.double() for k, t in w.items()}, drift=None)
+    return _one_b
+
+
+def one_b_drift(toks, ref):
+    """Rounding adds up over 16 layers: how far bfloat16 may drift on average is measured, not
+    guessed, by evaluating the plain implementation itself in bfloat16 (once). The engine
+    accumulates in 32-bit where that evaluation rounds, so it must not be further from the 64-bit
+    logits."""
+    m = one_b()
+    if m["drift"] is None:
+        rounded = P.forward_logits(m["w"], m["cfg"], toks, dtype=torch.bfloat16).double()
+        m["drift"] = ((rounded - ref).abs().max(dim=-1).values / ref.abs().max(dim=-1).values).mean().item()
+        assert 0.01 < m["drift"] < 0.08, m["drift"]
+    return m["drift"]
+
+
 def test_llama_3_2_1b_at_full_depth_and_vocabulary():
     """All 16 layers and all 128,256 vocabulary rows of Llama-3.2-1B (random weights written to a
     folder and loaded by name like a checkpoint), 32-bit and bfloat16 against the plain
@@ -196,19 +224,12 @@ def test_llama_3_2_1b_at_full_depth_and_vocabulary():
     from dli_amd.engine.core import build_core
     from dli_amd.trace import TraceSession
 
-    folder = model_folder("1B", device="cuda")  # a billion weights: drawn on the GPU
+    m = one_b()
+    folder = m["folder"]
     rng = random.Random(8)
     toks = [rng.randrange(128256) for _ in range(64)]
-    cfg, w = P.load_folder(folder)
-    assert cfg["num_hidden_layers"] == 16 and w["model.embed_tokens.weight"].shape == (128256, 2048)
-    ref = P.forward_logits(w, cfg, toks)
-    # Rounding adds up over 16 layers: how far bfloat16 may drift on average is measured, not
-    # guessed, by evaluating the plain implementation itself in bfloat16. The engine accumulates
-    # in 32-bit where that evaluation rounds, so it must not be further from the 64-bit logits.
-    rounded = P.forward_logits(w, cfg, toks, dtype=torch.bfloat16).double()
-    drift = ((rounded - ref).abs().max(dim=-1).values / ref.abs().max(dim=-1).values).mean().item()
-    assert 0.01 < drift < 0.08, drift
-    del w, rounded
+    ref = P.forward_logits(m["w64"], m["cfg"], toks)
+    drift = one_b_drift(toks, ref)
     for dtype in ("float32", "bfloat16"):
         core = build_core(folder, num_pages=8, page_size=16, max_seqs=2, dtype=dtype,
                           enable_prefix_caching=False, watermark=0.0)
@@ -223,3 +244,43 @@ def test_llama_3_2_1b_at_full_depth_and_vocabulary():
             check(got, ref[i:i + 1], dtype, f"1B decode at {i} {dtype}")
         del core, s
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_llama_3_2_1b_in_portions_and_in_mixed_batches(dtype):
+    """The same model cut the other two ways (the reference's
+    tests/parity/test_engine_parity.py:7-12 names all of them for its real checkpoint): one request
+    in portions of changing size down to two tokens, and five requests of 40 to 100 tokens mixed,
+    up to four live, portions of some beside single tokens of others, in a pool that the four
+    longest fill to the last page, so that the fifth runs in pages that another one wrote before;
+    decode graphs on in bfloat16, as serving has them."""
+    from test_model_gpu import mixed_trace
+    from dli_amd.engine.core import build_core
+    from dli_amd.trace import TraceSession
+
+    m = one_b()
+    rng = random.Random(18)
+    lengths = [100, 92, 70, 50, 40]
+    all_toks = [[rng.randrange(128256) for _ in range(n)] for n in lengths]
+    refs = [P.forward_logits(m["w64"], m["cfg"], t) for t in all_toks]
+    drift = one_b_drift(all_toks[2], refs[2])
+    pages = sum(-(-n // 16) for n in lengths[:4])
+    core = build_core(m["folder"], num_pages=pages, page_size=16, max_seqs=4, dtype=dtype,
+                      enable_prefix_caching=False, watermark=0.0)
+    core.step.enable_decode_graphs(4, pages * 16)
+    s = TraceSession(core)
+    toks, ref, pos = all_toks[0], refs[0], 0
+    sizes = [16, 7, 5, 3, 2, 9, 2, 31, 4, 2, 17]
+    for k in range(100):
+        n = min(sizes[k % len(sizes)], len(toks) - pos)
+        if len(toks) - pos - n == 1:  # never leave a single token: portions go down to two
+            n += 1
+        got = s.step([{"id": "r", "tokens": toks[pos:pos + n], "want": list(range(n))}])
+        check(got, ref[pos:pos + n], dtype, f"1B portion [{pos},{pos + n}) {dtype}", mean_rtol=drift)
+        pos += n
+        if pos == len(toks):
+            break
+    s.step([], end=["r"])
+    mixed_trace(core, all_toks, lambda r: refs[r], dtype, f"1B {dtype}", seed=19, mean_rtol=drift)
+    if dtype == "bfloat16":
+        assert core.step.graphs.replays > 0
