@@ -591,10 +591,17 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
 
   bf16x8 qreg[2][DK];
   ColumnTile<DCH> st[2];
+  // beside st[j].m: the value subtracted in the exponent (m, or 0 while m is -inf), and the raw
+  // score above which m has to rise
+  float m_ref[2], raise_at[2];
+  constexpr float LAZY_LOG2 = 8.f;
+  const float inv_scale_log2e = 1.f / scale_log2e;
   int pos[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     st[j].init();
+    m_ref[j] = 0.f;
+    raise_at[j] = -INFINITY;
     const int qi = q0 + j * 16 + col;
     pos[j] = qi < q_len ? first_pos + qi : -1;
 #pragma unroll
@@ -613,34 +620,34 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   const int end = first_pos + wg_q_hi + 1;
   const int n_tiles = (end - begin + 31) / 32;
 
-  // Staging: thread-constant description of the UCH chunks this thread moves per tile. Chunk u <
-  // 4D is 8 dims of key u/(D/8); chunk 4D+c is 8 keys of dim c/4.
-  const bf16_t* src_base[UCH];
-  int src_off[UCH], src_mul[UCH], lds_off[UCH];
-  bool second_half[UCH], is_v[UCH], live[UCH];
-  int v_key[UCH];
+  // Staging: the UCH chunks that this thread moves per tile. Chunk u < 4D is 8 dims of key
+  // u/(D/8); chunk 4D+c holds 8 keys of dim (c%2D)/2: those of the tile's first half of 16 keys
+  // for c < 2D, of its second half after that. 2D and 4D are multiples of 64, so whether a chunk
+  // is of K or of V, and which half of the tile it lies in, is the same for all lanes of a wave:
+  // the page's address is then made on the scalar unit and each lane adds a constant of its own.
+  const int wave_first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / DLI_WAVE)) * DLI_WAVE;
+  unsigned lane_off[UCH];   // elements from the half's first key in its page
+  int lds_off[UCH], v_key[UCH];
+  bool second_half[UCH], is_v[UCH], live[UCH];  // second_half and is_v are the same in all lanes
 #pragma unroll
   for (int r = 0; r < UCH; ++r) {
     const int u_raw = threadIdx.x + r * NT;
     live[r] = CHUNKS % NT == 0 || u_raw < CHUNKS;
     const int u = live[r] ? u_raw : CHUNKS - 1;
-    is_v[r] = u >= 4 * D;
+    const int u_wave = min(wave_first + r * NT, CHUNKS - 1);  // the wave's first chunk decides for all of it
+    is_v[r] = u_wave >= 4 * D;
     if (!is_v[r]) {
       const int kk = u / (D / 8), part = u % (D / 8);
-      second_half[r] = kk >= 16;
-      src_base[r] = k_pages;
-      src_mul[r] = D;
-      src_off[r] = (kk % 16) * D + part * 8;
+      second_half[r] = u_wave >= 2 * D;
+      lane_off[r] = (kk % 16) * D + part * 8;
       lds_off[r] = kk * KPAD + part * 8;
       v_key[r] = 0;
     } else {
-      const int c = u - 4 * D, d = c / 4, vk = (c % 4) * 8;
-      second_half[r] = vk >= 16;
-      src_base[r] = v_pages;
-      src_mul[r] = 1;
-      src_off[r] = d * page_size + vk % 16;
-      lds_off[r] = K_ELEMS + d * VPAD + vk;
-      v_key[r] = vk;
+      const int c = u - 4 * D, d = (c % (2 * D)) / 2, sub = c % 2;
+      second_half[r] = u_wave >= 6 * D;
+      lane_off[r] = d * page_size + sub * 8;
+      v_key[r] = (second_half[r] ? 16 : 0) + sub * 8;
+      lds_off[r] = K_ELEMS + d * VPAD + v_key[r];
     }
   }
   bf16x8 stage[RD][UCH];
@@ -668,6 +675,10 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   // time and a tile is awaited without draining the younger ones behind it. Keys past the last one
   // of a half-filled page may hold anything: K rows there are masked as later than every query, V
   // columns are cleared on the way into LDS.
+  // (Looking a tile's pages up earlier in the iteration, behind the first product, so that the
+  // scalar load's answer arrives during the softmax, needs the lookup inside the branch that a wave
+  // takes when it sees the tile: the compiler then keeps the pages in vector registers or, told
+  // that the branch is uniform, copies the accumulators at its end: 393 -> 529 us at 8,192 tokens.)
   const int64_t page_elems = (int64_t)page_size * D;
   auto fetch = [&](int t, bf16x8 (&sq)[UCH]) {
     const int64_t pa = ((int64_t)page_a * kv_heads + kvh) * page_elems;
@@ -676,9 +687,10 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
     lookup(t + 32);
 #pragma unroll
     for (int r = 0; r < UCH; ++r) {
-      const int64_t pg = second_half[r] ? pb : pa;
-      const int of = second_half[r] ? ob : oa;
-      sq[r] = *reinterpret_cast<const bf16x8*>(src_base[r] + pg + of * src_mul[r] + src_off[r]);
+      // the same for every lane of the wave: a key's row of K is D long, a key's column of V^T one element
+      const int64_t first = (second_half[r] ? pb : pa) + (second_half[r] ? ob : oa) * (is_v[r] ? 1 : D);
+      const bf16_t* base = (is_v[r] ? v_pages : k_pages) + first;
+      sq[r] = *reinterpret_cast<const bf16x8*>(base + lane_off[r]);
     }
   };
   auto stash = [&](int buf, int t, bf16x8 (&sq)[UCH]) {
@@ -769,36 +781,50 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
           }
         }
       }
-      float alpha[2];
+      // The reference point of the exponentials moves lazily: st[j].m is raised (and what has been
+      // accumulated rescaled) only when a score of the tile exceeds it by more than 2^LAZY_LOG2,
+      // which each lane can tell from its own eight scores. Most tiles then need neither the
+      // maximum over the four lanes of a column nor the factor exp2(m_old - m_new); probabilities
+      // lie below 2^LAZY_LOG2 instead of below one, which changes nothing in the quotient O / l
+      // (32-bit sums, and bfloat16 keeps its eight bits at any magnitude).
+      float lane_max[2];
+      bool rise = false;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        float tile_max = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]),
-                              max2(sv[j][6], sv[j][7]));
-        tile_max = column_max(tile_max) * scale_log2e;  // the scale is positive
-        const float m_new = max2(st[j].m, tile_max);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        alpha[j] = fast_exp2(st[j].m - m_safe);
+        lane_max[j] = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]),
+                           max2(sv[j][6], sv[j][7]));
+        rise |= lane_max[j] > raise_at[j];
+      }
+      if (__builtin_amdgcn_ballot_w64(rise) != 0) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const float tile_max = column_max(lane_max[j]) * scale_log2e;  // the scale is positive
+          const float m_new = max2(st[j].m, tile_max);
+          const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+          const float alpha = fast_exp2(st[j].m - m_safe);  // 0 while nothing was seen, else at most 1
+          st[j].l *= alpha;
+#pragma unroll
+          for (int c = 0; c < DCH; ++c) st[j].o[c] *= alpha;
+          st[j].m = m_new;
+          m_ref[j] = m_safe;
+          raise_at[j] = m_new == -INFINITY ? -INFINITY : (m_new + LAZY_LOG2) * inv_scale_log2e;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        // l stays a per-lane partial sum (the lanes of a column share m): the four partial sums of
+        // a column are added once, after the last tile. (Taking the sum from the matrix cores
+        // instead, as the product of P^T with a row of ones, saves sixteen additions a lane and
+        // tile and was slower, 62 against 59 us; so was computing S^T of the next tile before the
+        // softmax of this one inside a wave, 68 us.)
         float tile_sum = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const float p = fast_exp2(fmaf(sv[j][i], scale_log2e, -m_safe));
+          const float p = fast_exp2(fmaf(sv[j][i], scale_log2e, -m_ref[j]));
           tile_sum += p;
           pb[j][i] = (bf16_t)p;
         }
-        // l stays a per-lane partial sum (the lanes of a column share m, hence alpha): the
-        // four partial sums of a column are added once, after the last tile. (Taking the sum
-        // from the matrix cores instead, as the product of P^T with a row of ones, saves sixteen
-        // additions a lane and tile and was slower, 62 against 59 us; so was computing S^T of the
-        // next tile before the softmax of this one inside a wave, 68 us.)
-        st[j].l = st[j].l * alpha[j] + tile_sum;
-        st[j].m = m_new;
-      }
-      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.f || alpha[1] != 1.f) != 0) {
-        // the running maximum rose somewhere: rescale what has been accumulated
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int c = 0; c < DCH; ++c) st[j].o[c] *= alpha[j];
+        st[j].l += tile_sum;
       }
     }
   };
@@ -1046,16 +1072,17 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (hw > 0) {
     const dim3 sgrid(tiles, q_heads / hw);
-    // Mirror tiles are paired (pair_tiles 1, or -1 and a launch in the range where it was faster:
-    // with too few workgroups pairing leaves compute units idle; with many, the queue of
-    // workgroups evens the causal triangle out by itself. Heads of up to 64: from two to under
-    // four workgroups per unit (2,048 tokens at the 1B sizes: 58 against 70 us; 4,096: 192 against
-    // 179; 8,192: 697 against 550); larger heads, whose single-tile kernel holds one wave a SIMD:
-    // from one a unit on (heads of 128, 2,048 tokens: 84 against 129 us; 16,384: 2.9 against 4.0 ms).
+    // Mirror tiles are paired (pair_tiles 1, or -1 and a launch in the range where it was faster):
+    // with too few workgroups pairing leaves compute units idle; with three or more a unit, the
+    // tiles listed longest first even the causal triangle out through the queue of workgroups,
+    // and the single-tile kernel's waves do not wait for one another. Heads of up to 64: from two
+    // to under three workgroups per unit (2,048 tokens at the 1B sizes: 50 against 55 us; 3,072:
+    // 127 against 92; 4,096: 161 against 122; 8,192: 565 against 393); larger heads, whose
+    // single-tile kernel holds one wave a SIMD: from one to under three a unit (heads of 128, 24
+    // of them, 2,048 tokens: 74 against 103 us; 8,192: 675 against 615).
     // The tile list has to hold all tiles of a request.
     const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
-    const bool in_range = head_dim <= 64 ? (launch >= 2 * units && launch < 4 * units)
-                                         : launch >= units;
+    const bool in_range = launch < 3 * units && launch >= (head_dim <= 64 ? 2 : 1) * units;
     const bool pair = pair_tiles >= 0 ? pair_tiles != 0 : in_range;
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \

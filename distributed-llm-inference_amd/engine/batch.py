@@ -139,12 +139,15 @@ class StepContext:
         q0, q1 = self.entry_rows(e)
         return int(self.kv_len_host[e]) - (q1 - q0) == 0
 
-    def q_tiles(self, rows_per_tile: int, first_entry: int = 0,
-                last_entry: Optional[int] = None) -> tuple[torch.Tensor, torch.Tensor]:
+    def q_tiles(self, rows_per_tile: int, first_entry: int = 0, last_entry: Optional[int] = None,
+                arrange: Optional[Callable[[np.ndarray, np.ndarray], np.ndarray]] = None,
+                arranged_as: Hashable = None) -> tuple[torch.Tensor, torch.Tensor]:
         """Query tiles ``(entry, first query of the tile)`` of entries ``[first, last)``, as two
-        int32 device vectors; built once per step and tile height."""
+        int32 device vectors; built once per step and tile height. ``arrange(entries, firsts)``
+        may return the order in which a kernel wants the tiles listed (a permutation; the default
+        is by entry and then by query); ``arranged_as`` names that order for the memo."""
         last = self.num_entries if last_entry is None else last_entry
-        key = (rows_per_tile, first_entry, last)
+        key = (rows_per_tile, first_entry, last, arranged_as if arrange is not None else None)
         hit = self._tiles.get(key)
         if hit is None:
             ent: list[int] = []
@@ -154,6 +157,12 @@ class StepContext:
                 for q0 in range(0, length, rows_per_tile):
                     ent.append(e)
                     q0s.append(q0)
-            hit = tuple(upload([np.asarray(ent, np.int32), np.asarray(q0s, np.int32)], self.device))
+            ent_a, q0_a = np.asarray(ent, np.int32), np.asarray(q0s, np.int32)
+            if arrange is not None and ent_a.size > 1:
+                order = np.asarray(arrange(ent_a, q0_a))
+                if sorted(order.tolist()) != list(range(ent_a.size)):
+                    raise ValueError("arrange() must return a permutation of the tiles")
+                ent_a, q0_a = ent_a[order], q0_a[order]
+            hit = tuple(upload([ent_a, q0_a], self.device))
             self._tiles[key] = hit
         return hit

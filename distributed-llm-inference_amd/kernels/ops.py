@@ -1104,8 +1104,9 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
                       tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
                       window: int = 0, pair_tiles: Optional[bool] = None) -> None:
     """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
-    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height:
-    every tile of every listed request, in ascending order within a request). ``pair_tiles``:
+    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height and
+    hold every tile of every listed request, in any order: workgroups start in the list's order,
+    so the tiles with the most keys belong first). ``pair_tiles``:
     whether one workgroup takes a tile and its mirror within the request, which evens out the
     causal mask's triangle; ``None`` lets the kernel decide by the size of the launch."""
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 from typing import Any, Callable, Optional
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -44,6 +45,34 @@ def planned_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int 
     return coarse
 
 
+def longest_first(ctx: Any, rows: int, units: int = 256) -> Callable:
+    """The order in which the prefill kernel wants a step's query tiles: those that see the most
+    keys first. Workgroups start in the order of the list, and under a causal mask a tile's work
+    grows with its place in the request: listed by place, the longest workgroups start last and
+    the launch ends with a few of them alone on the device (a prompt of 8,192 tokens at the 1B
+    sizes: 521 us a layer by place, 393 us longest first). Within the sorted list every second
+    run of as many tiles as an XCD has compute units is turned round, so that a unit that got a
+    long tile in one round gets a short one in the next."""
+    per_xcd = max(1, units // 8)
+
+    def arrange(entries: np.ndarray, firsts: np.ndarray) -> np.ndarray:
+        q_len = (ctx.q_start_host[entries + 1] - ctx.q_start_host[entries]).astype(np.int64)
+        keys = ctx.kv_len_host[entries].astype(np.int64) - q_len + np.minimum(firsts + rows, q_len)
+        order = np.argsort(-keys, kind="stable")
+        for r0 in range(per_xcd, order.size, 2 * per_xcd):
+            order[r0:r0 + per_xcd] = order[r0:r0 + per_xcd][::-1].copy()
+        return order
+
+    return arrange
+
+
+def prefill_tiles(ctx: Any, head_dim: int, q_heads: int, kv_heads: int, first_entry: int, device: torch.device):
+    """The tile list of the step's portions for :func:`ops.attention_prefill`."""
+    rows = ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads)
+    return ctx.q_tiles(rows, first_entry=first_entry, arrange=longest_first(ctx, rows, ops.compute_units(device)),
+                       arranged_as="longest first")
+
+
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                     ctx: Any, grp: Any, q_heads: int, scale: float, window: int = 0,
                     arrival_counters: Optional[Callable[[int], Optional[torch.Tensor]]] = None,
@@ -70,7 +99,7 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
         ops.attention_decode(q[:nd], k_pages, v_pages, out[:nd], ctx.kv_len, grp.block_tables, q_heads,
                              scale, window, splits, part_o, part_ml, arrivals=arrivals)
     if ctx.num_entries > nd:
-        tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads), first_entry=nd)
+        tile_entry, tile_q0 = prefill_tiles(ctx, head_dim, q_heads, kv_heads, nd, q.device)
         ops.attention_prefill(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
                               tile_entry, tile_q0, q_heads, scale, window)
 

@@ -21,7 +21,7 @@ from typing import Any, Optional, Sequence
 import torch
 
 from ..kernels import ops
-from .attention_kernels import step_splits
+from .attention_kernels import prefill_tiles, step_splits
 
 MAX_GROUPS, MAX_SHAPES = 4, 4
 _p, _i32, _i64, _f = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
@@ -147,7 +147,7 @@ class NativeBlocks:
         for i, (d, qh, kvh) in enumerate(self.shapes):
             sh = s.shapes[i]
             if ctx.num_entries > nd:
-                tile_entry, tile_q0 = ctx.q_tiles(ops.attention_prefill_tile_rows(d, qh, kvh), first_entry=nd)
+                tile_entry, tile_q0 = prefill_tiles(ctx, d, qh, kvh, nd, self.device)
                 sh.tile_entry, sh.tile_q0, sh.tiles = tile_entry.data_ptr(), tile_q0.data_ptr(), tile_entry.shape[0]
             if nd > 0:
                 # mixers of one shape plan alike, so the first one's answer for a recorded step holds for all
