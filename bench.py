@@ -6,7 +6,12 @@ The default run is the Llama-3.2-1B shape with random weights in bfloat16: 8 req
 greedily at a context of about 4096 tokens through the engine's own step loop (schedule, one
 batched step, sampling), W untimed steps and then exactly K timed ones between device
 synchronisations. One JSON line reports decoded tokens a second, the time of a 2,048-token prefill
-step, the decode step's memory roofline, and decode throughput at batch 1 and 64.
+step, the decode step's memory roofline, and under ``points`` decode throughput at batch 1 and 64,
+at the baseline's own context (2,048 growing to 2,304) and at 32,768 keys, and the other
+workloads that the baseline names: the Llama-3.2-3B sizes (decode at batch 8, a 2,048-token
+prefill, 64 requests batched continuously under 2,048 tokens a step) and the SmolLM2-1.7B sizes
+(decode at batch 8, 32 requests that share a prefix of 1,024 tokens). ``--no-other-shapes`` leaves
+the other models out, ``--no-points`` everything but the headline.
 """
 
 from __future__ import annotations
@@ -47,28 +52,35 @@ SMOLLM2_1_7B = {
 SHAPES = {"Llama-3.2-1B": LLAMA_3_2_1B, "Llama-3.2-3B": LLAMA_3_2_3B, "SmolLM2-1.7B": SMOLLM2_1_7B}
 
 
-def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, num_pages=None,
-                prefix_caching=False):
-    import torch
-
+def load_random_model(raw, dtype):
+    """A model of the sizes ``raw`` with random weights, by the road that generation takes: a
+    folder with config.json and model.safetensors (drawn on the GPU, a few seconds for a billion
+    weights), read by the loader."""
     import tempfile
 
-    from dli_amd.engine import LLMEngine, SchedulerConfig
     from dli_amd.weights import load_model, write_random_model
 
-    # The weights take the road that generation takes: a folder with config.json and
-    # model.safetensors (drawn on the GPU, a few seconds for a billion), read by the loader.
     with tempfile.TemporaryDirectory(prefix="dli_amd_bench_") as folder:
         write_random_model(folder, raw, seed=0, std=0.02, device="cuda:0")
-        model = load_model(folder, dtype=dtype, device="cuda:0")
-    cfg = model.config
+        return load_model(folder, dtype=dtype, device="cuda:0")
+
+
+def engine_for(model, batch, context, block_size, budget, decode_steps=1, num_pages=None, prefix_caching=False):
+    from dli_amd.engine import LLMEngine, SchedulerConfig
+
     pages = num_pages or batch * (-(-(context + SLACK) // block_size) + 1) + 8
     pages += pages // 64  # room for the share of the pool that admission keeps back (1%)
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=prefix_caching,
         config=SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
                                decode_steps=decode_steps))
-    return engine, cfg
+    return engine, model.config
+
+
+def make_engine(raw, dtype, batch, context, block_size, budget, decode_steps=1, num_pages=None,
+                prefix_caching=False):
+    return engine_for(load_random_model(raw, dtype), batch, context, block_size, budget, decode_steps, num_pages,
+                      prefix_caching)
 
 
 def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
@@ -153,7 +165,7 @@ def prefill_run(engine, cfg, tokens, repeats=3):
     return best
 
 
-def serving_run(raw, dtype, workload, budget, decode_steps, rounds=2):
+def serving_run(raw, dtype, workload, budget, decode_steps, rounds=2, model=None):
     """Requests batched continuously under a budget of ``budget`` tokens a step. ``mixed``: 64 requests
     with prompts of 128 to 2,048 random tokens and 256 generated tokens each (the workload that the
     baseline names for the 3B sizes). ``shared-prefix``: 32 requests that share a prefix of 1,024 tokens
@@ -169,8 +181,9 @@ def serving_run(raw, dtype, workload, budget, decode_steps, rounds=2):
     shared = workload == "shared-prefix"
     requests, longest, out_tokens = (32, 1024 + 512, 128) if shared else (64, 2048, 256)
     pages = requests * (-(-(longest + out_tokens) // 16) + 1) + 8
-    engine, cfg = make_engine(raw, dtype, requests, longest + out_tokens - SLACK, 16, budget, decode_steps,
-                              num_pages=pages, prefix_caching=shared)
+    engine, cfg = engine_for(model if model is not None else load_random_model(raw, dtype), requests,
+                             longest + out_tokens - SLACK, 16, budget, decode_steps, num_pages=pages,
+                             prefix_caching=shared)
     rng = random.Random(0)
     prefix = [rng.randrange(cfg.vocab_size) for _ in range(1024)] if shared else []
     result = {}
@@ -195,6 +208,45 @@ def serving_run(raw, dtype, workload, budget, decode_steps, rounds=2):
                   "seconds": round(dt, 4), "engine_steps": steps, "generated_tok_s": round(generated / dt, 1),
                   "total_tok_s": round((prompt_tokens + generated) / dt, 1)}
     return result, cfg
+
+
+def other_shapes(args, short, itemsize):
+    """The baseline's other workloads, each on a model of its own sizes: flat entries for ``points``."""
+    import gc
+
+    import torch
+
+    out = {}
+    k = min(args.decode_steps, 8)
+    steps, warm = min(args.steps, 32), min(args.warmup, 4)
+    for key, shape in (("llama3b", "Llama-3.2-3B"), ("smollm2_1_7b", "SmolLM2-1.7B")):
+        model = load_random_model(dict(SHAPES[shape]), args.dtype)
+        engine, cfg = engine_for(model, 8, args.context, args.block_size, 8192, k)
+        tok_s, ms, _ = decode_run(engine, cfg, 8, args.context, steps, warm, k)
+        out[f"{key}_decode_b8"] = round(tok_s, 1)
+        out[f"{key}_decode_b8_ms"] = round(ms, 4)
+        out[f"{key}_decode_b8_frac"] = round(decode_bytes(cfg, 8, args.context, itemsize) / (ms * 1e-3) / 1e9 / HBM_GBPS, 4)
+        if key == "llama3b":
+            t = prefill_run(engine, cfg, 2048)
+            out[f"{key}_prefill2048"] = round(2048 / t, 1)
+            out[f"{key}_prefill2048_ms"] = round(t * 1e3, 3)
+            out[f"{key}_prefill2048_frac"] = round(prefill_flops(cfg, 2048) / t / PEAK_FLOPS[short], 4)
+        del engine
+        gc.collect()
+        workload, budget = ("mixed", 2048) if key == "llama3b" else ("shared-prefix", 4096)
+        got, _ = serving_run(None, args.dtype, workload, budget, k, model=model)
+        tag = f"{key}_serving_{workload.replace('-', '_')}_budget{budget}"
+        out[f"{tag}_generated_tok_s"] = got["generated_tok_s"]
+        out[f"{tag}_total_tok_s"] = got["total_tok_s"]
+        out[f"{tag}_seconds"] = got["seconds"]
+        out[f"{tag}_requests"] = got["requests"]
+        if workload == "shared-prefix":
+            out[f"{tag}_prompt_tokens"] = got["prompt_tokens"]
+            out[f"{tag}_prompt_tokens_from_cache"] = got["prompt_tokens_from_cache"]
+        del model
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
 
 
 def prefill_flops(cfg, tokens):
@@ -227,6 +279,8 @@ def main() -> int:
                     help="decode steps that one engine step runs on the device before the host looks "
                          "(the timed steps are cut into engine steps of at most this many)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
+    ap.add_argument("--no-other-shapes", action="store_true",
+                    help="skip the points on the Llama-3.2-3B and SmolLM2-1.7B sizes (each loads a model of its own)")
     ap.add_argument("--serving", nargs="?", const="mixed", default=None, choices=["mixed", "shared-prefix"],
                     help="instead of the decode steps, requests batched continuously under --budget tokens a "
                          "step. mixed: 64 requests, prompts of 128 to 2,048 tokens, 256 generated tokens each; "
@@ -310,10 +364,31 @@ def main() -> int:
         for b in (1, 64):   # the headline's context, other batch sizes
             point(f"decode_b{b}", b, args.context, args.decode_steps)
         for b in (1, 8, 64):
-            # one token per engine step, the default of generate() and of the command line
+            # one token per engine step, an engine's own default (generate() and the command line take eight)
             point(f"decode_b{b}_one_token_per_call", b, args.context, 1)
             # prompts of 2,048 tokens with 256 generated: the context grows from 2,048 to 2,304
             point(f"decode_b{b}_context2304", b, 2304, args.decode_steps)
+        if args.shape == "Llama-3.2-1B" and not args.layers:
+            # a long context: 8 requests of 32,768 keys each (attention reads 8.6 GB a step beside 2.5 GB of weights)
+            import gc
+
+            model = engine.core.model
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+            engine, _ = engine_for(model, 8, 32768, args.block_size, 8192, args.decode_steps)
+            point("decode_b8_context32768", 8, 32768, args.decode_steps)
+            del engine, model
+            gc.collect()
+            torch.cuda.empty_cache()
+            if not args.no_other_shapes:
+                points.update(other_shapes(args, short, itemsize))
+                line["config"]["other_shapes"] = (
+                    "llama3b: Llama-3.2-3B sizes (28 layers, hidden 3072, 24 heads of 128, 8 kv heads, intermediate "
+                    "8192, vocab 128256); smollm2_1_7b: SmolLM2-1.7B sizes (24 layers, hidden 2048, 32 heads of 64, "
+                    "32 kv heads, intermediate 8192, vocab 49152); serving: continuous batching, 64 requests with "
+                    "prompts of 128-2048 tokens and 256 generated (mixed) or 32 requests sharing 1024 tokens plus "
+                    "64-512 of their own and 128 generated, page reuse on (shared_prefix)")
         line["points"] = points
     print(json.dumps(line))
     return 0
