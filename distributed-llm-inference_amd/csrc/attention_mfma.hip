@@ -679,17 +679,21 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   // scalar load's answer arrives during the softmax, needs the lookup inside the branch that a wave
   // takes when it sees the tile: the compiler then keeps the pages in vector registers or, told
   // that the branch is uniform, copies the accumulators at its end: 393 -> 529 us at 8,192 tokens.)
-  const int64_t page_elems = (int64_t)page_size * D;
+  // Scalar arithmetic counts here: a wave issues it in turn with its vector instructions, and
+  // all waves of a compute unit share one scalar unit. So a page's offset is one 32 x 32-bit
+  // product onto the kv head's own base (the host checks that a page's elements fit 32 bits).
+  const unsigned page_stride = (unsigned)kv_heads * (unsigned)page_size * (unsigned)D;
+  const bf16_t* k_head = k_pages + (int64_t)kvh * page_size * D;
+  const bf16_t* v_head = v_pages + (int64_t)kvh * page_size * D;
   auto fetch = [&](int t, bf16x8 (&sq)[UCH]) {
-    const int64_t pa = ((int64_t)page_a * kv_heads + kvh) * page_elems;
-    const int64_t pb = ((int64_t)page_b * kv_heads + kvh) * page_elems;
-    const int oa = off_a, ob = off_b;
+    const uint64_t at_a = (uint64_t)(unsigned)page_a * page_stride, at_b = (uint64_t)(unsigned)page_b * page_stride;
+    const unsigned oa = off_a, ob = off_b;
     lookup(t + 32);
 #pragma unroll
     for (int r = 0; r < UCH; ++r) {
       // the same for every lane of the wave: a key's row of K is D long, a key's column of V^T one element
-      const int64_t first = (second_half[r] ? pb : pa) + (second_half[r] ? ob : oa) * (is_v[r] ? 1 : D);
-      const bf16_t* base = (is_v[r] ? v_pages : k_pages) + first;
+      const unsigned off = second_half[r] ? ob : oa;
+      const bf16_t* base = (is_v[r] ? v_head : k_head) + (second_half[r] ? at_b : at_a) + (is_v[r] ? off : off * D);
       sq[r] = *reinterpret_cast<const bf16x8*>(base + lane_off[r]);
     }
   };
@@ -891,6 +895,337 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   }
 }
 
+// ------------------------------------------------------------------------------------ prefill, keys split over two sets of waves
+// For launches of a few workgroups per compute unit. There the shared-tile kernel's time is the
+// time of its longest workgroup, and that is a chain of dependent steps per key tile (LDS reads,
+// first product, softmax, second product, the next tile's staging, the barrier) which one wave a
+// SIMD walks alone: some 1,900 cycles a tile of 32 keys, three times what its instructions take.
+// Here a workgroup has two sets of four waves that work on the SAME queries (a tile of the list,
+// 32 queries a wave as above): every turn stages 64 keys, of which the first set takes the first
+// 32 and the second set the other 32, so the chain is half as many turns long; after the last
+// turn the second set hands its running maximum, sum and output over through LDS and the first
+// set merges them with its own. A workgroup does that for a tile and then for its mirror tile
+// of the same request (tile b of n with tile n-1-b: together always n+1 key tiles, whatever b),
+// so all workgroups of a request take equally long; the workgroups of the lower half of the
+// tile list leave at once. Heads, products and layouts as in the shared-tile kernel.
+template <int DCH>
+__global__ __launch_bounds__(512) void attention_prefill_split_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
+    const int* __restrict__ q_start, const int* __restrict__ kv_len,
+    const int* __restrict__ block_tables, int table_stride, const int* __restrict__ tile_entry,
+    const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
+    int window, int heads_per_wg) {
+  constexpr int D = DCH * 16, DK = D / 32;
+  constexpr int KPAD = D + 8, VPAD = 32 + 8;
+  constexpr int NT = 512;
+  constexpr int CHUNKS = 8 * D;                 // 16-byte chunks of 32 keys: 4D of K, then 4D of V^T
+  constexpr int UCH = 2 * CHUNKS / NT;          // chunks per thread and turn (64 keys): D / 32
+  constexpr int RD = 3;                         // turns in flight from memory to registers
+  constexpr int K_ELEMS = 32 * KPAD, TILE_ELEMS = K_ELEMS + D * VPAD;
+  constexpr int STATE = 2 + 4 * DCH;            // floats of one column tile's state per lane
+  static_assert(2 * STATE * 256 * 4 <= 3 * 2 * TILE_ELEMS * 2, "the hand-over reuses the tile buffers");
+  __shared__ __attribute__((aligned(16))) bf16_t lds[3][2][TILE_ELEMS];  // per turn: keys 0..31, keys 32..63
+
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (gridDim.y % 8 == 0) {  // the tiles of one kv head on one XCD, as in the shared-tile kernel
+    const int linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int slot = linear / 8;
+    by = linear % 8 + 8 * (slot / (int)gridDim.x);
+    bx = slot % (int)gridDim.x;
+  }
+  const int e = tile_entry[bx];
+  const int tok0 = q_start[e];
+  const int q_len = q_start[e + 1] - tok0;
+  const int tile_rows = (4 / heads_per_wg) * 32;
+  const int q0_first = tile_q0[bx];
+  int q0_second = -1;
+  {
+    const int b = q0_first / tile_rows, mirror = (q_len + tile_rows - 1) / tile_rows - 1 - b;
+    if (b < mirror) return;  // the workgroup of the mirror tile does this one too
+    if (mirror < b) q0_second = mirror * tile_rows;
+  }
+  const int group = q_heads / kv_heads;
+  const int wg_per_kv = group / heads_per_wg;
+  const int kvh = by / wg_per_kv;
+  const int lane = threadIdx.x % DLI_WAVE, wave = (threadIdx.x / DLI_WAVE) % 4;
+  const int set = threadIdx.x / 256;  // which 32 of a turn's 64 keys
+  const int col = lane % 16, grp = lane / 16;
+  const int head = kvh * group + (by % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
+  const int n_keys = kv_len[e];
+  const int first_pos = n_keys - q_len;
+  const int* table = block_tables + (int64_t)e * table_stride;
+
+  // Staging: chunk u of a turn, u = thread + r * 512. u / CHUNKS says which 32 keys; within them
+  // chunk v < 4D is 8 dims of key v/(D/8) and chunk 4D+c holds 8 keys of dim (c%2D)/2, of the
+  // first 16 keys for c < 2D and of the other 16 after that. A run of 2D chunks (a multiple of 64)
+  // thus lies in one sixteenth-aligned run of 16 keys, i.e. in one page, and is K or V^T as a
+  // whole: per wave and r, the page's address is made on the scalar unit.
+  const int wave_first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / DLI_WAVE)) * DLI_WAVE;
+  unsigned lane_off[UCH];
+  int lds_off[UCH], v_key[UCH], first_key[UCH];  // first_key: of the chunk's run of 16 keys, within the turn's 64
+  bool is_v[UCH];
+#pragma unroll
+  for (int r = 0; r < UCH; ++r) {
+    const int u = threadIdx.x + r * NT, u_wave = wave_first + r * NT;
+    const int sub = u_wave / CHUNKS, v = u % CHUNKS, v_wave = u_wave % CHUNKS;
+    is_v[r] = v_wave >= 4 * D;
+    const bool second = is_v[r] ? v_wave >= 6 * D : v_wave >= 2 * D;
+    first_key[r] = sub * 32 + (second ? 16 : 0);
+    if (!is_v[r]) {
+      const int kk = v / (D / 8), part = v % (D / 8);
+      lane_off[r] = (kk % 16) * D + part * 8;
+      lds_off[r] = sub * TILE_ELEMS + kk * KPAD + part * 8;
+      v_key[r] = 0;
+    } else {
+      const int c = v - 4 * D, d = (c % (2 * D)) / 2, part = c % 2;
+      lane_off[r] = d * page_size + part * 8;
+      v_key[r] = (second ? 16 : 0) + part * 8;   // within the 32 keys
+      lds_off[r] = sub * TILE_ELEMS + K_ELEMS + d * VPAD + v_key[r];
+      v_key[r] += sub * 32;                       // within the turn's 64
+    }
+  }
+  const unsigned page_stride = (unsigned)kv_heads * (unsigned)page_size * (unsigned)D;
+  const bf16_t* k_head = k_pages + (int64_t)kvh * page_size * D;
+  const bf16_t* v_head = v_pages + (int64_t)kvh * page_size * D;
+  const int turn_pages = 64 / page_size, turn_rest = 64 % page_size;  // 64 keys on, in pages and keys
+
+  typedef short short4a __attribute__((ext_vector_type(4)));
+  union VFrag {
+    bf16x8 v;
+    short4a h[2];
+  };
+
+  for (int phase = 0; phase < 2; ++phase) {
+    const int q0_tile = phase == 0 ? q0_first : q0_second;
+    if (q0_tile < 0) break;
+    const int q0 = q0_tile + (wave / heads_per_wg) * 32;  // this wave's first query
+    const int wave_rows = max(0, min(32, q_len - q0));
+    bf16x8 qreg[2][DK];
+    ColumnTile<DCH> st[2];
+    float m_ref[2], raise_at[2];  // as in the shared-tile kernel: the exponent's reference, and the score that moves it
+    constexpr float LAZY_LOG2 = 8.f;
+    const float inv_scale_log2e = 1.f / scale_log2e;
+    int pos[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      st[j].init();
+      m_ref[j] = 0.f;
+      raise_at[j] = -INFINITY;
+      const int qi = q0 + j * 16 + col;
+      pos[j] = qi < q_len ? first_pos + qi : -1;
+#pragma unroll
+      for (int c = 0; c < DK; ++c) qreg[j][c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (qi < q_len) {
+        const bf16_t* qp = q + (int64_t)(tok0 + qi) * q_stride + (int64_t)head * D + grp * 8;
+#pragma unroll
+        for (int c = 0; c < DK; ++c) qreg[j][c] = *reinterpret_cast<const bf16x8*>(qp + c * 32);
+      }
+    }
+    const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + wave_rows - 1;
+    const int wg_q_hi = min(q_len, q0_tile + tile_rows) - 1;
+    const int begin = window > 0 ? max(0, first_pos + q0_tile - window + 1) / 64 * 64 : 0;
+    const int end = first_pos + wg_q_hi + 1;
+    const int n_turns = (end - begin + 63) / 64;
+
+    // Per chunk of this thread: where the run of 16 keys that it belongs to lies, turn after turn.
+    // Everything here is the same in all lanes of a wave, but it is computed per lane on purpose:
+    // on the scalar unit the table lookups and 64-bit address sums were more instructions a turn
+    // than the softmax, and a wave issues them in turn with its vector instructions.
+    int run_page[UCH], run_off[UCH], run_key[UCH];
+    int page_next[UCH];  // looked up one turn before the keys are fetched
+    int lane_zero;       // zero in a vector register: what is added to it is a value per lane for the compiler
+    asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
+    const int last_page = (n_keys - 1) / page_size;  // entries behind it may hold anything
+#pragma unroll
+    for (int r = 0; r < UCH; ++r) {
+      run_key[r] = begin + first_key[r] + lane_zero;
+      run_page[r] = run_key[r] / page_size;
+      run_off[r] = run_key[r] % page_size;
+      page_next[r] = table[min(run_page[r], last_page)];
+    }
+    bf16x8 stage[RD][UCH];
+    // The same loads whatever the turn, also past the last key (the request's last page again,
+    // never used), so that the count of loads in flight is known at compile time.
+    auto fetch = [&](bf16x8 (&sq)[UCH]) {
+#pragma unroll
+      for (int r = 0; r < UCH; ++r) {
+        const unsigned off = run_off[r];
+        const bf16_t* base = (is_v[r] ? v_head : k_head) + (uint64_t)(unsigned)page_next[r] * page_stride +
+                             (is_v[r] ? off : off * D);
+        sq[r] = *reinterpret_cast<const bf16x8*>(base + lane_off[r]);
+        run_key[r] += 64;
+        run_page[r] += turn_pages;
+        run_off[r] += turn_rest;
+        if (run_off[r] >= page_size) {
+          run_off[r] -= page_size;
+          ++run_page[r];
+        }
+        page_next[r] = table[min(run_page[r], last_page)];
+      }
+    };
+    auto stash = [&](int buf, int t, bf16x8 (&sq)[UCH]) {  // t: the turn's first key
+#pragma unroll
+      for (int r = 0; r < UCH; ++r) {
+        if (t + 64 > n_keys && is_v[r]) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (t + v_key[r] + i >= n_keys) sq[r][i] = (bf16_t)0.f;
+        }
+        *reinterpret_cast<bf16x8*>(&lds[buf][0][lds_off[r]]) = sq[r];
+      }
+    };
+#pragma unroll
+    for (int T = 0; T < 2 + RD; ++T) {
+      fetch(stage[T % RD]);
+      if (T < 2) stash(T, begin + T * 64, stage[T % RD]);
+    }
+    __syncthreads();
+
+    for (int it0 = 0; it0 < n_turns; it0 += RD) {
+#pragma unroll
+      for (int r3 = 0; r3 < RD; ++r3) {
+        const int it = it0 + r3;
+        if (it >= n_turns) break;
+        const int t = begin + it * 64 + set * 32;  // this set's 32 keys
+        if (wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1)) {
+          const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
+          const bf16_t* ks = &lds[it % 3][set][0];
+          const bf16_t* vs = ks + K_ELEMS;
+          bf16x8 kf0[DK], kf1[DK];
+          VFrag vf[DCH];
+#pragma unroll
+          for (int c = 0; c < DK; ++c) {
+            kf0[c] = *reinterpret_cast<const bf16x8*>(ks + col * KPAD + c * 32 + grp * 8);
+            kf1[c] = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KPAD + c * 32 + grp * 8);
+          }
+#pragma unroll
+          for (int c = 0; c < DCH; ++c) {
+            vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 4 * grp);
+            vf[c].h[1] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 16 + 4 * grp);
+          }
+          float4v sa[2], sb[2];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            sa[j] = float4v{0.f, 0.f, 0.f, 0.f};
+            sb[j] = float4v{0.f, 0.f, 0.f, 0.f};
+          }
+#pragma unroll
+          for (int c = 0; c < DK; ++c)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              sa[j] = mfma32(kf0[c], qreg[j][c], sa[j]);
+              sb[j] = mfma32(kf1[c], qreg[j][c], sb[j]);
+            }
+          float sv[2][8];
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              sv[j][i] = sa[j][i];
+              sv[j][4 + i] = sb[j][i];
+            }
+          if (need_mask) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int low = window > 0 ? pos[j] - window + 1 : 0;
+#pragma unroll
+              for (int i = 0; i < 8; ++i) {
+                const int key = t + (i < 4 ? 4 * grp + i : 16 + 4 * grp + i - 4);
+                if (key > pos[j] || key < low) sv[j][i] = -INFINITY;
+              }
+            }
+          }
+          float lane_max[2];
+          bool rise = false;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            lane_max[j] = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]),
+                               max2(sv[j][6], sv[j][7]));
+            rise |= lane_max[j] > raise_at[j];
+          }
+          if (__builtin_amdgcn_ballot_w64(rise) != 0) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const float tile_max = column_max(lane_max[j]) * scale_log2e;
+              const float m_new = max2(st[j].m, tile_max);
+              const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+              const float alpha = fast_exp2(st[j].m - m_safe);
+              st[j].l *= alpha;
+#pragma unroll
+              for (int c = 0; c < DCH; ++c) st[j].o[c] *= alpha;
+              st[j].m = m_new;
+              m_ref[j] = m_safe;
+              raise_at[j] = m_new == -INFINITY ? -INFINITY : (m_new + LAZY_LOG2) * inv_scale_log2e;
+            }
+          }
+          bf16x8 pb[2];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            float tile_sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const float p = fast_exp2(fmaf(sv[j][i], scale_log2e, -m_ref[j]));
+              tile_sum += p;
+              pb[j][i] = (bf16_t)p;
+            }
+            st[j].l += tile_sum;
+          }
+#pragma unroll
+          for (int c = 0; c < DCH; ++c)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
+        }
+        // turn it+2 leaves its register slot for LDS; the slot then receives turn it+2+RD
+        stash((it + 2) % 3, begin + (it + 2) * 64, stage[(r3 + 2) % RD]);
+        fetch(stage[(r3 + 2) % RD]);
+        __syncthreads();
+      }
+    }
+
+    // The second set hands over, the first merges: state v of lane l of wave w lies at
+    // [v][w * 64 + l], so that a wave's accesses are consecutive.
+    float* hand = reinterpret_cast<float*>(&lds[0][0][0]);
+    const int mine = wave * DLI_WAVE + lane;
+    if (set == 1) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        hand[(j * STATE + 0) * 256 + mine] = st[j].m;
+        hand[(j * STATE + 1) * 256 + mine] = st[j].l;
+#pragma unroll
+        for (int c = 0; c < DCH; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) hand[(j * STATE + 2 + 4 * c + i) * 256 + mine] = st[j].o[c][i];
+      }
+    }
+    __syncthreads();
+    if (set == 0) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float m_other = hand[(j * STATE + 0) * 256 + mine], l_other = hand[(j * STATE + 1) * 256 + mine];
+        const float m_all = max2(st[j].m, m_other);
+        const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+        const float a_mine = fast_exp2(st[j].m - m_safe), a_other = fast_exp2(m_other - m_safe);
+        const float l_sum = column_sum(st[j].l * a_mine + l_other * a_other);  // every lane takes part
+        const int qi = q0 + j * 16 + col;
+        if (qi >= q_len) continue;
+        const float inv = l_sum > 0.f ? 1.f / l_sum : 0.f;
+        bf16_t* op = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * D + 4 * grp;
+#pragma unroll
+        for (int c = 0; c < DCH; ++c) {
+          float o[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            o[i] = (st[j].o[c][i] * a_mine + hand[(j * STATE + 2 + 4 * c + i) * 256 + mine] * a_other) * inv;
+          const short4v packed = {bf16_bits(o[0]), bf16_bits(o[1]), bf16_bits(o[2]), bf16_bits(o[3])};
+          *reinterpret_cast<short4v*>(op + c * 16) = packed;
+        }
+      }
+    }
+    __syncthreads();  // the tile buffers are staged again for the mirror tile
+  }
+}
+
 // ------------------------------------------------------------------------------------ host side
 #define LOG2E 1.4426950408889634f
 
@@ -1071,22 +1406,30 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
     return DLI_ERR_ARGUMENT;
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (hw > 0) {
+    if ((int64_t)kv_heads * page_size * head_dim >= ((int64_t)1 << 31)) return DLI_ERR_ARGUMENT;  // the kernel's 32 bits
     const dim3 sgrid(tiles, q_heads / hw);
-    // Mirror tiles are paired (pair_tiles 1, or -1 and a launch in the range where it was faster):
-    // with too few workgroups pairing leaves compute units idle; with three or more a unit, the
-    // tiles listed longest first even the causal triangle out through the queue of workgroups,
-    // and the single-tile kernel's waves do not wait for one another. Heads of up to 64: from two
-    // to under three workgroups per unit (2,048 tokens at the 1B sizes: 50 against 55 us; 3,072:
-    // 127 against 92; 4,096: 161 against 122; 8,192: 565 against 393); larger heads, whose
-    // single-tile kernel holds one wave a SIMD: from one to under three a unit (heads of 128, 24
-    // of them, 2,048 tokens: 74 against 103 us; 8,192: 675 against 615).
-    // The tile list has to hold all tiles of a request.
+    // Which kernel (pair_tiles 0, 1 or 2; -1: by the size of the launch). With three or more
+    // workgroups a compute unit, every tile has a workgroup of its own (0): listed longest first,
+    // the tiles even the causal triangle out through the queue of workgroups, and no wave waits
+    // for a wave of another tile. With fewer, the launch is as long as its longest workgroup: then
+    // a workgroup takes a tile and its mirror tile, heads of up to 64 one after the other with the
+    // keys of each shared out to two sets of waves (2), larger heads, for which that kernel runs
+    // out of registers, side by side (1). Below one workgroup a unit pairing would leave units idle.
+    // Per layer at the 1B sizes, kernels 0 / 1 / 2: 2,048 tokens 57 / 52 / 46 us, 3,072 tokens
+    // 90 / 120 / 114, 4,096 tokens 129 / 173 / 148; 24 heads of 128: 2,048 tokens 104 / 76 / 83,
+    // 4,096 tokens 216 / 237 / 252. The tile list has to hold all tiles of a request.
     const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
-    const bool in_range = launch < 3 * units && launch >= (head_dim <= 64 ? 2 : 1) * units;
-    const bool pair = pair_tiles >= 0 ? pair_tiles != 0 : in_range;
+    const bool in_range = launch >= units && launch < 3 * units;
+    const int mode = pair_tiles >= 0 ? pair_tiles : (in_range ? (head_dim <= 64 ? 2 : 1) : 0);
+    const bool pair = mode == 1;
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \
-    if (pair)                                                                                     \
+    if (mode == 2)                                                                                \
+      attention_prefill_split_kernel<N><<<sgrid, 512, 0, stream>>>(                               \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
+          (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \
+          tile_q0, q_heads, kv_heads, page_size, scale * LOG2E, window, hw);                      \
+    else if (pair)                                                                                \
       attention_prefill_shared_kernel<N, true><<<sgrid, 512, 0, stream>>>(                        \
           (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
           (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \

@@ -1102,13 +1102,15 @@ def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, dtype: torch.dt
 def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
                       tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
-                      window: int = 0, pair_tiles: Optional[bool] = None) -> None:
+                      window: int = 0, pair_tiles: Optional[int] = None) -> None:
     """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
     :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height and
     hold every tile of every listed request, in any order: workgroups start in the list's order,
     so the tiles with the most keys belong first). ``pair_tiles``:
-    whether one workgroup takes a tile and its mirror within the request, which evens out the
-    causal mask's triangle; ``None`` lets the kernel decide by the size of the launch."""
+    1: one workgroup takes a tile and its mirror within the request side by side, which evens out
+    the causal mask's triangle; 2: it takes them one after the other with two sets of waves that
+    share each tile's keys (half as many dependent steps, for launches of few workgroups); 0:
+    every tile has its own workgroup; ``None`` lets the kernel decide by the size of the launch."""
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
     for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
         _dense(t, name, torch.int32, 1)

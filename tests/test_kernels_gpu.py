@@ -323,10 +323,11 @@ def test_the_merging_o_projection_refuses_what_it_does_not_take(ops):
 
 @pytest.mark.parametrize("qh,kvh,d,bs", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37])
-@pytest.mark.parametrize("pair", [False, True])
+@pytest.mark.parametrize("pair", [0, 1, 2])
 def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window, pair):
-    """Portions of every shape against their caches; `pair`: a workgroup takes a tile and its mirror
-    tile of the same request (odd and even numbers of tiles, one tile only, half-filled last tiles)."""
+    """Portions of every shape against their caches; `pair` 1: a workgroup takes a tile and its mirror
+    tile of the same request (odd and even numbers of tiles, one tile only, half-filled last tiles);
+    2: it takes them one after the other, two sets of waves sharing each tile's keys."""
     lens = [(2, 2), (7, 7), (33, 33), (5, 40), (2, 131), (129, 129), (16, 16), (31, 300), (140, 333), (1, 50),
             (257, 257), (200, 420)]
     q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=d + bs)
