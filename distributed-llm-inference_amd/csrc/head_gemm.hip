@@ -13,6 +13,10 @@
 // Weights in tile order (16 features x 128 k contiguous, see skinny_gemm.hip); 4 waves split k and
 // add up through LDS in wave order: the same sums in the same order as the tile-by-tile kernel's
 // shape of 4 k-waves x 2 tiles, to the bit. Rows: at most 16. K = 512 * KB.
+// The wave that stores the logits has every one of them in a register once: asked to, it keeps
+// each row's best (value, lowest index) among the logits of its workgroup and leaves it as one
+// part of the row's argmax, so that the sampler's first stage (a kernel that reads all logits
+// again) need not run.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -30,7 +34,7 @@ template <int KB, bool NORM>
 __global__ __launch_bounds__(HEAD_KS * 64) void head_gemm_kernel(
     const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
     const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w, float* __restrict__ out,
-    int64_t ldo, int M, int N, int K) {
+    int64_t ldo, int M, int N, int K, float* __restrict__ best_val, int* __restrict__ best_idx) {
   constexpr int KS = HEAD_KS;
   __shared__ float red[2][KS - 1][2][4][64];  // two pairs of tiles in turn
 
@@ -108,6 +112,8 @@ __global__ __launch_bounds__(HEAD_KS * 64) void head_gemm_kernel(
 
   static_assert(KB % 2 == 0, "the two weight buffers take turns in a fixed order");
   bf16x8 wf[2][2][4];
+  float top_v = -INFINITY;  // wave 0: the best logit of row col among those this lane stored, and its index
+  int top_i = 0x7fffffff;
   int pair = blockIdx.x;
   if (pair < pairs) load_block(wf[0], pair, 0);
   for (int turn = 0; pair < pairs; pair += gridDim.x, ++turn) {
@@ -148,11 +154,32 @@ __global__ __launch_bounds__(HEAD_KS * 64) void head_gemm_kernel(
           float v = acc[j][i];
           for (int wv = 0; wv < KS - 1; ++wv) v += red[buf][wv][j][i][lane];
           y[i] = v;
+          const int n = tile * 16 + 4 * grp + i;
+          if (v > top_v || (v == top_v && n < top_i)) {
+            top_v = v;
+            top_i = n;
+          }
         }
         // lane holds y[m = col][n = 16*tile + 4*grp + i] (storing whole lines of a row instead,
         // turned through LDS, changed nothing: the kernel's time is the table's)
         if (col < M) *reinterpret_cast<float4v*>(out + (int64_t)col * ldo + tile * 16 + 4 * grp) = y;
       }
+    }
+  }
+  if (best_val != nullptr && ks == 0) {
+    // part blockIdx.x of row col: the best of the four lanes that hold the row's logits
+#pragma unroll
+    for (int m = 16; m < 64; m <<= 1) {
+      const float ov = __shfl_xor(top_v, m, 64);
+      const int oi = __shfl_xor(top_i, m, 64);
+      if (ov > top_v || (ov == top_v && oi < top_i)) {
+        top_v = ov;
+        top_i = oi;
+      }
+    }
+    if (grp == 0 && col < M) {
+      best_val[(int64_t)col * gridDim.x + blockIdx.x] = top_v;
+      best_idx[(int64_t)col * gridDim.x + blockIdx.x] = top_i;
     }
   }
 }
@@ -168,27 +195,34 @@ extern "C" int dli_head_gemm_supports(int M, int N, int K) {
 // out float32 [M][N] (row stride ldo, a multiple of 4). norm_w float32 [K] or null (then xhat = x);
 // ssq_in float32 [ssq_parts][M]. workgroups: how many stay for the launch (0: one per compute unit,
 // which is ahead of two and more at every row count: 93 against 96 us at 8 rows, 97 against 100 at 16).
+// best_val / best_idx (both or neither): [M][dli_head_gemm_workgroups(N, workgroups)], each row's best
+// logit and its lowest index among the logits of each workgroup (the first stage of an argmax).
+extern "C" int dli_head_gemm_workgroups(int N, int workgroups) {
+  const int pairs = (N / 16 + 1) / 2;
+  const int grid = workgroups > 0 ? workgroups : dli_compute_units();
+  return grid > pairs ? pairs : grid;
+}
+
 extern "C" int dli_head_gemm(const void* x, int64_t ldx, const float* ssq_in, int ssq_parts, const float* norm_w,
                              float eps, const void* w_tiled, float* out, int64_t ldo, int M, int N, int K,
-                             int workgroups, hipStream_t stream) {
+                             int workgroups, float* best_val, int* best_idx, hipStream_t stream) {
   if (M <= 0 || N <= 0) return DLI_OK;
+  if ((best_val == nullptr) != (best_idx == nullptr)) return DLI_ERR_ARGUMENT;
   if (!dli_head_gemm_supports(M, N, K) || x == nullptr || w_tiled == nullptr || out == nullptr || ldx % 8 != 0 ||
       ldx < K || ldo % 4 != 0 || ldo < N || workgroups < 0 ||
       (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)))
     return DLI_ERR_ARGUMENT;
-  const int pairs = (N / 16 + 1) / 2;
-  int grid = workgroups > 0 ? workgroups : dli_compute_units();
-  if (grid > pairs) grid = pairs;
+  const int grid = dli_head_gemm_workgroups(N, workgroups);
 #define HEAD_CASE(KB)                                                                                          \
   case KB:                                                                                                     \
     if (norm_w != nullptr)                                                                                     \
       head_gemm_kernel<KB, true><<<grid, HEAD_KS * 64, 0, stream>>>((const bf16_t*)x, ldx, ssq_in, ssq_parts,   \
                                                                    norm_w, eps, (const bf16_t*)w_tiled, out,   \
-                                                                   ldo, M, N, K);                              \
+                                                                   ldo, M, N, K, best_val, best_idx);          \
     else                                                                                                       \
       head_gemm_kernel<KB, false><<<grid, HEAD_KS * 64, 0, stream>>>((const bf16_t*)x, ldx, ssq_in, ssq_parts,  \
                                                                     norm_w, eps, (const bf16_t*)w_tiled, out,  \
-                                                                    ldo, M, N, K);                             \
+                                                                    ldo, M, N, K, best_val, best_idx);         \
     break;
   switch (K / (128 * HEAD_KS)) {
     HEAD_CASE(2) HEAD_CASE(4) HEAD_CASE(6) HEAD_CASE(8)

@@ -94,12 +94,46 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
   }
 }
 
+// Between two decode steps that run back to back on the device: row i's sampled token becomes
+// its next input, its position and key count grow by one, its draw counter moves on, and its
+// cache slot in each group of layers is looked up in its block table. Rows without keys
+// (padding) are left alone. `tokens_out` receives the sampled tokens of the step that has just
+// run; with advance == 0 nothing else is done (the last step of a run).
+#define ADVANCE_MAX_GROUPS 4
+struct AdvanceGroups {
+  int* slots[ADVANCE_MAX_GROUPS];
+  const int* tables[ADVANCE_MAX_GROUPS];
+};
+struct AdvanceArgs {
+  int* tokens_out;  // null: the sampling kernel does none of this
+  int* token_ids;
+  int* positions;
+  int* kv_len;
+  uint64_t* counters;
+  AdvanceGroups groups;
+  int n_groups, table_stride, page_size, advance;
+};
+
+__device__ __forceinline__ void advance_row(const AdvanceArgs& a, int i, int tok) {
+  a.tokens_out[i] = tok;
+  if (!a.advance || a.kv_len[i] <= 0) return;
+  const int pos = a.positions[i] + 1;
+  a.token_ids[i] = tok;
+  a.positions[i] = pos;
+  a.kv_len[i] += 1;
+  a.counters[i] += 1;
+  for (int g = 0; g < a.n_groups; ++g) {
+    const int page = a.groups.tables[g][(int64_t)i * a.table_stride + pos / a.page_size];
+    a.groups.slots[g][i] = page * a.page_size + pos % a.page_size;
+  }
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int64_t row_stride, int vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint64_t* __restrict__ seeds,
     const uint64_t* __restrict__ counters, const float* __restrict__ part_val,
-    const int* __restrict__ part_idx, int* __restrict__ out) {
+    const int* __restrict__ part_idx, int parts, int* __restrict__ out, AdvanceArgs next) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
   __shared__ ArgBest best[16];
@@ -112,10 +146,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int k = top_k[row];
   const bool greedy = temp == 0.f || k == 1;
 
-  // maximum (and its lowest index), from the chunks' results of stage one
+  // maximum (and its lowest index), from the `parts` results of stage one
   ArgBest mine = {-INFINITY, 0x7fffffff};
-  if (tid < ARGMAX_CHUNKS)
-    mine = ArgBest{part_val[row * ARGMAX_CHUNKS + tid], part_idx[row * ARGMAX_CHUNKS + tid]};
+  if (tid < parts) mine = ArgBest{part_val[(int64_t)row * parts + tid], part_idx[(int64_t)row * parts + tid]};
 #pragma unroll
   for (int m = DLI_WAVE / 2; m > 0; m >>= 1) {
     ArgBest o;
@@ -128,9 +161,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   ArgBest top = best[0];
   for (int w = 1; w < (int)(blockDim.x / DLI_WAVE); ++w) top = better(top, best[w]);
   if (greedy) {
-    if (tid == 0) out[row] = top.i;
+    if (tid == 0) {
+      out[row] = top.i;
+      if (next.tokens_out != nullptr) advance_row(next, row, top.i);
+    }
     return;
   }
+  // the draw's counter, before this row moves on to its next draw
+  const uint64_t draw = counters[row];
 
   const float inv_t = 1.f / temp;
   const float xmax = top.v * inv_t;
@@ -187,7 +225,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (tid == 0) {
     float total = 0.f;
     for (int i = 0; i < (int)blockDim.x; ++i) total += chunk_sums[i];
-    const float u = (float)(philox_first_word(seeds[row], counters[row]) >> 8) * (1.0f / 16777216.0f);
+    const float u = (float)(philox_first_word(seeds[row], draw) >> 8) * (1.0f / 16777216.0f);
     const float target = u * total;
     float run = 0.f;
     int owner = -1;
@@ -215,8 +253,12 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       }
     }
     out[row] = pick;
+    if (next.tokens_out != nullptr) advance_row(next, row, pick);
   }
-  if (chosen < 0 && tid == 0) out[row] = top.i;  // no mass at all (cannot happen: the maximum is kept)
+  if (chosen < 0 && tid == 0) {  // no mass at all (cannot happen: the maximum is kept)
+    out[row] = top.i;
+    if (next.tokens_out != nullptr) advance_row(next, row, top.i);
+  }
 }
 
 // Floats and ints of scratch that dli_sample needs per row.
@@ -232,40 +274,55 @@ extern "C" int dli_sample(const float* logits, int64_t row_stride, int rows, int
   argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, rows), 256, 0, stream>>>(logits, row_stride, vocab,
                                                                        part_val, part_idx);
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
-  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab, temperature, top_k,
-                                                     top_p, seeds, counters, part_val, part_idx, out);
+  AdvanceArgs none = {};
+  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab, temperature, top_k, top_p, seeds,
+                                                     counters, part_val, part_idx, ARGMAX_CHUNKS, out, none);
   return dli_launch_status();
 }
 
-// Between two decode steps that run back to back on the device: row i's sampled token becomes
-// its next input, its position and key count grow by one, its draw counter moves on, and its
-// cache slot in each group of layers is looked up in its block table. Rows without keys
-// (padding) are left alone. `tokens_out` receives the sampled tokens of the step that has just
-// run; with advance == 0 nothing else is done (the last step of a run).
-#define ADVANCE_MAX_GROUPS 4
-struct AdvanceGroups {
-  int* slots[ADVANCE_MAX_GROUPS];
-  const int* tables[ADVANCE_MAX_GROUPS];
-};
-__global__ void decode_advance_kernel(const int* __restrict__ sampled, int* __restrict__ tokens_out,
-                                      int* __restrict__ token_ids, int* __restrict__ positions,
-                                      int* __restrict__ kv_len, uint64_t* __restrict__ counters,
-                                      AdvanceGroups groups, int n_groups, int table_stride,
-                                      int page_size, int rows, int advance) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= rows) return;
-  const int tok = sampled[i];
-  tokens_out[i] = tok;
-  if (!advance || kv_len[i] <= 0) return;
-  const int pos = positions[i] + 1;
-  token_ids[i] = tok;
-  positions[i] = pos;
-  kv_len[i] += 1;
-  counters[i] += 1;
-  for (int g = 0; g < n_groups; ++g) {
-    const int page = groups.tables[g][(int64_t)i * table_stride + pos / page_size];
-    groups.slots[g][i] = page * page_size + pos % page_size;
+static bool fill_groups(AdvanceGroups& groups, int* const* slots, const int* const* tables, int n_groups) {
+  if (n_groups < 0 || n_groups > ADVANCE_MAX_GROUPS) return false;
+  for (int g = 0; g < ADVANCE_MAX_GROUPS; ++g) {
+    groups.slots[g] = g < n_groups ? slots[g] : nullptr;
+    groups.tables[g] = g < n_groups ? tables[g] : nullptr;
+    if (g < n_groups && (groups.slots[g] == nullptr || groups.tables[g] == nullptr)) return false;
   }
+  return true;
+}
+
+// dli_sample and dli_decode_advance in one: the thread that chooses a row's token also hands it to
+// the row's next step, so a decode step inside a graph ends with one kernel less. `parts` > 0:
+// stage one of the argmax has been done by whoever made the logits (dli_head_gemm), part_val and
+// part_idx hold [rows][parts]; 0: it runs here (they then need dli_sample_scratch_per_row() per row).
+extern "C" int dli_sample_and_advance(const float* logits, int64_t row_stride, int rows, int vocab,
+                                      const float* temperature, const int* top_k, const float* top_p,
+                                      const uint64_t* seeds, uint64_t* counters, float* part_val, int* part_idx,
+                                      int parts, int* out, int* tokens_out, int* token_ids, int* positions,
+                                      int* kv_len, int* const* slots, const int* const* tables, int n_groups,
+                                      int table_stride, int page_size, int advance, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (vocab <= 0 || row_stride < vocab || rows > 65535 || part_val == nullptr || part_idx == nullptr ||
+      parts < 0 || parts > SAMPLE_THREADS || out == nullptr || tokens_out == nullptr || token_ids == nullptr ||
+      positions == nullptr || kv_len == nullptr || counters == nullptr || page_size <= 0 || table_stride <= 0)
+    return DLI_ERR_ARGUMENT;
+  AdvanceArgs next = {tokens_out, token_ids, positions, kv_len, counters, {}, n_groups, table_stride, page_size,
+                      advance};
+  if (!fill_groups(next.groups, slots, tables, n_groups)) return DLI_ERR_ARGUMENT;
+  if (parts == 0) {
+    argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, rows), 256, 0, stream>>>(logits, row_stride, vocab, part_val,
+                                                                         part_idx);
+    if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
+    parts = ARGMAX_CHUNKS;
+  }
+  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab, temperature, top_k, top_p, seeds,
+                                                     counters, part_val, part_idx, parts, out, next);
+  return dli_launch_status();
+}
+
+// The same hand-over as a kernel of its own (for steps whose tokens were chosen elsewhere).
+__global__ void decode_advance_kernel(const int* __restrict__ sampled, AdvanceArgs next, int rows) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < rows) advance_row(next, i, sampled[i]);
 }
 
 extern "C" int dli_decode_advance(const int* sampled, int* tokens_out, int* token_ids, int* positions,
@@ -273,15 +330,10 @@ extern "C" int dli_decode_advance(const int* sampled, int* tokens_out, int* toke
                                   const int* const* tables, int n_groups, int table_stride,
                                   int page_size, int rows, int advance, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
-  if (n_groups < 0 || n_groups > ADVANCE_MAX_GROUPS || page_size <= 0 || table_stride <= 0)
-    return DLI_ERR_ARGUMENT;
-  AdvanceGroups groups;
-  for (int g = 0; g < ADVANCE_MAX_GROUPS; ++g) {
-    groups.slots[g] = g < n_groups ? slots[g] : nullptr;
-    groups.tables[g] = g < n_groups ? tables[g] : nullptr;
-  }
-  decode_advance_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(sampled, tokens_out, token_ids, positions,
-                                                                kv_len, counters, groups, n_groups,
-                                                                table_stride, page_size, rows, advance);
+  if (page_size <= 0 || table_stride <= 0 || tokens_out == nullptr) return DLI_ERR_ARGUMENT;
+  AdvanceArgs next = {tokens_out, token_ids, positions, kv_len, counters, {}, n_groups, table_stride, page_size,
+                      advance};
+  if (!fill_groups(next.groups, slots, tables, n_groups)) return DLI_ERR_ARGUMENT;
+  decode_advance_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(sampled, next, rows);
   return dli_launch_status();
 }

@@ -106,6 +106,9 @@ class StepContext:
     # per mixer (``id(mixer)``), what it answered to ``Mixer.decode_plan`` for this step: set only
     # on the context of a recorded step, whose host arrays say nothing about the steps it will replay
     decode_plans: dict = field(default_factory=dict)
+    # where the head may leave the first stage of every row's argmax (``parts.base.ArgmaxStage``):
+    # offered by a step that chooses every row's token on the device right after the forward pass
+    argmax_stage: Any = None
     _tiles: dict = field(default_factory=dict)
     _memo: dict = field(default_factory=dict)
 

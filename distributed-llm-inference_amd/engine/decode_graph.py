@@ -26,6 +26,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
+from ..parts.base import ArgmaxStage
 from .batch import GroupView, StepContext, StepEntry
 from .table_rows import TableRows
 
@@ -130,20 +131,23 @@ class DecodeGraphs:
             tokens_dev = torch.zeros(b, dtype=torch.int32, device=dev_name)
             tokens_all = torch.zeros(steps, b, dtype=torch.int32, device=dev_name)
             scratch = ops.sample_scratch(b, dev_name)
+            stage = ArgmaxStage(scratch)
+            ctx.argmax_stage = stage
         ps = self.step_fn.manager.page_size
 
         def body(steps=steps):
             # `steps` decode steps back to back: after each, the sampled tokens become the next
             # inputs and positions, lengths, slots and draw counters move on, all on the device
             for j in range(steps):
+                if sampled:
+                    stage.parts = 0  # the head may do the first stage of the argmax and say so
                 logits = model.forward(ctx, caches)
                 if sampled:
-                    ops.sample(logits, dv["temperature"].view(torch.float32), dv["top_k"],
-                               dv["top_p"].view(torch.float32), dv["seeds"].view(torch.int64),
-                               dv["counters"].view(torch.int64), tokens_dev, scratch)
-                    ops.decode_advance(tokens_dev, tokens_all[j], dv["token_ids"], dv["positions"], dv["kv_len"],
-                                       dv["counters"].view(torch.int64), [g.slots for g in groups],
-                                       [g.block_tables for g in groups], ps, advance=j + 1 < steps)
+                    ops.sample_and_advance(
+                        logits, dv["temperature"].view(torch.float32), dv["top_k"], dv["top_p"].view(torch.float32),
+                        dv["seeds"].view(torch.int64), dv["counters"].view(torch.int64), tokens_dev, scratch,
+                        stage.parts, tokens_all[j], dv["token_ids"], dv["positions"], dv["kv_len"],
+                        [g.slots for g in groups], [g.block_tables for g in groups], ps, advance=j + 1 < steps)
             if sampled:
                 tokens_host.copy_(tokens_all.view(-1), non_blocking=True)
             return logits

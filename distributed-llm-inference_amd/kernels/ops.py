@@ -45,6 +45,9 @@ _SIGNATURES = {
     "dli_sample": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                    _c_ptr],
     "dli_sample_scratch_per_row": [],
+    "dli_sample_and_advance": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                               _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                               _c_int, _c_ptr],
     "dli_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
                            _c_int, _c_int, _c_ptr],
     "dli_skinny_gemm_max_rows": [],
@@ -55,7 +58,8 @@ _SIGNATURES = {
                                  _c_int, _c_ptr],
     "dli_head_gemm_supports": [_c_int, _c_int, _c_int],
     "dli_head_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int,
-                      _c_int, _c_ptr],
+                      _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "dli_head_gemm_workgroups": [_c_int, _c_int],
     "dli_skinny_gemm_merged": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int,
                                _c_int, _c_int, _c_ptr],
     "dli_mid_gemm": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_int,
@@ -516,13 +520,17 @@ def head_gemm_supports(rows: int, n: int, k: int, dtype: torch.dtype) -> bool:
 
 
 def head_gemm(x: torch.Tensor, w_tiled: torch.Tensor, out: torch.Tensor, norm_w: Optional[torch.Tensor] = None,
-              eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None, workgroups: int = 0) -> None:
+              eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None, workgroups: int = 0,
+              best: Optional[tuple[torch.Tensor, torch.Tensor]] = None) -> int:
     """``out = xhat @ w.T`` as float32 for at most 16 rows and the many rows of a vocabulary:
     workgroups that stay for the whole launch walk the tiles of ``w_tiled`` (:func:`tile_weights`
     of ``w [n, k]``) in turn, each wave keeping its normalised activations in registers. ``norm_w``,
     ``eps``, ``ssq_in [parts, rows]``: the RMSNorm of ``x`` as in :func:`skinny_gemm`. The sums are
     those of :func:`skinny_gemm` with ``shape=4``, to the bit. ``workgroups``: how many (0: one per
-    compute unit)."""
+    compute unit). ``best``: float32 values and int32 indices (the scratch of :func:`sample_scratch`); each
+    workgroup then leaves every row's best logit and its lowest index among the logits it made, as
+    ``[rows, parts]`` at the start of both, and the number of parts comes back (the first stage of
+    :func:`sample_and_advance`'s argmax); without it 0."""
     _rows(x, "x", torch.bfloat16)
     m, k = x.shape
     _rows(out, "out", torch.float32)
@@ -542,8 +550,17 @@ def head_gemm(x: torch.Tensor, w_tiled: torch.Tensor, out: torch.Tensor, norm_w:
         _dense(ssq_in, "ssq_in", torch.float32, 2)
         _require(ssq_in.shape[1] == m and ssq_in.shape[0] >= 1, "ssq_in must be [parts, rows]")
         parts = ssq_in.shape[0]
+    groups = 0
+    if best is not None:
+        groups = int(library().dli_head_gemm_workgroups(n, int(workgroups)))
+        _dense(best[0], "best values", torch.float32)
+        _dense(best[1], "best indices", torch.int32)
+        _require(best[0].numel() >= m * groups and best[1].numel() >= m * groups, "the argmax's scratch is too small")
     _check(library().dli_head_gemm(_ptr(x), x.stride(0), _ptr(ssq_in), parts, _ptr(norm_w), float(eps), _ptr(w_tiled),
-                                   _ptr(out), out.stride(0), m, n, k, int(workgroups), _stream()), "head_gemm")
+                                   _ptr(out), out.stride(0), m, n, k, int(workgroups),
+                                   _ptr(best[0]) if best is not None else None,
+                                   _ptr(best[1]) if best is not None else None, _stream()), "head_gemm")
+    return groups
 
 
 MERGED_ROWS, MERGED_SPLITS, _MERGED_RANGE = 4, 16, 512  # csrc/skinny_gemm.hip: MERGE_ROWS, MERGE_SPLITS, MERGE_RANGE
@@ -1129,8 +1146,8 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
 
 def sample_scratch(rows: int, device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
     """Scratch that :func:`sample` needs for ``rows`` rows (values and indices of the argmax's
-    first stage)."""
-    per = int(library().dli_sample_scratch_per_row())
+    first stage: its own chunks, or one part per workgroup of a logits kernel that does that stage)."""
+    per = max(int(library().dli_sample_scratch_per_row()), compute_units(device))
     return (torch.empty(rows * per, device=device, dtype=torch.float32),
             torch.empty(rows * per, device=device, dtype=torch.int32))
 
@@ -1163,6 +1180,53 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _check(library().dli_sample(_ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k),
                                 _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(scratch[0]), _ptr(scratch[1]),
                                 _ptr(out), _stream()), "sample")
+
+
+def sample_and_advance(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+                       seeds: torch.Tensor, counters: torch.Tensor, out: torch.Tensor,
+                       scratch: tuple[torch.Tensor, torch.Tensor], parts: int, tokens_out: torch.Tensor,
+                       token_ids: torch.Tensor, positions: torch.Tensor, kv_len: torch.Tensor,
+                       slots: Sequence[torch.Tensor], tables: Sequence[torch.Tensor], page_size: int,
+                       advance: bool) -> None:
+    """:func:`sample` and :func:`decode_advance` in one launch (for decode steps recorded into a
+    graph): the thread that chooses a row's token hands it on. ``parts`` > 0: ``scratch`` already
+    holds the first stage of every row's argmax as ``[rows, parts]`` (:func:`head_gemm` with
+    ``best``), and the kernel that reads all logits for it does not run."""
+    _rows(logits, "logits", torch.float32)
+    rows, vocab = logits.shape
+    _dense(temperature, "temperature", torch.float32, 1)
+    _dense(top_p, "top_p", torch.float32, 1)
+    _dense(seeds, "seeds", torch.int64, 1)
+    _dense(counters, "counters", torch.int64, 1)
+    for name, t in (("top_k", top_k), ("out", out), ("tokens_out", tokens_out), ("token_ids", token_ids),
+                    ("positions", positions), ("kv_len", kv_len)):
+        _dense(t, name, torch.int32, 1)
+    for name, t in (("temperature", temperature), ("top_k", top_k), ("top_p", top_p), ("seeds", seeds),
+                    ("counters", counters), ("out", out), ("tokens_out", tokens_out), ("token_ids", token_ids),
+                    ("positions", positions), ("kv_len", kv_len)):
+        _require(t.shape[0] == rows, f"{name} must have one value per row")
+    per = int(library().dli_sample_scratch_per_row())
+    _dense(scratch[0], "scratch values", torch.float32)
+    _dense(scratch[1], "scratch indices", torch.int32)
+    need = rows * (parts if parts > 0 else per)
+    _require(0 <= parts <= 1024 and scratch[0].numel() >= need and scratch[1].numel() >= need,
+             "sampling scratch is too small")
+    _require(len(slots) == len(tables) <= 4, "one slot vector and one table per group, at most 4 groups")
+    width = 1
+    for g, (sl, tb) in enumerate(zip(slots, tables)):
+        _dense(sl, f"slots[{g}]", torch.int32, 1)
+        _dense(tb, f"tables[{g}]", torch.int32, 2)
+        _require(sl.shape[0] == rows and tb.shape[0] == rows, "slots and tables must have one row per request")
+        _require(g == 0 or tb.shape[1] == width, "the groups' tables differ in width")
+        width = tb.shape[1]
+    n = len(slots)
+    slot_ptrs = (ctypes.c_void_p * 4)(*([t.data_ptr() for t in slots] + [None] * (4 - n)))
+    table_ptrs = (ctypes.c_void_p * 4)(*([t.data_ptr() for t in tables] + [None] * (4 - n)))
+    _check(library().dli_sample_and_advance(
+        _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
+        _ptr(counters), _ptr(scratch[0]), _ptr(scratch[1]), int(parts), _ptr(out), _ptr(tokens_out), _ptr(token_ids),
+        _ptr(positions), _ptr(kv_len), ctypes.cast(slot_ptrs, ctypes.c_void_p), ctypes.cast(table_ptrs, ctypes.c_void_p),
+        n, width, int(page_size), int(bool(advance)), _stream()), "sample_and_advance")
 
 
 def decode_advance(sampled: torch.Tensor, tokens_out: torch.Tensor, token_ids: torch.Tensor,

@@ -280,9 +280,22 @@ class Block(Part):
         return None
 
 
+@dataclass
+class ArgmaxStage:
+    """What a step's sampler offers the head: ``scratch``, float32 values and int32 indices with
+    room for ``[rows, compute units]`` each. A head whose kernel has every logit in a register
+    anyway may leave each row's best (value, lowest index) per workgroup there, as
+    ``[rows, parts]``, and say how many ``parts`` there are; the sampler then skips the kernel that
+    reads all logits once more for that. 0 parts: nothing was left."""
+
+    scratch: tuple
+    parts: int = 0
+
+
 class Head(Part):
     """Rows to logits: ``forward(x [k, hidden]) -> float32 [k, vocab]``. ``tie(table)`` gives a
-    tied head the embedding's table."""
+    tied head the embedding's table. The fused decode form, ``forward_stream(stream, norm,
+    argmax=None)``, may fill an :class:`ArgmaxStage`."""
 
     def tie(self, table: torch.Tensor) -> None:
         raise NotImplementedError

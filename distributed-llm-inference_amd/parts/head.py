@@ -8,7 +8,7 @@ from typing import Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .base import DecodeStream, Head, Norm, Runtime
+from .base import ArgmaxStage, DecodeStream, Head, Norm, Runtime
 from .linear import decode_copy, linear
 from .registry import register_part
 from .spec import WeightSpec
@@ -65,22 +65,26 @@ class LinearHead(Head):
         return self.rt.is_bf16 and (ctx.num_tokens > self.FEW_ROWS
                                     or ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype))
 
-    def forward_stream(self, stream: DecodeStream, norm: Norm) -> torch.Tensor:
+    def forward_stream(self, stream: DecodeStream, norm: Norm, argmax: Optional[ArgmaxStage] = None) -> torch.Tensor:
         """Logits of every row of the stream, the final norm computed inside the product (with
-        more than a few rows: the norm kernel, then the library product)."""
+        more than a few rows: the norm kernel, then the library product). ``argmax``: where the
+        kernel that makes the logits may leave the first stage of every row's argmax."""
         if stream.x.shape[0] > self.FEW_ROWS:
             ready = stream.normed_by(norm)  # the last residual sum's kernel may have normalised already
             return self.forward(ready if ready is not None else norm.forward(stream.x))
         norm_w, eps = norm.fused_params()
         out = torch.empty(stream.x.shape[0], self.vocab_size, device=self.rt.device, dtype=torch.float32)
-        self._few_rows(stream.x, out, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        parts = self._few_rows(stream.x, out, best=argmax.scratch if argmax is not None else None,
+                               norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
+        if argmax is not None:
+            argmax.parts = parts
         return out
 
-    def _few_rows(self, x: torch.Tensor, out: torch.Tensor, **norm) -> None:
+    def _few_rows(self, x: torch.Tensor, out: torch.Tensor, best=None, **norm) -> int:
         """At most 16 rows: the kernel whose workgroups stay and walk the table (a long stream:
         at the 1B sizes 89 to 100 us for 1 to 16 rows against 92 to 112 with a workgroup per pair
         of tiles), where it takes the sizes; else the few-row product."""
         if self.weight_tiled is not None and ops.head_gemm_supports(x.shape[0], self.vocab_size, self.hidden_size, x.dtype):
-            ops.head_gemm(x, self.weight_tiled, out, **norm)
-        else:
-            ops.skinny_gemm(x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out, **norm)
+            return ops.head_gemm(x, self.weight_tiled, out, best=best, **norm)
+        ops.skinny_gemm(x, self.weight, w_tiled=self.weight_tiled, epilogue=ops.SKINNY_F32, out=out, **norm)
+        return 0

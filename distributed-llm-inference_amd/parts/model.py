@@ -163,7 +163,10 @@ class Model:
             # the norm that the stream meets next: the following entry's first, or the final one
             after = order[i + 1].block.first_norm(order[i + 1].parts) if i + 1 < len(order) else self.final_norm
             layer.block.forward_stream(stream, ctx, cache, layer.parts, following=after)
-        logits = self.head.forward_stream(stream, self.final_norm)
+        if ctx.argmax_stage is not None:  # offered by a step that samples every row on the device
+            logits = self.head.forward_stream(stream, self.final_norm, ctx.argmax_stage)
+        else:
+            logits = self.head.forward_stream(stream, self.final_norm)
         k = ctx.logit_rows.shape[0]
         if getattr(ctx, "all_rows_wanted", False):
             return logits

@@ -118,3 +118,95 @@ def test_invalid_params():
         with pytest.raises(ValueError, match="must"):
             SamplingParams(**kw)
     assert SamplingParams(top_k=1, temperature=1.0).greedy and SamplingParams().greedy
+
+
+@pytest.mark.parametrize("rows,n,k,workgroups", [(1, 3088, 2048, 0), (8, 1008, 1024, 5), (16, 272, 4096, 1), (5, 128256, 2048, 0)])
+def test_the_logits_kernel_leaves_the_first_stage_of_the_argmax(rows, n, k, workgroups):
+    """The kernel that makes the logits of a few rows has each of them in a register once: asked
+    to, every workgroup leaves each row's best logit and its lowest index, and the best of those
+    parts is the row's argmax (ties to the lowest index: several logits are made equal and the
+    largest on purpose, far apart, so that they fall to different workgroups)."""
+    from dli_amd.kernels import ops
+
+    torch.manual_seed(rows + n)
+    x = torch.randn(rows, k, device="cuda").bfloat16()
+    w = (torch.randn(n, k, device="cuda") / k ** 0.5).bfloat16()
+    for r in range(rows):  # equal weight rows give equal logits: a tie between n//5 + r and 4n//5 + r, above the rest
+        lo, hi = n // 5 + r, 4 * n // 5 + r
+        w[lo] = w[hi] = (x[r].float() / x[r].float().norm() * 8).bfloat16()
+    wt = ops.tile_weights(w)
+    out = torch.empty(rows, n, device="cuda", dtype=torch.float32)
+    scratch = ops.sample_scratch(rows, x.device)
+    scratch[0].fill_(float("nan"))
+    scratch[1].fill_(-7)
+    parts = ops.head_gemm(x, wt, out, workgroups=workgroups, best=scratch)
+    assert parts == min(workgroups or ops.compute_units(x.device), (n // 16 + 1) // 2)
+    vals = scratch[0][:rows * parts].view(rows, parts).cpu()
+    idxs = scratch[1][:rows * parts].view(rows, parts).cpu()
+    logits = out.cpu()
+    for r in range(rows):
+        top = logits[r].max()
+        first = int((logits[r] == top).nonzero()[0])
+        assert first == n // 5 + r, "the tie was meant to hold the row's largest logit"
+        assert vals[r].max() == top
+        assert int(idxs[r][vals[r] == top].min()) == first
+        for p in range(parts):  # every part is a logit of the row at the index it names
+            assert logits[r, idxs[r, p]] == vals[r, p]
+    assert ops.head_gemm(x, wt, out) == 0
+
+
+@pytest.mark.parametrize("stage_one", ["own", "given"])
+def test_sampling_and_handing_on_in_one_kernel_equals_the_two(stage_one):
+    """`sample_and_advance` against `sample` followed by `decode_advance`: greedy and seeded rows,
+    a padding row without keys, two groups of layers, with the first stage of the argmax done by
+    its own kernel or given as parts (here: the best of every seven logits)."""
+    from dli_amd.kernels import ops
+
+    rows, vocab, ps, width = 6, 1000, 8, 5
+    g = torch.Generator().manual_seed(5)
+    logits = (torch.randn(rows, vocab, generator=g) * 3).cuda()
+    temperature = torch.tensor([0.0, 0.8, 1.0, 0.0, 1.3, 0.7]).cuda()
+    top_k = torch.tensor([-1, 20, -1, 1, 50, -1], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 1.0, 0.9, 1.0, 0.8, 1.0]).cuda()
+    seeds = torch.arange(11, 11 + rows, dtype=torch.int64).cuda()
+
+    def state():
+        tables = [torch.randint(0, 40, (rows, width), generator=torch.Generator().manual_seed(9 + i), dtype=torch.int32).cuda()
+                  for i in range(2)]
+        return dict(counters=torch.tensor([0, 3, 7, 1, 2, 4], dtype=torch.int64).cuda(),
+                    token_ids=torch.full((rows,), 5, dtype=torch.int32).cuda(),
+                    positions=torch.tensor([6, 7, 15, 22, 31, 0], dtype=torch.int32).cuda(),
+                    kv_len=torch.tensor([7, 8, 16, 23, 32, 0], dtype=torch.int32).cuda(),  # the last row is padding
+                    slots=[torch.full((rows,), -1, dtype=torch.int32).cuda() for _ in range(2)], tables=tables,
+                    tokens_out=torch.full((rows,), -3, dtype=torch.int32).cuda())
+
+    for advance in (True, False):
+        a, b = state(), state()
+        out_a = torch.empty(rows, dtype=torch.int32, device="cuda")
+        ops.sample(logits, temperature, top_k, top_p, seeds, a["counters"], out_a)
+        ops.decode_advance(out_a, a["tokens_out"], a["token_ids"], a["positions"], a["kv_len"], a["counters"],
+                           a["slots"], a["tables"], ps, advance)
+        out_b = torch.empty(rows, dtype=torch.int32, device="cuda")
+        scratch = ops.sample_scratch(rows, logits.device)
+        parts = 0
+        if stage_one == "given":
+            parts = 143
+            vals = torch.full((rows, parts), float("-inf"), device="cuda")
+            idxs = torch.full((rows, parts), 2 ** 31 - 1, dtype=torch.int32, device="cuda")
+            for p in range(parts):  # parts of seven logits each; the last holds the six that are left
+                lo, hi = 7 * p, min(vocab, 7 * p + 7)
+                v, i = logits[:, lo:hi].max(dim=1)
+                vals[:, p], idxs[:, p] = v, (i + lo).int()
+            scratch[0][:rows * parts] = vals.reshape(-1)
+            scratch[1][:rows * parts] = idxs.reshape(-1)
+        ops.sample_and_advance(logits, temperature, top_k, top_p, seeds, b["counters"], out_b, scratch, parts,
+                               b["tokens_out"], b["token_ids"], b["positions"], b["kv_len"], b["slots"], b["tables"],
+                               ps, advance)
+        assert torch.equal(out_a, out_b)
+        for key in ("counters", "token_ids", "positions", "kv_len", "tokens_out"):
+            assert torch.equal(a[key], b[key]), (key, advance)
+        for sa, sb in zip(a["slots"], b["slots"]):
+            assert torch.equal(sa, sb)
+        assert (a["kv_len"][-1] == 0) and (a["slots"][0][-1] == -1)  # the padding row was left alone
+        if advance:
+            assert torch.equal(a["positions"][:5].cpu(), torch.tensor([7, 8, 16, 23, 32], dtype=torch.int32))
