@@ -224,6 +224,9 @@ def test_shared_prefix_sampling_preemption_config_b():
     without, _ = run(ps, params, enable_prefix_caching=False, **tight)
     assert with_reuse == alone and without == alone
     assert all(len(o) == 32 for o in alone) and len({tuple(o) for o in alone}) > 1
+    # and what they agree on is what the plain implementation's distributions and the requests' own draws give
+    for p, q, out in zip(ps, params, alone):
+        assert_draws_follow_the_plain_distribution(name, p, out, q, q.seed, 1e-3)
 
 
 def assert_same_or_near_cell_edge(name, prompt, a, b, params, seed, tol):
@@ -270,6 +273,7 @@ def test_seeded_request_is_the_same_alone_and_in_a_busy_batch(dtype):
         return out
 
     alone, busy, pair = run([2]), run([0, 1, 2, 3, 4]), run([2, 4])
+    assert_draws_follow_the_plain_distribution(name, ps[2], alone, sp, 7, 1e-3 if dtype == "float32" else 0.05)
     if dtype == "float32":
         assert alone == busy == pair
     else:
