@@ -829,3 +829,117 @@ def test_a_subclass_of_a_built_in_part_is_not_taken_for_it_by_the_loop_in_c():
         outs.append(TraceSession(core).step([{"id": "r", "tokens": toks, "want": [89]}]).clone())
     assert halved.native_runs == 0 and plain_model.native_runs == 1
     assert not torch.allclose(outs[0], outs[1], atol=1e-3)
+
+
+# ------------------------------------------------------------------ a toy norm
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_norm_is_registered_built_and_stepped(dtype):
+    """Another norm, defined here and nowhere in the framework: a layer norm with mean, variance,
+    weight and bias, as the three norms of a pre-norm model. It has no ``fused_params`` (the fused
+    decode kernels and the loop in C compute an RMS norm), so every step must take the parts' plain
+    ``forward``; its ``forward(x, delta)`` makes the residual sum in place as the interface asks.
+    Whole, in portions, mixed and token by token against a plain float64 model."""
+    import tempfile
+    from typing import Mapping, Optional
+
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import LayerSpec, ModelSpec, Norm, PartSpec, ScheduleEntry, WeightSpec, register_part, unregister_part
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    @register_part("norm", "toy_layer_norm")
+    class ToyLayerNorm(Norm):
+        def __init__(self, runtime, *, width: int, eps: float) -> None:
+            super().__init__(runtime)
+            self.width, self.eps = width, eps
+            self.w = self.b = None
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.width,), role="float32", init="norm"),
+                    "bias": WeightSpec((self.width,), role="float32")}
+
+        def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+            self.w, self.b = tensors["weight"], tensors["bias"]
+
+        def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+            if delta is not None:
+                x.copy_((x.float() + delta.float()).to(x.dtype))  # the residual sum, in place, 32-bit
+            h = x.float()
+            h = (h - h.mean(-1, keepdim=True)) * torch.rsqrt(h.var(-1, unbiased=False, keepdim=True) + self.eps)
+            return (h * self.w + self.b).to(x.dtype)
+
+    h, heads, kv_heads, d, inter, vocab, eps, theta, n_layers = 40, 2, 2, 16, 56, 45, 1e-5, 10000.0, 2
+
+    def build(cfg):
+        norm = dict(width=h, eps=eps)
+        pos = PartSpec("rotary", dict(dim=d, theta=theta))
+        layers = []
+        for i in range(n_layers):
+            p = f"layers.{i}."
+            layers.append(LayerSpec(PartSpec("pre_norm"), {
+                "mixer_norm": ("norm", PartSpec("toy_layer_norm", norm, p + "n1.")),
+                "mixer": ("mixer", PartSpec("gqa_attention", dict(hidden_size=h, num_heads=heads, num_kv_heads=kv_heads,
+                                                                 head_dim=d, position=pos), p + "attn.")),
+                "feed_forward_norm": ("norm", PartSpec("toy_layer_norm", norm, p + "n2.")),
+                "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=inter), p + "mlp."))}))
+        return ModelSpec(
+            architecture="ToyLayerNormForCausalLM", vocab_size=vocab, hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=vocab, hidden_size=h), "embed."),
+            layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(n_layers)),
+            final_norm=PartSpec("toy_layer_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=vocab, hidden_size=h, tied=False), "head."))
+
+    def layer_norm(x, w, b):
+        return (x - x.mean(-1, keepdim=True)) / torch.sqrt(x.var(-1, unbiased=False, keepdim=True) + eps) * w + b
+
+    def plain(w, tokens):
+        w = {k: v.double() for k, v in w.items()}
+        sizes = dict(num_heads=heads, num_kv_heads=kv_heads, head_dim=d)
+        cos, sin = P.rope_cos_sin(P.inverse_frequencies({"rope_type": "default", "theta": theta}, d),
+                                  torch.arange(len(tokens)), torch.float64)
+        x = w["embed.weight"][torch.tensor(tokens)]
+        for i in range(n_layers):
+            p = f"layers.{i}."
+            x = x + P.attention_block(layer_norm(x, w[p + "n1.weight"], w[p + "n1.bias"]), w, p + "attn.", sizes, cos, sin)
+            x = x + P.swiglu_mlp(layer_norm(x, w[p + "n2.weight"], w[p + "n2.bias"]), w, p + "mlp.")
+        return P.linear(layer_norm(x, w["norm.weight"], w["norm.bias"]), w["head.weight"])
+
+    register_architecture("ToyLayerNormForCausalLM", dict, build)
+    try:
+        from test_model_gpu import check
+
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, {"architectures": ["ToyLayerNormForCausalLM"]}, seed=14, std=0.2,
+                                        norm_jitter=0.1)
+            _, weights = P.load_folder(folder)
+            rng = torch.Generator().manual_seed(4)
+            toks = {rid: torch.randint(0, vocab, (n,), generator=rng).tolist() for rid, n in (("a", 41), ("b", 19))}
+            ref = {rid: plain(weights, t) for rid, t in toks.items()}
+            model = load_model(folder, dtype=dtype)
+            core = build_core(model, num_pages=10, page_size=8, max_seqs=4, enable_prefix_caching=False, watermark=0.0)
+            core.step.enable_decode_graphs(4, 80)
+            assert core.step.graphs is None, "a part that does not say so is not recorded into graphs"
+            s = TraceSession(core)
+            for rid, t in toks.items():
+                got = s.step([{"id": rid, "tokens": t, "want": list(range(len(t)))}], end=[rid])
+                check(got, ref[rid], dtype, f"toy norm, {rid} whole")
+            fed = {"a": 0, "b": 0}
+            for plan in ({"a": 13}, {"a": 7, "b": 5}, {"a": 2, "b": 9}, {"a": 5, "b": 2}):
+                entries = [{"id": rid, "tokens": toks[rid][fed[rid]:fed[rid] + n], "want": list(range(n))}
+                           for rid, n in plan.items()]
+                got = s.step(entries)
+                check(got, torch.cat([ref[rid][fed[rid]:fed[rid] + n] for rid, n in plan.items()]), dtype,
+                      f"toy norm, portions {plan} at {fed}")
+                for rid, n in plan.items():
+                    fed[rid] += n
+            while fed["b"] < len(toks["b"]):
+                got = s.step([{"id": rid, "tokens": [toks[rid][fed[rid]]], "want": [0]} for rid in ("a", "b")])
+                check(got, torch.stack([ref[rid][fed[rid]] for rid in ("a", "b")]), dtype, f"toy norm, decode at {fed}")
+                fed = {rid: n + 1 for rid, n in fed.items()}
+            assert model.native_runs == 0
+            core.manager.check_invariants()
+    finally:
+        unregister_architecture("ToyLayerNormForCausalLM")
+        unregister_part("norm", "toy_layer_norm")
