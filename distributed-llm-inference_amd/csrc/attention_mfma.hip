@@ -524,9 +524,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // set of four waves that takes the mirror tile of the same request (tile b of n pairs with tile
 // n-1-b): under a causal mask the two together always have the same number of key tiles to visit,
 // whatever b, so that all workgroups take equally long; the workgroups of the lower half of the
-// tile list leave at once. Tiles of 32 keys are pipelined: while tile i is consumed from LDS, tile
-// i+1 already lies there, tile i+2 is being written there from registers and tiles i+3.. are on
-// their way from memory into registers.
+// tile list leave at once. Tiles of 32 keys are pipelined through a ring of NB buffers in LDS:
+// while tile i is consumed, tile i+1 already lies there and tiles i+2..i+NB-1 are on their way
+// from memory, written into LDS by the loads themselves (no registers, no second instruction; moving
+// a tile through registers took a third of the kernel's time at 8,192 tokens).
 // Products use v_mfma_f32_16x16x32_bf16 (lane l: row/column l%16, k-indices 8*(l/16)..+7). For
 // P*V the eight k-indices of lane group g stand for the keys 4g..4g+3 and 16+4g..16+4g+3 of the
 // tile, which is how the two 16-key halves of S^T leave the first product.
@@ -537,8 +538,38 @@ __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+// Which chunk of its row (R chunks of 16 bytes) a K chunk changes places with in LDS: the 16 lanes
+// that read chunk c of keys 0..15 (or 16..31) then read 16 different 16-byte columns of the 256
+// bytes that LDS serves at a time. Rows of 4 or 12 chunks: four rows share a column; of 8: two;
+// of 16: all.
+template <int R>
+__device__ __forceinline__ int k_swizzle(int key) {
+  static_assert(R == 4 || R == 8 || R == 12 || R == 16, "rows of 32, 64, 96 or 128 dims");
+  return R == 8 ? (key >> 1) & 7 : (R == 16 ? key & 15 : (key >> 2) & 3);
+}
+
+// waits until at most `n` of the wave's vector memory loads are outstanding (nothing else awaited)
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  static_assert(N >= 0 && N < 64, "6 bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// The barrier between two tiles, without the fence of __syncthreads(): that fence would wait for
+// every load that is still writing LDS, the later tiles' too. What the barrier orders is stated by
+// hand instead: wait_loads() before it for the tile that is read next; a buffer is written again
+// only after the barrier that follows its last read, whose values the wave has used by then.
+__device__ __forceinline__ void tile_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// (The single-tile kernel for heads of up to 64 is held to the registers that let three waves
+// share a SIMD: 130 instead of 176, nothing spilled, no copies between the two register files.)
 template <int DCH, bool PAIR>
-__global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_kernel(
+__global__ __launch_bounds__(PAIR ? 512 : 256) __attribute__((amdgpu_waves_per_eu(!PAIR && DCH <= 4 ? 3 : 1)))
+void attention_prefill_shared_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len,
@@ -546,13 +577,15 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
     const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
     int window, int heads_per_wg) {
   constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of the first product
-  constexpr int KPAD = D + 8, VPAD = 32 + 8;    // padded rows against bank conflicts
+  constexpr int R = D / 8;                      // 16-byte chunks in a key's row of K
   constexpr int NT = PAIR ? 512 : 256;          // threads
-  constexpr int CHUNKS = 8 * D;                 // 16-byte chunks of a tile: 4D of K, then 4D of V^T
-  constexpr int UCH = (CHUNKS + NT - 1) / NT;   // chunks per thread and tile
-  constexpr int RD = 3;                         // tiles in flight from memory to registers
-  constexpr int K_ELEMS = 32 * KPAD, TILE_ELEMS = K_ELEMS + D * VPAD;
-  __shared__ __attribute__((aligned(16))) bf16_t lds[3][TILE_ELEMS];  // K rows, then V^T rows
+  constexpr int NW = NT / DLI_WAVE;             // waves
+  constexpr int BLOCKS = 2 * DCH;               // 1 KB blocks of a tile (64 chunks of 16 bytes): DCH of K, DCH of V^T
+  constexpr int UCH = (BLOCKS + NW - 1) / NW;   // blocks per wave and tile
+  constexpr int NB = DCH <= 4 ? 6 : (DCH <= 6 ? 5 : 4);  // tiles in LDS: one in use, the others on their way
+  constexpr int K_ELEMS = 32 * D, VH_ELEMS = 16 * D, TILE_ELEMS = 64 * D;
+  // a tile: K rows of 32 keys; V^T rows (one a dim) of the first 16 keys; V^T rows of the other 16
+  __shared__ __attribute__((aligned(1024))) bf16_t lds[NB][TILE_ELEMS];
 
   // Workgroups are dealt to the eight XCDs in turn by their linear index, and each XCD has an L2
   // of its own: the tiles of one kv head are therefore given to one XCD (when the heads divide
@@ -620,37 +653,36 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   const int end = first_pos + wg_q_hi + 1;
   const int n_tiles = (end - begin + 31) / 32;
 
-  // Staging: the UCH chunks that this thread moves per tile. Chunk u < 4D is 8 dims of key
-  // u/(D/8); chunk 4D+c holds 8 keys of dim (c%2D)/2: those of the tile's first half of 16 keys
-  // for c < 2D, of its second half after that. 2D and 4D are multiples of 64, so whether a chunk
-  // is of K or of V, and which half of the tile it lies in, is the same for all lanes of a wave:
-  // the page's address is then made on the scalar unit and each lane adds a constant of its own.
-  const int wave_first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / DLI_WAVE)) * DLI_WAVE;
+  // Staging: a wave moves a block of 64 chunks with one load that writes LDS directly (lane i's 16
+  // bytes land at the block's address + 16 i). Blocks 0..DCH-1 are the K rows in order (16-byte
+  // chunk p of the region is part p % R of key p / R), blocks DCH.. the two V^T halves (chunk p of
+  // a half is 8 keys of dim p / 2). DCH is even, so whether a block is of K or of V, and which half
+  // of the tile's keys it holds, is the same for all lanes of a wave: the page's address is made on
+  // the scalar unit and each lane adds a constant of its own. Rows are not padded. Instead the
+  // chunks of a row change places (an XOR of the chunk's number with bits of the row's number,
+  // applied here to the address a lane reads from and below to the address a fragment is read
+  // at) so that the 16 lanes that read one column of chunks hit 16 different bank groups.
+  const int wave_id = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / DLI_WAVE));
   unsigned lane_off[UCH];   // elements from the half's first key in its page
-  int lds_off[UCH], v_key[UCH];
-  bool second_half[UCH], is_v[UCH], live[UCH];  // second_half and is_v are the same in all lanes
+  int block_at[UCH];        // the block's first element in a tile
+  bool second_half[UCH], is_v[UCH];  // the same in all lanes
 #pragma unroll
   for (int r = 0; r < UCH; ++r) {
-    const int u_raw = threadIdx.x + r * NT;
-    live[r] = CHUNKS % NT == 0 || u_raw < CHUNKS;
-    const int u = live[r] ? u_raw : CHUNKS - 1;
-    const int u_wave = min(wave_first + r * NT, CHUNKS - 1);  // the wave's first chunk decides for all of it
-    is_v[r] = u_wave >= 4 * D;
+    // with more waves than blocks, the others load a block a second time (same bytes, same place):
+    // every wave then has the same number of loads in flight
+    const int blk = (wave_id + r * NW) % BLOCKS;
+    is_v[r] = blk >= DCH;
+    second_half[r] = blk % DCH >= DCH / 2;
+    block_at[r] = blk * 512;
+    const int p = (blk % (DCH / 2)) * 64 + lane;  // the lane's chunk within the half's region
     if (!is_v[r]) {
-      const int kk = u / (D / 8), part = u % (D / 8);
-      second_half[r] = u_wave >= 2 * D;
-      lane_off[r] = (kk % 16) * D + part * 8;
-      lds_off[r] = kk * KPAD + part * 8;
-      v_key[r] = 0;
+      const int kk = p / R, part = (p % R) ^ k_swizzle<R>(kk);
+      lane_off[r] = kk * D + part * 8;
     } else {
-      const int c = u - 4 * D, d = (c % (2 * D)) / 2, sub = c % 2;
-      second_half[r] = u_wave >= 6 * D;
+      const int d = p / 2, sub = (p % 2) ^ ((d >> 3) & 1);
       lane_off[r] = d * page_size + sub * 8;
-      v_key[r] = (second_half[r] ? 16 : 0) + sub * 8;
-      lds_off[r] = K_ELEMS + d * VPAD + v_key[r];
     }
   }
-  bf16x8 stage[RD][UCH];
   // Tiles are fetched in order, so the page of the tile's first key is tracked by addition
   // instead of division: `tile_page` indexes the block table, `tile_off` is the key's offset in it.
   // Tiles start at multiples of 32 and pages hold a multiple of 16 keys, so each half of a tile
@@ -674,7 +706,7 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   // halves read page 0 and are never used): the count of loads in flight is then known at compile
   // time and a tile is awaited without draining the younger ones behind it. Keys past the last one
   // of a half-filled page may hold anything: K rows there are masked as later than every query, V
-  // columns are cleared on the way into LDS.
+  // columns are cleared in the fragments that a wave has read from LDS.
   // (Looking a tile's pages up earlier in the iteration, behind the first product, so that the
   // scalar load's answer arrives during the softmax, needs the lookup inside the branch that a wave
   // takes when it sees the tile: the compiler then keeps the pages in vector registers or, told
@@ -685,7 +717,7 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   const unsigned page_stride = (unsigned)kv_heads * (unsigned)page_size * (unsigned)D;
   const bf16_t* k_head = k_pages + (int64_t)kvh * page_size * D;
   const bf16_t* v_head = v_pages + (int64_t)kvh * page_size * D;
-  auto fetch = [&](int t, bf16x8 (&sq)[UCH]) {
+  auto fetch = [&](int t, int buf) __attribute__((always_inline)) {
     const uint64_t at_a = (uint64_t)(unsigned)page_a * page_stride, at_b = (uint64_t)(unsigned)page_b * page_stride;
     const unsigned oa = off_a, ob = off_b;
     lookup(t + 32);
@@ -694,30 +726,17 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
       // the same for every lane of the wave: a key's row of K is D long, a key's column of V^T one element
       const unsigned off = second_half[r] ? ob : oa;
       const bf16_t* base = (is_v[r] ? v_head : k_head) + (second_half[r] ? at_b : at_a) + (is_v[r] ? off : off * D);
-      sq[r] = *reinterpret_cast<const bf16x8*>(base + lane_off[r]);
-    }
-  };
-  auto stash = [&](int buf, int t, bf16x8 (&sq)[UCH]) {
-#pragma unroll
-    for (int r = 0; r < UCH; ++r) {
-      if (live[r]) {
-        if (t + 32 > n_keys && is_v[r]) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i)
-            if (t + v_key[r] + i >= n_keys) sq[r][i] = (bf16_t)0.f;
-        }
-        *reinterpret_cast<bf16x8*>(&lds[buf][lds_off[r]]) = sq[r];
-      }
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(base + lane_off[r]),
+          (__attribute__((address_space(3))) void*)&lds[buf][block_at[r]], 16, 0, 0);
     }
   };
 
-  // tiles 0 and 1 go straight to LDS; tile T >= 2 waits in register slot T % RD
+  // tiles 0..NB-2 set out for LDS; the loop needs the first of them there
 #pragma unroll
-  for (int T = 0; T < 2 + RD; ++T) {
-    fetch(begin + T * 32, stage[T % RD]);
-    if (T < 2) stash(T, begin + T * 32, stage[T % RD]);
-  }
-  __syncthreads();
+  for (int T = 0; T < NB - 1; ++T) fetch(begin + T * 32, T);
+  wait_loads<(NB - 2) * UCH>();
+  tile_barrier();
   typedef short short4a __attribute__((ext_vector_type(4)));
   union VFrag {
     bf16x8 v;
@@ -729,12 +748,18 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   VFrag vf_kept[DCH];
   bf16x8 pb_kept[2];
   bool active = false;
+  // where this lane's fragments lie in a tile: chunk 4c+g of key row `col` (and of row 16+col, 16
+  // rows on), and keys 4g..4g+3 of dim row 16c+col in either half
+  int k_at[DK];
+#pragma unroll
+  for (int c = 0; c < DK; ++c) k_at[c] = col * D + ((c * 4 + grp) ^ k_swizzle<R>(col)) * 8;
+  const int v_at = col * 16 + ((grp >> 1) ^ (col >> 3)) * 8 + (grp & 1) * 4;
   auto sees = [&](int it) __attribute__((always_inline)) {  // whether any of the wave's queries sees a key of the tile
     const int t = begin + it * 32;
     return wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1);
   };
   auto scores = [&](int it, VFrag (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
-    const int t = begin + it * 32, buf = it % 3;
+    const int t = begin + it * 32, buf = it % NB;
     {
       const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
       const bf16_t* ks = &lds[buf][0];
@@ -744,13 +769,13 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
       bf16x8 kf0[DK], kf1[DK];
 #pragma unroll
       for (int c = 0; c < DK; ++c) {
-        kf0[c] = *reinterpret_cast<const bf16x8*>(ks + col * KPAD + c * 32 + grp * 8);
-        kf1[c] = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KPAD + c * 32 + grp * 8);
+        kf0[c] = *reinterpret_cast<const bf16x8*>(ks + k_at[c]);
+        kf1[c] = *reinterpret_cast<const bf16x8*>(ks + 16 * D + k_at[c]);
       }
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
-        vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 4 * grp);
-        vf[c].h[1] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 16 + 4 * grp);
+        vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + c * 256 + v_at);
+        vf[c].h[1] = *reinterpret_cast<const short4a*>(vs + VH_ELEMS + c * 256 + v_at);
       }
       // S^T of both column tiles, for the two halves of the tile: keys t+4g+i and t+16+4g+i
       float4v sa[2], sb[2];
@@ -830,6 +855,17 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
         }
         st[j].l += tile_sum;
       }
+      // keys past the request's last one (the rest of a half-filled page) may hold anything, also
+      // what no product with zero clears
+      if (t + 32 > n_keys) {
+#pragma unroll
+        for (int c = 0; c < DCH; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (t + 4 * grp + i >= n_keys) vf[c].h[0][i] = 0;
+            if (t + 16 + 4 * grp + i >= n_keys) vf[c].h[1][i] = 0;
+          }
+      }
     }
   };
   auto values = [&](VFrag (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
@@ -838,18 +874,19 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
 #pragma unroll
       for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
   };
-  auto move_on = [&](int it, int slot) __attribute__((always_inline)) {
-    // tile it+2 leaves its register slot for LDS; the slot then receives tile it+2+RD
-    stash((it + 2) % 3, begin + (it + 2) * 32, stage[slot]);
-    fetch(begin + (it + 2 + RD) * 32, stage[slot]);
+  auto move_on = [&](int it) __attribute__((always_inline)) {
+    // tile it+NB-1 sets out for the buffer that tile it-1 left at the last barrier; tile it+1 has
+    // to be there before the next one
+    fetch(begin + (it + NB - 1) * 32, (it + NB - 1) % NB);
+    wait_loads<(NB - 2) * UCH>();
   };
   auto scores_half = [&](int it) __attribute__((always_inline)) {
     active = sees(it);
     if (active) scores(it, vf_kept, pb_kept);
   };
-  auto values_half = [&](int it, int slot) __attribute__((always_inline)) {
+  auto values_half = [&](int it) __attribute__((always_inline)) {
     if (active) values(vf_kept, pb_kept);
-    move_on(it, slot);
+    move_on(it);
   };
   // The paired kernel tests once per tile whether the wave has work, the single one before each
   // half: the same work either way, but the compiler orders the two forms differently, and each
@@ -858,9 +895,9 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
   // tile), so that one set's products run beside the other's softmax; and the pair's key tiles
   // dealt out evenly to the two sets with a merge of their states at the end. Slower by 45% in the
   // single-tile kernel: S^T of tile it+1 sent to the matrix cores before the softmax of tile it.
-  for (int it0 = 0; it0 < n_tiles; it0 += RD) {
+  for (int it0 = 0; it0 < n_tiles; it0 += NB) {
 #pragma unroll
-    for (int r = 0; r < RD; ++r) {
+    for (int r = 0; r < NB; ++r) {
       const int it = it0 + r;
       if (it >= n_tiles) break;
       if constexpr (PAIR) {
@@ -870,12 +907,12 @@ __global__ __launch_bounds__(PAIR ? 512 : 256) void attention_prefill_shared_ker
           scores(it, vf, pb);
           values(vf, pb);
         }
-        move_on(it, (r + 2) % RD);
+        move_on(it);
       } else {
         scores_half(it);
-        values_half(it, (r + 2) % RD);
+        values_half(it);
       }
-      __syncthreads();
+      tile_barrier();
     }
   }
 
@@ -1415,9 +1452,10 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
     // a workgroup takes a tile and its mirror tile, heads of up to 64 one after the other with the
     // keys of each shared out to two sets of waves (2), larger heads, for which that kernel runs
     // out of registers, side by side (1). Below one workgroup a unit pairing would leave units idle.
-    // Per layer at the 1B sizes, kernels 0 / 1 / 2: 2,048 tokens 57 / 52 / 46 us, 3,072 tokens
-    // 90 / 120 / 114, 4,096 tokens 129 / 173 / 148; 24 heads of 128: 2,048 tokens 104 / 76 / 83,
-    // 4,096 tokens 216 / 237 / 252. The tile list has to hold all tiles of a request.
+    // Per layer at the 1B sizes, kernels 0 / 1 / 2: 2,048 tokens 58 / 54 / 46 us, 4,096 tokens
+    // 130 / 125 / 150, 8,192 tokens 436 / 438 / 509, 16,384 tokens 1,517 / 1,453 / 1,888; 24 heads of
+    // 128: 2,048 tokens 96 / 72 / 83, 8,192 tokens 613 / 651 / 676. The tile list has to hold all
+    // tiles of a request.
     const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
     const bool in_range = launch >= units && launch < 3 * units;
     const int mode = pair_tiles >= 0 ? pair_tiles : (in_range ? (head_dim <= 64 ? 2 : 1) : 0);
