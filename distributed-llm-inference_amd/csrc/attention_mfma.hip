@@ -691,17 +691,21 @@ void attention_prefill_shared_kernel(
   // vector memory queue where it would wait behind the tiles in flight.
   int tile_page = begin / page_size, tile_off = begin % page_size;
   int page_a = 0, page_b = 0, off_a = 0, off_b = 0;
-  auto lookup = [&](int t) {
-    // table entries exist only for pages that hold keys
+  // Table entries exist only for pages that hold keys: a tile past them reads the last one's.
+  // No branch goes around the loads: a condition that outlives its block becomes a lane mask, and
+  // what is computed from it (the second entry's index) went through the vector unit and back,
+  // which cost 7% of the kernel's time at 8,192 tokens.
+  const int last_page = max(n_keys - 1, 0) / page_size;
+  auto lookup = [&]() {
     off_a = tile_off;
     const int second = tile_off + 16 >= page_size ? 1 : 0;
-    off_b = tile_off + 16 - (second ? page_size : 0);
-    page_a = t < n_keys ? table[tile_page] : 0;
-    page_b = t + 16 < n_keys ? table[tile_page + second] : 0;
+    off_b = tile_off + 16 - second * page_size;
+    page_a = table[min(tile_page, last_page)];
+    page_b = table[min(tile_page + second, last_page)];
     tile_off += 32;
     while (tile_off >= page_size) { tile_off -= page_size; ++tile_page; }
   };
-  lookup(begin);
+  lookup();
   // Every fetch issues the same loads whatever the tile, also for tiles past the last one (their
   // halves read page 0 and are never used): the count of loads in flight is then known at compile
   // time and a tile is awaited without draining the younger ones behind it. Keys past the last one
@@ -717,10 +721,10 @@ void attention_prefill_shared_kernel(
   const unsigned page_stride = (unsigned)kv_heads * (unsigned)page_size * (unsigned)D;
   const bf16_t* k_head = k_pages + (int64_t)kvh * page_size * D;
   const bf16_t* v_head = v_pages + (int64_t)kvh * page_size * D;
-  auto fetch = [&](int t, int buf) __attribute__((always_inline)) {
+  auto fetch = [&](int buf) __attribute__((always_inline)) {  // the next tile in order
     const uint64_t at_a = (uint64_t)(unsigned)page_a * page_stride, at_b = (uint64_t)(unsigned)page_b * page_stride;
     const unsigned oa = off_a, ob = off_b;
-    lookup(t + 32);
+    lookup();
 #pragma unroll
     for (int r = 0; r < UCH; ++r) {
       // the same for every lane of the wave: a key's row of K is D long, a key's column of V^T one element
@@ -734,7 +738,7 @@ void attention_prefill_shared_kernel(
 
   // tiles 0..NB-2 set out for LDS; the loop needs the first of them there
 #pragma unroll
-  for (int T = 0; T < NB - 1; ++T) fetch(begin + T * 32, T);
+  for (int T = 0; T < NB - 1; ++T) fetch(T);
   wait_loads<(NB - 2) * UCH>();
   tile_barrier();
   typedef short short4a __attribute__((ext_vector_type(4)));
@@ -742,12 +746,8 @@ void attention_prefill_shared_kernel(
     bf16x8 v;
     short4a h[2];
   };
-  // A tile's work in two halves. The first reads the tile's fragments from LDS, makes S^T and the
-  // softmax (vector unit, mostly); the second makes P*V (matrix cores) and moves tile it+2 on its
-  // way (memory and LDS). What a wave carries from one to the other:
-  VFrag vf_kept[DCH];
-  bf16x8 pb_kept[2];
-  bool active = false;
+  // A tile's work in two parts: `scores` reads the tile's fragments from LDS, makes S^T and the
+  // softmax (vector unit, mostly); `values` makes P*V (matrix cores).
   // where this lane's fragments lie in a tile: chunk 4c+g of key row `col` (and of row 16+col, 16
   // rows on), and keys 4g..4g+3 of dim row 16c+col in either half
   int k_at[DK];
@@ -877,20 +877,9 @@ void attention_prefill_shared_kernel(
   auto move_on = [&](int it) __attribute__((always_inline)) {
     // tile it+NB-1 sets out for the buffer that tile it-1 left at the last barrier; tile it+1 has
     // to be there before the next one
-    fetch(begin + (it + NB - 1) * 32, (it + NB - 1) % NB);
+    fetch((it + NB - 1) % NB);
     wait_loads<(NB - 2) * UCH>();
   };
-  auto scores_half = [&](int it) __attribute__((always_inline)) {
-    active = sees(it);
-    if (active) scores(it, vf_kept, pb_kept);
-  };
-  auto values_half = [&](int it) __attribute__((always_inline)) {
-    if (active) values(vf_kept, pb_kept);
-    move_on(it);
-  };
-  // The paired kernel tests once per tile whether the wave has work, the single one before each
-  // half: the same work either way, but the compiler orders the two forms differently, and each
-  // kernel is 5 to 15% faster in its form (timed at 2,048 to 16,384 tokens, heads of 64 and 128).
   // Tried and slower by 10 to 15%: the second set half a tile behind the first (two barriers a
   // tile), so that one set's products run beside the other's softmax; and the pair's key tiles
   // dealt out evenly to the two sets with a merge of their states at the end. Slower by 45% in the
@@ -900,18 +889,13 @@ void attention_prefill_shared_kernel(
     for (int r = 0; r < NB; ++r) {
       const int it = it0 + r;
       if (it >= n_tiles) break;
-      if constexpr (PAIR) {
-        if (sees(it)) {
-          VFrag vf[DCH];
-          bf16x8 pb[2];
-          scores(it, vf, pb);
-          values(vf, pb);
-        }
-        move_on(it);
-      } else {
-        scores_half(it);
-        values_half(it);
+      if (sees(it)) {
+        VFrag vf[DCH];
+        bf16x8 pb[2];
+        scores(it, vf, pb);
+        values(vf, pb);
       }
+      move_on(it);
       tile_barrier();
     }
   }
