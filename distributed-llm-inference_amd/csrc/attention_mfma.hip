@@ -568,7 +568,7 @@ __device__ __forceinline__ void tile_barrier() {
 // (The single-tile kernel for heads of up to 64 is held to the registers that let three waves
 // share a SIMD: 130 instead of 176, nothing spilled, no copies between the two register files.)
 template <int DCH, bool PAIR>
-__global__ __launch_bounds__(PAIR ? 512 : 256) __attribute__((amdgpu_waves_per_eu(!PAIR && DCH <= 4 ? 3 : 1)))
+__global__ __launch_bounds__(PAIR ? 512 : 256) __attribute__((amdgpu_waves_per_eu(PAIR ? 1 : (DCH <= 4 ? 3 : 2))))
 void attention_prefill_shared_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
@@ -1429,20 +1429,29 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   if (hw > 0) {
     if ((int64_t)kv_heads * page_size * head_dim >= ((int64_t)1 << 31)) return DLI_ERR_ARGUMENT;  // the kernel's 32 bits
     const dim3 sgrid(tiles, q_heads / hw);
-    // Which kernel (pair_tiles 0, 1 or 2; -1: by the size of the launch). With three or more
-    // workgroups a compute unit, every tile has a workgroup of its own (0): listed longest first,
-    // the tiles even the causal triangle out through the queue of workgroups, and no wave waits
-    // for a wave of another tile. With fewer, the launch is as long as its longest workgroup: then
-    // a workgroup takes a tile and its mirror tile, heads of up to 64 one after the other with the
-    // keys of each shared out to two sets of waves (2), larger heads, for which that kernel runs
-    // out of registers, side by side (1). Below one workgroup a unit pairing would leave units idle.
-    // Per layer at the 1B sizes, kernels 0 / 1 / 2: 2,048 tokens 58 / 54 / 46 us, 4,096 tokens
-    // 130 / 125 / 150, 8,192 tokens 436 / 438 / 509, 16,384 tokens 1,517 / 1,453 / 1,888; 24 heads of
-    // 128: 2,048 tokens 96 / 72 / 83, 8,192 tokens 613 / 651 / 676. The tile list has to hold all
-    // tiles of a request.
+    // Which kernel (pair_tiles 0, 1 or 2; -1: by the size of the launch). As a rule every tile has
+    // a workgroup of its own (0): listed longest first, the tiles even the causal triangle out
+    // through the queue of workgroups, and no wave waits for a wave of another tile. Where the
+    // launch has between one and two workgroups a compute unit, the units that get a second long
+    // tile decide its length: then a workgroup takes a tile and its mirror tile, which halves
+    // the workgroups that do anything, one to a unit: heads of up to 64 one after the other with
+    // the keys of each shared out to two sets of waves (2), larger heads, for which that kernel
+    // runs out of registers, side by side (1). These two fall off a cliff as soon as a unit would
+    // need a second such workgroup (they fill its registers), earlier for the larger heads, so
+    // their windows are kept to what was measured. Per layer, kernels 0 / 1 / 2, each timed in
+    // the steady state of a loop of launches, workgroups a unit in brackets:
+    //   32 heads of 64 on 8: 1,024 tokens [1.0] 25.5 / 27.0 / 26.0 us, 1,536 [1.5] 35.3 / 36.7 / 33.3,
+    //     2,048 [2.0] 45.5 / 46.8 / 41.1, 2,304 [2.2] 51.6 / 54.9 / 84.8, 3,072 [3.0] 67.5 / 75.1 / 105,
+    //     4,096 103 / 101 / 136, 8,192 334 / 368 / 491 (824 TFLOP/s), 16,384 1,241 / 1,376 / 1,870 (886)
+    //   24 heads of 128 on 8: 1,408 tokens [1.0] 48.5 / 49.5 / 62.8, 1,728 [1.3] 58.1 / 57.1 / 73.6,
+    //     2,048 [1.5] 83.3 / 66.3 / 79.2, 2,304 [1.7] 88.6 / 73.1 / 85.7, 2,560 [1.9] 93.6 / 121 / 173,
+    //     3,072 [2.2] 104 / 147 / 198, 8,192 498 / 604 / 664 (828 TFLOP/s)
+    // The tile list has to hold all tiles of a request.
     const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
-    const bool in_range = launch >= units && launch < 3 * units;
-    const int mode = pair_tiles >= 0 ? pair_tiles : (in_range ? (head_dim <= 64 ? 2 : 1) : 0);
+    const bool small_heads = head_dim <= 64;
+    const bool in_range = small_heads ? 4 * launch >= 5 * units && launch <= 2 * units
+                                      : 5 * launch >= 7 * units && 4 * launch <= 7 * units;
+    const int mode = pair_tiles >= 0 ? pair_tiles : (in_range ? (small_heads ? 2 : 1) : 0);
     const bool pair = mode == 1;
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \

@@ -286,9 +286,9 @@ def test_llama_3_2_1b_in_portions_and_in_mixed_batches(dtype):
         assert core.step.graphs.replays > 0
 
 
-def test_a_prompt_of_a_thousand_tokens_takes_the_kernel_that_shares_keys_between_two_sets_of_waves(monkeypatch):
-    """1,100 tokens at the 1B widths are 35 query tiles of eight kv heads each: between one and
-    three workgroups a compute unit, where the prefill attention lets a workgroup take a tile and
+def test_a_prompt_of_1700_tokens_takes_the_kernel_that_shares_keys_between_two_sets_of_waves(monkeypatch):
+    """1,700 tokens at the 1B widths are 54 query tiles of eight kv heads each: between 1.25 and
+    two workgroups a compute unit, where the prefill attention lets a workgroup take a tile and
     then its mirror tile with each turn's keys shared out to two sets of waves. The whole model
     through that kernel (chosen by the launch's size, not asked for), whole and as a portion on top
     of cached keys, against the plain implementation."""
@@ -296,7 +296,7 @@ def test_a_prompt_of_a_thousand_tokens_takes_the_kernel_that_shares_keys_between
     from dli_amd.trace import TraceSession
 
     rng = random.Random(29)
-    toks = [rng.randrange(32003) for _ in range(1100)]
+    toks = [rng.randrange(32003) for _ in range(1700)]
     ref = plain(toks)
     seen = []
     real = ops.attention_prefill
@@ -306,16 +306,16 @@ def test_a_prompt_of_a_thousand_tokens_takes_the_kernel_that_shares_keys_between
         return real(*a, **k)
 
     monkeypatch.setattr(ops, "attention_prefill", counted)
-    core = make_core("bfloat16", pages=72)
+    core = make_core("bfloat16", pages=110)
     core.model.native_steps = False  # through the parts, so that the launches can be counted here
     s = TraceSession(core)
-    want = [0, 17, 511, 512, 1023, 1099]
+    want = [0, 17, 511, 512, 1023, 1699]
     got = s.step([{"id": "w", "tokens": toks, "want": want}], end=["w"])
-    check(got, ref[want], "bfloat16", "1,100 tokens whole")
-    assert seen and all(tiles == 35 and forced is None for tiles, forced in seen)
+    check(got, ref[want], "bfloat16", "1,700 tokens whole")
+    assert seen and all(tiles == 54 and forced is None for tiles, forced in seen)
     units = ops.compute_units(torch.device("cuda"))
-    assert units <= 35 * 8 < 3 * units, "the launch was meant to fall into the range of the split-key kernel"
+    assert 5 * units <= 4 * 54 * 8 and 54 * 8 <= 2 * units, "the launch was meant to fall into the range of the split-key kernel"
     got = s.step([{"id": "p", "tokens": toks[:60], "want": [59]}])
     check(got, ref[59:60], "bfloat16", "first portion")
     got = s.step([{"id": "p", "tokens": toks[60:], "want": [w - 60 for w in want[2:]]}], end=["p"])
-    check(got, ref[want[2:]], "bfloat16", "1,040 tokens on top of 60 cached keys")
+    check(got, ref[want[2:]], "bfloat16", "1,640 tokens on top of 60 cached keys")
