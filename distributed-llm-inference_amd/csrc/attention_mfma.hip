@@ -529,8 +529,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // from memory, written into LDS by the loads themselves (no registers, no second instruction; moving
 // a tile through registers took a third of the kernel's time at 8,192 tokens).
 // Products use v_mfma_f32_16x16x32_bf16 (lane l: row/column l%16, k-indices 8*(l/16)..+7). For
-// P*V the eight k-indices of lane group g stand for the keys 4g..4g+3 and 16+4g..16+4g+3 of the
-// tile, which is how the two 16-key halves of S^T leave the first product.
+// P*V the eight k-indices of lane group g stand for the keys 8g..8g+7 of the tile here (in the
+// kernel further down that splits a turn's keys: for the keys 4g..4g+3 and 16+4g..16+4g+3, which
+// is how two products of 16 consecutive keys each leave S^T).
 // Needs head_dim % 32 == 0.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
@@ -538,14 +539,16 @@ __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// Which chunk of its row (R chunks of 16 bytes) a K chunk changes places with in LDS: the 16 lanes
-// that read chunk c of keys 0..15 (or 16..31) then read 16 different 16-byte columns of the 256
-// bytes that LDS serves at a time. Rows of 4 or 12 chunks: four rows share a column; of 8: two;
-// of 16: all.
+// Which chunk of its row (R chunks of 16 bytes) a K chunk changes places with in LDS. A product
+// reads chunk c of the sixteen key rows 8a + 4b + r (a, r = 0..3; b says which of the tile's two
+// products), one row a lane: with this the sixteen lanes read sixteen different 16-byte columns
+// of the 256 bytes that LDS serves at a time. Rows of 4 or 12 chunks: the four rows of one r share
+// a column; of 8: the two of one r / 2; of 16: all.
 template <int R>
-__device__ __forceinline__ int k_swizzle(int key) {
+__device__ __forceinline__ int k_swizzle(int key) {  // key: 0..31 within the tile
   static_assert(R == 4 || R == 8 || R == 12 || R == 16, "rows of 32, 64, 96 or 128 dims");
-  return R == 8 ? (key >> 1) & 7 : (R == 16 ? key & 15 : (key >> 2) & 3);
+  const int a = key >> 3;
+  return R == 8 ? (a << 1) | ((key >> 1) & 1) : (R == 16 ? (a << 2) | (key & 3) : a);
 }
 
 // waits until at most `n` of the wave's vector memory loads are outstanding (nothing else awaited)
@@ -645,7 +648,10 @@ void attention_prefill_shared_kernel(
       for (int c = 0; c < DK; ++c) qreg[j][c] = *reinterpret_cast<const bf16x8*>(qp + c * 32);
     }
   }
-  const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + wave_rows - 1;  // this wave's span
+  // this wave's span, the same in all its lanes and said so: what is decided from it per tile
+  // (whether the wave sees the tile, whether it needs the mask) is then scalar work
+  const int pos_lo = __builtin_amdgcn_readfirstlane(first_pos + q0);
+  const int pos_hi = __builtin_amdgcn_readfirstlane(first_pos + q0 + wave_rows - 1);
   // the workgroup walks the keys that any of its queries sees
   const int wg_q_lo = q0_second >= 0 ? q0_second : q0_first;
   const int wg_q_hi = min(q_len, q0_first + tile_rows) - 1;
@@ -676,7 +682,7 @@ void attention_prefill_shared_kernel(
     block_at[r] = blk * 512;
     const int p = (blk % (DCH / 2)) * 64 + lane;  // the lane's chunk within the half's region
     if (!is_v[r]) {
-      const int kk = p / R, part = (p % R) ^ k_swizzle<R>(kk);
+      const int kk = p / R, part = (p % R) ^ k_swizzle<R>(kk + (second_half[r] ? 16 : 0));
       lane_off[r] = kk * D + part * 8;
     } else {
       const int d = p / 2, sub = (p % 2) ^ ((d >> 3) & 1);
@@ -741,27 +747,36 @@ void attention_prefill_shared_kernel(
   for (int T = 0; T < NB - 1; ++T) fetch(T);
   wait_loads<(NB - 2) * UCH>();
   tile_barrier();
-  typedef short short4a __attribute__((ext_vector_type(4)));
-  union VFrag {
-    bf16x8 v;
-    short4a h[2];
-  };
   // A tile's work in two parts: `scores` reads the tile's fragments from LDS, makes S^T and the
   // softmax (vector unit, mostly); `values` makes P*V (matrix cores).
-  // where this lane's fragments lie in a tile: chunk 4c+g of key row `col` (and of row 16+col, 16
-  // rows on), and keys 4g..4g+3 of dim row 16c+col in either half
-  int k_at[DK];
+  // Where this lane's fragments lie in a tile. Which sixteen keys a product of S^T takes is free,
+  // since every lane reads its own key's row: rows 4g..4g+3 of the first product are the keys
+  // 8g..8g+3 and those of the second the keys 8g+4..8g+7, so that lane group g ends up with the
+  // probabilities of the eight consecutive keys 8g..8g+7, whose values (dim row 16c+col) lie in
+  // LDS as one chunk of 16 bytes.
+  int k_at[2][DK];
+  const int key_row = 8 * (col / 4) + col % 4;  // of the first product; the second's: four rows on
 #pragma unroll
-  for (int c = 0; c < DK; ++c) k_at[c] = col * D + ((c * 4 + grp) ^ k_swizzle<R>(col)) * 8;
-  const int v_at = col * 16 + ((grp >> 1) ^ (col >> 3)) * 8 + (grp & 1) * 4;
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int c = 0; c < DK; ++c)
+      k_at[b][c] = (key_row + 4 * b) * D + ((c * 4 + grp) ^ k_swizzle<R>(key_row + 4 * b)) * 8;
+  const int v_at = (grp >> 1) * VH_ELEMS + col * 16 + ((grp & 1) ^ (col >> 3)) * 8;
+  // the tiles that the wave sees, [see_from, see_until], and among them those that need no mask,
+  // [plain_until, plain_from] (tile starts; an empty range where there is no such tile)
+  const bool has_rows = pos_hi >= pos_lo;
+  const int see_until = has_rows ? pos_hi : -1;
+  const int see_from = window > 0 ? pos_lo - window + 1 - 31 : 0;
+  const int plain_from = pos_hi - pos_lo == 31 ? pos_lo - 31 : -1;
+  const int plain_until = window > 0 ? pos_hi - window + 1 : 0;
   auto sees = [&](int it) __attribute__((always_inline)) {  // whether any of the wave's queries sees a key of the tile
     const int t = begin + it * 32;
-    return wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1);
+    return t <= see_until && t >= see_from;
   };
-  auto scores = [&](int it, VFrag (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
+  auto scores = [&](int it, bf16x8 (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
     const int t = begin + it * 32, buf = it % NB;
     {
-      const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
+      const bool need_mask = t > plain_from || t < plain_until;
       const bf16_t* ks = &lds[buf][0];
       const bf16_t* vs = &lds[buf][K_ELEMS];
       // all operand fragments of the tile are requested from LDS first, so that the reads of V
@@ -769,13 +784,12 @@ void attention_prefill_shared_kernel(
       bf16x8 kf0[DK], kf1[DK];
 #pragma unroll
       for (int c = 0; c < DK; ++c) {
-        kf0[c] = *reinterpret_cast<const bf16x8*>(ks + k_at[c]);
-        kf1[c] = *reinterpret_cast<const bf16x8*>(ks + 16 * D + k_at[c]);
+        kf0[c] = *reinterpret_cast<const bf16x8*>(ks + k_at[0][c]);
+        kf1[c] = *reinterpret_cast<const bf16x8*>(ks + k_at[1][c]);
       }
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
-        vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + c * 256 + v_at);
-        vf[c].h[1] = *reinterpret_cast<const short4a*>(vs + VH_ELEMS + c * 256 + v_at);
+        vf[c] = *reinterpret_cast<const bf16x8*>(vs + c * 256 + v_at);
       }
       // S^T of both column tiles, for the two halves of the tile: keys t+4g+i and t+16+4g+i
       float4v sa[2], sb[2];
@@ -805,7 +819,7 @@ void attention_prefill_shared_kernel(
           const int low = window > 0 ? pos[j] - window + 1 : 0;
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            const int key = t + (i < 4 ? 4 * grp + i : 16 + 4 * grp + i - 4);
+            const int key = t + 8 * grp + i;
             if (key > pos[j] || key < low) sv[j][i] = -INFINITY;
           }
         }
@@ -861,18 +875,16 @@ void attention_prefill_shared_kernel(
 #pragma unroll
         for (int c = 0; c < DCH; ++c)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (t + 4 * grp + i >= n_keys) vf[c].h[0][i] = 0;
-            if (t + 16 + 4 * grp + i >= n_keys) vf[c].h[1][i] = 0;
-          }
+          for (int i = 0; i < 8; ++i)
+            if (t + 8 * grp + i >= n_keys) vf[c][i] = (__bf16)0.f;
       }
     }
   };
-  auto values = [&](VFrag (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
+  auto values = [&](bf16x8 (&vf)[DCH], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
 #pragma unroll
     for (int c = 0; c < DCH; ++c)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
+      for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c], pb[j], st[j].o[c]);
   };
   auto move_on = [&](int it) __attribute__((always_inline)) {
     // tile it+NB-1 sets out for the buffer that tile it-1 left at the last barrier; tile it+1 has
@@ -890,7 +902,7 @@ void attention_prefill_shared_kernel(
       const int it = it0 + r;
       if (it >= n_tiles) break;
       if (sees(it)) {
-        VFrag vf[DCH];
+        bf16x8 vf[DCH];
         bf16x8 pb[2];
         scores(it, vf, pb);
         values(vf, pb);
@@ -1413,6 +1425,44 @@ extern "C" int dli_attention_decode_bf16_static(const void* q, int64_t q_stride,
                                    scale, window, splits, stream);
 }
 
+// Which of the shared-tile kernels a launch of `launch` workgroups takes (hw: query heads that a
+// workgroup takes, 4, 2 or 1). As a rule every tile has a workgroup of its own (0): listed
+// longest first, the tiles even the causal triangle out through the queue of workgroups, and no
+// wave waits for a wave of another tile. Two kernels let a workgroup take a tile and its mirror
+// tile, which halves the workgroups that do anything: one after the other with the keys of each
+// shared out to two sets of waves (2; heads of up to 64, it runs out of registers above), or side
+// by side (1). They win where a launch has between one and two workgroups a compute unit and a
+// workgroup's four waves take different blocks of queries (hw < 4: the waves with the later
+// queries decide how long the workgroup takes, and the two kernels even that out), or the heads
+// are large; they fall off a cliff as soon as a unit would need a second such workgroup (they
+// fill its registers), earlier for the larger heads, so their windows are kept to what was
+// measured. Per layer, kernels 0 / 1 / 2 in us, each timed in the steady state of a loop of
+// launches, workgroups a unit in brackets:
+//   32 heads of 64 on 8 (hw 4): 1,024 tokens [1.0] 23.4 / 24.7 / 26.4, 1,536 [1.5] 32.2 / 33.1 / 33.8,
+//     2,048 [2.0] 41.2 / 41.7 / 41.6, 2,304 [2.2] 46.2 / 51.1 / 85.3, 3,072 [3.0] 61.5 / 69.7 / 107,
+//     4,096 98.8 / 94.9 / 136, 8,192 316 / 330 / 491 (869 TFLOP/s), 16,384 1,216 / 1,253 / 1,870 (904)
+//   32 heads of 64 on 32 (hw 1): 1,024 [1.0] 23.7 / 26.3 / 27.7, 1,536 [1.5] 39.8 / 47.4 / 36.3,
+//     2,048 [2.0] 55.2 / 59.9 / 46.0, 2,560 [2.5] 65.6 / 70.2 / 95.7
+//   16 heads of 32 on 8 (hw 2): 2,048 [1.0] 35.8 / 38.3 / 27.8, 4,096 [2.0] 66.8 / 70.4 / 47.8
+//   24 heads of 128 on 8 (hw 1): 1,408 [1.0] 42.5 / 43.7 / 63.1, 1,728 [1.3] 52.3 / 50.8 / 73.0,
+//     2,048 [1.5] 77.2 / 59.1 / 80.1, 2,304 [1.7] 80.4 / 64.7 / 86.1, 2,560 [1.9] 84.9 / 105 / 174,
+//     3,072 [2.2] 92.9 / 127 / 199, 8,192 455 / 517 / 664 (906 TFLOP/s)
+static int prefill_kernel_choice(int head_dim, int hw, int64_t launch) {
+  const int64_t units = dli_compute_units();
+  if (head_dim > 64) return 5 * launch >= 7 * units && 4 * launch <= 7 * units ? 1 : 0;
+  return hw < 4 && launch >= units && launch <= 2 * units ? 2 : 0;
+}
+
+// The kernel that dli_attention_prefill_bf16 takes for this shape and this many tiles when it is
+// left the choice: 0 every tile a workgroup, 1 a tile and its mirror tile side by side, 2 one after
+// the other with the keys shared out; 3: none of the three (head_dim not a multiple of 32: the
+// kernel without shared tiles).
+extern "C" int dli_attention_prefill_kernel_choice(int head_dim, int q_heads, int kv_heads, int tiles) {
+  if (kv_heads <= 0 || q_heads % kv_heads != 0) return DLI_ERR_ARGUMENT;
+  const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
+  return hw == 0 ? 3 : prefill_kernel_choice(head_dim, hw, (int64_t)tiles * (q_heads / hw));
+}
+
 extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages,
                                           const void* v_pages, void* out, int64_t out_stride,
                                           const int* q_start, const int* kv_len,
@@ -1429,29 +1479,7 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   if (hw > 0) {
     if ((int64_t)kv_heads * page_size * head_dim >= ((int64_t)1 << 31)) return DLI_ERR_ARGUMENT;  // the kernel's 32 bits
     const dim3 sgrid(tiles, q_heads / hw);
-    // Which kernel (pair_tiles 0, 1 or 2; -1: by the size of the launch). As a rule every tile has
-    // a workgroup of its own (0): listed longest first, the tiles even the causal triangle out
-    // through the queue of workgroups, and no wave waits for a wave of another tile. Where the
-    // launch has between one and two workgroups a compute unit, the units that get a second long
-    // tile decide its length: then a workgroup takes a tile and its mirror tile, which halves
-    // the workgroups that do anything, one to a unit: heads of up to 64 one after the other with
-    // the keys of each shared out to two sets of waves (2), larger heads, for which that kernel
-    // runs out of registers, side by side (1). These two fall off a cliff as soon as a unit would
-    // need a second such workgroup (they fill its registers), earlier for the larger heads, so
-    // their windows are kept to what was measured. Per layer, kernels 0 / 1 / 2, each timed in
-    // the steady state of a loop of launches, workgroups a unit in brackets:
-    //   32 heads of 64 on 8: 1,024 tokens [1.0] 25.5 / 27.0 / 26.0 us, 1,536 [1.5] 35.3 / 36.7 / 33.3,
-    //     2,048 [2.0] 45.5 / 46.8 / 41.1, 2,304 [2.2] 51.6 / 54.9 / 84.8, 3,072 [3.0] 67.5 / 75.1 / 105,
-    //     4,096 103 / 101 / 136, 8,192 334 / 368 / 491 (824 TFLOP/s), 16,384 1,241 / 1,376 / 1,870 (886)
-    //   24 heads of 128 on 8: 1,408 tokens [1.0] 48.5 / 49.5 / 62.8, 1,728 [1.3] 58.1 / 57.1 / 73.6,
-    //     2,048 [1.5] 83.3 / 66.3 / 79.2, 2,304 [1.7] 88.6 / 73.1 / 85.7, 2,560 [1.9] 93.6 / 121 / 173,
-    //     3,072 [2.2] 104 / 147 / 198, 8,192 498 / 604 / 664 (828 TFLOP/s)
-    // The tile list has to hold all tiles of a request.
-    const int64_t launch = (int64_t)tiles * (q_heads / hw), units = dli_compute_units();
-    const bool small_heads = head_dim <= 64;
-    const bool in_range = small_heads ? 4 * launch >= 5 * units && launch <= 2 * units
-                                      : 5 * launch >= 7 * units && 4 * launch <= 7 * units;
-    const int mode = pair_tiles >= 0 ? pair_tiles : (in_range ? (small_heads ? 2 : 1) : 0);
+    const int mode = pair_tiles >= 0 ? pair_tiles : prefill_kernel_choice(head_dim, hw, (int64_t)tiles * (q_heads / hw));
     const bool pair = mode == 1;
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \

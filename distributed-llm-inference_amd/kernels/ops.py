@@ -79,6 +79,7 @@ _SIGNATURES = {
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
     "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
+    "dli_attention_prefill_kernel_choice": [_c_int, _c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_decode_self_merging_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
@@ -1005,6 +1006,17 @@ def attention_prefill_tile_rows(head_dim: int, q_heads: int, kv_heads: int) -> i
     rows = int(library().dli_attention_prefill_tile_rows(head_dim, q_heads, kv_heads))
     _require(rows > 0, "query heads are not a multiple of kv heads")
     return rows
+
+
+def attention_prefill_kernel_choice(head_dim: int, q_heads: int, kv_heads: int, tiles: int) -> int:
+    """Which kernel :func:`attention_prefill` takes for a tile list of ``tiles`` entries when it is
+    left the choice (``pair_tiles=None``): 0 every tile a workgroup of its own, 1 a tile and its
+    mirror tile side by side in one workgroup, 2 one after the other with each turn's keys shared
+    out to two sets of waves, 3 the kernel without shared tiles (head sizes that are no multiple
+    of 32)."""
+    choice = int(library().dli_attention_prefill_kernel_choice(head_dim, q_heads, kv_heads, tiles))
+    _require(choice >= 0, "query heads are not a multiple of kv heads")
+    return choice
 
 
 def _check_paged(q, k_pages, v_pages, out, q_heads):

@@ -342,6 +342,45 @@ def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window, pair):
     assert err < tol(torch.bfloat16), err
 
 
+@pytest.mark.parametrize("qh,kvh,d,want_kernel", [(16, 16, 64, 2), (8, 4, 32, 2), (12, 4, 128, 1), (16, 4, 64, 0)])
+def test_attention_prefill_kernel_chosen_by_the_size_of_the_launch(ops, qh, kvh, d, want_kernel):
+    """Left the choice, the prefill attention takes another kernel where a launch has between one and
+    two workgroups a compute unit (a tile and its mirror tile in one workgroup): one prompt whose
+    length puts the launch there, and a short one beside it; against the kernel with a workgroup per
+    tile, and rows of both against a 32-bit softmax over their keys."""
+    units = ops.compute_units(torch.device("cuda"))
+    rows = ops.attention_prefill_tile_rows(d, qh, kvh)
+    per_tile = qh // (4 * 32 // rows)             # workgroups that a tile of the list becomes
+    tiles = -(-units * 3 // (2 * per_tile))        # 1.5 workgroups a unit
+    bs = 16
+    lens = [(tiles * rows - 40 - rows, tiles * rows - 40 - rows), (40, 77)]
+    q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=qh + d)
+    te, tq = _tiles(q_start, rows)
+    assert len(te) == tiles
+    assert ops.attention_prefill_kernel_choice(d, qh, kvh, tiles) == want_kernel
+    assert ops.attention_prefill_kernel_choice(d, qh, kvh, 4 * tiles) == 0
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    scale = 1.0 / math.sqrt(d)
+    args = (q.cuda(), kp.cuda(), vp.cuda())
+    rest = (dev(q_start), dev(kv_len), dev(tables), dev(te), dev(tq), qh, scale, 0)
+    chosen = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
+    ops.attention_prefill(*args, chosen, *rest)
+    single = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
+    ops.attention_prefill(*args, single, *rest, pair_tiles=0)
+    assert (chosen.float() - single.float()).abs().max().item() < tol(torch.bfloat16)
+    # rows of the long request and the short one's last, from their keys gathered out of the pages
+    kd, vd = kp.cuda().float(), vp.cuda().float()
+    for e, row in ((0, 0), (0, 31), (0, 32), (0, lens[0][0] // 2 + 3), (0, lens[0][0] - 1), (1, 39)):
+        n_keys = kv_len[e] - (q_start[e + 1] - q_start[e]) + row + 1
+        pages = torch.tensor(tables[e][:-(-n_keys // bs)], device="cuda")
+        keys = kd[pages].permute(1, 0, 2, 3).reshape(kvh, -1, d)[:, :n_keys]         # [kvh, keys, d]
+        vals = vd[pages].permute(1, 2, 0, 3).reshape(kvh, d, -1)[:, :, :n_keys]      # [kvh, d, keys]
+        qrow = q[q_start[e] + row].cuda().float().view(kvh, qh // kvh, d)
+        p = torch.softmax(torch.einsum("hgd,hkd->hgk", qrow, keys) * scale, dim=-1)
+        ref = torch.einsum("hgk,hdk->hgd", p, vals).reshape(-1)
+        assert (chosen[q_start[e] + row].float() - ref).abs().max().item() < tol(torch.bfloat16), (e, row)
+
+
 def test_attention_finds_one_far_key_among_hundreds(ops):
     """One key far back is made to dominate (its q.k is scaled up); the output must be its value.
     A kernel that drops, misplaces or mis-masks a page cannot pass."""

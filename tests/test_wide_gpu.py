@@ -286,12 +286,11 @@ def test_llama_3_2_1b_in_portions_and_in_mixed_batches(dtype):
         assert core.step.graphs.replays > 0
 
 
-def test_a_prompt_of_1700_tokens_takes_the_kernel_that_shares_keys_between_two_sets_of_waves(monkeypatch):
-    """1,700 tokens at the 1B widths are 54 query tiles of eight kv heads each: between 1.25 and
-    two workgroups a compute unit, where the prefill attention lets a workgroup take a tile and
-    then its mirror tile with each turn's keys shared out to two sets of waves. The whole model
-    through that kernel (chosen by the launch's size, not asked for), whole and as a portion on top
-    of cached keys, against the plain implementation."""
+def test_a_prompt_of_1700_tokens_whole_and_on_top_of_cached_keys(monkeypatch):
+    """1,700 tokens at the 1B widths are 54 query tiles of eight kv heads each: between one and two
+    workgroups a compute unit, so that units work on two tiles of different lengths at a time.
+    The whole model through the prefill attention kernel that the launch's size selects (not asked
+    for), whole and as a portion on top of cached keys, against the plain implementation."""
     from dli_amd.kernels import ops
     from dli_amd.trace import TraceSession
 
@@ -313,8 +312,6 @@ def test_a_prompt_of_1700_tokens_takes_the_kernel_that_shares_keys_between_two_s
     got = s.step([{"id": "w", "tokens": toks, "want": want}], end=["w"])
     check(got, ref[want], "bfloat16", "1,700 tokens whole")
     assert seen and all(tiles == 54 and forced is None for tiles, forced in seen)
-    units = ops.compute_units(torch.device("cuda"))
-    assert 5 * units <= 4 * 54 * 8 and 54 * 8 <= 2 * units, "the launch was meant to fall into the range of the split-key kernel"
     got = s.step([{"id": "p", "tokens": toks[:60], "want": [59]}])
     check(got, ref[59:60], "bfloat16", "first portion")
     got = s.step([{"id": "p", "tokens": toks[60:], "want": [w - 60 for w in want[2:]]}], end=["p"])
