@@ -520,18 +520,15 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // ------------------------------------------------------------------------------------ prefill, shared tiles
 // The waves of a workgroup share every key tile through LDS. Four waves take HW query heads of
 // one kv head (HW = 4, 2 or 1, whatever divides the group) times 4/HW blocks of 32 queries, so
-// each K/V tile is fetched from memory once for 128 query rows. With PAIR a workgroup has a second
-// set of four waves that takes the mirror tile of the same request (tile b of n pairs with tile
-// n-1-b): under a causal mask the two together always have the same number of key tiles to visit,
-// whatever b, so that all workgroups take equally long; the workgroups of the lower half of the
-// tile list leave at once. Tiles of 32 keys are pipelined through a ring of NB buffers in LDS:
+// each K/V tile is fetched from memory once for 128 query rows. Every tile of the list has a
+// workgroup of its own: listed longest first, the tiles even the causal triangle out through the
+// queue of workgroups, and no wave waits for a wave of another tile. Tiles of 32 keys are
+// pipelined through a ring of NB buffers in LDS:
 // while tile i is consumed, tile i+1 already lies there and tiles i+2..i+NB-1 are on their way
 // from memory, written into LDS by the loads themselves (no registers, no second instruction; moving
 // a tile through registers took a third of the kernel's time at 8,192 tokens).
 // Products use v_mfma_f32_16x16x32_bf16 (lane l: row/column l%16, k-indices 8*(l/16)..+7). For
-// P*V the eight k-indices of lane group g stand for the keys 8g..8g+7 of the tile here (in the
-// kernel further down that splits a turn's keys: for the keys 4g..4g+3 and 16+4g..16+4g+3, which
-// is how two products of 16 consecutive keys each leave S^T).
+// P*V the eight k-indices of lane group g stand for the keys 8g..8g+7 of the tile.
 // Needs head_dim % 32 == 0.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
@@ -568,10 +565,11 @@ __device__ __forceinline__ void tile_barrier() {
   asm volatile("" ::: "memory");
 }
 
-// (The single-tile kernel for heads of up to 64 is held to the registers that let three waves
-// share a SIMD: 130 instead of 176, nothing spilled, no copies between the two register files.)
-template <int DCH, bool PAIR>
-__global__ __launch_bounds__(PAIR ? 512 : 256) __attribute__((amdgpu_waves_per_eu(PAIR ? 1 : (DCH <= 4 ? 3 : 2))))
+// (Held to the registers that let three waves share a SIMD for heads of up to 64 and two for
+// larger ones: 126 instead of 176 and 196 instead of 276, nothing spilled, no copies between
+// the two register files.)
+template <int DCH>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DCH <= 4 ? 3 : 2)))
 void attention_prefill_shared_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
@@ -581,7 +579,7 @@ void attention_prefill_shared_kernel(
     int window, int heads_per_wg) {
   constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of the first product
   constexpr int R = D / 8;                      // 16-byte chunks in a key's row of K
-  constexpr int NT = PAIR ? 512 : 256;          // threads
+  constexpr int NT = 256;                       // threads
   constexpr int NW = NT / DLI_WAVE;             // waves
   constexpr int BLOCKS = 2 * DCH;               // 1 KB blocks of a tile (64 chunks of 16 bytes): DCH of K, DCH of V^T
   constexpr int UCH = (BLOCKS + NW - 1) / NW;   // blocks per wave and tile
@@ -593,35 +591,33 @@ void attention_prefill_shared_kernel(
   // Workgroups are dealt to the eight XCDs in turn by their linear index, and each XCD has an L2
   // of its own: the tiles of one kv head are therefore given to one XCD (when the heads divide
   // evenly), so that a head's keys and values are fetched into one L2 instead of all eight.
+  // Eight workgroups in a row (one an XCD) take the same tile for eight heads; the next eight the
+  // same tile for the next eight heads, and only then the list's next tile: workgroups start in
+  // the order of the tile list whatever the number of heads.
   int bx = blockIdx.x, by = blockIdx.y;
+  const int linear = blockIdx.x + gridDim.x * blockIdx.y;
   if (gridDim.y % 8 == 0) {
-    const int linear = blockIdx.x + gridDim.x * blockIdx.y;
-    const int slot = linear / 8;
-    by = linear % 8 + 8 * (slot / (int)gridDim.x);
-    bx = slot % (int)gridDim.x;
+    const int slot = linear / 8, head_blocks = gridDim.y / 8;
+    by = linear % 8 + 8 * (slot % head_blocks);
+    bx = slot / head_blocks;
+  } else {  // the list's order at least: a tile for all heads, then the next tile
+    by = linear % (int)gridDim.y;
+    bx = linear / (int)gridDim.y;
   }
   const int e = tile_entry[bx];
   const int tok0 = q_start[e];
   const int q_len = q_start[e + 1] - tok0;
   const int tile_rows = (4 / heads_per_wg) * 32;
   const int q0_first = tile_q0[bx];
-  int q0_second = -1;
-  if (PAIR) {
-    const int b = q0_first / tile_rows, mirror = (q_len + tile_rows - 1) / tile_rows - 1 - b;
-    if (b < mirror) return;  // the workgroup of the mirror tile does this one too
-    if (mirror < b) q0_second = mirror * tile_rows;
-  }
   const int group = q_heads / kv_heads;
   const int wg_per_kv = group / heads_per_wg;
   const int kvh = by / wg_per_kv;
-  const int lane = threadIdx.x % DLI_WAVE, wave = (threadIdx.x / DLI_WAVE) % 4;
-  const int set = threadIdx.x / 256;  // which of the workgroup's two tiles
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
   const int col = lane % 16, grp = lane / 16;
   const int head = kvh * group + (by % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
   const int n_keys = kv_len[e];
   const int first_pos = n_keys - q_len;
-  const int set_q0 = set == 0 ? q0_first : q0_second;
-  const int q0 = set_q0 < 0 ? q_len : set_q0 + (wave / heads_per_wg) * 32;  // this wave's first query
+  const int q0 = q0_first + (wave / heads_per_wg) * 32;  // this wave's first query
   const int wave_rows = max(0, min(32, q_len - q0));
   const int* table = block_tables + (int64_t)e * table_stride;
 
@@ -653,7 +649,7 @@ void attention_prefill_shared_kernel(
   const int pos_lo = __builtin_amdgcn_readfirstlane(first_pos + q0);
   const int pos_hi = __builtin_amdgcn_readfirstlane(first_pos + q0 + wave_rows - 1);
   // the workgroup walks the keys that any of its queries sees
-  const int wg_q_lo = q0_second >= 0 ? q0_second : q0_first;
+  const int wg_q_lo = q0_first;
   const int wg_q_hi = min(q_len, q0_first + tile_rows) - 1;
   const int begin = window > 0 ? max(0, first_pos + wg_q_lo - window + 1) / 32 * 32 : 0;
   const int end = first_pos + wg_q_hi + 1;
@@ -892,10 +888,7 @@ void attention_prefill_shared_kernel(
     fetch((it + NB - 1) % NB);
     wait_loads<(NB - 2) * UCH>();
   };
-  // Tried and slower by 10 to 15%: the second set half a tile behind the first (two barriers a
-  // tile), so that one set's products run beside the other's softmax; and the pair's key tiles
-  // dealt out evenly to the two sets with a merge of their states at the end. Slower by 45% in the
-  // single-tile kernel: S^T of tile it+1 sent to the matrix cores before the softmax of tile it.
+  // (Tried and 45% slower: S^T of tile it+1 sent to the matrix cores before the softmax of tile it.)
   for (int it0 = 0; it0 < n_tiles; it0 += NB) {
 #pragma unroll
     for (int r = 0; r < NB; ++r) {
@@ -925,337 +918,6 @@ void attention_prefill_shared_kernel(
                               bf16_bits(st[j].o[c][2] * inv), bf16_bits(st[j].o[c][3] * inv)};
       *reinterpret_cast<short4v*>(op + c * 16) = packed;
     }
-  }
-}
-
-// ------------------------------------------------------------------------------------ prefill, keys split over two sets of waves
-// For launches of a few workgroups per compute unit. There the shared-tile kernel's time is the
-// time of its longest workgroup, and that is a chain of dependent steps per key tile (LDS reads,
-// first product, softmax, second product, the next tile's staging, the barrier) which one wave a
-// SIMD walks alone: some 1,900 cycles a tile of 32 keys, three times what its instructions take.
-// Here a workgroup has two sets of four waves that work on the SAME queries (a tile of the list,
-// 32 queries a wave as above): every turn stages 64 keys, of which the first set takes the first
-// 32 and the second set the other 32, so the chain is half as many turns long; after the last
-// turn the second set hands its running maximum, sum and output over through LDS and the first
-// set merges them with its own. A workgroup does that for a tile and then for its mirror tile
-// of the same request (tile b of n with tile n-1-b: together always n+1 key tiles, whatever b),
-// so all workgroups of a request take equally long; the workgroups of the lower half of the
-// tile list leave at once. Heads, products and layouts as in the shared-tile kernel.
-template <int DCH>
-__global__ __launch_bounds__(512) void attention_prefill_split_kernel(
-    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
-    const bf16_t* __restrict__ v_pages, bf16_t* __restrict__ out, int64_t out_stride,
-    const int* __restrict__ q_start, const int* __restrict__ kv_len,
-    const int* __restrict__ block_tables, int table_stride, const int* __restrict__ tile_entry,
-    const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
-    int window, int heads_per_wg) {
-  constexpr int D = DCH * 16, DK = D / 32;
-  constexpr int KPAD = D + 8, VPAD = 32 + 8;
-  constexpr int NT = 512;
-  constexpr int CHUNKS = 8 * D;                 // 16-byte chunks of 32 keys: 4D of K, then 4D of V^T
-  constexpr int UCH = 2 * CHUNKS / NT;          // chunks per thread and turn (64 keys): D / 32
-  constexpr int RD = 3;                         // turns in flight from memory to registers
-  constexpr int K_ELEMS = 32 * KPAD, TILE_ELEMS = K_ELEMS + D * VPAD;
-  constexpr int STATE = 2 + 4 * DCH;            // floats of one column tile's state per lane
-  static_assert(2 * STATE * 256 * 4 <= 3 * 2 * TILE_ELEMS * 2, "the hand-over reuses the tile buffers");
-  __shared__ __attribute__((aligned(16))) bf16_t lds[3][2][TILE_ELEMS];  // per turn: keys 0..31, keys 32..63
-
-  int bx = blockIdx.x, by = blockIdx.y;
-  if (gridDim.y % 8 == 0) {  // the tiles of one kv head on one XCD, as in the shared-tile kernel
-    const int linear = blockIdx.x + gridDim.x * blockIdx.y;
-    const int slot = linear / 8;
-    by = linear % 8 + 8 * (slot / (int)gridDim.x);
-    bx = slot % (int)gridDim.x;
-  }
-  const int e = tile_entry[bx];
-  const int tok0 = q_start[e];
-  const int q_len = q_start[e + 1] - tok0;
-  const int tile_rows = (4 / heads_per_wg) * 32;
-  const int q0_first = tile_q0[bx];
-  int q0_second = -1;
-  {
-    const int b = q0_first / tile_rows, mirror = (q_len + tile_rows - 1) / tile_rows - 1 - b;
-    if (b < mirror) return;  // the workgroup of the mirror tile does this one too
-    if (mirror < b) q0_second = mirror * tile_rows;
-  }
-  const int group = q_heads / kv_heads;
-  const int wg_per_kv = group / heads_per_wg;
-  const int kvh = by / wg_per_kv;
-  const int lane = threadIdx.x % DLI_WAVE, wave = (threadIdx.x / DLI_WAVE) % 4;
-  const int set = threadIdx.x / 256;  // which 32 of a turn's 64 keys
-  const int col = lane % 16, grp = lane / 16;
-  const int head = kvh * group + (by % wg_per_kv) * heads_per_wg + wave % heads_per_wg;
-  const int n_keys = kv_len[e];
-  const int first_pos = n_keys - q_len;
-  const int* table = block_tables + (int64_t)e * table_stride;
-
-  // Staging: chunk u of a turn, u = thread + r * 512. u / CHUNKS says which 32 keys; within them
-  // chunk v < 4D is 8 dims of key v/(D/8) and chunk 4D+c holds 8 keys of dim (c%2D)/2, of the
-  // first 16 keys for c < 2D and of the other 16 after that. A run of 2D chunks (a multiple of 64)
-  // thus lies in one sixteenth-aligned run of 16 keys, i.e. in one page, and is K or V^T as a
-  // whole: per wave and r, the page's address is made on the scalar unit.
-  const int wave_first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / DLI_WAVE)) * DLI_WAVE;
-  unsigned lane_off[UCH];
-  int lds_off[UCH], v_key[UCH], first_key[UCH];  // first_key: of the chunk's run of 16 keys, within the turn's 64
-  bool is_v[UCH];
-#pragma unroll
-  for (int r = 0; r < UCH; ++r) {
-    const int u = threadIdx.x + r * NT, u_wave = wave_first + r * NT;
-    const int sub = u_wave / CHUNKS, v = u % CHUNKS, v_wave = u_wave % CHUNKS;
-    is_v[r] = v_wave >= 4 * D;
-    const bool second = is_v[r] ? v_wave >= 6 * D : v_wave >= 2 * D;
-    first_key[r] = sub * 32 + (second ? 16 : 0);
-    if (!is_v[r]) {
-      const int kk = v / (D / 8), part = v % (D / 8);
-      lane_off[r] = (kk % 16) * D + part * 8;
-      lds_off[r] = sub * TILE_ELEMS + kk * KPAD + part * 8;
-      v_key[r] = 0;
-    } else {
-      const int c = v - 4 * D, d = (c % (2 * D)) / 2, part = c % 2;
-      lane_off[r] = d * page_size + part * 8;
-      v_key[r] = (second ? 16 : 0) + part * 8;   // within the 32 keys
-      lds_off[r] = sub * TILE_ELEMS + K_ELEMS + d * VPAD + v_key[r];
-      v_key[r] += sub * 32;                       // within the turn's 64
-    }
-  }
-  const unsigned page_stride = (unsigned)kv_heads * (unsigned)page_size * (unsigned)D;
-  const bf16_t* k_head = k_pages + (int64_t)kvh * page_size * D;
-  const bf16_t* v_head = v_pages + (int64_t)kvh * page_size * D;
-  const int turn_pages = 64 / page_size, turn_rest = 64 % page_size;  // 64 keys on, in pages and keys
-
-  typedef short short4a __attribute__((ext_vector_type(4)));
-  union VFrag {
-    bf16x8 v;
-    short4a h[2];
-  };
-
-  for (int phase = 0; phase < 2; ++phase) {
-    const int q0_tile = phase == 0 ? q0_first : q0_second;
-    if (q0_tile < 0) break;
-    const int q0 = q0_tile + (wave / heads_per_wg) * 32;  // this wave's first query
-    const int wave_rows = max(0, min(32, q_len - q0));
-    bf16x8 qreg[2][DK];
-    ColumnTile<DCH> st[2];
-    float m_ref[2], raise_at[2];  // as in the shared-tile kernel: the exponent's reference, and the score that moves it
-    constexpr float LAZY_LOG2 = 8.f;
-    const float inv_scale_log2e = 1.f / scale_log2e;
-    int pos[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      st[j].init();
-      m_ref[j] = 0.f;
-      raise_at[j] = -INFINITY;
-      const int qi = q0 + j * 16 + col;
-      pos[j] = qi < q_len ? first_pos + qi : -1;
-#pragma unroll
-      for (int c = 0; c < DK; ++c) qreg[j][c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (qi < q_len) {
-        const bf16_t* qp = q + (int64_t)(tok0 + qi) * q_stride + (int64_t)head * D + grp * 8;
-#pragma unroll
-        for (int c = 0; c < DK; ++c) qreg[j][c] = *reinterpret_cast<const bf16x8*>(qp + c * 32);
-      }
-    }
-    const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + wave_rows - 1;
-    const int wg_q_hi = min(q_len, q0_tile + tile_rows) - 1;
-    const int begin = window > 0 ? max(0, first_pos + q0_tile - window + 1) / 64 * 64 : 0;
-    const int end = first_pos + wg_q_hi + 1;
-    const int n_turns = (end - begin + 63) / 64;
-
-    // Per chunk of this thread: where the run of 16 keys that it belongs to lies, turn after turn.
-    // Everything here is the same in all lanes of a wave, but it is computed per lane on purpose:
-    // on the scalar unit the table lookups and 64-bit address sums were more instructions a turn
-    // than the softmax, and a wave issues them in turn with its vector instructions.
-    int run_page[UCH], run_off[UCH], run_key[UCH];
-    int page_next[UCH];  // looked up one turn before the keys are fetched
-    int lane_zero;       // zero in a vector register: what is added to it is a value per lane for the compiler
-    asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
-    const int last_page = (n_keys - 1) / page_size;  // entries behind it may hold anything
-#pragma unroll
-    for (int r = 0; r < UCH; ++r) {
-      run_key[r] = begin + first_key[r] + lane_zero;
-      run_page[r] = run_key[r] / page_size;
-      run_off[r] = run_key[r] % page_size;
-      page_next[r] = table[min(run_page[r], last_page)];
-    }
-    bf16x8 stage[RD][UCH];
-    // The same loads whatever the turn, also past the last key (the request's last page again,
-    // never used), so that the count of loads in flight is known at compile time.
-    auto fetch = [&](bf16x8 (&sq)[UCH]) {
-#pragma unroll
-      for (int r = 0; r < UCH; ++r) {
-        const unsigned off = run_off[r];
-        const bf16_t* base = (is_v[r] ? v_head : k_head) + (uint64_t)(unsigned)page_next[r] * page_stride +
-                             (is_v[r] ? off : off * D);
-        sq[r] = *reinterpret_cast<const bf16x8*>(base + lane_off[r]);
-        run_key[r] += 64;
-        run_page[r] += turn_pages;
-        run_off[r] += turn_rest;
-        if (run_off[r] >= page_size) {
-          run_off[r] -= page_size;
-          ++run_page[r];
-        }
-        page_next[r] = table[min(run_page[r], last_page)];
-      }
-    };
-    auto stash = [&](int buf, int t, bf16x8 (&sq)[UCH]) {  // t: the turn's first key
-#pragma unroll
-      for (int r = 0; r < UCH; ++r) {
-        if (t + 64 > n_keys && is_v[r]) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i)
-            if (t + v_key[r] + i >= n_keys) sq[r][i] = (bf16_t)0.f;
-        }
-        *reinterpret_cast<bf16x8*>(&lds[buf][0][lds_off[r]]) = sq[r];
-      }
-    };
-#pragma unroll
-    for (int T = 0; T < 2 + RD; ++T) {
-      fetch(stage[T % RD]);
-      if (T < 2) stash(T, begin + T * 64, stage[T % RD]);
-    }
-    __syncthreads();
-
-    for (int it0 = 0; it0 < n_turns; it0 += RD) {
-#pragma unroll
-      for (int r3 = 0; r3 < RD; ++r3) {
-        const int it = it0 + r3;
-        if (it >= n_turns) break;
-        const int t = begin + it * 64 + set * 32;  // this set's 32 keys
-        if (wave_rows > 0 && t <= pos_hi && (window <= 0 || t + 31 >= pos_lo - window + 1)) {
-          const bool need_mask = t + 31 > pos_lo || (window > 0 && t < pos_hi - window + 1) || wave_rows < 32;
-          const bf16_t* ks = &lds[it % 3][set][0];
-          const bf16_t* vs = ks + K_ELEMS;
-          bf16x8 kf0[DK], kf1[DK];
-          VFrag vf[DCH];
-#pragma unroll
-          for (int c = 0; c < DK; ++c) {
-            kf0[c] = *reinterpret_cast<const bf16x8*>(ks + col * KPAD + c * 32 + grp * 8);
-            kf1[c] = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KPAD + c * 32 + grp * 8);
-          }
-#pragma unroll
-          for (int c = 0; c < DCH; ++c) {
-            vf[c].h[0] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 4 * grp);
-            vf[c].h[1] = *reinterpret_cast<const short4a*>(vs + (c * 16 + col) * VPAD + 16 + 4 * grp);
-          }
-          float4v sa[2], sb[2];
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            sa[j] = float4v{0.f, 0.f, 0.f, 0.f};
-            sb[j] = float4v{0.f, 0.f, 0.f, 0.f};
-          }
-#pragma unroll
-          for (int c = 0; c < DK; ++c)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              sa[j] = mfma32(kf0[c], qreg[j][c], sa[j]);
-              sb[j] = mfma32(kf1[c], qreg[j][c], sb[j]);
-            }
-          float sv[2][8];
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              sv[j][i] = sa[j][i];
-              sv[j][4 + i] = sb[j][i];
-            }
-          if (need_mask) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const int low = window > 0 ? pos[j] - window + 1 : 0;
-#pragma unroll
-              for (int i = 0; i < 8; ++i) {
-                const int key = t + (i < 4 ? 4 * grp + i : 16 + 4 * grp + i - 4);
-                if (key > pos[j] || key < low) sv[j][i] = -INFINITY;
-              }
-            }
-          }
-          float lane_max[2];
-          bool rise = false;
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            lane_max[j] = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]),
-                               max2(sv[j][6], sv[j][7]));
-            rise |= lane_max[j] > raise_at[j];
-          }
-          if (__builtin_amdgcn_ballot_w64(rise) != 0) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const float tile_max = column_max(lane_max[j]) * scale_log2e;
-              const float m_new = max2(st[j].m, tile_max);
-              const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-              const float alpha = fast_exp2(st[j].m - m_safe);
-              st[j].l *= alpha;
-#pragma unroll
-              for (int c = 0; c < DCH; ++c) st[j].o[c] *= alpha;
-              st[j].m = m_new;
-              m_ref[j] = m_safe;
-              raise_at[j] = m_new == -INFINITY ? -INFINITY : (m_new + LAZY_LOG2) * inv_scale_log2e;
-            }
-          }
-          bf16x8 pb[2];
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            float tile_sum = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              const float p = fast_exp2(fmaf(sv[j][i], scale_log2e, -m_ref[j]));
-              tile_sum += p;
-              pb[j][i] = (bf16_t)p;
-            }
-            st[j].l += tile_sum;
-          }
-#pragma unroll
-          for (int c = 0; c < DCH; ++c)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) st[j].o[c] = mfma32(vf[c].v, pb[j], st[j].o[c]);
-        }
-        // turn it+2 leaves its register slot for LDS; the slot then receives turn it+2+RD
-        stash((it + 2) % 3, begin + (it + 2) * 64, stage[(r3 + 2) % RD]);
-        fetch(stage[(r3 + 2) % RD]);
-        __syncthreads();
-      }
-    }
-
-    // The second set hands over, the first merges: state v of lane l of wave w lies at
-    // [v][w * 64 + l], so that a wave's accesses are consecutive.
-    float* hand = reinterpret_cast<float*>(&lds[0][0][0]);
-    const int mine = wave * DLI_WAVE + lane;
-    if (set == 1) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        hand[(j * STATE + 0) * 256 + mine] = st[j].m;
-        hand[(j * STATE + 1) * 256 + mine] = st[j].l;
-#pragma unroll
-        for (int c = 0; c < DCH; ++c)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) hand[(j * STATE + 2 + 4 * c + i) * 256 + mine] = st[j].o[c][i];
-      }
-    }
-    __syncthreads();
-    if (set == 0) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const float m_other = hand[(j * STATE + 0) * 256 + mine], l_other = hand[(j * STATE + 1) * 256 + mine];
-        const float m_all = max2(st[j].m, m_other);
-        const float m_safe = m_all == -INFINITY ? 0.f : m_all;
-        const float a_mine = fast_exp2(st[j].m - m_safe), a_other = fast_exp2(m_other - m_safe);
-        const float l_sum = column_sum(st[j].l * a_mine + l_other * a_other);  // every lane takes part
-        const int qi = q0 + j * 16 + col;
-        if (qi >= q_len) continue;
-        const float inv = l_sum > 0.f ? 1.f / l_sum : 0.f;
-        bf16_t* op = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * D + 4 * grp;
-#pragma unroll
-        for (int c = 0; c < DCH; ++c) {
-          float o[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            o[i] = (st[j].o[c][i] * a_mine + hand[(j * STATE + 2 + 4 * c + i) * 256 + mine] * a_other) * inv;
-          const short4v packed = {bf16_bits(o[0]), bf16_bits(o[1]), bf16_bits(o[2]), bf16_bits(o[3])};
-          *reinterpret_cast<short4v*>(op + c * 16) = packed;
-        }
-      }
-    }
-    __syncthreads();  // the tile buffers are staged again for the mirror tile
   }
 }
 
@@ -1425,52 +1087,13 @@ extern "C" int dli_attention_decode_bf16_static(const void* q, int64_t q_stride,
                                    scale, window, splits, stream);
 }
 
-// Which of the shared-tile kernels a launch of `launch` workgroups takes (hw: query heads that a
-// workgroup takes, 4, 2 or 1). As a rule every tile has a workgroup of its own (0): listed
-// longest first, the tiles even the causal triangle out through the queue of workgroups, and no
-// wave waits for a wave of another tile. Two kernels let a workgroup take a tile and its mirror
-// tile, which halves the workgroups that do anything: one after the other with the keys of each
-// shared out to two sets of waves (2; heads of up to 64, it runs out of registers above), or side
-// by side (1). They win where a launch has between one and two workgroups a compute unit and a
-// workgroup's four waves take different blocks of queries (hw < 4: the waves with the later
-// queries decide how long the workgroup takes, and the two kernels even that out), or the heads
-// are large; they fall off a cliff as soon as a unit would need a second such workgroup (they
-// fill its registers), earlier for the larger heads, so their windows are kept to what was
-// measured. Per layer, kernels 0 / 1 / 2 in us, each timed in the steady state of a loop of
-// launches, workgroups a unit in brackets:
-//   32 heads of 64 on 8 (hw 4): 1,024 tokens [1.0] 23.4 / 24.7 / 26.4, 1,536 [1.5] 32.2 / 33.1 / 33.8,
-//     2,048 [2.0] 41.2 / 41.7 / 41.6, 2,304 [2.2] 46.2 / 51.1 / 85.3, 3,072 [3.0] 61.5 / 69.7 / 107,
-//     4,096 98.8 / 94.9 / 136, 8,192 316 / 330 / 491 (869 TFLOP/s), 16,384 1,216 / 1,253 / 1,870 (904)
-//   32 heads of 64 on 32 (hw 1): 1,024 [1.0] 23.7 / 26.3 / 27.7, 1,536 [1.5] 39.8 / 47.4 / 36.3,
-//     2,048 [2.0] 55.2 / 59.9 / 46.0, 2,560 [2.5] 65.6 / 70.2 / 95.7
-//   16 heads of 32 on 8 (hw 2): 2,048 [1.0] 35.8 / 38.3 / 27.8, 4,096 [2.0] 66.8 / 70.4 / 47.8
-//   24 heads of 128 on 8 (hw 1): 1,408 [1.0] 42.5 / 43.7 / 63.1, 1,728 [1.3] 52.3 / 50.8 / 73.0,
-//     2,048 [1.5] 77.2 / 59.1 / 80.1, 2,304 [1.7] 80.4 / 64.7 / 86.1, 2,560 [1.9] 84.9 / 105 / 174,
-//     3,072 [2.2] 92.9 / 127 / 199, 8,192 455 / 517 / 664 (906 TFLOP/s)
-static int prefill_kernel_choice(int head_dim, int hw, int64_t launch) {
-  const int64_t units = dli_compute_units();
-  if (head_dim > 64) return 5 * launch >= 7 * units && 4 * launch <= 7 * units ? 1 : 0;
-  return hw < 4 && launch >= units && launch <= 2 * units ? 2 : 0;
-}
-
-// The kernel that dli_attention_prefill_bf16 takes for this shape and this many tiles when it is
-// left the choice: 0 every tile a workgroup, 1 a tile and its mirror tile side by side, 2 one after
-// the other with the keys shared out; 3: none of the three (head_dim not a multiple of 32: the
-// kernel without shared tiles).
-extern "C" int dli_attention_prefill_kernel_choice(int head_dim, int q_heads, int kv_heads, int tiles) {
-  if (kv_heads <= 0 || q_heads % kv_heads != 0) return DLI_ERR_ARGUMENT;
-  const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
-  return hw == 0 ? 3 : prefill_kernel_choice(head_dim, hw, (int64_t)tiles * (q_heads / hw));
-}
-
 extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages,
                                           const void* v_pages, void* out, int64_t out_stride,
                                           const int* q_start, const int* kv_len,
                                           const int* block_tables, int table_stride,
                                           const int* tile_entry, const int* tile_q0, int tiles,
                                           int q_heads, int kv_heads, int head_dim, int page_size,
-                                          float scale, int window, int pair_tiles,
-                                          hipStream_t stream) {
+                                          float scale, int window, hipStream_t stream) {
   if (tiles <= 0) return DLI_OK;
   if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || q_heads > 65535 || q_stride % 4 != 0 || out_stride % 4 != 0)
@@ -1479,25 +1102,12 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
   if (hw > 0) {
     if ((int64_t)kv_heads * page_size * head_dim >= ((int64_t)1 << 31)) return DLI_ERR_ARGUMENT;  // the kernel's 32 bits
     const dim3 sgrid(tiles, q_heads / hw);
-    const int mode = pair_tiles >= 0 ? pair_tiles : prefill_kernel_choice(head_dim, hw, (int64_t)tiles * (q_heads / hw));
-    const bool pair = mode == 1;
 #define SHARED_CASE(N)                                                                            \
   case N:                                                                                         \
-    if (mode == 2)                                                                                \
-      attention_prefill_split_kernel<N><<<sgrid, 512, 0, stream>>>(                               \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
-          (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \
-          tile_q0, q_heads, kv_heads, page_size, scale * LOG2E, window, hw);                      \
-    else if (pair)                                                                                \
-      attention_prefill_shared_kernel<N, true><<<sgrid, 512, 0, stream>>>(                        \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
-          (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \
-          tile_q0, q_heads, kv_heads, page_size, scale * LOG2E, window, hw);                      \
-    else                                                                                          \
-      attention_prefill_shared_kernel<N, false><<<sgrid, 256, 0, stream>>>(                       \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
-          (bf16_t*)out, out_stride, q_start, kv_len, block_tables, table_stride, tile_entry,      \
-          tile_q0, q_heads, kv_heads, page_size, scale * LOG2E, window, hw);                      \
+    attention_prefill_shared_kernel<N><<<sgrid, 256, 0, stream>>>(                                \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
+        out_stride, q_start, kv_len, block_tables, table_stride, tile_entry, tile_q0, q_heads,    \
+        kv_heads, page_size, scale * LOG2E, window, hw);                                          \
     break;
     switch (head_dim / 16) {
       SHARED_CASE(2) SHARED_CASE(4) SHARED_CASE(6) SHARED_CASE(8)

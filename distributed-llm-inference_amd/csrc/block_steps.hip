@@ -36,8 +36,7 @@ int dli_attention_decode_bf16(const void* q, int64_t q_stride, const void* k_pag
 int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages, void* out,
                                int64_t out_stride, const int* q_start, const int* kv_len, const int* block_tables,
                                int table_stride, const int* tile_entry, const int* tile_q0, int tiles, int q_heads,
-                               int kv_heads, int head_dim, int page_size, float scale, int window, int pair_tiles,
-                               hipStream_t stream);
+                               int kv_heads, int head_dim, int page_size, float scale, int window, hipStream_t stream);
 }
 
 namespace {
@@ -111,8 +110,7 @@ extern "C" int dli_prenorm_blocks_bf16(void* x, const DliBlockArgs* blocks, int 
     if (s.num_entries > s.num_decode)
       STEP(dli_attention_prefill_bf16(s.qkv, qkv_w, b.k_pages, b.v_pages, s.attn, q_w, s.q_start, s.kv_len,
                                       s.block_tables[b.group], s.table_stride[b.group], sh.tile_entry, sh.tile_q0,
-                                      sh.tiles, b.q_heads, b.kv_heads, b.head_dim, s.page_size, b.scale, b.window, -1,
-                                      stream));
+                                      sh.tiles, b.q_heads, b.kv_heads, b.head_dim, s.page_size, b.scale, b.window, stream));
     STEP(dli_gemm_bf16(s.attn, q_w, b.w_o, q_w, b.b_o, s.mixed, h, s.rows, h, q_w, s.gemm_workspace,
                        s.gemm_workspace_bytes, s.device, stream));
     STEP(dli_rms_norm(x, s.mixed, b.norm2_w, x, s.normed, s.rows, b.hidden, b.eps2, 1, stream));

@@ -79,7 +79,6 @@ _SIGNATURES = {
     "dli_attention_generic_tile_rows": [_c_int],
     "dli_attention_mfma_supports": [_c_int, _c_int],
     "dli_attention_prefill_tile_rows": [_c_int, _c_int, _c_int],
-    "dli_attention_prefill_kernel_choice": [_c_int, _c_int, _c_int, _c_int],
     "dli_attention_decode_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_attention_decode_self_merging_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
@@ -91,8 +90,7 @@ _SIGNATURES = {
                                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_rope_angles": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                                   _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
-                                   _c_ptr],
+                                   _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                               _c_int, _c_int, _c_ptr],
@@ -1008,17 +1006,6 @@ def attention_prefill_tile_rows(head_dim: int, q_heads: int, kv_heads: int) -> i
     return rows
 
 
-def attention_prefill_kernel_choice(head_dim: int, q_heads: int, kv_heads: int, tiles: int) -> int:
-    """Which kernel :func:`attention_prefill` takes for a tile list of ``tiles`` entries when it is
-    left the choice (``pair_tiles=None``): 0 every tile a workgroup of its own, 1 a tile and its
-    mirror tile side by side in one workgroup, 2 one after the other with each turn's keys shared
-    out to two sets of waves, 3 the kernel without shared tiles (head sizes that are no multiple
-    of 32)."""
-    choice = int(library().dli_attention_prefill_kernel_choice(head_dim, q_heads, kv_heads, tiles))
-    _require(choice >= 0, "query heads are not a multiple of kv heads")
-    return choice
-
-
 def _check_paged(q, k_pages, v_pages, out, q_heads):
     _dense(k_pages, "k_pages", torch.bfloat16, 4)
     _rows(q, "q", torch.bfloat16)
@@ -1131,15 +1118,11 @@ def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, dtype: torch.dt
 def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
                       tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
-                      window: int = 0, pair_tiles: Optional[int] = None) -> None:
+                      window: int = 0) -> None:
     """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
-    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height and
-    hold every tile of every listed request, in any order: workgroups start in the list's order,
-    so the tiles with the most keys belong first). ``pair_tiles``:
-    1: one workgroup takes a tile and its mirror within the request side by side, which evens out
-    the causal mask's triangle; 2: it takes them one after the other with two sets of waves that
-    share each tile's keys (half as many dependent steps, for launches of few workgroups); 0:
-    every tile has its own workgroup; ``None`` lets the kernel decide by the size of the launch."""
+    :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height, in
+    any order: every tile has a workgroup of its own and workgroups start in the list's order, so
+    the tiles with the most keys belong first)."""
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
     for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
         _dense(t, name, torch.int32, 1)
@@ -1151,8 +1134,7 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
     _check(library().dli_attention_prefill_bf16(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tile_entry.shape[0], q_heads,
-        kv_heads, head_dim, page_size, float(scale), int(window), -1 if pair_tiles is None else int(pair_tiles),
-        _stream()), "attention_prefill")
+        kv_heads, head_dim, page_size, float(scale), int(window), _stream()), "attention_prefill")
 
 # ----------------------------------------------------------------------------- sampling
 

@@ -45,15 +45,16 @@ def planned_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int 
     return coarse
 
 
-def longest_first(ctx: Any, rows: int, units: int = 256) -> Callable:
+def longest_first(ctx: Any, rows: int, units: int = 256, workgroups_per_tile: int = 8) -> Callable:
     """The order in which the prefill kernel wants a step's query tiles: those that see the most
     keys first. Workgroups start in the order of the list, and under a causal mask a tile's work
     grows with its place in the request: listed by place, the longest workgroups start last and
     the launch ends with a few of them alone on the device (a prompt of 8,192 tokens at the 1B
     sizes: 521 us a layer by place, 393 us longest first). Within the sorted list every second
-    run of as many tiles as an XCD has compute units is turned round, so that a unit that got a
-    long tile in one round gets a short one in the next."""
-    per_xcd = max(1, units // 8)
+    run of as many tiles as give every compute unit one workgroup (a tile of the list becomes
+    ``workgroups_per_tile`` workgroups, one per group of query heads) is turned round, so that a
+    unit that got a long tile in one round gets a short one in the next."""
+    per_xcd = max(1, units // max(1, workgroups_per_tile))
 
     def arrange(entries: np.ndarray, firsts: np.ndarray) -> np.ndarray:
         q_len = (ctx.q_start_host[entries + 1] - ctx.q_start_host[entries]).astype(np.int64)
@@ -69,8 +70,12 @@ def longest_first(ctx: Any, rows: int, units: int = 256) -> Callable:
 def prefill_tiles(ctx: Any, head_dim: int, q_heads: int, kv_heads: int, first_entry: int, device: torch.device):
     """The tile list of the step's portions for :func:`ops.attention_prefill`."""
     rows = ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads)
-    return ctx.q_tiles(rows, first_entry=first_entry, arrange=longest_first(ctx, rows, ops.compute_units(device)),
-                       arranged_as="longest first")
+    # a workgroup takes a tile for 4 * 32 / rows query heads where it shares tiles (head sizes that
+    # are multiples of 32), else for one
+    per_tile = q_heads * rows // 128 if head_dim % 32 == 0 else q_heads
+    units = ops.compute_units(device)
+    return ctx.q_tiles(rows, first_entry=first_entry, arrange=longest_first(ctx, rows, units, per_tile),
+                       arranged_as=f"longest first, rounds of {max(1, units // max(1, per_tile))}")
 
 
 def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,

@@ -301,7 +301,7 @@ def test_a_prompt_of_1700_tokens_whole_and_on_top_of_cached_keys(monkeypatch):
     real = ops.attention_prefill
 
     def counted(*a, **k):
-        seen.append((a[7].shape[0], k.get("pair_tiles")))  # tiles in the list, and that nobody forces a kernel
+        seen.append(a[7].shape[0])  # tiles in the list
         return real(*a, **k)
 
     monkeypatch.setattr(ops, "attention_prefill", counted)
@@ -311,7 +311,7 @@ def test_a_prompt_of_1700_tokens_whole_and_on_top_of_cached_keys(monkeypatch):
     want = [0, 17, 511, 512, 1023, 1699]
     got = s.step([{"id": "w", "tokens": toks, "want": want}], end=["w"])
     check(got, ref[want], "bfloat16", "1,700 tokens whole")
-    assert seen and all(tiles == 54 and forced is None for tiles, forced in seen)
+    assert seen and all(tiles == 54 for tiles in seen)
     got = s.step([{"id": "p", "tokens": toks[:60], "want": [59]}])
     check(got, ref[59:60], "bfloat16", "first portion")
     got = s.step([{"id": "p", "tokens": toks[60:], "want": [w - 60 for w in want[2:]]}], end=["p"])
