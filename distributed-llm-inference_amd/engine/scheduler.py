@@ -181,6 +181,11 @@ class Scheduler:
         if not plan.preempted:  # memory that was just freed serves running requests first
             self._admit_waiting(plan, left)
         plan.decode_steps = self._decode_steps(plan)
+        # The step runs its chunks in this order: single tokens first (as the step function lays
+        # them out anyway), those with the most keys first. The decode attention's workgroups start
+        # in row order, and with rows of 128 to 2,300 keys as they come the launch ended with a few
+        # long rows alone on the device (64 such rows at the 3B sizes: 69 us a layer, 59 sorted).
+        plan.chunks.sort(key=lambda c: (0, -c.start) if c.num_tokens == 1 else (1, 0))
         self._step += 1
         return plan
 

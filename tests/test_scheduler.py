@@ -72,6 +72,24 @@ def test_long_prompt_is_cut_into_portions_while_decoding_goes_on():
     assert long.output_ids == alone(list(range(40)), 2)
 
 
+def test_a_step_lists_decoding_requests_first_and_the_longest_of_them_first():
+    """The plan's order is the order of the step's rows: single tokens before portions, the rows with
+    the most keys first (the decode attention's workgroups start in row order)."""
+    eng, runner, _ = make(budget=64)
+    lens = [5, 23, 11, 17]
+    for i, n in enumerate(lens):
+        eng.add_request(f"r{i}", list(range(n)), SamplingParams(max_tokens=6))
+    eng.step()                       # all four prompts whole
+    eng.add_request("late", list(range(100, 130)), SamplingParams(max_tokens=2))
+    eng.step()
+    chunks = runner.calls[-1].chunks
+    assert [c.request.request_id for c in chunks] == ["r1", "r3", "r2", "r0", "late"]
+    assert [c.num_tokens for c in chunks] == [1, 1, 1, 1, 30]
+    starts = [c.start for c in chunks[:4]]
+    assert starts == sorted(starts, reverse=True) == [23, 17, 11, 5]
+    run(eng)
+
+
 def test_content_reuse_starts_the_portion_after_the_cached_pages():
     eng, runner, _ = make(budget=64)
     p = list(range(30))
