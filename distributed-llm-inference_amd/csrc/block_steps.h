@@ -7,12 +7,19 @@
 #define DLI_MAX_SHAPES 4   // distinct attention shapes (head size, heads, kv heads) in one model
 
 // What depends on the step's batch and an attention shape: the query tiles of the portions (for
-// this shape's tile height) and the key splits of the single-token rows.
+// this shape's tile height), which of them have their keys cut into two runs (tile_cut null: none;
+// see dli_attention_prefill_bf16) with the memory for that, and the key splits of the
+// single-token rows.
 struct DliStepShape {
   const int32_t* tile_entry;
   const int32_t* tile_q0;
   int32_t tiles;
   int32_t decode_splits;
+  const int32_t* tile_cut;
+  float* cut_buf;
+  uint32_t* cut_count;
+  int32_t cut_tiles;
+  int32_t pad0;
 };
 
 // One step: the batch's arrays on the device (as the step context holds them) and the scratch

@@ -142,6 +142,19 @@ class StepContext:
         q0, q1 = self.entry_rows(e)
         return int(self.kv_len_host[e]) - (q1 - q0) == 0
 
+    def upload(self, arrays: Sequence[np.ndarray]) -> list[torch.Tensor]:
+        """The host arrays as device tensors on the step's device (one copy for all of them)."""
+        return upload(arrays, self.device)
+
+    def step_lists(self, key: Hashable, make: Callable[[], Any]) -> Any:
+        """``make()``, made once per key and kept as long as the context: for lists that depend on
+        the step's host arrays alone (which entry brings how many tokens over how many keys),
+        such as the tile lists of the attention kernels."""
+        hit = self._tiles.get(key)
+        if hit is None:
+            hit = self._tiles[key] = make()
+        return hit
+
     def q_tiles(self, rows_per_tile: int, first_entry: int = 0, last_entry: Optional[int] = None,
                 arrange: Optional[Callable[[np.ndarray, np.ndarray], np.ndarray]] = None,
                 arranged_as: Hashable = None) -> tuple[torch.Tensor, torch.Tensor]:

@@ -28,7 +28,8 @@ _p, _i32, _i64, _f = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_f
 
 
 class StepShape(ctypes.Structure):
-    _fields_ = [("tile_entry", _p), ("tile_q0", _p), ("tiles", _i32), ("decode_splits", _i32)]
+    _fields_ = [("tile_entry", _p), ("tile_q0", _p), ("tiles", _i32), ("decode_splits", _i32), ("tile_cut", _p),
+                ("cut_buf", _p), ("cut_count", _p), ("cut_tiles", _i32), ("pad0", _i32)]
 
 
 class StepArgs(ctypes.Structure):
@@ -68,12 +69,13 @@ class NativeBlocks:
     def __init__(self, blocks: Sequence[dict], caches: Sequence[Any], device: torch.device) -> None:
         self.device = device
         self.array = (BlockArgs * len(blocks))()
-        self.shapes: list[tuple[int, int, int]] = []   # (head_dim, q_heads, kv_heads), by shape index
+        # (head_dim, q_heads, kv_heads, whether a window is set: such layers' tiles are never cut), by shape index
+        self.shapes: list[tuple[int, int, int, bool]] = []
         self.plan_owners: list[int] = []                 # per shape, the first mixer of that shape
         self.keep = []                                   # tensors whose addresses the array holds
         self.widths = dict(hidden=0, qkv=0, attn=0, gate_up=0, act=0)
         for a, f, cache in zip(self.array, blocks, caches):
-            shape = (f["head_dim"], f["q_heads"], f["kv_heads"])
+            shape = (f["head_dim"], f["q_heads"], f["kv_heads"], f["window"] > 0)
             if shape not in self.shapes:
                 self.shapes.append(shape)
                 self.plan_owners.append(f.get("plan_owner", 0))
@@ -87,7 +89,7 @@ class NativeBlocks:
                          "intermediate", "window"):
                 setattr(a, name, f[name])
             a.group, a.shape, a.kind = cache.group, self.shapes.index(shape), f["kind"]
-            d, qh, kvh = shape
+            d, qh, kvh, _ = shape
             w = self.widths
             w["hidden"] = max(w["hidden"], f["hidden"])
             w["qkv"] = max(w["qkv"], (qh + 2 * kvh) * d)
@@ -144,11 +146,14 @@ class NativeBlocks:
         nd = ctx.num_decode
         parts_o = parts_ml = 0
         keep = [scratch]
-        for i, (d, qh, kvh) in enumerate(self.shapes):
+        for i, (d, qh, kvh, windowed) in enumerate(self.shapes):
             sh = s.shapes[i]
             if ctx.num_entries > nd:
-                tile_entry, tile_q0 = prefill_tiles(ctx, d, qh, kvh, nd, self.device)
-                sh.tile_entry, sh.tile_q0, sh.tiles = tile_entry.data_ptr(), tile_q0.data_ptr(), tile_entry.shape[0]
+                t = prefill_tiles(ctx, d, qh, kvh, nd, self.device, window=1 if windowed else 0)
+                sh.tile_entry, sh.tile_q0, sh.tiles = t.entry.data_ptr(), t.q0.data_ptr(), t.tiles
+                if t.cut is not None:
+                    sh.tile_cut, sh.cut_tiles = t.cut.data_ptr(), t.cut_tiles
+                    sh.cut_buf, sh.cut_count = t.cut_buf.data_ptr(), t.cut_count.data_ptr()
             if nd > 0:
                 # mixers of one shape plan alike, so the first one's answer for a recorded step holds for all
                 splits = step_splits(ctx, nd, qh, kvh, self.device, ctx.decode_plans.get(self.plan_owners[i]))

@@ -75,3 +75,59 @@ def test_a_call_records_graphs_where_it_decodes_long_enough():
     assert graphs_pay([16, GRAPHS_PAY_FROM], 256)
     assert graphs_pay([256] * 600, 256)                        # three rounds of 256 steps
     assert not graphs_pay([256] * 256, 256) and graphs_pay([256] * 257, 256)
+
+
+def test_which_tiles_of_a_short_launch_have_their_keys_cut():
+    """One prompt of 2,048 tokens at the 1B sizes (a tile of 32 queries is 8 workgroups, 256 compute
+    units): the 32 tiles that walk more than half of the longest one's key tiles are cut, which
+    brings the launch to three workgroups a unit; from 3,072 tokens on nothing is cut; never a tile
+    too short for two runs, never more than the launch has room for."""
+    import numpy as np
+
+    from dli_amd.parts.attention_kernels import MIN_RUN_TILES, tiles_to_cut
+
+    key_tiles = np.arange(1, 65)
+    cut = tiles_to_cut(key_tiles, 8, 256)
+    assert cut.sum() == 32 and cut[32:].all() and not cut[:32].any()
+    assert not tiles_to_cut(np.arange(1, 97), 8, 256).any()
+    cut = tiles_to_cut(np.arange(1, 81), 8, 256)           # room for 16 more entries
+    assert cut.sum() == 16 and cut[64:].all()
+    cut = tiles_to_cut(np.arange(1, 21), 8, 256)           # 640 tokens: only tiles of 16 key tiles and more
+    assert cut.tolist() == [n >= 2 * MIN_RUN_TILES for n in range(1, 21)]
+    assert not tiles_to_cut(np.arange(1, 9), 8, 256).any() and not tiles_to_cut(np.zeros(0, np.int64), 8, 256).any()
+
+
+def test_the_tile_list_of_a_step_lists_every_tile_once_or_both_of_its_runs():
+    """Random steps: every tile of every portion is in the list, whole or as run 0 and run 1 with
+    the same place; places count the cut tiles from 0; the entries' shares of keys never grow
+    within a round of the list (every second round is turned round)."""
+    import random
+
+    import numpy as np
+
+    from dli_amd.parts.attention_kernels import list_tiles
+
+    rng = random.Random(3)
+    for trial in range(200):
+        n = rng.randrange(1, 6)
+        first = rng.randrange(0, n)
+        q_len = np.asarray([1] * first + [rng.randrange(2, 3000) for _ in range(n - first)], np.int64)
+        kv_len = q_len + np.asarray([rng.randrange(0, 500) for _ in range(n)], np.int64)
+        rows, per_tile, units = rng.choice([(32, 8), (128, 24), (64, 4), (128, 9)]) + (rng.choice([64, 256, 304]),)
+        may_cut = rng.random() < 0.8
+        ent, q0, code, n_cut = list_tiles(q_len, kv_len, first, rows, per_tile, units, may_cut)
+        want = {(e, t) for e in range(first, n) for t in range(0, int(q_len[e]), rows)}
+        if code is None:
+            assert n_cut == 0 and sorted(zip(ent.tolist(), q0.tolist())) == sorted(want)
+            continue
+        assert may_cut and n_cut > 0 and len(ent) == len(want) + n_cut
+        whole = [(e, t) for e, t, c in zip(ent.tolist(), q0.tolist(), code.tolist()) if c < 0]
+        runs = {}
+        for e, t, c in zip(ent.tolist(), q0.tolist(), code.tolist()):
+            if c >= 0:
+                assert (c >> 4) & 15 == 2
+                runs.setdefault((e, t), []).append((c & 15, c >> 8))
+        assert len(whole) == len(set(whole)) and set(whole) | set(runs) == want and not set(whole) & set(runs)
+        assert all(sorted(r) == [(0, r[0][1]), (1, r[0][1])] for r in runs.values())
+        assert sorted(r[0][1] for r in runs.values()) == list(range(n_cut))
+        assert len(ent) * per_tile <= 3 * units

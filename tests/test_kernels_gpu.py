@@ -340,32 +340,51 @@ def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window):
     assert err < tol(torch.bfloat16), err
 
 
-@pytest.mark.parametrize("qh,kvh,d", [(16, 16, 64), (8, 4, 32), (12, 4, 128), (16, 4, 64), (9, 3, 64)])
+@pytest.mark.parametrize("qh,kvh,d", [(16, 16, 64), (8, 4, 32), (12, 4, 128), (16, 4, 64), (9, 3, 64), (8, 2, 96)])
 def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, qh, kvh, d):
     """A launch in which compute units work on two tiles of different lengths at a time (and, with
-    many heads, in which the order of the workgroups differs from the grid's): one prompt whose
-    length puts the launch there, and a short one beside it; rows of both against a 32-bit softmax
-    over their keys."""
+    many heads, in which the order of the workgroups differs from the grid's), listed as the engine
+    lists it: one prompt whose length puts the launch there, on top of 24 cached keys, and a short
+    one beside it. Once with every tile whole and once with the keys of the longest tiles cut
+    into two runs that two workgroups share (twice on the same counters: each launch leaves them
+    zero): the two agree, and rows of both requests agree with a 32-bit softmax over their keys."""
+    import numpy as np
+    from dli_amd.parts.attention_kernels import list_tiles
+
     units = ops.compute_units(torch.device("cuda"))
     rows = ops.attention_prefill_tile_rows(d, qh, kvh)
     per_tile = qh // (4 * 32 // rows)             # workgroups that a tile of the list becomes
     tiles = -(-units * 3 // (2 * per_tile))        # 1.5 workgroups a unit
     bs = 16
-    lens = [(tiles * rows - 40 - rows, tiles * rows - 40 - rows), (40, 77)]
+    long_q = tiles * rows - 40 - rows
+    lens = [(long_q, long_q + 24), (40, 77)]
     q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=qh + d)
-    te, tq = _tiles(q_start, rows)
-    assert len(te) == tiles
-    order = sorted(range(tiles), key=lambda i: -(kv_len[te[i]] - (q_start[te[i] + 1] - q_start[te[i]]) + tq[i]))
-    te, tq = [te[i] for i in order], [tq[i] for i in order]   # longest first, as the engine lists them
-    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    dev = lambda x: torch.tensor(np.asarray(x), dtype=torch.int32, device="cuda")
     scale = 1.0 / math.sqrt(d)
-    out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
-    ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables), dev(te),
-                          dev(tq), qh, scale, 0)
-    assert torch.isfinite(out.float()).all() and (out.float().abs() < 8).all()   # every row was written
+    q_len = np.asarray([n for n, _ in lens], np.int64)
+    outs = []
+    for may_cut in (False, True):
+        te, tq, code, n_cut = list_tiles(q_len, np.asarray(kv_len, np.int64), 0, rows, per_tile, units, may_cut)
+        assert (code is not None) == may_cut and len(te) == tiles + n_cut
+        extra = {}
+        if may_cut:
+            assert n_cut > 0 and sorted(c & 15 for c in code if c >= 0) == [0] * n_cut + [1] * n_cut
+            extra = dict(tile_cut=dev(code), cut_tiles=n_cut,
+                         cut_buf=torch.full((n_cut * ops.attention_prefill_cut_floats(d, qh, kvh),), float("nan"), device="cuda"),
+                         cut_count=torch.zeros(n_cut * qh, dtype=torch.int32, device="cuda"))
+        for again in range(2 if may_cut else 1):
+            out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
+            ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables), dev(te),
+                                  dev(tq), qh, scale, 0, **extra)
+            assert torch.isfinite(out.float()).all() and (out.float().abs() < 8).all()   # every row was written
+            outs.append(out)
+        if may_cut:
+            assert int(extra["cut_count"].abs().sum()) == 0
+    assert torch.equal(outs[1], outs[2])
+    assert (outs[0].float() - outs[1].float()).abs().max().item() < tol(torch.bfloat16)
     # rows of the long request and the short one's last, from their keys gathered out of the pages
     kd, vd = kp.cuda().float(), vp.cuda().float()
-    for e, row in ((0, 0), (0, 31), (0, 32), (0, 127), (0, 128), (0, lens[0][0] // 2 + 3), (0, lens[0][0] - 1), (1, 39)):
+    for e, row in ((0, 0), (0, 31), (0, 32), (0, 127), (0, 128), (0, long_q // 2 + 3), (0, long_q - 1), (1, 39)):
         n_keys = kv_len[e] - (q_start[e + 1] - q_start[e]) + row + 1
         pages = torch.tensor(tables[e][:-(-n_keys // bs)], device="cuda")
         keys = kd[pages].permute(1, 0, 2, 3).reshape(kvh, -1, d)[:, :n_keys]         # [kvh, keys, d]
@@ -373,7 +392,8 @@ def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, 
         qrow = q[q_start[e] + row].cuda().float().view(kvh, qh // kvh, d)
         p = torch.softmax(torch.einsum("hgd,hkd->hgk", qrow, keys) * scale, dim=-1)
         ref = torch.einsum("hgk,hdk->hgd", p, vals).reshape(-1)
-        assert (out[q_start[e] + row].float() - ref).abs().max().item() < tol(torch.bfloat16), (e, row)
+        for out in outs[:2]:
+            assert (out[q_start[e] + row].float() - ref).abs().max().item() < tol(torch.bfloat16), (e, row)
 
 
 def test_attention_finds_one_far_key_among_hundreds(ops):

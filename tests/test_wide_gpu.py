@@ -288,9 +288,10 @@ def test_llama_3_2_1b_in_portions_and_in_mixed_batches(dtype):
 
 def test_a_prompt_of_1700_tokens_whole_and_on_top_of_cached_keys(monkeypatch):
     """1,700 tokens at the 1B widths are 54 query tiles of eight kv heads each: between one and two
-    workgroups a compute unit, so that units work on two tiles of different lengths at a time.
-    The whole model through the prefill attention kernel that the launch's size selects (not asked
-    for), whole and as a portion on top of cached keys, against the plain implementation."""
+    workgroups a compute unit, so that units work on two tiles of different lengths at a time and
+    the longest tiles have their keys cut into two runs that two workgroups share. The whole model
+    through the prefill attention as the step lists its tiles, whole and as a portion on top of
+    cached keys, against the plain implementation."""
     from dli_amd.kernels import ops
     from dli_amd.trace import TraceSession
 
@@ -301,7 +302,7 @@ def test_a_prompt_of_1700_tokens_whole_and_on_top_of_cached_keys(monkeypatch):
     real = ops.attention_prefill
 
     def counted(*a, **k):
-        seen.append(a[7].shape[0])  # tiles in the list
+        seen.append((a[7].shape[0], a[13]))  # entries of the tile list, and how many tiles are listed twice, with half their keys each
         return real(*a, **k)
 
     monkeypatch.setattr(ops, "attention_prefill", counted)
@@ -311,7 +312,7 @@ def test_a_prompt_of_1700_tokens_whole_and_on_top_of_cached_keys(monkeypatch):
     want = [0, 17, 511, 512, 1023, 1699]
     got = s.step([{"id": "w", "tokens": toks, "want": want}], end=["w"])
     check(got, ref[want], "bfloat16", "1,700 tokens whole")
-    assert seen and all(tiles == 54 for tiles in seen)
+    assert seen and all(entries == 54 + cut and cut > 0 for entries, cut in seen)
     got = s.step([{"id": "p", "tokens": toks[:60], "want": [59]}])
     check(got, ref[59:60], "bfloat16", "first portion")
     got = s.step([{"id": "p", "tokens": toks[60:], "want": [w - 60 for w in want[2:]]}], end=["p"])
