@@ -568,6 +568,8 @@ __device__ __forceinline__ void tile_barrier() {
 // (Held to the registers that let three waves share a SIMD for heads of up to 64 and two for
 // larger ones: 126 instead of 176 and 196 instead of 276, nothing spilled, no copies between
 // the two register files.)
+#define PREFILL_MAX_CUTS 8  // the most runs that a tile's keys are cut into
+
 template <int DCH>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DCH <= 4 ? 3 : 2)))
 void attention_prefill_shared_kernel(
@@ -576,7 +578,8 @@ void attention_prefill_shared_kernel(
     const int* __restrict__ q_start, const int* __restrict__ kv_len,
     const int* __restrict__ block_tables, int table_stride, const int* __restrict__ tile_entry,
     const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
-    int window, int heads_per_wg, const int* __restrict__ tile_cut, float* cut_buf, unsigned* cut_count) {
+    int window, int heads_per_wg, const int* __restrict__ tile_cut, int cut_room, float* cut_buf,
+    unsigned* cut_count) {
   constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of the first product
   constexpr int R = D / 8;                      // 16-byte chunks in a key's row of K
   constexpr int NT = 256;                       // threads
@@ -609,10 +612,10 @@ void attention_prefill_shared_kernel(
   const int q_len = q_start[e + 1] - tok0;
   const int tile_rows = (4 / heads_per_wg) * 32;
   const int q0_first = tile_q0[bx];
-  // A tile whose keys are cut into runs (short launches: the longest workgroups are then half or
-  // a quarter as long): this workgroup takes run `cut` of `cuts`, and the workgroup that finishes
-  // second of a tile's two runs adds them up. code: cut | cuts << 4 | place of the tile among the
-  // cut ones << 8; cuts is 1 or 2.
+  // A tile whose keys are cut into runs (short launches: the longest workgroups are then a
+  // fraction as long): this workgroup takes run `cut` of `cuts`, and the workgroup that finishes
+  // last of a tile's runs adds them up. code: cut | cuts << 4 | place of the tile among the cut
+  // ones << 8; cuts is at most PREFILL_MAX_CUTS, and the buffer has room for cut_room runs a tile.
   const int cut_code = tile_cut != nullptr ? tile_cut[bx] : -1;
   const int cut = cut_code >= 0 ? cut_code & 15 : 0, cuts = cut_code >= 0 ? (cut_code >> 4) & 15 : 1;
   const int cut_place = cut_code >= 0 ? cut_code >> 8 : 0;
@@ -917,17 +920,17 @@ void attention_prefill_shared_kernel(
   float l_sum[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) l_sum[j] = column_sum(st[j].l);  // every lane takes part
-  if (cuts == 2) {
+  if (cuts > 1) {
     // This run's state goes to memory at the device's scope: per wave and column tile DCH + 1
     // quads a lane (the output's, then the sum and the exponent's reference point). Then the
-    // workgroup counts itself in; the one that counts second reads the other run's state, adds the
-    // two in the order of the runs (its own from its registers: the same values), and leaves the
-    // counter zero for the next launch.
+    // workgroup counts itself in; the one that counts last reads the other runs' states, adds all
+    // of them up in the order of the runs (its own from its registers: the same values), and
+    // leaves the counter zero for the next launch.
     constexpr int QUADS = DCH + 1;
     __shared__ unsigned arrived_before;
     const __amdgpu_buffer_rsrc_t cb = device_scope_buffer(cut_buf);
     const unsigned wg_quads = 8u * QUADS * 64u;   // 4 waves x 2 column tiles
-    const unsigned tile_at = ((unsigned)cut_place * gridDim.y + (unsigned)by) * 2u;
+    const unsigned tile_at = ((unsigned)cut_place * gridDim.y + (unsigned)by) * (unsigned)cut_room;
     auto at = [&](int run, int j, int quad) {
       return ((tile_at + (unsigned)run) * wg_quads + ((unsigned)(wave * 2 + j) * QUADS + (unsigned)quad) * 64u + (unsigned)lane) * 16u;
     };
@@ -943,37 +946,55 @@ void attention_prefill_shared_kernel(
     unsigned* counter = cut_count + (size_t)cut_place * gridDim.y + by;
     if (threadIdx.x == 0) arrived_before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (arrived_before != 1u) return;
+    if (arrived_before != (unsigned)cuts - 1) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    float4v o_other[2][DCH], stat[2];   // all loads leave before the first is used
+    // the runs' sums and reference points first (all loads leave before the first is used) ...
+    merge_float2 stat[2][PREFILL_MAX_CUTS];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int c = 0; c < DCH; ++c) o_other[j][c] = device_load4(cb, at(1 - cut, j, c));
-      stat[j] = device_load4(cb, at(1 - cut, j, DCH));
-    }
+      for (int run = 0; run < PREFILL_MAX_CUTS; ++run)
+        stat[j][run] = run < cuts ? device_load2(cb, at(run, j, DCH)) : merge_float2{0.f, 0.f};
+    float wgt[2][PREFILL_MAX_CUTS];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       // a run that saw no key of a query (sum 0) has no say in the reference point
-      const float l_o = stat[j][0], m_o = stat[j][1];
-      const float m_all = max2(l_sum[j] > 0.f ? m_ref[j] : -INFINITY, l_o > 0.f ? m_o : -INFINITY);
+      float m_all = -INFINITY;
+#pragma unroll
+      for (int run = 0; run < PREFILL_MAX_CUTS; ++run) m_all = max2(m_all, stat[j][run][0] > 0.f ? stat[j][run][1] : -INFINITY);
       const float m_safe = m_all == -INFINITY ? 0.f : m_all;
-      const float w_own = l_sum[j] > 0.f ? fast_exp2(m_ref[j] - m_safe) : 0.f;
-      const float w_other = l_o > 0.f ? fast_exp2(m_o - m_safe) : 0.f;
-      // Products and sums in the order of the runs and each rounded by itself, so that the result
-      // does not depend on which of the two workgroups does the adding (left to itself the
-      // compiler fuses one product into the sum, the merging workgroup's own or the other's).
-      const float w0 = cut == 0 ? w_own : w_other, w1 = cut == 0 ? w_other : w_own;
-      const float l0 = cut == 0 ? l_sum[j] : l_o, l1 = cut == 0 ? l_o : l_sum[j];
-      l_sum[j] = __fadd_rn(__fmul_rn(l0, w0), __fmul_rn(l1, w1));
+      float l_all = 0.f;
 #pragma unroll
-      for (int c = 0; c < DCH; ++c)
+      for (int run = 0; run < PREFILL_MAX_CUTS; ++run) {
+        wgt[j][run] = stat[j][run][0] > 0.f ? fast_exp2(stat[j][run][1] - m_safe) : 0.f;
+        l_all = __fadd_rn(l_all, __fmul_rn(stat[j][run][0], wgt[j][run]));
+      }
+      l_sum[j] = l_all;
+    }
+    // ... then their outputs, run by run. Products and sums in the order of the runs and each
+    // rounded by itself, so that the result does not depend on which of the workgroups does the
+    // adding (left to itself the compiler fuses a product into the sum, and which one depends on
+    // whose values sit in registers).
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float a = cut == 0 ? st[j].o[c][i] : o_other[j][c][i], b = cut == 0 ? o_other[j][c][i] : st[j].o[c][i];
-          st[j].o[c][i] = __fadd_rn(__fmul_rn(a, w0), __fmul_rn(b, w1));
-        }
+    for (int j = 0; j < 2; ++j) {
+      float4v acc[DCH];
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) acc[c] = float4v{0.f, 0.f, 0.f, 0.f};
+      for (int run = 0; run < cuts; ++run) {
+        float4v o_run[DCH];
+#pragma unroll
+        for (int c = 0; c < DCH; ++c) o_run[c] = device_load4(cb, at(run, j, c));
+        float w = 0.f;
+#pragma unroll
+        for (int u = 0; u < PREFILL_MAX_CUTS; ++u) w = u == run ? wgt[j][u] : w;
+#pragma unroll
+        for (int c = 0; c < DCH; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[c][i] = __fadd_rn(acc[c][i], __fmul_rn(o_run[c][i], w));
+      }
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) st[j].o[c] = acc[c];
     }
   }
 #pragma unroll
@@ -1157,22 +1178,26 @@ extern "C" int dli_attention_decode_bf16_static(const void* q, int64_t q_stride,
                                    scale, window, splits, stream);
 }
 
-// 32-bit values that the kernel wants per tile whose keys are cut into two runs (the states of both
-// runs of every workgroup of the tile), or 0 where this shape's kernel cuts no tiles.
+// 32-bit values that the kernel wants per run of a tile whose keys are cut into runs (the state
+// of every workgroup of the tile), or 0 where this shape's kernel cuts no tiles.
 extern "C" int dli_attention_prefill_cut_floats(int head_dim, int q_heads, int kv_heads) {
   if (kv_heads <= 0 || q_heads % kv_heads != 0 || q_heads > 65535 || head_dim > 128) return DLI_ERR_ARGUMENT;
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (hw == 0) return 0;
-  return (q_heads / hw) * 2 * 8 * (head_dim / 16 + 1) * 64 * 4;
+  return (q_heads / hw) * 8 * (head_dim / 16 + 1) * 64 * 4;
 }
 
-// tile_cut (or null: every tile whole): per entry of the tile list -1, or run | 2 << 4 | place << 8
-// for run 0 or 1 of a tile whose keys two workgroups share, `place` numbering the cut tiles from 0
-// to cut_tiles - 1; both runs must be listed. Only without a window and for head sizes that are
-// multiples of 32. cut_buf: cut_tiles * dli_attention_prefill_cut_floats() values; cut_count: one
-// counter per cut tile and workgroup of a tile (cut_tiles * q_heads / (heads a workgroup takes);
-// q_heads is enough), zero before the first launch; every launch leaves them zero, and launches
-// that share them or cut_buf must not overlap.
+// The most runs that a tile's keys can be cut into.
+extern "C" int dli_attention_prefill_max_cuts() { return PREFILL_MAX_CUTS; }
+
+// tile_cut (or null: every tile whole): per entry of the tile list -1, or run | runs << 4 |
+// place << 8 for one of the 2 to dli_attention_prefill_max_cuts() runs of a tile whose keys that
+// many workgroups share, `place` numbering the cut tiles from 0 to cut_tiles - 1; all runs of a
+// tile must be listed. Only without a window and for head sizes that are multiples of 32.
+// cut_room: the most runs of any tile; cut_buf: cut_tiles * cut_room *
+// dli_attention_prefill_cut_floats() values; cut_count: one counter per cut tile and workgroup of
+// a tile (cut_tiles * q_heads is enough), zero before the first launch; every launch leaves them
+// zero, and launches that share them or cut_buf must not overlap.
 extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pages,
                                           const void* v_pages, void* out, int64_t out_stride,
                                           const int* q_start, const int* kv_len,
@@ -1180,15 +1205,16 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
                                           const int* tile_entry, const int* tile_q0, int tiles,
                                           int q_heads, int kv_heads, int head_dim, int page_size,
                                           float scale, int window, const int* tile_cut, int cut_tiles,
-                                          float* cut_buf, unsigned* cut_count, hipStream_t stream) {
+                                          int cut_room, float* cut_buf, unsigned* cut_count, hipStream_t stream) {
   if (tiles <= 0) return DLI_OK;
   if (!dli_attention_mfma_supports(head_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || q_heads > 65535 || q_stride % 4 != 0 || out_stride % 4 != 0)
     return DLI_ERR_ARGUMENT;
   const int hw = shared_heads_per_wg(head_dim, q_heads / kv_heads);
   if (tile_cut != nullptr &&
-      (hw == 0 || window > 0 || cut_tiles <= 0 || cut_tiles >= (1 << 23) || cut_buf == nullptr || cut_count == nullptr ||
-       (int64_t)cut_tiles * dli_attention_prefill_cut_floats(head_dim, q_heads, kv_heads) * 4 >= ((int64_t)1 << 32)))
+      (hw == 0 || window > 0 || cut_tiles <= 0 || cut_tiles >= (1 << 23) || cut_room < 2 || cut_room > PREFILL_MAX_CUTS ||
+       cut_buf == nullptr || cut_count == nullptr ||
+       (int64_t)cut_tiles * cut_room * dli_attention_prefill_cut_floats(head_dim, q_heads, kv_heads) * 4 >= ((int64_t)1 << 32)))
     return DLI_ERR_ARGUMENT;
   if (hw > 0) {
     if ((int64_t)kv_heads * page_size * head_dim >= ((int64_t)1 << 31)) return DLI_ERR_ARGUMENT;  // the kernel's 32 bits
@@ -1198,7 +1224,7 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
     attention_prefill_shared_kernel<N><<<sgrid, 256, 0, stream>>>(                                \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, \
         out_stride, q_start, kv_len, block_tables, table_stride, tile_entry, tile_q0, q_heads,    \
-        kv_heads, page_size, scale * LOG2E, window, hw, tile_cut, cut_buf, cut_count);            \
+        kv_heads, page_size, scale * LOG2E, window, hw, tile_cut, cut_room, cut_buf, cut_count);  \
     break;
     switch (head_dim / 16) {
       SHARED_CASE(2) SHARED_CASE(4) SHARED_CASE(6) SHARED_CASE(8)

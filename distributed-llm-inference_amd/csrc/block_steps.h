@@ -19,7 +19,7 @@ struct DliStepShape {
   float* cut_buf;
   uint32_t* cut_count;
   int32_t cut_tiles;
-  int32_t pad0;
+  int32_t cut_room;   // the most runs of any cut tile
 };
 
 // One step: the batch's arrays on the device (as the step context holds them) and the scratch

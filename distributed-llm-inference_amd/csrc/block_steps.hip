@@ -37,7 +37,7 @@ int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const void* k_pa
                                int64_t out_stride, const int* q_start, const int* kv_len, const int* block_tables,
                                int table_stride, const int* tile_entry, const int* tile_q0, int tiles, int q_heads,
                                int kv_heads, int head_dim, int page_size, float scale, int window, const int* tile_cut,
-                               int cut_tiles, float* cut_buf, unsigned* cut_count, hipStream_t stream);
+                               int cut_tiles, int cut_room, float* cut_buf, unsigned* cut_count, hipStream_t stream);
 }
 
 namespace {
@@ -55,7 +55,8 @@ bool block_is_sane(const DliBlockArgs& b, const DliStepArgs& s) {
   if (s.slots[b.group] == nullptr || s.block_tables[b.group] == nullptr || s.table_stride[b.group] <= 0) return false;
   const DliStepShape& sh = s.shapes[b.shape];
   if (s.num_entries > s.num_decode && (sh.tiles <= 0 || sh.tile_entry == nullptr || sh.tile_q0 == nullptr)) return false;
-  if (sh.tile_cut != nullptr && (b.window > 0 || sh.cut_tiles <= 0 || sh.cut_buf == nullptr || sh.cut_count == nullptr)) return false;
+  if (sh.tile_cut != nullptr && (b.window > 0 || sh.cut_tiles <= 0 || sh.cut_room < 2 || sh.cut_buf == nullptr || sh.cut_count == nullptr))
+    return false;
   if (s.num_decode > 0 && (sh.decode_splits < 1 || (sh.decode_splits > 1 && (s.part_o == nullptr || s.part_ml == nullptr))))
     return false;
   return dli_attention_mfma_supports(b.head_dim, s.page_size) != 0;
@@ -113,7 +114,7 @@ extern "C" int dli_prenorm_blocks_bf16(void* x, const DliBlockArgs* blocks, int 
       STEP(dli_attention_prefill_bf16(s.qkv, qkv_w, b.k_pages, b.v_pages, s.attn, q_w, s.q_start, s.kv_len,
                                       s.block_tables[b.group], s.table_stride[b.group], sh.tile_entry, sh.tile_q0,
                                       sh.tiles, b.q_heads, b.kv_heads, b.head_dim, s.page_size, b.scale, b.window,
-                                      sh.tile_cut, sh.cut_tiles, sh.cut_buf, sh.cut_count, stream));
+                                      sh.tile_cut, sh.cut_tiles, sh.cut_room, sh.cut_buf, sh.cut_count, stream));
     STEP(dli_gemm_bf16(s.attn, q_w, b.w_o, q_w, b.b_o, s.mixed, h, s.rows, h, q_w, s.gemm_workspace,
                        s.gemm_workspace_bytes, s.device, stream));
     STEP(dli_rms_norm(x, s.mixed, b.norm2_w, x, s.normed, s.rows, b.hidden, b.eps2, 1, stream));

@@ -155,17 +155,13 @@ class StepContext:
             hit = self._tiles[key] = make()
         return hit
 
-    def q_tiles(self, rows_per_tile: int, first_entry: int = 0, last_entry: Optional[int] = None,
-                arrange: Optional[Callable[[np.ndarray, np.ndarray], np.ndarray]] = None,
-                arranged_as: Hashable = None) -> tuple[torch.Tensor, torch.Tensor]:
-        """Query tiles ``(entry, first query of the tile)`` of entries ``[first, last)``, as two
-        int32 device vectors; built once per step and tile height. ``arrange(entries, firsts)``
-        may return the order in which a kernel wants the tiles listed (a permutation; the default
-        is by entry and then by query); ``arranged_as`` names that order for the memo."""
+    def q_tiles(self, rows_per_tile: int, first_entry: int = 0,
+                last_entry: Optional[int] = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """Query tiles ``(entry, first query of the tile)`` of entries ``[first, last)``, by entry
+        and then by query, as two int32 device vectors; built once per step and tile height."""
         last = self.num_entries if last_entry is None else last_entry
-        key = (rows_per_tile, first_entry, last, arranged_as if arrange is not None else None)
-        hit = self._tiles.get(key)
-        if hit is None:
+
+        def make() -> tuple[torch.Tensor, torch.Tensor]:
             ent: list[int] = []
             q0s: list[int] = []
             for e in range(first_entry, last):
@@ -173,12 +169,6 @@ class StepContext:
                 for q0 in range(0, length, rows_per_tile):
                     ent.append(e)
                     q0s.append(q0)
-            ent_a, q0_a = np.asarray(ent, np.int32), np.asarray(q0s, np.int32)
-            if arrange is not None and ent_a.size > 1:
-                order = np.asarray(arrange(ent_a, q0_a))
-                if sorted(order.tolist()) != list(range(ent_a.size)):
-                    raise ValueError("arrange() must return a permutation of the tiles")
-                ent_a, q0_a = ent_a[order], q0_a[order]
-            hit = tuple(upload([ent_a, q0_a], self.device))
-            self._tiles[key] = hit
-        return hit
+            return tuple(self.upload([np.asarray(ent, np.int32), np.asarray(q0s, np.int32)]))
+
+        return self.step_lists(("query tiles", rows_per_tile, first_entry, last), make)

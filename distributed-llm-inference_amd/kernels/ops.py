@@ -91,8 +91,9 @@ _SIGNATURES = {
     "dli_rope_angles": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "dli_attention_prefill_bf16": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr,
-                                   _c_int, _c_ptr, _c_ptr, _c_ptr],
+                                   _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "dli_attention_prefill_cut_floats": [_c_int, _c_int, _c_int],
+    "dli_attention_prefill_max_cuts": [],
     "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                               _c_int, _c_int, _c_ptr],
@@ -1009,11 +1010,16 @@ def attention_prefill_tile_rows(head_dim: int, q_heads: int, kv_heads: int) -> i
 
 
 def attention_prefill_cut_floats(head_dim: int, q_heads: int, kv_heads: int) -> int:
-    """float32 values that :func:`attention_prefill` wants in ``cut_buf`` per tile whose keys are
-    cut into two runs; 0 where this shape's kernel cuts no tiles."""
+    """float32 values that :func:`attention_prefill` wants in ``cut_buf`` per run of a tile whose
+    keys are cut into runs; 0 where this shape's kernel cuts no tiles."""
     n = int(library().dli_attention_prefill_cut_floats(head_dim, q_heads, kv_heads))
     _require(n >= 0, "query heads are not a multiple of kv heads")
     return n
+
+
+def attention_prefill_max_cuts() -> int:
+    """The most runs that :func:`attention_prefill` lets a tile's keys be cut into."""
+    return int(library().dli_attention_prefill_max_cuts())
 
 
 def _check_paged(q, k_pages, v_pages, out, q_heads):
@@ -1128,7 +1134,7 @@ def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, dtype: torch.dt
 def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
                       tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float,
-                      window: int = 0, tile_cut: Optional[torch.Tensor] = None, cut_tiles: int = 0,
+                      window: int = 0, tile_cut: Optional[torch.Tensor] = None, cut_tiles: int = 0, cut_room: int = 0,
                       cut_buf: Optional[torch.Tensor] = None, cut_count: Optional[torch.Tensor] = None) -> None:
     """Matrix-core attention for portions; operands as :func:`attention_generic`, tiles of
     :func:`attention_prefill_tile_rows` queries (the tile list must be built with that height, in
@@ -1136,12 +1142,13 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
     the tiles with the most keys belong first).
 
     ``tile_cut`` (int32, one per list entry; only without a window and where
-    :func:`attention_prefill_cut_floats` is not 0): -1 for a whole tile, or ``run | 2 << 4 |
-    place << 8`` for run 0 or 1 of a tile that is listed twice and whose keys the two workgroups
-    share, ``place`` numbering the ``cut_tiles`` cut tiles from 0. ``cut_buf``: float32,
-    ``cut_tiles * attention_prefill_cut_floats(...)`` values; ``cut_count``: int32, ``cut_tiles *
-    q_heads`` counters, zero before the first launch (every launch leaves them zero; launches that
-    share them must not overlap)."""
+    :func:`attention_prefill_cut_floats` is not 0): -1 for a whole tile, or ``run | runs << 4 |
+    place << 8`` for one of the 2 to :func:`attention_prefill_max_cuts` runs of a tile that is
+    listed once per run and whose keys that many workgroups share, ``place`` numbering the
+    ``cut_tiles`` cut tiles from 0. ``cut_room``: the most runs of any tile; ``cut_buf``: float32,
+    ``cut_tiles * cut_room * attention_prefill_cut_floats(...)`` values; ``cut_count``: int32,
+    ``cut_tiles * q_heads`` counters, zero before the first launch (every launch leaves them zero;
+    launches that share them must not overlap)."""
     kv_heads, page_size, head_dim = _check_paged(q, k_pages, v_pages, out, q_heads)
     for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
         _dense(t, name, torch.int32, 1)
@@ -1156,15 +1163,16 @@ def attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Ten
         per = attention_prefill_cut_floats(head_dim, q_heads, kv_heads)
         _require(per > 0 and window == 0, "this shape's kernel cuts no tiles, or a window is set")
         _require(cut_buf is not None and cut_count is not None and cut_tiles > 0, "cut tiles need their buffers")
+        _require(2 <= cut_room <= attention_prefill_max_cuts(), "cut_room outside what the kernel takes")
         _dense(cut_buf, "cut_buf", torch.float32, 1)
         _dense(cut_count, "cut_count", torch.int32, 1)
-        _require(cut_buf.shape[0] >= cut_tiles * per and cut_count.shape[0] >= cut_tiles * q_heads,
+        _require(cut_buf.shape[0] >= cut_tiles * cut_room * per and cut_count.shape[0] >= cut_tiles * q_heads,
                  "cut_buf or cut_count too small for the cut tiles")
     _check(library().dli_attention_prefill_bf16(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tile_entry.shape[0], q_heads,
-        kv_heads, head_dim, page_size, float(scale), int(window), _ptr(tile_cut), int(cut_tiles), _ptr(cut_buf),
-        _ptr(cut_count), _stream()), "attention_prefill")
+        kv_heads, head_dim, page_size, float(scale), int(window), _ptr(tile_cut), int(cut_tiles), int(cut_room),
+        _ptr(cut_buf), _ptr(cut_count), _stream()), "attention_prefill")
 
 # ----------------------------------------------------------------------------- sampling
 

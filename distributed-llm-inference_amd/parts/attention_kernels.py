@@ -46,28 +46,56 @@ def planned_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int 
 
 
 # A launch of fewer workgroups than this per compute unit is as long as its longest workgroup, and
-# cutting the keys of its longest tiles into two runs, each a workgroup, shortens that (one prompt
-# of 2,048 tokens at the 1B sizes: 43 -> 32 us a layer before the runs are added up); with more, the
-# workgroups queue anyway and the cut only costs its merge. A run is not shorter than MIN_RUN_TILES
-# tiles of 32 keys.
+# cutting the keys of its longest tiles into runs, each a workgroup, shortens that (one prompt of
+# 2,048 tokens at the 1B sizes: 43 -> 33 us a layer); with more, the workgroups queue anyway and
+# the cut only costs its merge (3,072 tokens: 62 -> 69 us with room for four a unit). A run is not
+# shorter than MIN_RUN_TILES tiles of 32 keys, and a tile has at most MAX_RUNS runs (the kernel's
+# limit is asked at the first use).
 CUT_BELOW_WORKGROUPS_PER_UNIT = 3
 MIN_RUN_TILES = 8
+MAX_RUNS = 8
+LONE_TILE_COST = 1.5   # a tile of a workgroup alone on its SIMDs, in tiles of a busy compute unit
 
 
-def tiles_to_cut(key_tiles: np.ndarray, workgroups_per_tile: int, units: int) -> np.ndarray:
-    """Which tiles of a launch have their keys cut into two runs (a mask over ``key_tiles``, the
-    number of 32-key tiles that each query tile walks): the longest ones, as many as keep the
-    launch under three workgroups a compute unit, and only those longer than half the longest
-    (cutting a shorter one would not shorten the longest workgroup) and long enough for two runs."""
-    cut = np.zeros(key_tiles.size, bool)
+def runs_of_tiles(key_tiles: np.ndarray, workgroups_per_tile: int, units: int, most: int = MAX_RUNS) -> np.ndarray:
+    """Into how many runs each tile of a launch has its keys cut (1: whole; ``key_tiles``: the
+    number of 32-key tiles that each query tile walks). While the launch stays under three
+    workgroups a compute unit, and the longest workgroup is still what the launch waits for (it
+    takes longer than the units' work in all), the tile with the longest run gets one more, as long
+    as its runs stay long enough; nothing is cut where that does not make the longest workgroup at
+    least 15% shorter (tiles of much the same length and no room for all of them: a large portion on top of
+    a long context)."""
+    import heapq
+
+    runs = np.ones(key_tiles.size, np.int64)
     spare = CUT_BELOW_WORKGROUPS_PER_UNIT * units // max(1, workgroups_per_tile) - key_tiles.size
     if spare <= 0 or key_tiles.size == 0:
-        return cut
+        return runs
+    share = lambda i: -(-int(key_tiles[i]) // int(runs[i]))   # the tile's longest run
+    heap = [(-share(i), i) for i in range(key_tiles.size)]
+    heapq.heapify(heap)
+    # What a compute unit has to do in all, in tiles of 32 keys of one workgroup. Under a causal
+    # mask from the prompt's start, the short tiles' workgroups leave early and the longest runs end
+    # alone on their SIMDs, where a tile takes about one and a half times what a full unit needs
+    # per tile: cutting stops when the longest run is no longer what the launch waits for. Tiles of
+    # much the same length (a portion on top of a long context) all live to the end, and more runs
+    # pay until the units are full (512 tokens on 8,192 keys: 155 us whole, 66 with four runs
+    # a tile, 57 with six; one prompt of 2,048 tokens: 31.6 us with 21 tiles cut, 33.0 with 32).
+    per_unit = float(key_tiles.sum()) * workgroups_per_tile / units
+    lone_cost = LONE_TILE_COST if float(key_tiles.mean()) < 0.75 * float(key_tiles.max()) else 2 * LONE_TILE_COST
+    while spare > 0:
+        longest_run, i = heapq.heappop(heap)
+        if -longest_run * lone_cost <= per_unit:
+            break   # the launch is as long as its work by now, not as its longest workgroup
+        if runs[i] >= most or int(key_tiles[i]) // (int(runs[i]) + 1) < MIN_RUN_TILES:
+            break   # the longest workgroup cannot get shorter
+        runs[i] += 1
+        spare -= 1
+        heapq.heappush(heap, (-share(i), i))
     longest = int(key_tiles.max())
-    wanted = np.flatnonzero((key_tiles > -(-longest // 2)) & (key_tiles >= 2 * MIN_RUN_TILES))
-    wanted = wanted[np.argsort(-key_tiles[wanted], kind="stable")][:spare]
-    cut[wanted] = True
-    return cut
+    if max(share(i) for i in range(key_tiles.size)) * 20 > longest * 17:
+        runs[:] = 1
+    return runs
 
 
 def round_about(order: np.ndarray, per_round: int) -> np.ndarray:
@@ -83,8 +111,9 @@ class PrefillTiles:
     needs for the tiles whose keys are cut (``cut`` None: none are)."""
 
     def __init__(self, entry: torch.Tensor, q0: torch.Tensor, cut: Optional[torch.Tensor] = None, cut_tiles: int = 0,
-                 cut_buf: Optional[torch.Tensor] = None, cut_count: Optional[torch.Tensor] = None) -> None:
-        self.entry, self.q0, self.cut, self.cut_tiles = entry, q0, cut, cut_tiles
+                 cut_room: int = 0, cut_buf: Optional[torch.Tensor] = None,
+                 cut_count: Optional[torch.Tensor] = None) -> None:
+        self.entry, self.q0, self.cut, self.cut_tiles, self.cut_room = entry, q0, cut, cut_tiles, cut_room
         self.cut_buf, self.cut_count = cut_buf, cut_count
 
     @property
@@ -93,17 +122,17 @@ class PrefillTiles:
 
 
 def list_tiles(q_len: np.ndarray, kv_len: np.ndarray, first_entry: int, rows: int, workgroups_per_tile: int,
-               units: int, may_cut: bool) -> tuple[np.ndarray, np.ndarray, Optional[np.ndarray], int]:
+               units: int, may_cut: bool) -> tuple[np.ndarray, np.ndarray, Optional[np.ndarray], int, int]:
     """The tiles of entries ``first_entry..`` (``q_len`` new tokens over ``kv_len`` keys each) in the
     order in which the prefill kernel wants them: ``(entry, first query, cut code or None, number of
-    cut tiles)``. Those that see the most keys come first: workgroups start in the order of the list,
+    cut tiles, most runs of a tile)``. Those that see the most keys come first: workgroups start in the order of the list,
     and under a causal mask a tile's work grows with its place in the request; listed by place, the
     longest workgroups start last and the launch ends with a few of them alone on the device (a
     prompt of 8,192 tokens at the 1B sizes: 521 us a layer by place, 393 us longest first). Within
     the sorted list every second run of as many tiles as give every compute unit one workgroup (a
     tile becomes ``workgroups_per_tile`` workgroups, one per group of query heads) is turned round,
     so that a unit that got a long tile in one round gets a short one in the next. A cut tile is
-    listed twice, each time with half its keys."""
+    listed once per run, each time with its share of the keys."""
     ent, q0s = [], []
     for e in range(first_entry, q_len.size):
         for q0 in range(0, int(q_len[e]), rows):
@@ -111,26 +140,25 @@ def list_tiles(q_len: np.ndarray, kv_len: np.ndarray, first_entry: int, rows: in
             q0s.append(q0)
     ent_a, q0_a = np.asarray(ent, np.int32), np.asarray(q0s, np.int32)
     if ent_a.size == 0:
-        return ent_a, q0_a, None, 0
+        return ent_a, q0_a, None, 0, 0
     length = q_len[ent_a].astype(np.int64)
     keys = kv_len[ent_a].astype(np.int64) - length + np.minimum(q0_a + rows, length)
     key_tiles = -(-keys // 32)
-    cut = tiles_to_cut(key_tiles, workgroups_per_tile, units) if may_cut else np.zeros(ent_a.size, bool)
-    n_cut = int(cut.sum())
+    runs = runs_of_tiles(key_tiles, workgroups_per_tile, units) if may_cut else np.ones(ent_a.size, np.int64)
     per_round = max(1, units // max(1, workgroups_per_tile))
+    cut = runs > 1
+    n_cut = int(cut.sum())
     if n_cut == 0:
         order = round_about(np.argsort(-keys, kind="stable"), per_round)
-        return ent_a[order], q0_a[order], None, 0
-    # the list's entries: whole tiles once, cut tiles twice (run 0 and run 1), each with its share of the keys
-    which = np.concatenate([np.flatnonzero(~cut), np.flatnonzero(cut), np.flatnonzero(cut)])
+        return ent_a[order], q0_a[order], None, 0, 0
+    # the list's entries: a tile once per run, each with its share of the keys
+    which = np.repeat(np.arange(ent_a.size), runs)
+    run = np.concatenate([np.arange(r) for r in runs])
     place = np.cumsum(cut) - 1                       # the cut tiles numbered in list order
-    code = np.full(which.size, -1, np.int64)
-    n_whole = int((~cut).sum())
-    code[n_whole:n_whole + n_cut] = 0 | 2 << 4 | place[cut] << 8
-    code[n_whole + n_cut:] = 1 | 2 << 4 | place[cut] << 8
-    share = np.where(code >= 0, -(-key_tiles[which] // 2), key_tiles[which])
+    code = np.where(cut[which], run | runs[which] << 4 | place[which] << 8, -1)
+    share = -(-key_tiles[which] // runs[which])
     order = round_about(np.argsort(-share, kind="stable"), per_round)
-    return ent_a[which][order], q0_a[which][order], code[order].astype(np.int32), n_cut
+    return ent_a[which][order], q0_a[which][order], code[order].astype(np.int32), n_cut, int(runs.max())
 
 
 def prefill_tiles(ctx: Any, head_dim: int, q_heads: int, kv_heads: int, first_entry: int, device: torch.device,
@@ -147,12 +175,13 @@ def prefill_tiles(ctx: Any, head_dim: int, q_heads: int, kv_heads: int, first_en
 
     def make() -> PrefillTiles:
         q_len = (ctx.q_start_host[1:] - ctx.q_start_host[:-1]).astype(np.int64)
-        ent, q0, code, n_cut = list_tiles(q_len, np.asarray(ctx.kv_len_host), first_entry, rows, per_tile, units, may_cut)
+        ent, q0, code, n_cut, room = list_tiles(q_len, np.asarray(ctx.kv_len_host), first_entry, rows, per_tile,
+                                                units, may_cut)
         if code is None:
             return PrefillTiles(*ctx.upload([ent, q0]))
         entry_t, q0_t, code_t = ctx.upload([ent, q0, code])
-        return PrefillTiles(entry_t, q0_t, code_t, n_cut,
-                            torch.empty(n_cut * cut_floats, device=device, dtype=torch.float32),
+        return PrefillTiles(entry_t, q0_t, code_t, n_cut, room,
+                            torch.empty(n_cut * room * cut_floats, device=device, dtype=torch.float32),
                             torch.zeros(n_cut * q_heads, device=device, dtype=torch.int32))
 
     return ctx.step_lists(("prefill tiles", rows, per_tile, first_entry, may_cut), make)
@@ -186,7 +215,7 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
     if ctx.num_entries > nd:
         t = prefill_tiles(ctx, head_dim, q_heads, kv_heads, nd, q.device, window)
         ops.attention_prefill(q, k_pages, v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables, t.entry, t.q0,
-                              q_heads, scale, window, t.cut, t.cut_tiles, t.cut_buf, t.cut_count)
+                              q_heads, scale, window, t.cut, t.cut_tiles, t.cut_room, t.cut_buf, t.cut_count)
 
 
 def decode_attention_unmerged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, ctx: Any, grp: Any,

@@ -29,7 +29,7 @@ _p, _i32, _i64, _f = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_f
 
 class StepShape(ctypes.Structure):
     _fields_ = [("tile_entry", _p), ("tile_q0", _p), ("tiles", _i32), ("decode_splits", _i32), ("tile_cut", _p),
-                ("cut_buf", _p), ("cut_count", _p), ("cut_tiles", _i32), ("pad0", _i32)]
+                ("cut_buf", _p), ("cut_count", _p), ("cut_tiles", _i32), ("cut_room", _i32)]
 
 
 class StepArgs(ctypes.Structure):
@@ -152,7 +152,7 @@ class NativeBlocks:
                 t = prefill_tiles(ctx, d, qh, kvh, nd, self.device, window=1 if windowed else 0)
                 sh.tile_entry, sh.tile_q0, sh.tiles = t.entry.data_ptr(), t.q0.data_ptr(), t.tiles
                 if t.cut is not None:
-                    sh.tile_cut, sh.cut_tiles = t.cut.data_ptr(), t.cut_tiles
+                    sh.tile_cut, sh.cut_tiles, sh.cut_room = t.cut.data_ptr(), t.cut_tiles, t.cut_room
                     sh.cut_buf, sh.cut_count = t.cut_buf.data_ptr(), t.cut_count.data_ptr()
             if nd > 0:
                 # mixers of one shape plan alike, so the first one's answer for a recorded step holds for all

@@ -79,28 +79,41 @@ def test_a_call_records_graphs_where_it_decodes_long_enough():
 
 def test_which_tiles_of_a_short_launch_have_their_keys_cut():
     """One prompt of 2,048 tokens at the 1B sizes (a tile of 32 queries is 8 workgroups, 256 compute
-    units): the 32 tiles that walk more than half of the longest one's key tiles are cut, which
-    brings the launch to three workgroups a unit; from 3,072 tokens on nothing is cut; never a tile
-    too short for two runs, never more than the launch has room for."""
+    units): the 21 longest tiles are cut in two, after which no workgroup is longer than two
+    thirds of a unit's work; from 3,072 tokens on nothing is cut; shorter launches cut into more
+    runs, never runs of fewer than eight key tiles, never more workgroups than three a unit, and
+    nothing where the longest workgroup would stay about as long."""
     import numpy as np
 
-    from dli_amd.parts.attention_kernels import MIN_RUN_TILES, tiles_to_cut
+    from dli_amd.parts.attention_kernels import MAX_RUNS, MIN_RUN_TILES, runs_of_tiles
 
-    key_tiles = np.arange(1, 65)
-    cut = tiles_to_cut(key_tiles, 8, 256)
-    assert cut.sum() == 32 and cut[32:].all() and not cut[:32].any()
-    assert not tiles_to_cut(np.arange(1, 97), 8, 256).any()
-    cut = tiles_to_cut(np.arange(1, 81), 8, 256)           # room for 16 more entries
-    assert cut.sum() == 16 and cut[64:].all()
-    cut = tiles_to_cut(np.arange(1, 21), 8, 256)           # 640 tokens: only tiles of 16 key tiles and more
-    assert cut.tolist() == [n >= 2 * MIN_RUN_TILES for n in range(1, 21)]
-    assert not tiles_to_cut(np.arange(1, 9), 8, 256).any() and not tiles_to_cut(np.zeros(0, np.int64), 8, 256).any()
+    runs = runs_of_tiles(np.arange(1, 65), 8, 256)       # the launch's work: 65 tiles a unit; runs of up to 43 may stay
+    assert runs[:43].tolist() == [1] * 43 and runs[43:].tolist() == [2] * 21
+    assert runs_of_tiles(np.arange(1, 97), 8, 256).tolist() == [1] * 96
+    runs = runs_of_tiles(np.arange(1, 81), 8, 256)           # room for 16 more entries, 13 used
+    assert runs.sum() == 93 and runs[67:].tolist() == [2] * 13
+    for tokens in (512, 640, 1024, 1536):
+        key_tiles = np.arange(1, tokens // 32 + 1)
+        runs = runs_of_tiles(key_tiles, 8, 256)
+        assert runs.sum() * 8 <= 3 * 256 and runs.max() <= MAX_RUNS
+        assert all(r == 1 or n // r >= MIN_RUN_TILES for n, r in zip(key_tiles.tolist(), runs.tolist()))
+        longest = max(-(-n // r) for n, r in zip(key_tiles.tolist(), runs.tolist()))
+        assert longest <= 0.85 * key_tiles.max() or runs.max() == 1
+    assert runs_of_tiles(np.arange(1, 33), 8, 256).max() >= 3    # 1,024 tokens: more than two runs for the longest
+    assert runs_of_tiles(np.arange(1, 9), 8, 256).max() == 1 and runs_of_tiles(np.zeros(0, np.int64), 8, 256).size == 0
+    # a portion of 2,048 tokens on top of 14K cached keys: 64 tiles of 450 to 512 key tiles, room for 32 more
+    # workgroups a head group, after which the longest whole tile would still walk 480: nothing is cut
+    assert runs_of_tiles(np.arange(449, 513), 8, 256).max() == 1
+    # 512 tokens on top of 8K keys: 16 tiles of much the same length, room for 80 more entries: six runs each
+    assert runs_of_tiles(np.arange(257, 273), 8, 256).tolist() == [6] * 16
+    # one prompt of 1,536 tokens: two runs for the upper half, as at 2,048
+    assert runs_of_tiles(np.arange(1, 49), 8, 256).tolist() == [1] * 24 + [2] * 24
 
 
-def test_the_tile_list_of_a_step_lists_every_tile_once_or_both_of_its_runs():
-    """Random steps: every tile of every portion is in the list, whole or as run 0 and run 1 with
-    the same place; places count the cut tiles from 0; the entries' shares of keys never grow
-    within a round of the list (every second round is turned round)."""
+def test_the_tile_list_of_a_step_lists_every_tile_once_or_all_of_its_runs():
+    """Random steps: every tile of every portion is in the list, whole or once per run with the
+    same place and number of runs; places count the cut tiles from 0; the launch stays under three
+    workgroups a compute unit where anything is cut."""
     import random
 
     import numpy as np
@@ -115,19 +128,21 @@ def test_the_tile_list_of_a_step_lists_every_tile_once_or_both_of_its_runs():
         kv_len = q_len + np.asarray([rng.randrange(0, 500) for _ in range(n)], np.int64)
         rows, per_tile, units = rng.choice([(32, 8), (128, 24), (64, 4), (128, 9)]) + (rng.choice([64, 256, 304]),)
         may_cut = rng.random() < 0.8
-        ent, q0, code, n_cut = list_tiles(q_len, kv_len, first, rows, per_tile, units, may_cut)
+        ent, q0, code, n_cut, room = list_tiles(q_len, kv_len, first, rows, per_tile, units, may_cut)
         want = {(e, t) for e in range(first, n) for t in range(0, int(q_len[e]), rows)}
         if code is None:
-            assert n_cut == 0 and sorted(zip(ent.tolist(), q0.tolist())) == sorted(want)
+            assert n_cut == 0 and room == 0 and sorted(zip(ent.tolist(), q0.tolist())) == sorted(want)
             continue
-        assert may_cut and n_cut > 0 and len(ent) == len(want) + n_cut
+        assert may_cut and n_cut > 0
         whole = [(e, t) for e, t, c in zip(ent.tolist(), q0.tolist(), code.tolist()) if c < 0]
         runs = {}
         for e, t, c in zip(ent.tolist(), q0.tolist(), code.tolist()):
             if c >= 0:
-                assert (c >> 4) & 15 == 2
-                runs.setdefault((e, t), []).append((c & 15, c >> 8))
+                runs.setdefault((e, t), []).append((c & 15, (c >> 4) & 15, c >> 8))
         assert len(whole) == len(set(whole)) and set(whole) | set(runs) == want and not set(whole) & set(runs)
-        assert all(sorted(r) == [(0, r[0][1]), (1, r[0][1])] for r in runs.values())
-        assert sorted(r[0][1] for r in runs.values()) == list(range(n_cut))
+        for r in runs.values():
+            n, place = r[0][1], r[0][2]
+            assert 2 <= n <= room and sorted(r) == [(i, n, place) for i in range(n)]
+        assert max(r[0][1] for r in runs.values()) == room
+        assert sorted(r[0][2] for r in runs.values()) == list(range(n_cut))
         assert len(ent) * per_tile <= 3 * units

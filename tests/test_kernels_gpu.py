@@ -346,31 +346,39 @@ def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, 
     many heads, in which the order of the workgroups differs from the grid's), listed as the engine
     lists it: one prompt whose length puts the launch there, on top of 24 cached keys, and a short
     one beside it. Once with every tile whole and once with the keys of the longest tiles cut
-    into two runs that two workgroups share (twice on the same counters: each launch leaves them
-    zero): the two agree, and rows of both requests agree with a 32-bit softmax over their keys."""
-    import numpy as np
-    from dli_amd.parts.attention_kernels import list_tiles
-
+    into runs that as many workgroups share (twice on the same counters: each launch leaves them
+    zero, and the two launches give the same bits): whole and cut agree, and rows of both requests
+    agree with a 32-bit softmax over their keys. The same again for a portion of 100 tokens on top of
+    3,000 cached keys, whose few tiles are cut into many runs."""
     units = ops.compute_units(torch.device("cuda"))
     rows = ops.attention_prefill_tile_rows(d, qh, kvh)
     per_tile = qh // (4 * 32 // rows)             # workgroups that a tile of the list becomes
     tiles = -(-units * 3 // (2 * per_tile))        # 1.5 workgroups a unit
     bs = 16
     long_q = tiles * rows - 40 - rows
-    lens = [(long_q, long_q + 24), (40, 77)]
+    for lens, most_runs in (([(long_q, long_q + 24), (40, 77)], 2), ([(100, 3100), (40, 77)], 3)):
+        _check_cut_and_whole(ops, qh, kvh, d, bs, lens, rows, per_tile, units, most_runs)
+
+
+def _check_cut_and_whole(ops, qh, kvh, d, bs, lens, rows, per_tile, units, most_runs):
+    import numpy as np
+    from dli_amd.parts.attention_kernels import list_tiles
+
+    long_q = lens[0][0]
     q, kp, vp, q_start, kv_len, tables = _paged_case(torch.bfloat16, qh, kvh, d, bs, lens, seed=qh + d)
     dev = lambda x: torch.tensor(np.asarray(x), dtype=torch.int32, device="cuda")
     scale = 1.0 / math.sqrt(d)
     q_len = np.asarray([n for n, _ in lens], np.int64)
     outs = []
     for may_cut in (False, True):
-        te, tq, code, n_cut = list_tiles(q_len, np.asarray(kv_len, np.int64), 0, rows, per_tile, units, may_cut)
-        assert (code is not None) == may_cut and len(te) == tiles + n_cut
+        te, tq, code, n_cut, room = list_tiles(q_len, np.asarray(kv_len, np.int64), 0, rows, per_tile, units, may_cut)
+        assert (code is not None) == may_cut
         extra = {}
         if may_cut:
-            assert n_cut > 0 and sorted(c & 15 for c in code if c >= 0) == [0] * n_cut + [1] * n_cut
-            extra = dict(tile_cut=dev(code), cut_tiles=n_cut,
-                         cut_buf=torch.full((n_cut * ops.attention_prefill_cut_floats(d, qh, kvh),), float("nan"), device="cuda"),
+            assert n_cut > 0 and room >= most_runs
+            extra = dict(tile_cut=dev(code), cut_tiles=n_cut, cut_room=room,
+                         cut_buf=torch.full((n_cut * room * ops.attention_prefill_cut_floats(d, qh, kvh),), float("nan"),
+                                            device="cuda"),
                          cut_count=torch.zeros(n_cut * qh, dtype=torch.int32, device="cuda"))
         for again in range(2 if may_cut else 1):
             out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
@@ -384,7 +392,8 @@ def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, 
     assert (outs[0].float() - outs[1].float()).abs().max().item() < tol(torch.bfloat16)
     # rows of the long request and the short one's last, from their keys gathered out of the pages
     kd, vd = kp.cuda().float(), vp.cuda().float()
-    for e, row in ((0, 0), (0, 31), (0, 32), (0, 127), (0, 128), (0, long_q // 2 + 3), (0, long_q - 1), (1, 39)):
+    for e, row in ((0, 0), (0, 31), (0, 32), (0, min(127, long_q - 2)), (0, min(128, long_q - 2)), (0, long_q // 2 + 3),
+                   (0, long_q - 1), (1, 39)):
         n_keys = kv_len[e] - (q_start[e + 1] - q_start[e]) + row + 1
         pages = torch.tensor(tables[e][:-(-n_keys // bs)], device="cuda")
         keys = kd[pages].permute(1, 0, 2, 3).reshape(kvh, -1, d)[:, :n_keys]         # [kvh, keys, d]
