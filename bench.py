@@ -7,7 +7,8 @@ greedily at a context of about 4096 tokens through the engine's own step loop (s
 batched step, sampling), W untimed steps and then exactly K timed ones between device
 synchronisations. One JSON line reports decoded tokens a second, the time of a 2,048-token prefill
 step, the decode step's memory roofline, and under ``points`` decode throughput at batch 1 and 64,
-at the baseline's own context (2,048 growing to 2,304) and at 32,768 keys, and the other
+at the baseline's own context (2,048 growing to 2,304) and at 32,768 keys, a prompt of 16,384
+tokens in portions of 2,048 and of 512, and the other
 workloads that the baseline names: the Llama-3.2-3B sizes (decode at batch 8, a 2,048-token
 prefill, 64 requests batched continuously under 2,048 tokens a step) and the SmolLM2-1.7B sizes
 (decode at batch 8, 32 requests that share a prefix of 1,024 tokens). ``--no-other-shapes`` leaves
@@ -144,11 +145,20 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     return batch * steps / dt, dt / steps * 1e3, per
 
 
-def prefill_run(engine, cfg, tokens, repeats=3):
+def prefill_run(engine, cfg, tokens, repeats=3, portion=None):
+    """Seconds for one prompt of ``tokens`` tokens (the best of ``repeats``, after one untimed run):
+    in one step, or with ``portion`` in steps of at most that many tokens, each on top of the keys
+    that the earlier ones left in the cache."""
+    import dataclasses
+
     import torch
 
     from dli_amd.sampling import SamplingParams
 
+    config = engine.scheduler.config
+    assert (portion or tokens) <= config.max_num_batched_tokens, "the engine's buffers are made for its own budget"
+    if portion:
+        engine.scheduler.config = dataclasses.replace(config, max_num_batched_tokens=portion)
     gen = torch.Generator().manual_seed(99)
     best = float("inf")
     for r in range(repeats + 1):
@@ -156,12 +166,16 @@ def prefill_run(engine, cfg, tokens, repeats=3):
         engine.add_request(f"p{r}", prompt, SamplingParams(max_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        engine.step()  # the whole prompt is one portion: budget >= tokens
+        steps = 0
+        while engine.has_unfinished():
+            engine.step()
+            steps += 1
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        assert not engine.has_unfinished()
+        assert steps == -(-tokens // (portion or tokens))
         if r > 0:
             best = min(best, dt)
+    engine.scheduler.config = config
     return best
 
 
@@ -291,6 +305,8 @@ def main() -> int:
                     help="run only prefill steps of --prefill-tokens tokens (for profiling) and print their time")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="prompt length of --only-prefill (the line of the default run always has 2,048)")
+    ap.add_argument("--portion", type=int, default=None,
+                    help="with --only-prefill: the prompt runs in steps of at most this many tokens")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
@@ -323,8 +339,9 @@ def main() -> int:
 
     if args.only_prefill:
         n = args.prefill_tokens
-        t = prefill_run(engine, cfg, n, repeats=args.steps)
-        print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": n, "tok_s": round(n / t, 1),
+        t = prefill_run(engine, cfg, n, repeats=args.steps, portion=args.portion)
+        print(json.dumps({"prefill_ms": round(t * 1e3, 3), "tokens": n, "portion": args.portion or n,
+                          "tok_s": round(n / t, 1),
                           "frac": round(prefill_flops(cfg, n) / t / PEAK_FLOPS[short], 4),
                           "attention_gflop_per_layer": round(2 * cfg.num_heads * cfg.head_dim * n * (n + 1) / 1e9, 2)}))
         return 0
@@ -378,6 +395,13 @@ def main() -> int:
             torch.cuda.empty_cache()
             engine, _ = engine_for(model, 8, 32768, args.block_size, 8192, args.decode_steps)
             point("decode_b8_context32768", 8, 32768, args.decode_steps)
+            # a long prompt in portions, each on top of the keys of the earlier ones
+            for portion in (2048, 512):   # 512 is the scheduler's own default budget
+                t = prefill_run(engine, cfg, 16384, repeats=2, portion=portion)
+                key = f"prefill16384_in_portions_of_{portion}"
+                points[key] = round(16384 / t, 1)
+                points[key + "_ms"] = round(t * 1e3, 3)
+                points[key + "_frac"] = round(prefill_flops(cfg, 16384) / t / PEAK_FLOPS[short], 4)
             del engine, model
             gc.collect()
             torch.cuda.empty_cache()

@@ -7,7 +7,7 @@
 #define DLI_MAX_SHAPES 4   // distinct attention shapes (head size, heads, kv heads) in one model
 
 // What depends on the step's batch and an attention shape: the query tiles of the portions (for
-// this shape's tile height), which of them have their keys cut into two runs (tile_cut null: none;
+// this shape's tile height), which of them have their keys cut into runs (tile_cut null: none;
 // see dli_attention_prefill_bf16) with the memory for that, and the key splits of the
 // single-token rows.
 struct DliStepShape {
