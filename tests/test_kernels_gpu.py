@@ -349,14 +349,16 @@ def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, 
     into runs that as many workgroups share (twice on the same counters: each launch leaves them
     zero, and the two launches give the same bits): whole and cut agree, and rows of both requests
     agree with a 32-bit softmax over their keys. The same again for a portion of 100 tokens on top of
-    3,000 cached keys, whose few tiles are cut into many runs."""
+    3,000 cached keys, whose few tiles are cut into many runs, and for 40 tokens on top of 8,960,
+    whose two tiles get as many runs as the kernel takes."""
     units = ops.compute_units(torch.device("cuda"))
     rows = ops.attention_prefill_tile_rows(d, qh, kvh)
     per_tile = qh // (4 * 32 // rows)             # workgroups that a tile of the list becomes
     tiles = -(-units * 3 // (2 * per_tile))        # 1.5 workgroups a unit
     bs = 16
     long_q = tiles * rows - 40 - rows
-    for lens, most_runs in (([(long_q, long_q + 24), (40, 77)], 2), ([(100, 3100), (40, 77)], 3)):
+    for lens, most_runs in (([(long_q, long_q + 24), (40, 77)], 2), ([(100, 3100), (40, 77)], 3),
+                            ([(40, 9000), (40, 77)], ops.attention_prefill_max_cuts())):
         _check_cut_and_whole(ops, qh, kvh, d, bs, lens, rows, per_tile, units, most_runs)
 
 
