@@ -346,9 +346,9 @@ def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, 
     many heads, in which the order of the workgroups differs from the grid's), listed as the engine
     lists it: one prompt whose length puts the launch there, on top of 24 cached keys, and a short
     one beside it. Once with every tile whole and once with the keys of the longest tiles cut
-    into runs that as many workgroups share (twice on the same counters: each launch leaves them
-    zero, and the two launches give the same bits): whole and cut agree, and rows of both requests
-    agree with a 32-bit softmax over their keys. The same again for a portion of 100 tokens on top of
+    into runs that as many workgroups share (twice on the same counters and buffers, with a launch
+    for other queries in between: each launch leaves the counters zero, and the two give the same
+    bits): whole and cut agree, and rows of both requests agree with a 32-bit softmax over their keys. The same again for a portion of 100 tokens on top of
     3,000 cached keys, whose few tiles are cut into many runs, and for 40 tokens on top of 8,960,
     whose two tiles get as many runs as the kernel takes."""
     units = ops.compute_units(torch.device("cuda"))
@@ -383,6 +383,9 @@ def _check_cut_and_whole(ops, qh, kvh, d, bs, lens, rows, per_tile, units, most_
                                             device="cuda"),
                          cut_count=torch.zeros(n_cut * qh, dtype=torch.int32, device="cuda"))
         for again in range(2 if may_cut else 1):
+            if again:   # other queries through the same buffers in between: nothing of them may be left behind
+                ops.attention_prefill(-q.cuda(), kp.cuda(), vp.cuda(), torch.empty_like(out), dev(q_start), dev(kv_len),
+                                      dev(tables), dev(te), dev(tq), qh, scale, 0, **extra)
             out = torch.full(q.shape, 9.0, dtype=torch.bfloat16, device="cuda")
             ops.attention_prefill(q.cuda(), kp.cuda(), vp.cuda(), out, dev(q_start), dev(kv_len), dev(tables), dev(te),
                                   dev(tq), qh, scale, 0, **extra)
