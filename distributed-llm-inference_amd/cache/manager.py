@@ -14,15 +14,21 @@ one at a time as a request grows; a request's full, computed pages are entered i
 operation that cannot get its pages raises :class:`NoFreePagesError` before it changes anything.
 
 Content reuse needs the cached pages to be a pure function of the token prefix in *every* group,
-and the request to have no other per-request state: it is active only when there is exactly one
-group, of kind ``full``, and the model is not ``stateful``.
+and the request to have no other per-request state: it is off for a ``stateful`` model. Every
+group keeps a content index of its own, under the same identities (the hash chain over the token
+prefix). A prompt's leading pages are served from the indexes only as far as *all* groups can
+serve them: a ``full`` group must hold every page of the run, a ``window`` group the pages that the
+first computed token's window still reaches (the pages before those start out as released, as
+they would be had the request computed the run itself).
 
 Rules of the content index (each prevents a concrete fault; block_manager.py:17-29):
 only full pages are entered; only after their keys have been computed; a prompt is never served
 wholly from the index (the page with its last token is always computed, since a step must run at
-least one token to give logits); a page is entered only under its own request's cached parent, and
-only leaves are reclaimed, so every cached page is reachable from the root; shared pages are never
-written.
+least one token to give logits); in a full group a page is entered only under its own request's
+cached parent, and only leaves are reclaimed, so every cached page is reachable from the root (a
+window group gives its oldest pages back first, so there a page stands by itself: no parent, any
+idle one may be reclaimed, and a lookup asks for each page it needs by name); shared pages are
+never written.
 """
 
 from __future__ import annotations
@@ -144,8 +150,18 @@ class _Seq:
     reserved: int = 0  # tokens that the tables have room for, where that exceeds num_tokens
 
 
+@dataclass
+class _Hits:
+    """What the content indexes hold of a prompt: ``pages`` leading pages need no computing;
+    group g's table starts with ``first[g]`` released entries, then the cached pages ``found[g]``."""
+
+    pages: int
+    first: list[int]
+    found: list[list[int]]
+
+
 class CacheManager:
-    """Hands out pages and state slots to requests and keeps the content index.
+    """Hands out pages and state slots to requests and keeps the content indexes.
 
     Args:
         groups: one :class:`GroupSpec` per group of layers (the dense Llama decoder has one).
@@ -153,6 +169,7 @@ class CacheManager:
         page_size: token slots per page.
         max_seqs: number of state slots, i.e. the most requests that hold cache at once.
         stateful: the model keeps per-request state outside the pages (disables content reuse).
+        enable_prefix_caching: content reuse, in all groups or in none.
         watermark: fraction of each group's pages kept back when *admitting* prompts, so running
             requests can still grow (block_manager.py:138-139).
         confine_to_thread: every call that changes the manager must come from the thread that
@@ -184,11 +201,11 @@ class CacheManager:
         if len(counts) != len(self.groups) or any(c <= 0 for c in counts):
             raise ValueError("num_pages must be positive, one number or one per group")
         self.page_size = page_size
-        self.pools = [PagePool(c, eviction_policy if i == 0 else "lru") for i, c in enumerate(counts)]
+        # a policy given by name is made once per group; an order handed in serves the first group
+        self.pools = [PagePool(c, eviction_policy if i == 0 or isinstance(eviction_policy, str) else "lru")
+                      for i, c in enumerate(counts)]
         self.slots = StateSlots(max_seqs)
-        self.prefix_caching = bool(
-            enable_prefix_caching and len(self.groups) == 1 and self.groups[0].kind == "full" and not stateful
-        )
+        self.prefix_caching = bool(enable_prefix_caching and not stateful)
         self._reserve = [int(watermark * c) for c in counts]
         self._seqs: dict[SeqId, _Seq] = {}
         self._stats = CacheStats()
@@ -252,7 +269,7 @@ class CacheManager:
 
     def pages_needed_for_prompt(self, token_ids: Sequence[int], namespace: bytes = b"") -> int:
         hits, _ = self._lookup(token_ids, namespace)
-        return self._ceil(len(token_ids)) - len(hits)
+        return self._ceil(len(token_ids)) - hits.pages
 
     def can_allocate(self, token_ids: Sequence[int], namespace: bytes = b"") -> bool:
         """Whether :meth:`allocate` would succeed with the watermark respected."""
@@ -298,14 +315,14 @@ class CacheManager:
         pages = self._ceil(n)
         if not self._admissible(n, hits, respect_watermark=respect_watermark):
             raise NoFreePagesError(
-                f"request {seq_id!r} needs {pages - len(hits)} more pages for its {n} tokens; "
+                f"request {seq_id!r} needs {pages - hits.pages} more pages for its {n} tokens; "
                 f"{self.num_available_pages} can be had ({max(self._reserve)} kept back)")
         # Everything below succeeds: the checks above have counted the pages.
-        tables = [self._fill_table(pool, hits if g == 0 else (), pages) for g, pool in enumerate(self.pools)]
-        seq = _Seq(tables=tables, num_tokens=n, num_computed=len(hits) * self.page_size, namespace=namespace,
-                   state_slot=self.slots.take(), released=[0] * len(self.pools))
+        tables = [self._fill_table(pool, hits.first[g], hits.found[g], pages) for g, pool in enumerate(self.pools)]
+        seq = _Seq(tables=tables, num_tokens=n, num_computed=hits.pages * self.page_size, namespace=namespace,
+                   state_slot=self.slots.take(), released=list(hits.first))
         if self.prefix_caching:
-            seq.page_hashes, seq.num_registered = hashes, len(hits)
+            seq.page_hashes, seq.num_registered = hashes, hits.pages
             seq.tail_tokens = list(token_ids[len(hashes) * self.page_size:])
         self._stats.prompt_tokens_queried += n
         self._stats.prompt_tokens_hit += seq.num_computed
@@ -313,14 +330,15 @@ class CacheManager:
         return Allocation(tuple(map(tuple, tables)), seq.num_computed, seq.state_slot)
 
     @staticmethod
-    def _fill_table(pool: PagePool, hits: Sequence[int], pages: int) -> list[int]:
-        """A new request's table in one group: the cached pages that its prompt matched, then
-        fresh ones up to ``pages``. The matched pages are taken hold of first, so that none of
-        them can be reclaimed to make room for the fresh ones."""
+    def _fill_table(pool: PagePool, first: int, hits: Sequence[int], pages: int) -> list[int]:
+        """A new request's table in one group: ``first`` entries for pages that the window has
+        passed already, the cached pages that its prompt matched, then fresh ones up to ``pages``.
+        The matched pages are taken hold of first, so that none of them can be reclaimed to make
+        room for the fresh ones."""
         for page in hits:
             pool.incref(page)
             pool.order.found(page)
-        return [*hits, *(pool.take() for _ in range(pages - len(hits)))]
+        return [*([RELEASED] * first), *hits, *(pool.take() for _ in range(pages - first - len(hits)))]
 
     @_confined
     def append_slots(self, seq_id: SeqId, token_ids: Sequence[int]) -> list[CopyOp]:
@@ -464,35 +482,52 @@ class CacheManager:
         except KeyError:
             raise SequenceError(f"unknown sequence {seq_id!r}") from None
 
-    def _lookup(self, token_ids: Sequence[int], namespace: bytes) -> tuple[list[int], list[PageHash]]:
-        """Longest cached run of leading full pages, never the page with the last token."""
+    def _first_needed_page(self, g: int, computed_pages: int) -> int:
+        """The first page of group ``g`` that a request with ``computed_pages`` full pages computed
+        still reads: its next query sits at the first position after them."""
+        spec = self.groups[g]
+        if spec.kind != "window":
+            return 0
+        return max(0, computed_pages * self.page_size - spec.window + 1) // self.page_size
+
+    def _lookup(self, token_ids: Sequence[int], namespace: bytes) -> tuple[_Hits, list[PageHash]]:
+        """The longest run of leading full pages that every group can serve from its index,
+        never the page with the last token."""
+        none = _Hits(0, [0] * len(self.pools), [[] for _ in self.pools])
         if not self.prefix_caching:
-            return [], []
+            return none, []
         eligible = (len(token_ids) - 1) // self.page_size * self.page_size
         hashes = chain_hashes(namespace, token_ids[:eligible], self.page_size)
-        hits: list[int] = []
-        index = self.pools[0].by_identity
-        for h in hashes:
-            page = index.get(h)
-            if page is None:
+        run = len(hashes)   # full groups: the run ends at the first page that one of them lacks
+        for g, pool in enumerate(self.pools):
+            if self.groups[g].kind == "full":
+                run = next((i for i, h in enumerate(hashes[:run]) if h not in pool.by_identity), run)
+        while run > 0:      # window groups: the pages that the window at the run's end reaches
+            short = False
+            for g, pool in enumerate(self.pools):
+                if self.groups[g].kind == "window":
+                    short = short or any(hashes[i] not in pool.by_identity
+                                         for i in range(self._first_needed_page(g, run), run))
+            if not short:
                 break
-            hits.append(page)
-        return hits, hashes
+            run -= 1
+        if run == 0:
+            return none, hashes
+        first = [self._first_needed_page(g, run) for g in range(len(self.pools))]
+        found = [[pool.by_identity[h] for h in hashes[first[g]:run]] for g, pool in enumerate(self.pools)]
+        return _Hits(run, first, found), hashes
 
-    def _admissible(self, n_tokens: int, hits: list[int], *, respect_watermark: bool) -> bool:
-        total = self._ceil(n_tokens)
+    def _admissible(self, n_tokens: int, hits: _Hits, *, respect_watermark: bool) -> bool:
+        fresh = self._ceil(n_tokens) - hits.pages
         for g, pool in enumerate(self.pools):
             reserve = self._reserve[g] if respect_watermark else 0
-            if g == 0:
-                revived = sum(1 for p in hits if pool.ref[p] == 0)  # idle hits stop being reclaimable
-                if pool.num_available - revived - (total - len(hits)) < reserve:
-                    return False
-            elif pool.num_available - total < reserve:
+            revived = sum(1 for p in hits.found[g] if pool.ref[p] == 0)  # idle hits stop being reclaimable
+            if pool.num_available - revived - fresh < reserve:
                 return False
         return True
 
     def _register_full_pages(self, seq: _Seq) -> None:
-        ps, pool = self.page_size, self.pools[0]
+        ps = self.page_size
         full_computed = seq.num_computed // ps
         while seq.num_registered < full_computed:
             i = seq.num_registered
@@ -500,11 +535,15 @@ class CacheManager:
                 parent_hash = seq.page_hashes[-1] if seq.page_hashes else ROOT_PARENT
                 seq.page_hashes.append(page_hash(seq.namespace, parent_hash, seq.tail_tokens[:ps]))
                 del seq.tail_tokens[:ps]
-            outcome = pool.register(
-                seq.tables[0][i], seq.page_hashes[i],
-                seq.page_hashes[i - 1] if i else None, seq.tables[0][i - 1] if i else None, i)
-            if outcome == "duplicate":
-                self._stats.duplicate_registrations += 1
+            for g, pool in enumerate(self.pools):
+                table = seq.tables[g]
+                if table[i] == RELEASED:
+                    continue
+                chained = self.groups[g].kind == "full" and i > 0
+                outcome = pool.register(table[i], seq.page_hashes[i], seq.page_hashes[i - 1] if chained else None,
+                                        table[i - 1] if chained else None, i)
+                if outcome == "duplicate":
+                    self._stats.duplicate_registrations += 1
             seq.num_registered += 1
 
     def _release_passed(self, seq: _Seq, g: int, window: int) -> None:

@@ -245,7 +245,6 @@ def test_reclaim_orders():
 
 def test_window_group_gives_pages_back_while_the_request_runs():
     m = CacheManager([GroupSpec(), GroupSpec("window", 6)], num_pages=[32, 8], page_size=4, watermark=0.0)
-    assert not m.prefix_caching  # content reuse needs a single full group
     m.allocate("a", list(range(10)))
     assert len(m.block_table("a", 0)) == 3 and len(m.block_table("a", 1)) == 3
     m.mark_computed("a", 10)
@@ -264,6 +263,68 @@ def test_window_group_gives_pages_back_while_the_request_runs():
     m.free("a")
     m.check_invariants()
     assert all(p.num_available == p.num_pages for p in m.pools)
+
+
+def test_two_full_groups_serve_a_prompt_as_far_as_both_hold_it():
+    m = CacheManager([GroupSpec(), GroupSpec()], num_pages=[16, 5], page_size=4, watermark=0.0)
+    assert m.prefix_caching
+    a = list(range(17))                       # four full pages and the page of the last token
+    m.allocate("a", a)
+    m.mark_computed("a", 17)
+    m.free("a")
+    got = m.allocate("b", a + [99])
+    assert got.num_cached_tokens == 16
+    assert all(len(t) == 5 for t in got.block_tables)
+    m.free("b")
+    # the small group loses pages of the run to another prompt (leaves first): the run ends there in both
+    m.allocate("c", [50, 51, 52, 53, 54, 55, 56, 57, 58])        # three pages of the second group's five
+    m.check_invariants()
+    assert sum(1 for h in chain_hashes(b"", a[:16], 4) if h in m.pools[1].by_identity) == 2
+    assert sum(1 for h in chain_hashes(b"", a[:16], 4) if h in m.pools[0].by_identity) == 4
+    m.free("c")
+    got = m.allocate("d", a)
+    assert got.num_cached_tokens == 8
+    assert got.block_tables[0][:2] != got.block_tables[0][2:4] and len(got.block_tables[1]) == 5
+    m.check_invariants()
+
+
+def test_a_window_group_serves_the_pages_that_the_first_computed_token_still_reaches():
+    ps, window = 4, 6
+    m = CacheManager([GroupSpec(), GroupSpec("window", window)], num_pages=[32, 12], page_size=ps, watermark=0.0)
+    a = list(range(30))
+    m.allocate("a", a)
+    for upto in (7, 19, 30):                  # in portions: pages are entered before the window passes them
+        m.mark_computed("a", upto)
+        m.check_invariants()
+    held = m.block_table("a", 1)
+    assert held[:6] == (RELEASED,) * 6        # next query at 30 sees keys 25..: pages 0..5 are passed
+    m.free("a")
+    # 22 tokens in common, then others: five full pages match; a query at 20 sees keys 15..20: from page 3 on
+    b = a[:22] + [77, 78, 79]
+    got = m.allocate("b", b)
+    assert got.num_cached_tokens == 20
+    full, win = got.block_tables
+    assert RELEASED not in full and len(full) == len(win) == 7
+    assert win[:3] == (RELEASED,) * 3 and RELEASED not in win[3:]
+    assert m.slot_mapping("b", 15, 25, group=1)
+    with pytest.raises(ValueError):
+        m.slot_mapping("b", 11, 12, group=1)
+    m.check_invariants()
+    m.mark_computed("b", 25)
+    m.check_invariants()
+    # the window group has lost a page that such a run needs: the run is cut back to where both can serve it
+    m.free("b")
+    h = chain_hashes(b"", a[:20], ps)
+    pool = m.pools[1]
+    victim = pool.by_identity[h[4]]
+    while victim in pool.cached:              # reclaim idle pages until that one has gone
+        pool.free.append(pool._evict(pool.order.take()))
+    m.check_invariants()
+    got = m.allocate("c", b)
+    assert got.num_cached_tokens < 20
+    first = max(0, got.num_cached_tokens - window + 1) // ps
+    assert got.block_tables[1][:first] == (RELEASED,) * first and RELEASED not in got.block_tables[1][first:]
+    m.check_invariants()
 
 
 def test_state_slots_are_taken_and_given_back():
@@ -338,18 +399,29 @@ def test_random_orders_of_requests_keep_every_invariant(seed, policy):
     assert m.slots.num_free == 5, "state slots were lost"
 
 
-def test_shadow_cache_never_serves_wrong_or_unwritten_content():
-    """A shadow of the device memory: slot -> (token prefix that was written there). A hit must
-    point at pages whose shadow equals the new prompt's prefix, and a write must never land in a
-    page that another request holds."""
-    rng = random.Random(7)
+@pytest.mark.parametrize("groups,pages", [
+    ([GroupSpec()], [24]),
+    ([GroupSpec(), GroupSpec()], [24, 17]),
+    ([GroupSpec(), GroupSpec("window", 6)], [24, 14]),
+    ([GroupSpec("window", 9), GroupSpec(), GroupSpec("window", 3)], [20, 24, 12]),
+])
+def test_shadow_cache_never_serves_wrong_or_unwritten_content(groups, pages):
+    """A shadow of the device memory of every group: slot -> (token prefix that was written there).
+    A hit must point at pages whose shadow equals the new prompt's prefix, in every group, for
+    every key that the request's first computed token and the ones after it read there (all
+    of them, or those inside the window); and a write must never land in a page that another
+    request holds. Steps compute in portions of any length, as an engine's would."""
+    rng = random.Random(7 + len(groups))
     ps = 4
-    m = mk(num_pages=24, page_size=ps)
-    written: dict[int, tuple] = {}
+    m = CacheManager(groups, num_pages=pages, page_size=ps, watermark=0.0)
+    assert m.prefix_caching
+    written: list[dict[int, tuple]] = [{} for _ in groups]
     live: dict = {}
-    for step in range(800):
+    hits = 0
+    stems = [[rng.randrange(3) for _ in range(22)] for _ in range(3)]
+    for step in range(1200):
         if rng.random() < 0.4 or not live:
-            toks = [rng.randrange(3) for _ in range(rng.randrange(1, 25))]
+            toks = (rng.choice(stems)[:rng.randrange(0, 22)] + [rng.randrange(3) for _ in range(rng.randrange(1, 12))])[:28]
             try:
                 alloc = m.allocate(step, toks)
             except (NoFreePagesError, NoFreeSlotError):
@@ -358,26 +430,36 @@ def test_shadow_cache_never_serves_wrong_or_unwritten_content():
                     m.free(rid)
                     del live[rid]
                 continue
-            for p in range(alloc.num_cached_tokens):
-                slot = m.slot_mapping(step, p, p + 1)[0]
-                assert written.get(slot) == tuple(toks[:p + 1]), "a hit serves wrong or unwritten content"
+            cached = alloc.num_cached_tokens
+            hits += cached > 0
+            for g, spec in enumerate(groups):
+                first_read = max(0, cached - spec.window + 1) if spec.kind == "window" else 0
+                for p in range(first_read, cached):
+                    slot = m.slot_mapping(step, p, p + 1, group=g)[0]
+                    assert written[g].get(slot) == tuple(toks[:p + 1]), "a hit serves wrong or unwritten content"
             live[step] = toks
         else:
             rid = rng.choice(list(live))
             toks = live[rid]
             lo = m.num_computed_tokens(rid)
             hi = rng.randrange(lo, len(toks) + 1)
-            for p in range(lo, hi):  # the step function writes these slots
-                slot = m.slot_mapping(rid, p, p + 1)[0]
-                page = slot // ps
-                holders = sum(1 for other in live if page in m.block_table(other))
-                assert holders == 1, "a write lands in a page that another request holds"
-                written[slot] = tuple(toks[:p + 1])
+            for g, spec in enumerate(groups):
+                for p in range(lo, hi):  # the step function writes these slots
+                    slot = m.slot_mapping(rid, p, p + 1, group=g)[0]
+                    page = slot // ps
+                    holders = sum(1 for other in live if page in m.block_table(other, g))
+                    assert holders == 1, "a write lands in a page that another request holds"
+                    written[g][slot] = tuple(toks[:p + 1])
+                if spec.kind == "window" and hi > lo:   # and every key that the portion's queries read is in place
+                    for p in range(max(0, lo - spec.window + 1), lo):
+                        slot = m.slot_mapping(rid, p, p + 1, group=g)[0]
+                        assert written[g].get(slot) == tuple(toks[:p + 1])
             m.mark_computed(rid, hi)
             if hi == len(toks) and rng.random() < 0.5:
                 m.free(rid)
                 del live[rid]
         m.check_invariants()
+    assert hits > 40
 
 
 def test_reserving_ahead_takes_pages_now_and_appends_use_them():

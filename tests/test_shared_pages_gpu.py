@@ -128,3 +128,136 @@ def test_live_requests_on_the_same_prefix_pages(name, page, dtype):
     s.step([], end=["a", "b", "c"])
     mgr.reset_prefix_cache()
     assert mgr.stats().used_pages == 0 and mgr.stats().free_pages == mgr.stats().num_pages
+
+
+@pytest.mark.parametrize("dtype,page,window", [("float32", 4, 10), ("bfloat16", 16, 24)])
+def test_a_toy_model_of_three_cache_groups_is_served_a_prefix_from_all_of_them(dtype, page, window):
+    """A toy architecture defined here whose three attention layers form three cache groups: every
+    key, a window of keys, every key with other head sizes. Its requests are served a prefix that
+    an earlier request left behind, from all three groups at once (the window group gives only the
+    pages that the first computed token still reaches; the table starts with released entries);
+    they step in portions and token by token beside each other against a plain 64-bit model of the
+    toy, written below with the plain implementation's parts and a band mask of its own. The pool
+    has no page to spare while the two run, so the groups that keep every key lose the rest of the
+    prefix, and a later request is served the shorter run that all three can still give."""
+    import math
+    import tempfile
+
+    import plain_llama as P
+    from dli_amd.cache import RELEASED
+    from dli_amd.config import register_architecture, unregister_architecture
+    from dli_amd.engine.core import build_core
+    from dli_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from dli_amd.trace import TraceSession
+    from dli_amd.weights import load_model, write_random_model
+
+    h, inter, vocab, eps, theta = 48, 80, 53, 1e-5, 1000.0
+    shapes = [dict(num_heads=3, num_kv_heads=1, head_dim=16, window=0),
+              dict(num_heads=3, num_kv_heads=1, head_dim=16, window=window),
+              dict(num_heads=2, num_kv_heads=2, head_dim=32, window=0)]
+
+    def build(cfg):
+        norm = dict(width=h, eps=eps)
+        layers = []
+        for i, shape in enumerate(shapes):
+            p = f"layers.{i}."
+            pos = PartSpec("rotary", dict(dim=shape["head_dim"], theta=theta))
+            layers.append(LayerSpec(PartSpec("pre_norm"), {
+                "mixer_norm": ("norm", PartSpec("rms_norm", norm, p + "n1.")),
+                "mixer": ("mixer", PartSpec("gqa_attention", dict(shape, hidden_size=h, position=pos), p + "attn.")),
+                "feed_forward_norm": ("norm", PartSpec("rms_norm", norm, p + "n2.")),
+                "feed_forward": ("feed_forward", PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=inter),
+                                                          p + "mlp."))}))
+        return ModelSpec(
+            architecture="ToyThreeGroupsForCausalLM", vocab_size=vocab, hidden_size=h,
+            embedding=PartSpec("token_embedding", dict(vocab_size=vocab, hidden_size=h), "embed."),
+            layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(3)),
+            final_norm=PartSpec("rms_norm", norm, "norm."),
+            head=PartSpec("linear_head", dict(vocab_size=vocab, hidden_size=h, tied=True), "head."))
+
+    def banded_attention(x, w, prefix, shape):
+        """Projections, rotation, softmax over the keys j with i - window < j <= i, output projection."""
+        n, nh, nkv, d = x.shape[0], shape["num_heads"], shape["num_kv_heads"], shape["head_dim"]
+        cos, sin = P.rope_cos_sin(P.inverse_frequencies({"rope_type": "default", "theta": theta}, d),
+                                  torch.arange(n), torch.float64)
+        q = P.apply_rope(P.linear(x, w[prefix + "q_proj.weight"]).view(n, nh, d).transpose(0, 1), cos, sin)
+        k = P.apply_rope(P.linear(x, w[prefix + "k_proj.weight"]).view(n, nkv, d).transpose(0, 1), cos, sin)
+        v = P.linear(x, w[prefix + "v_proj.weight"]).view(n, nkv, d).transpose(0, 1)
+        i, j = torch.arange(n)[:, None], torch.arange(n)[None, :]
+        seen = (j <= i) & ((j > i - shape["window"]) if shape["window"] else (j >= 0))
+        out = torch.empty_like(q)
+        for head in range(nh):
+            scores = (q[head] @ k[head // (nh // nkv)].T) / math.sqrt(d)
+            out[head] = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1) @ v[head // (nh // nkv)]
+        return P.linear(out.transpose(0, 1).reshape(n, nh * d), w[prefix + "o_proj.weight"])
+
+    def plain(w, tokens):
+        x = w["embed.weight"][torch.tensor(tokens)]
+        for i, shape in enumerate(shapes):
+            p = f"layers.{i}."
+            x = x + banded_attention(P.rms_norm(x, w[p + "n1.weight"], eps), w, p + "attn.", shape)
+            x = x + P.swiglu_mlp(P.rms_norm(x, w[p + "n2.weight"], eps), w, p + "mlp.")
+        return P.linear(P.rms_norm(x, w["norm.weight"], eps), w["embed.weight"])
+
+    register_architecture("ToyThreeGroupsForCausalLM", dict, build)
+    try:
+        with tempfile.TemporaryDirectory() as tmp:
+            folder = write_random_model(tmp, {"architectures": ["ToyThreeGroupsForCausalLM"]}, seed=21, std=0.15,
+                                        norm_jitter=0.1)
+            weights = {k: v.double() for k, v in P.load_folder(folder)[1].items()}
+            rng = torch.Generator().manual_seed(5)
+            rand = lambda n: torch.randint(0, vocab, (n,), generator=rng).tolist()
+            prefix = rand(5 * page + 3)
+            toks = {"a": prefix[:4 * page] + rand(21), "b": prefix[:3 * page] + rand(14), "c": prefix + rand(9)}
+            ref = {rid: plain(weights, t) for rid, t in toks.items()}
+            # as many pages as the two live requests need together, three of them shared: whatever
+            # else the index holds has to go while they run
+            pages = -(-len(toks["a"]) // page) + -(-len(toks["b"]) // page) - 3
+            core = build_core(load_model(folder, dtype=dtype), num_pages=pages, page_size=page, max_seqs=4, watermark=0.0)
+            mgr = core.manager
+            assert mgr.prefix_caching and [g.kind for g in mgr.groups] == ["full", "window", "full"]
+            core.step.enable_decode_graphs(4, pages * page)
+            s = TraceSession(core)
+            got = s.step([{"id": "w", "tokens": prefix, "want": [len(prefix) - 1]}], end=["w"])
+            check(got, plain(weights, prefix)[-1:], dtype, "three groups, the prefix")
+            fed = {}
+
+            def run(plan):
+                entries, want = [], []
+                for rid, n in plan:
+                    lo = fed.get(rid, 0)
+                    start = shared[rid] if rid not in fed else lo      # a new request is fed from its first token
+                    hi = min(len(toks[rid]), start + n)
+                    entries.append({"id": rid, "tokens": toks[rid][lo:hi], "want": list(range(start - lo, hi - lo))})
+                    want.append(ref[rid][start:hi])
+                    fed[rid] = hi
+                check(s.step(entries), torch.cat(want), dtype, f"three groups, {plan} up to {fed}")
+                mgr.check_invariants()
+
+            shared = {"a": 4 * page, "b": 3 * page}
+            run([("a", 6)])
+            first = max(0, 4 * page - window + 1) // page       # the window at a's first computed token
+            assert first > 0
+            assert mgr.block_table("a", 1)[:first] == (RELEASED,) * first and RELEASED not in mgr.block_table("a", 0)
+            run([("a", 3), ("b", 5)])
+            assert mgr.stats().prompt_tokens_hit == 7 * page
+            for g in (0, 2):
+                assert mgr.block_table("a", g)[:3] == mgr.block_table("b", g)[:3]
+            run([("b", 2), ("a", 5)])
+            while fed["a"] < len(toks["a"]) or fed["b"] < len(toks["b"]):
+                run([(rid, 1) for rid in ("a", "b") if fed[rid] < len(toks[rid])])
+            if dtype == "bfloat16":
+                assert core.step.graphs.replays > 0
+            assert mgr.stats().window_pages_released > 0
+            s.step([], end=["a", "b"])
+            # the whole prefix again: what the pools still hold of it decides how much is served
+            served = -(-len(toks["c"]) // page) - mgr.pages_needed_for_prompt(toks["c"])
+            assert mgr.pools[0].evictions > 0 and served == 4
+            shared["c"] = served * page
+            run([("c", 4)])
+            run([("c", 100)])
+            s.step([], end=["c"])
+            mgr.reset_prefix_cache()
+            assert mgr.stats().used_pages == 0 and mgr.stats().free_pages == mgr.stats().num_pages
+    finally:
+        unregister_architecture("ToyThreeGroupsForCausalLM")
