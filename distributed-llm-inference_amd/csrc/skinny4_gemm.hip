@@ -50,7 +50,7 @@ __device__ __forceinline__ float4v mfma4(short4v a, short4v b, float4v c) {
   return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
 }
 
-template <int KS, int FQ, int MG, int EPI, bool NORM, bool XL>
+template <int KS, int FQ, int MG, int EPI, bool NORM, bool XL, int DEPTH>
 __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
     const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ ssq_in, int ssq_parts,
     const float* __restrict__ norm_w, float eps, const bf16_t* __restrict__ w,
@@ -147,7 +147,10 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
   // DEPTH chunks are on their way at a time, each in registers of its own: the loop is written
   // out for all of them, so that no chunk is copied (a copy waits for its loads) and each is
   // waited for only when its turn has come.
-  constexpr int DEPTH = 4;  // (2 is as fast, 3 and 8 are slower: 11.1, 11.8 and 12.7 us for down at the 1B sizes, 8 rows)
+  // (4 or 2, as fast as each other where a wave's chunks are a multiple of four: the launch takes 2
+  // where they are not, since a wave's turns are a multiple of DEPTH; 3 and 8 are slower: 11.1,
+  // 11.8 and 12.7 us for down at the 1B sizes, 8 rows)
+  static_assert(DEPTH == 2 || DEPTH == 4, "chunks on their way at a time");
   Stage st[DEPTH];
   auto fetch_first = [&]() __attribute__((always_inline)) {
 #pragma unroll
@@ -300,7 +303,8 @@ __global__ __launch_bounds__(KS * 64) void skinny4_kernel(
       }
     }
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) multiply(st[d], c + d);  // the last group (turns past the end add zeros)
+    for (int d = 0; d < DEPTH; ++d)
+      if (c + d < c1) multiply(st[d], c + d);  // the last group (what was loaded past the end is not waited for)
   }
 
   // blocks l/4 that differ in their upper two bits are added by lane swaps, the remaining four
@@ -416,14 +420,22 @@ static void launch4(S4_PARAMS) {
   // tiles: staging costs a workgroup a barrier and a trip to memory before its first product, which
   // pays when each compute unit works through several workgroups, and does not for a short kernel.
   const int64_t x_lds = (int64_t)M * ((K + 127) / 128 * 128 + 32) * 2;
-  if (x_lds <= 64 * 1024 && tiles >= 4 * dli_compute_units())
-    skinny4_kernel<KS, FQ, MG, EPI, NORM, true><<<tiles, KS * 64, (size_t)x_lds, stream>>>(
-        (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
-        out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
-  else
-    skinny4_kernel<KS, FQ, MG, EPI, NORM, false><<<tiles, KS * 64, 0, stream>>>(
-        (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias,
-        out, ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset);
+  const bool staged = x_lds <= 64 * 1024 && tiles >= 4 * dli_compute_units();
+  // A wave walks its chunks of 128 k in groups of DEPTH turns: four at a time where every wave's
+  // share is a multiple of four, else two (rows of 2,560 or 3,072 k on four waves are five or six
+  // chunks a wave: eight turns in groups of four, six in groups of two; the sums are the same
+  // whichever way, each wave adds its chunks in their order).
+  const int chunks = (K + 127) / 128;
+  const bool by_four = chunks % (4 * KS) == 0;
+#define S4_LAUNCH(XL_, DEPTH_)                                                                              \
+  skinny4_kernel<KS, FQ, MG, EPI, NORM, XL_, DEPTH_><<<tiles, KS * 64, XL_ ? (size_t)x_lds : 0, stream>>>( \
+      (const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, (const bf16_t*)bias, out,    \
+      ldo, (bf16_t*)stream_buf, lds_, ssq_out, M, N, K, up_offset)
+  if (staged && by_four) S4_LAUNCH(true, 4);
+  else if (staged) S4_LAUNCH(true, 2);
+  else if (by_four) S4_LAUNCH(false, 4);
+  else S4_LAUNCH(false, 2);
+#undef S4_LAUNCH
 }
 
 template <int KS, int FQ, int EPI, bool NORM>
