@@ -460,6 +460,30 @@ def test_a_graph_of_more_than_64_rows_cuts_the_keys_as_its_mixer_planned(monkeyp
     assert seen and all(rows == 80 and nd == 80 and splits == min(planned) for rows, nd, splits in seen), seen
 
 
+def test_a_recorded_step_is_planned_for_its_requests_and_not_for_the_padded_rows():
+    """17 requests decode on a graph of 32 rows. What the mixers plan for the recording (into how
+    many runs the attention cuts a request's keys) is asked for 17 requests: the padded rows bring
+    no work, and a plan for 32 would leave compute units idle."""
+    from dli_amd.engine.core import build_core
+    from dli_amd.trace import TraceSession
+
+    name, count, n = "B", 17, 2060
+    toks = prompts(name, [n + 2] * count, seed=300)
+    core = build_core(model_folder(name), num_pages=count * (-(-(n + 2) // 16)) + 4, page_size=16, max_seqs=32,
+                      dtype="bfloat16", enable_prefix_caching=False, watermark=0.0)
+    core.step.enable_decode_graphs(32, n + 4)
+    s = TraceSession(core)
+    for r in range(count):
+        s.step([{"id": r, "tokens": toks[r][:n], "want": []}])
+    out = s.step([{"id": r, "tokens": [toks[r][n]], "want": [0]} for r in range(count)])
+    assert out.shape[0] == count and torch.isfinite(out).all()
+    (key,) = core.step.graphs.captured
+    owners = core.step.plan_owners
+    assert key[0] == 32 and owners
+    assert key[1] == tuple(part.decode_plan(count, n + 1) for part in owners)
+    assert key[1] != tuple(part.decode_plan(32, n + 1) for part in owners), "the test's sizes no longer tell the two apart"
+
+
 def test_trace_run_program(tmp_path):
     """bin/trace_run as a user runs it: steps on standard input, `done` lines, <step>.f32 files."""
     import json
