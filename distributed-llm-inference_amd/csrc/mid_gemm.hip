@@ -1,5 +1,8 @@
 // Matrix product for a decode step of 17 to 64 rows (it takes 1 to 64):
 //   y[m][n] = sum_k xhat[m][k] * w[n][k]
+// k is walked in blocks of 128; where k is no multiple of 128 the last block is part empty: the
+// activations past k count as zeros (so what the weights hold there does not matter, as long as
+// it is finite: row by row it is the next row's start, in tile order the copy's zero filling).
 // With this many rows the activations are no longer small beside the weights: a workgroup that
 // owns few features and reads every row for them moves more activation bytes than weight bytes.
 // So the activations of a block of 128 k are brought into LDS once per workgroup (normalised on
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   const int tile = blockIdx.x * NW + nw;
   const bool owns = tile < tiles;
   const int split = blockIdx.y;
-  const int nblk = K / 128;
+  const int nblk = (K + 127) / 128;
   const int b0 = (int)((int64_t)nblk * split / p.splits), b1 = (int)((int64_t)nblk * (split + 1) / p.splits);
   const int cnt = b1 - b0;
   const int steps = (cnt + KW - 1) / KW;       // the same for every wave: all keep the barriers
@@ -110,7 +113,8 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   // is sent past the end, where it returns zeros and costs no memory traffic. So every step
   // issues the same loads, the number of loads on their way is known at every wait, and a step
   // waits for its own block only.
-  const unsigned w_bytes = (unsigned)((int64_t)p.w_rows * K * 2);
+  const int KP = nblk * 128;           // a row of the tile-ordered copy: whole blocks
+  const unsigned w_bytes = (unsigned)((int64_t)p.w_rows * (p.tiled ? KP : K) * 2);
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc((void*)p.w, 0, w_bytes, 0x00020000);
   const unsigned x_bytes = (unsigned)(((int64_t)(M - 1) * p.ldx + K) * 2);
   const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, x_bytes, 0x00020000);
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   for (int a = 0; a < NA; ++a) {
     const int tl = min(tile, tiles - 1);
     if (p.tiled) {
-      wbase[a] = (unsigned)(((int64_t)(tl + a * (p.up_offset / 16)) * 16 * K + lane * 8) * 2);
+      wbase[a] = (unsigned)(((int64_t)(tl + a * (p.up_offset / 16)) * 16 * KP + lane * 8) * 2);
     } else {
       const int n = min(tl * 16 + col, N - 1) + a * p.up_offset;
       wbase[a] = (unsigned)(((int64_t)n * K + grp * 32) * 2);
@@ -157,12 +161,15 @@ __global__ __launch_bounds__(NW * KW * 64) void mid_gemm_kernel(MidArgs p) {
   auto fetch_x = [&](Staged& st, int b, bool wanted) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < PP; ++i) {
-      const unsigned at = wanted && prow[i] < M ? (unsigned)(((int64_t)prow[i] * p.ldx + b * 128 + pk[i]) * 2) : x_bytes;
+      const unsigned at = wanted && prow[i] < M && b * 128 + pk[i] < K
+                              ? (unsigned)(((int64_t)prow[i] * p.ldx + b * 128 + pk[i]) * 2) : x_bytes;
       st.v[i] = as_bf16x8(__builtin_amdgcn_raw_buffer_load_b128(xres, (int)at, 0, 0));
     }
-    // (without a norm the same two loads, of anything: no load hangs on a condition)
-    st.nw0 = *reinterpret_cast<const float4v*>(nw_at + b * 128 + pk[0]);
-    st.nw1 = *reinterpret_cast<const float4v*>(nw_at + b * 128 + pk[0] + 4);
+    // (without a norm the same two loads, of anything: no load hangs on a condition; past k the
+    // last eight weights, for activations that are zero)
+    const int nk = min(b * 128 + pk[0], K - 8);
+    st.nw0 = *reinterpret_cast<const float4v*>(nw_at + nk);
+    st.nw1 = *reinterpret_cast<const float4v*>(nw_at + nk + 4);
   };
   auto stash_x = [&](const Staged& st, int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -527,8 +534,9 @@ int launch_mid_rows(int nw, int kw, const MidArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-// x [M, K] bfloat16 (row stride ldx), M <= 64, K % 128 == 0. w: [N (+ up part), K] row by row, or
-// in tile order if `tiled` (then N % 16 == 0 and up_offset % 16 == 0). norm_w == nullptr: no norm.
+// x [M, K] bfloat16 (row stride ldx), M <= 64, K % 8 == 0. w: [N (+ up part), K] row by row, or
+// in tile order if `tiled` (then N % 16 == 0 and up_offset % 16 == 0, and a row of the copy is K
+// rounded up to whole blocks of 128, zeros past K). norm_w == nullptr: no norm.
 // epilogue 0: out is float32 [splits][M][N] (ldo == N); 1 (gated) and 2 (store): out is bfloat16
 // [M][N] with row stride ldo, one split. waves: feature tiles per workgroup; kwaves: waves that
 // share a feature tile and split the workgroup's k (the built pairs are listed in launch_mid).
@@ -537,8 +545,8 @@ extern "C" int dli_mid_gemm(const void* x, int64_t ldx, const float* ssq_in, int
                             void* out, int64_t ldo, int M, int N, int K, int up_offset, int epilogue,
                             int splits, int waves, int kwaves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return DLI_OK;
-  if (M > 64 || K <= 0 || K % 128 != 0 || ldx % 8 != 0 || ldx < K || out == nullptr || epilogue < 0 ||
-      epilogue > 2 || splits < 1 || splits > K / 128 || waves < 1 || kwaves < 1 ||
+  if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0 || ldx < K || out == nullptr || epilogue < 0 ||
+      epilogue > 2 || splits < 1 || splits > (K + 127) / 128 || waves < 1 || kwaves < 1 ||
       (epilogue != MID_PARTIAL && splits != 1) || (epilogue == MID_PARTIAL && (ldo != N || bias != nullptr)) ||
       (epilogue != MID_PARTIAL && (ldo < N || ldo % 4 != 0)) ||
       (norm_w != nullptr && (ssq_in == nullptr || ssq_parts <= 0)) ||
@@ -547,7 +555,7 @@ extern "C" int dli_mid_gemm(const void* x, int64_t ldx, const float* ssq_in, int
     return DLI_ERR_ARGUMENT;
   // the kernel addresses the matrix and the rows with 32-bit byte offsets
   const int64_t w_rows = epilogue == MID_SWIGLU ? (int64_t)up_offset + N : N;
-  if (w_rows * K * 2 >= ((int64_t)1 << 32) - 4096 || ((int64_t)(M - 1) * ldx + K) * 2 >= ((int64_t)1 << 31))
+  if (w_rows * ((K + 127) / 128 * 128) * 2 >= ((int64_t)1 << 32) - 4096 || ((int64_t)(M - 1) * ldx + K) * 2 >= ((int64_t)1 << 31))
     return DLI_ERR_ARGUMENT;
   const MidArgs a{(const bf16_t*)x, ldx, ssq_in, ssq_parts, norm_w, eps, (const bf16_t*)w, tiled, (int)w_rows,
                   (const bf16_t*)bias, out, ldo, M, N, K, up_offset, splits};

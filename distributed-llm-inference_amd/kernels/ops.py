@@ -369,15 +369,26 @@ def tiled_weights_help(w_rows: int, k: int, epilogue: int, device: torch.device)
     return skinny_gemm_plan(8, n, k, epilogue, device)[0] == "tiles16"
 
 
-def tile_weights(w: torch.Tensor) -> torch.Tensor:
+def tile_weights(w: torch.Tensor, whole_blocks: bool = True) -> torch.Tensor:
     """``w [n, k]`` (bfloat16, n % 16 == 0, k % 128 == 0) in the order in which the 16x16-tile
     kernel's lanes read it: ``t[tile][block][q][g][c][8] = w[16*tile + c][128*block + 32*g + 8*q + ...]``,
-    so that each load of a wave is 1 KB of consecutive memory. Same number of elements, flat."""
+    so that each load of a wave is 1 KB of consecutive memory. Same number of elements, flat.
+    ``whole_blocks=False`` takes any k % 8 == 0 and fills the last block of 128 with zeros (the copy
+    then has ``n * padded_k(k)`` elements; only :func:`mid_gemm` reads such a copy)."""
     _dense(w, "w", torch.bfloat16, 2)
     n, k = w.shape
+    if k % 128 != 0 and not whole_blocks:
+        _require(k % 8 == 0, "tile order needs k % 8 == 0")
+        w = torch.nn.functional.pad(w, (0, padded_k(k) - k))
+        k = w.shape[1]
     _require(n % 16 == 0 and k % 128 == 0, "tile order needs n % 16 == 0 and k % 128 == 0")
     t = w.view(n // 16, 16, k // 128, 4, 4, 8)       # tile, c, block, g, q, 8
     return t.permute(0, 2, 4, 3, 1, 5).contiguous().view(-1)
+
+
+def padded_k(k: int) -> int:
+    """``k`` rounded up to whole blocks of 128."""
+    return -(-k // 128) * 128
 
 
 _compute_units: dict[int, int] = {}
@@ -464,6 +475,8 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, out: Optiona
     if bias is not None:
         _dense(bias, "bias", torch.bfloat16, 1)
         _require(bias.shape[0] == w.shape[0], "bias length differs from rows of w")
+    if k % 128 != 0:
+        w_tiled = None   # a copy in whole blocks with a zero-filled last one: the 17-to-64-row kernel's alone
     if shape is not None:
         _require(shape in (0, 1, 2, 3, 4), "shape must be 0..4")
         kernel, a, n_parts = "tiles16", shape, -(-n // 16)
@@ -636,7 +649,7 @@ MID_ROWS = 64
 
 def mid_gemm_supports(rows: int, k: int, dtype: torch.dtype) -> bool:
     """Whether the product kernel for decode steps of up to 64 rows takes this shape."""
-    return dtype == torch.bfloat16 and 0 < rows <= MID_ROWS and k > 0 and k % 128 == 0
+    return dtype == torch.bfloat16 and 0 < rows <= MID_ROWS and k > 0 and k % 8 == 0
 
 
 MID_SHAPES = ((4, 1), (4, 2))              # (waves, kwaves) that are built for the plain products
@@ -651,7 +664,7 @@ def mid_gemm_plan(n: int, k: int, epilogue: int, units: int, rows: int = 64) -> 
     split: its epilogue needs whole sums). These launches last a few trips to memory, so the plan
     aims at one workgroup on every compute unit with eight to sixteen waves, each with few blocks
     of 128 k to fetch."""
-    tiles, blocks = -(-n // 16), k // 128
+    tiles, blocks = -(-n // 16), -(-k // 128)
     if epilogue == MID_SWIGLU:
         # (two against four k-waves a tile, cold weights: 21.1 and 21.4 us at 32 rows, 23.4 and 23.0
         # at 48, 28.7 and 26.1 at 64 at the 1B sizes; with k of 3072 24.8 and 24.5, 29.9 and 27.2, 37.4
@@ -670,9 +683,10 @@ def mid_gemm_plan(n: int, k: int, epilogue: int, units: int, rows: int = 64) -> 
 
 def mid_tiles_help(w_rows: int, k: int, epilogue: int) -> bool:
     """Whether decode steps of 17 to 64 rows would read a copy of a ``[w_rows, k]`` weight in tile
-    order (:func:`tile_weights`): the layer products do, where the sizes tile."""
+    order (:func:`tile_weights`, of whole blocks of k, zero-filled): the layer products do, where
+    the features tile."""
     n = w_rows // 2 if epilogue == SKINNY_SWIGLU else w_rows
-    return epilogue in (SKINNY_STORE, SKINNY_SWIGLU, SKINNY_RESIDUAL) and k % 128 == 0 and n % 16 == 0 and n > 0
+    return epilogue in (SKINNY_STORE, SKINNY_SWIGLU, SKINNY_RESIDUAL) and k % 8 == 0 and n % 16 == 0 and n > 0
 
 
 def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = False, n: Optional[int] = None,
@@ -680,22 +694,24 @@ def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = F
              norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None,
              splits: Optional[int] = None, waves: Optional[int] = None,
              kwaves: Optional[int] = None) -> torch.Tensor:
-    """``y = xhat @ w.T`` for at most 64 rows of bfloat16 ``x [rows, k]``, k a multiple of 128.
+    """``y = xhat @ w.T`` for at most 64 rows of bfloat16 ``x [rows, k]``, k a multiple of 8.
 
     ``w`` is ``[n, k]`` (``[2n, k]``, gate rows then up rows, for ``MID_SWIGLU``), or the same in
-    tile order (:func:`tile_weights`, flat) with ``tiled`` and ``n`` given. ``norm_w``/``eps``/
+    tile order (:func:`tile_weights`, flat; of whole blocks, zero-filled where k is no multiple
+    of 128) with ``tiled`` and ``n`` given. ``norm_w``/``eps``/
     ``ssq_in [parts, rows]``: xhat is the RMSNorm of x. ``MID_PARTIAL`` returns float32
     ``[splits, rows, n]`` whose sum over the splits, in their order, is the product (no bias; the
     finishing kernels add them up); ``MID_STORE`` and ``MID_SWIGLU`` return bfloat16 ``[rows, n]``.
     """
     _rows(x, "x", torch.bfloat16)
     m, k = x.shape
-    _require(mid_gemm_supports(m, k, x.dtype), f"this product takes 1..64 rows and k % 128 == 0, not {m} x {k}")
+    _require(mid_gemm_supports(m, k, x.dtype), f"this product takes 1..64 rows and k % 8 == 0, not {m} x {k}")
     _require(x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
     sets = 2 if epilogue == MID_SWIGLU else 1
     if tiled:
         _dense(w, "w", torch.bfloat16, 1)
-        _require(n is not None and n % 16 == 0 and w.numel() == sets * n * k, "tiled weights need n % 16 == 0 features of depth k")
+        _require(n is not None and n % 16 == 0 and w.numel() == sets * n * padded_k(k),
+                 "tiled weights need n % 16 == 0 features of depth k, in whole blocks of 128")
     else:
         _dense(w, "w", torch.bfloat16, 2)
         _require(w.shape[1] == k and w.shape[0] % sets == 0, "x and w differ in inner size")
@@ -706,7 +722,7 @@ def mid_gemm(x: torch.Tensor, w: torch.Tensor, *, epilogue: int, tiled: bool = F
     kwaves = plan_kwaves if kwaves is None else kwaves
     splits = plan_splits if splits is None else splits
     built = MID_SHAPES_GATED if epilogue == MID_SWIGLU else MID_SHAPES
-    _require((waves, kwaves) in built and 1 <= splits <= k // 128,
+    _require((waves, kwaves) in built and 1 <= splits <= -(-k // 128),
              f"(waves, kwaves) must be one of {built}, splits 1..k/128")
     if epilogue == MID_PARTIAL:
         _require(bias is None and n % 4 == 0, "partial products take no bias, n % 4 == 0")
@@ -886,7 +902,7 @@ def tile_weights_qkv_rope(w: torch.Tensor, q_heads: int, kv_heads: int, head_dim
     _dense(w, "w", torch.bfloat16, 2)
     _require(w.shape[0] == (q_heads + 2 * kv_heads) * head_dim, "w must hold the q, k and v heads")
     order = qkv_rope_feature_order(q_heads, kv_heads, head_dim).to(w.device)
-    return tile_weights(w[order].contiguous())
+    return tile_weights(w[order].contiguous(), whole_blocks=False)
 
 
 def skinny_gemm_qkv_rope(x: torch.Tensor, w_tiled: torch.Tensor, q_out: torch.Tensor, angles: torch.Tensor,

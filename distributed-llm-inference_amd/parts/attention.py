@@ -210,7 +210,7 @@ class GQAttention(Mixer):
             self._forward_stream_mid(stream, norm, ctx, cache, grp, following)
             return
         qkv = self.rt.empty(n, (nh + 2 * nkv) * d)
-        if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS:
+        if self.w_qkv_rope is not None and n in ROPE_IN_PRODUCT_ROWS and self.hidden_size % 128 == 0:
             # product, rotation and cache write in one kernel; only q comes back
             angles = self.position.step_angles(ctx, qkv.dtype)
             ops.skinny_gemm_qkv_rope(stream.x, self.w_qkv_rope, qkv, angles, grp.slots, cache.k_pages, cache.v_pages,

@@ -50,7 +50,8 @@ def decode_copy(rt: Runtime, weight: Optional[torch.Tensor], epilogue: int) -> O
     if not (ops.tiled_weights_help(weight.shape[0], weight.shape[1], epilogue, weight.device)
             or ops.mid_tiles_help(weight.shape[0], weight.shape[1], epilogue)):
         return None
-    return ops.tile_weights(weight)
+    # (rows that are no whole blocks of 128: zero-filled to whole blocks, for the 17-to-64-row kernel alone)
+    return ops.tile_weights(weight, whole_blocks=False)
 
 
 # From this many rows on, the kernel that makes the residual sum also applies the norm that follows
