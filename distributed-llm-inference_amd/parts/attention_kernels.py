@@ -17,8 +17,11 @@ from ..kernels import ops
 # From decode steps at batch 1 to 64: two workgroups per compute unit, and at 4K keys at most 16
 # runs, were ahead of more of either (the partial results cost a merge that grows with them); a
 # request with 32K keys did better with 64 runs than with 16, so the limit grows with the keys.
+# Runs of at least 256 keys: with 128, steps at contexts of 512 to 2,048 keys were 0.5 to 2% slower
+# at the 1B and 3B sizes and 6% at four kv heads (8 requests of 2,048 keys: 16 runs of 128 keys
+# against 8 of 256); with 512 they were 1 to 3% slower again.
 WORKGROUPS_PER_UNIT = 2
-MIN_KEYS_PER_SPLIT = 128
+MIN_KEYS_PER_SPLIT = 256
 FEW_SPLITS = 16          # the limit up to 8K keys
 KEYS_PER_EXTRA_SPLIT = 512
 MAX_SPLITS = 64
@@ -26,7 +29,7 @@ MAX_SPLITS = 64
 
 def choose_splits(requests: int, kv_head_tiles: int, max_keys: int, units: int = 256) -> int:
     """How many runs to cut each request's keys into for the decode kernel: enough workgroups
-    to give every compute unit two workgroups, never runs under 128 keys (reference's rule of the
+    to give every compute unit two workgroups, never runs under 256 keys (reference's rule of the
     same kind: src/dli/model/paged_attention.py:63-74). ``units``: the device's compute units."""
     programs = max(1, requests * kv_head_tiles)
     want = -(-WORKGROUPS_PER_UNIT * units // programs)

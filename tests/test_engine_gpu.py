@@ -467,7 +467,7 @@ def test_a_recorded_step_is_planned_for_its_requests_and_not_for_the_padded_rows
     from dli_amd.engine.core import build_core
     from dli_amd.trace import TraceSession
 
-    name, count, n = "B", 17, 2060
+    name, count, n = "B", 17, 4100
     toks = prompts(name, [n + 2] * count, seed=300)
     core = build_core(model_folder(name), num_pages=count * (-(-(n + 2) // 16)) + 4, page_size=16, max_seqs=32,
                       dtype="bfloat16", enable_prefix_caching=False, watermark=0.0)

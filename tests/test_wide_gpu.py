@@ -112,7 +112,7 @@ def test_one_and_two_requests_decode_without_a_merge_kernel(count, monkeypatch):
     from dli_amd.trace import TraceSession
 
     rng = random.Random(11 + count)
-    lens = [300, 270][:count]
+    lens = [600, 540][:count]
     steps = 6
     toks = [[rng.randrange(32003) for _ in range(n + steps)] for n in lens]
     calls = []
@@ -121,7 +121,7 @@ def test_one_and_two_requests_decode_without_a_merge_kernel(count, monkeypatch):
 
     def run(limit):
         monkeypatch.setattr(attention, "MERGE_IN_PRODUCT_ROWS", limit)
-        core = make_core("bfloat16", pages=48, graphs=count)
+        core = make_core("bfloat16", pages=80, graphs=count)
         s = TraceSession(core)
         s.step([{"id": r, "tokens": toks[r][:lens[r]], "want": []} for r in range(count)])
         outs = []
@@ -151,7 +151,7 @@ def test_decode_attention_merges_its_runs_of_keys_in_the_launch(monkeypatch):
     from dli_amd.trace import TraceSession
 
     rng = random.Random(23)
-    lens = [300, 270, 140, 17]
+    lens = [600, 540, 280, 17]
     steps = 6
     toks = [[rng.randrange(32003) for _ in range(n + steps)] for n in lens]
     seen = []
@@ -166,7 +166,7 @@ def test_decode_attention_merges_its_runs_of_keys_in_the_launch(monkeypatch):
     def run(self_merging):
         if not self_merging:
             monkeypatch.setattr(attention.GQAttention, "arrival_counters", lambda self, needed: None)
-        core = make_core("bfloat16", pages=64, graphs=4)
+        core = make_core("bfloat16", pages=100, graphs=4)
         s = TraceSession(core)
         s.step([{"id": r, "tokens": toks[r][:lens[r]], "want": []} for r in range(4)])
         outs = []
