@@ -94,6 +94,8 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     # Requests admitted first decode a token a step while the others still prefill; the prompts are
     # shortened by that many steps so that no request outgrows `context` while the clock runs.
     budget = engine.scheduler.config.max_num_batched_tokens
+    # (the engine has brought this down to what its runner can do: the 32-bit path decodes one token a step)
+    decode_steps = min(decode_steps, engine.scheduler.config.decode_steps)
     # An engine step may decode several tokens of every request (SchedulerConfig.decode_steps): the
     # clock runs over exactly `steps` decode steps of the model, cut into engine steps of 8, 4, 2 or 1
     # (the largest first), and the warm-up runs every such size once so that its graph exists.
