@@ -50,7 +50,13 @@ SMOLLM2_1_7B = {
     "head_dim": 64, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "rope_theta": 130000.0,
     "tie_word_embeddings": True, "hidden_act": "silu",
 }
-SHAPES = {"Llama-3.2-1B": LLAMA_3_2_1B, "Llama-3.2-3B": LLAMA_3_2_3B, "SmolLM2-1.7B": SMOLLM2_1_7B}
+# the small members of the family (widths that are no multiple of 128), for --shape
+SMOLLM2_135M = dict(SMOLLM2_1_7B, hidden_size=576, intermediate_size=1536, num_hidden_layers=30,
+                    num_attention_heads=9, num_key_value_heads=3, rope_theta=100000.0)
+SMOLLM2_360M = dict(SMOLLM2_1_7B, hidden_size=960, intermediate_size=2560, num_hidden_layers=32,
+                    num_attention_heads=15, num_key_value_heads=5, rope_theta=100000.0)
+SHAPES = {"Llama-3.2-1B": LLAMA_3_2_1B, "Llama-3.2-3B": LLAMA_3_2_3B, "SmolLM2-1.7B": SMOLLM2_1_7B,
+          "SmolLM2-360M": SMOLLM2_360M, "SmolLM2-135M": SMOLLM2_135M}
 
 
 def load_random_model(raw, dtype):
