@@ -31,6 +31,9 @@ from .batch import GroupView, StepContext, StepEntry
 from .table_rows import TableRows
 
 
+RECORD_AT = 3  # a shape is recorded when it is asked for the third time (or when no recorded shape can stand in)
+
+
 def _bucket(n: int) -> int:
     b = 1
     while b < n:
@@ -66,6 +69,7 @@ class DecodeGraphs:
         self.max_width = max(1, max_blocks_per_seq)
         self.n_groups = step_fn.manager.num_groups
         self.captured: dict[tuple, _Captured] = {}
+        self._asked: dict[tuple, int] = {}   # how often a shape that is not recorded has been asked for
         self.replays = 0
         self.enabled = self._supported()
 
@@ -188,6 +192,18 @@ class DecodeGraphs:
         plans = tuple(part.decode_plan(requests, max_kv) for part in self.step_fn.plan_owners)
         return (b, plans, width, sampled, steps)
 
+    def _stand_in(self, key: tuple, requests: int) -> Optional[tuple]:
+        """The recorded shape with the fewest rows (then the narrowest block table) that can run a
+        step of ``key``'s kind for ``requests`` requests: as many tokens a step, sampled alike,
+        rows and table width at least as large. What its parts planned was planned for another
+        batch: that costs speed, never a result."""
+        best = None
+        for other, cap in self.captured.items():
+            if other[3:] == key[3:] and other[0] >= requests and other[2] >= key[2]:
+                if best is None or (other[0], other[2]) < (best[0][0], best[0][2]):
+                    best = (other, cap)
+        return best
+
     def warm_up(self, batches: Sequence[int], max_len: int, *, sampled: bool = True,
                 steps: Sequence[int] = (1,)) -> int:
         """Capture now every graph that decode steps of ``batches`` requests with up to ``max_len``
@@ -229,10 +245,18 @@ class DecodeGraphs:
         if steps > 1 and not sampled:
             raise ValueError("several steps in a row need the sampling parameters")
         key = self._shape_key(n, max(e.start + steps for e in entries), sampled, steps)
-        b = key[0]
         cap = self.captured.get(key)
         if cap is None:
-            cap = self.captured[key] = self._capture(*key)
+            # A recording costs as much time as ten to thirty steps. A shape that has been asked for
+            # fewer than RECORD_AT times (the tail of a batch, whose requests end one by one) is
+            # served by a recorded shape of more rows or a wider block table where there is one.
+            self._asked[key] = self._asked.get(key, 0) + 1
+            stand_in = self._stand_in(key, n) if self._asked[key] < RECORD_AT else None
+            if stand_in is not None:
+                key, cap = stand_in
+            else:
+                cap = self.captured[key] = self._capture(*key)
+        b = key[0]
         v = cap.views
         if cap.staged is not None:
             # a caller that used the last logits without waiting for them (a copy on the stream,

@@ -484,6 +484,40 @@ def test_a_recorded_step_is_planned_for_its_requests_and_not_for_the_padded_rows
     assert key[1] != tuple(part.decode_plan(32, n + 1) for part in owners), "the test's sizes no longer tell the two apart"
 
 
+def test_a_shape_that_is_asked_for_rarely_is_served_by_a_recorded_shape_of_more_rows():
+    """Eight requests decode on a graph of eight rows; five of them end, and the three that go on
+    are served by that graph for the first two steps (a recording costs as much as many steps, and
+    the tail of a batch changes its shape every few steps) and by a recording of their own from
+    the third step on. The logits are the plain implementation's all along."""
+    from test_model_gpu import check, plain_logits
+    from dli_amd.engine.core import build_core
+    from dli_amd.trace import TraceSession
+
+    name, count, n = "B", 8, 40
+    toks = prompts(name, [n + 6] * count, seed=310)
+    core = build_core(model_folder(name), num_pages=count * 4 + 4, page_size=16, max_seqs=8, dtype="bfloat16",
+                      enable_prefix_caching=False, watermark=0.0)
+    core.step.enable_decode_graphs(8, 64)
+    graphs = core.step.graphs
+    s = TraceSession(core)
+    s.step([{"id": r, "tokens": toks[r][:n], "want": []} for r in range(count)])
+
+    def decode(rows, i, end=()):
+        out = s.step([{"id": r, "tokens": [toks[r][n + i]], "want": [0]} for r in rows], end=end)
+        check(out, torch.stack([plain_logits(name, toks[r])[n + i] for r in rows]), "bfloat16", f"step {i}, rows {rows}")
+
+    decode(range(8), 0, end=range(3, 8))
+    assert len(graphs.captured) == 1 and graphs.replays == 1
+    decode(range(3), 1)
+    decode(range(3), 2)
+    assert len(graphs.captured) == 1 and graphs.replays == 3, "the graph of eight rows stands in twice"
+    decode(range(3), 3)
+    assert len(graphs.captured) == 2 and graphs.replays == 4
+    assert sorted(k[0] for k in graphs.captured) == [4, 8]
+    decode(range(3), 4)
+    assert len(graphs.captured) == 2 and graphs.replays == 5
+
+
 def test_trace_run_program(tmp_path):
     """bin/trace_run as a user runs it: steps on standard input, `done` lines, <step>.f32 files."""
     import json
