@@ -104,9 +104,9 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     decode_steps = min(decode_steps, engine.scheduler.config.decode_steps)
     # An engine step may decode several tokens of every request (SchedulerConfig.decode_steps): the
     # clock runs over exactly `steps` decode steps of the model, cut into engine steps of 8, 4, 2 or 1
-    # (the largest first), and the warm-up runs every such size three times so that its graph exists
-    # (a shape is recorded when it is asked for the third time; before, a recorded shape of more
-    # rows stands in).
+    # (the largest first), and the warm-up runs every such size once so that its graph exists (a
+    # shape is recorded at once where no recorded shape of up to four times its rows can stand in:
+    # measure batches that lie further apart on one engine).
     def chunks_of(n):
         out = []
         while n > 0:
@@ -115,7 +115,7 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
         return out
 
     timed = chunks_of(steps)
-    warm_chunks = sorted(set(timed), reverse=True) * 3
+    warm_chunks = sorted(set(timed), reverse=True)
     while sum(warm_chunks) < warmup:
         warm_chunks.append(timed[0])
     warm, per = sum(warm_chunks), timed[0]

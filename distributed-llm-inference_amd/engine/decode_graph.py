@@ -31,7 +31,12 @@ from .batch import GroupView, StepContext, StepEntry
 from .table_rows import TableRows
 
 
-RECORD_AT = 3  # a shape is recorded when it is asked for the third time (or when no recorded shape can stand in)
+# A recording costs as much time as fifteen to thirty decode steps; a recorded shape of more rows that
+# stands in costs a tenth to a third of a step more. A shape is recorded once it has been asked for
+# RECORD_AFTER_STEPS decode steps, at once if nothing recorded can stand in, or if what can has more
+# than STAND_IN_ROWS times its rows.
+RECORD_AFTER_STEPS = 64
+STAND_IN_ROWS = 4
 
 
 def _bucket(n: int) -> int:
@@ -69,7 +74,7 @@ class DecodeGraphs:
         self.max_width = max(1, max_blocks_per_seq)
         self.n_groups = step_fn.manager.num_groups
         self.captured: dict[tuple, _Captured] = {}
-        self._asked: dict[tuple, int] = {}   # how often a shape that is not recorded has been asked for
+        self._asked: dict[tuple, int] = {}   # decode steps that a shape that is not recorded has been asked for
         self.replays = 0
         self.enabled = self._supported()
 
@@ -193,14 +198,18 @@ class DecodeGraphs:
         return (b, plans, width, sampled, steps)
 
     def _stand_in(self, key: tuple, requests: int) -> Optional[tuple]:
-        """The recorded shape with the fewest rows (then the narrowest block table) that can run a
-        step of ``key``'s kind for ``requests`` requests: as many tokens a step, sampled alike,
-        rows and table width at least as large. What its parts planned was planned for another
-        batch: that costs speed, never a result."""
+        """The recorded shape with the fewest rows (then with the same plans, then the narrowest
+        block table) that can run a step of ``key``'s kind for ``requests`` requests: as many
+        tokens a step, sampled alike, rows and table width at least as large. What its parts
+        planned may have been planned for another batch: that costs speed, never a result."""
+        def order(k):
+            return (k[0], k[1] != key[1], k[2])
+
         best = None
         for other, cap in self.captured.items():
-            if other[3:] == key[3:] and other[0] >= requests and other[2] >= key[2]:
-                if best is None or (other[0], other[2]) < (best[0][0], best[0][2]):
+            if (other[3:] == key[3:] and requests <= other[0] <= STAND_IN_ROWS * key[0]
+                    and other[2] >= key[2]):
+                if best is None or order(other) < order(best[0]):
                     best = (other, cap)
         return best
 
@@ -247,11 +256,10 @@ class DecodeGraphs:
         key = self._shape_key(n, max(e.start + steps for e in entries), sampled, steps)
         cap = self.captured.get(key)
         if cap is None:
-            # A recording costs as much time as ten to thirty steps. A shape that has been asked for
-            # fewer than RECORD_AT times (the tail of a batch, whose requests end one by one) is
-            # served by a recorded shape of more rows or a wider block table where there is one.
-            self._asked[key] = self._asked.get(key, 0) + 1
-            stand_in = self._stand_in(key, n) if self._asked[key] < RECORD_AT else None
+            # A shape that has been asked for little (the tail of a batch, whose requests end one
+            # by one) is served by a recorded shape of more rows or a wider block table.
+            self._asked[key] = self._asked.get(key, 0) + steps
+            stand_in = self._stand_in(key, n) if self._asked[key] < RECORD_AFTER_STEPS else None
             if stand_in is not None:
                 key, cap = stand_in
             else:

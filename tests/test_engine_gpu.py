@@ -484,17 +484,21 @@ def test_a_recorded_step_is_planned_for_its_requests_and_not_for_the_padded_rows
     assert key[1] != tuple(part.decode_plan(32, n + 1) for part in owners), "the test's sizes no longer tell the two apart"
 
 
-def test_a_shape_that_is_asked_for_rarely_is_served_by_a_recorded_shape_of_more_rows():
+def test_a_shape_that_is_asked_for_rarely_is_served_by_a_recorded_shape_of_more_rows(monkeypatch):
     """Eight requests decode on a graph of eight rows; five of them end, and the three that go on
-    are served by that graph for the first two steps (a recording costs as much as many steps, and
-    the tail of a batch changes its shape every few steps) and by a recording of their own from
-    the third step on. The logits are the plain implementation's all along."""
+    are served by that graph until they have asked for as many steps as a recording is taken to
+    be worth (three here; a recording costs as much as many steps, and the tail of a batch changes
+    its shape every few steps), then by a recording of their own. A graph of more than four times
+    the rows does not stand in. The logits are the plain implementation's all along."""
     from test_model_gpu import check, plain_logits
+    from dli_amd.engine import decode_graph
     from dli_amd.engine.core import build_core
     from dli_amd.trace import TraceSession
 
+    monkeypatch.setattr(decode_graph, "RECORD_AFTER_STEPS", 3)
+
     name, count, n = "B", 8, 40
-    toks = prompts(name, [n + 6] * count, seed=310)
+    toks = prompts(name, [n + 8] * count, seed=310)
     core = build_core(model_folder(name), num_pages=count * 4 + 4, page_size=16, max_seqs=8, dtype="bfloat16",
                       enable_prefix_caching=False, watermark=0.0)
     core.step.enable_decode_graphs(8, 64)
@@ -514,8 +518,14 @@ def test_a_shape_that_is_asked_for_rarely_is_served_by_a_recorded_shape_of_more_
     decode(range(3), 3)
     assert len(graphs.captured) == 2 and graphs.replays == 4
     assert sorted(k[0] for k in graphs.captured) == [4, 8]
-    decode(range(3), 4)
+    decode(range(3), 4, end=range(1, 3))
     assert len(graphs.captured) == 2 and graphs.replays == 5
+    decode(range(1), 5)
+    assert len(graphs.captured) == 2 and graphs.replays == 6, "the graph of four rows stands in for one request"
+    monkeypatch.setattr(decode_graph, "STAND_IN_ROWS", 2)
+    graphs._asked.clear()
+    decode(range(1), 6)
+    assert sorted(k[0] for k in graphs.captured) == [1, 4, 8], "four rows are more than twice one row"
 
 
 def test_trace_run_program(tmp_path):
