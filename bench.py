@@ -31,7 +31,13 @@ if str(ROOT) not in sys.path:
 HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-SLACK = 96  # decode steps that early requests may run before the timed ones
+SLACK = 96  # decode steps that early requests may run before the timed ones (at least)
+
+
+def slack_for(batch, context, budget):
+    """Decode steps that the requests admitted first may run while the others' prompts are still
+    computed ``budget`` tokens a step."""
+    return max(SLACK, -(-batch * context // budget) + 8)
 
 LLAMA_3_2_1B = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 128256, "hidden_size": 2048,
@@ -75,7 +81,7 @@ def load_random_model(raw, dtype):
 def engine_for(model, batch, context, block_size, budget, decode_steps=1, num_pages=None, prefix_caching=False):
     from dli_amd.engine import LLMEngine, SchedulerConfig
 
-    pages = num_pages or batch * (-(-(context + SLACK) // block_size) + 1) + 8
+    pages = num_pages or batch * (-(-(context + slack_for(batch, context, budget)) // block_size) + 1) + 8
     pages += pages // 64  # room for the share of the pool that admission keeps back (1%)
     engine = LLMEngine.for_model(
         model, num_blocks=pages, block_size=block_size, enable_prefix_caching=prefix_caching,
@@ -100,6 +106,7 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
     # Requests admitted first decode a token a step while the others still prefill; the prompts are
     # shortened by that many steps so that no request outgrows `context` while the clock runs.
     budget = engine.scheduler.config.max_num_batched_tokens
+    slack = slack_for(batch, context, budget)
     # (the engine has brought this down to what its runner can do: the 32-bit path decodes one token a step)
     decode_steps = min(decode_steps, engine.scheduler.config.decode_steps)
     # An engine step may decode several tokens of every request (SchedulerConfig.decode_steps): the
@@ -126,12 +133,12 @@ def decode_run(engine, cfg, batch, context, steps, warmup, decode_steps=1):
         prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).tolist()
         ids.append(f"b{batch}-{i}")
         # requests that were admitted first decode a few tokens while the others still prefill
-        engine.add_request(ids[-1], prompt, SamplingParams(max_tokens=steps + warm + per + 1 + SLACK, ignore_eos=True))
+        engine.add_request(ids[-1], prompt, SamplingParams(max_tokens=steps + warm + per + 1 + slack, ignore_eos=True))
     guard = 0
     while engine.scheduler.waiting or any(r.num_computed_tokens < prompt_len for r in engine.scheduler.running):
         engine.step()  # prefill, in portions under the token budget
         guard += 1
-        assert guard < SLACK, "prefill took more steps than the pool has slack for"
+        assert guard < slack, "prefill took more steps than the pool has slack for"
     import dataclasses
 
     def advance(chunks):
