@@ -31,7 +31,7 @@ from .batch import GroupView, StepContext, StepEntry
 from .table_rows import TableRows
 
 
-# A recording costs as much time as fifteen to thirty decode steps; a recorded shape of more rows that
+# A recording costs as much time as ten to twenty decode steps; a recorded shape of more rows that
 # stands in costs a tenth to a third of a step more. A shape is recorded once it has been asked for
 # RECORD_AFTER_STEPS decode steps, at once if nothing recorded can stand in, or if what can has more
 # than STAND_IN_ROWS times its rows.
@@ -173,9 +173,9 @@ class DecodeGraphs:
         # No cyclic garbage collection while the stream is capturing: a dead cycle that holds
         # device memory or an older graph (an engine that was dropped) would be destroyed in the
         # middle of the capture, and freeing those is not allowed there (the process aborts).
-        # Such cycles are collected before the capture instead.
+        # Such cycles wait for the first collection after the capture (collecting them here, before
+        # it, took 30 ms beside a loaded model: three times what the recording itself takes).
         collecting = gc.isenabled()
-        gc.collect()
         gc.disable()
         try:
             with torch.cuda.graph(graph):
