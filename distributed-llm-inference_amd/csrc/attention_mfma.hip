@@ -529,7 +529,12 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // a tile through registers took a third of the kernel's time at 8,192 tokens).
 // Products use v_mfma_f32_16x16x32_bf16 (lane l: row/column l%16, k-indices 8*(l/16)..+7). For
 // P*V the eight k-indices of lane group g stand for the keys 8g..8g+7 of the tile.
-// Needs head_dim % 32 == 0.
+// Head sizes of 32 to 128 in steps of 16. Where the size is no multiple of 32 (48, 80, 112) the
+// first product's last sixteen dims take one v_mfma_f32_16x16x16_bf16, and K lies in LDS part by
+// part (chunk `part` of the tile's 32 keys side by side, the sixteen keys of a product next to
+// each other: sixteen lanes then read 256 consecutive bytes whatever the row length), which the
+// loads arrange by the address each lane reads from; a block of 64 chunks then holds keys of
+// both halves of the tile, so the half's page is chosen lane by lane.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ float4v mfma32(bf16x8 a, bf16x8 b, float4v c) {
@@ -580,7 +585,9 @@ void attention_prefill_shared_kernel(
     const int* __restrict__ tile_q0, int q_heads, int kv_heads, int page_size, float scale_log2e,
     int window, int heads_per_wg, const int* __restrict__ tile_cut, int cut_room, float* cut_buf,
     unsigned* cut_count) {
-  constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of the first product
+  constexpr int D = DCH * 16, DK = D / 32;      // DK: k-steps of 32 dims of the first product
+  constexpr bool ODD = DCH % 2 != 0;            // sixteen dims more, and K part by part in LDS
+  static_assert(DCH >= 2 && DCH <= 8, "heads of 32 to 128");
   constexpr int R = D / 8;                      // 16-byte chunks in a key's row of K
   constexpr int NT = 256;                       // threads
   constexpr int NW = NT / DLI_WAVE;             // waves
@@ -632,6 +639,7 @@ void attention_prefill_shared_kernel(
   const int* table = block_tables + (int64_t)e * table_stride;
 
   bf16x8 qreg[2][DK];
+  short4v qtail[2];   // dims 32 DK + 4 grp .. + 3 (ODD)
   ColumnTile<DCH> st[2];
   // beside st[j].m: the value subtracted in the exponent (m, or 0 while m is -inf), and the raw
   // score above which m has to rise
@@ -648,10 +656,12 @@ void attention_prefill_shared_kernel(
     pos[j] = qi < q_len ? first_pos + qi : -1;
 #pragma unroll
     for (int c = 0; c < DK; ++c) qreg[j][c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    qtail[j] = short4v{0, 0, 0, 0};
     if (qi < q_len) {
       const bf16_t* qp = q + (int64_t)(tok0 + qi) * q_stride + (int64_t)head * D + grp * 8;
 #pragma unroll
       for (int c = 0; c < DK; ++c) qreg[j][c] = *reinterpret_cast<const bf16x8*>(qp + c * 32);
+      if constexpr (ODD) qtail[j] = *reinterpret_cast<const short4v*>(qp - grp * 8 + 32 * DK + grp * 4);
     }
   }
   // this wave's span, the same in all its lanes and said so: what is decided from it per tile
@@ -680,21 +690,40 @@ void attention_prefill_shared_kernel(
   unsigned lane_off[UCH];   // elements from the half's first key in its page
   int block_at[UCH];        // the block's first element in a tile
   bool second_half[UCH], is_v[UCH];  // the same in all lanes
+  bool lane_second[UCH];    // ODD: the half of the tile that this lane's chunk belongs to
 #pragma unroll
   for (int r = 0; r < UCH; ++r) {
     // with more waves than blocks, the others load a block a second time (same bytes, same place):
     // every wave then has the same number of loads in flight
     const int blk = (wave_id + r * NW) % BLOCKS;
     is_v[r] = blk >= DCH;
-    second_half[r] = blk % DCH >= DCH / 2;
     block_at[r] = blk * 512;
-    const int p = (blk % (DCH / 2)) * 64 + lane;  // the lane's chunk within the half's region
-    if (!is_v[r]) {
-      const int kk = p / R, part = (p % R) ^ k_swizzle<R>(kk + (second_half[r] ? 16 : 0));
-      lane_off[r] = kk * D + part * 8;
+    if constexpr (!ODD) {
+      second_half[r] = blk % DCH >= DCH / 2;
+      lane_second[r] = second_half[r];
+      const int p = (blk % (DCH / 2)) * 64 + lane;  // the lane's chunk within the half's region
+      if (!is_v[r]) {
+        const int kk = p / R, part = (p % R) ^ k_swizzle<R>(kk + (second_half[r] ? 16 : 0));
+        lane_off[r] = kk * D + part * 8;
+      } else {
+        const int d = p / 2, sub = (p % 2) ^ ((d >> 3) & 1);
+        lane_off[r] = d * page_size + sub * 8;
+      }
     } else {
-      const int d = p / 2, sub = (p % 2) ^ ((d >> 3) & 1);
-      lane_off[r] = d * page_size + sub * 8;
+      second_half[r] = false;
+      const int pg = (blk % DCH) * 64 + lane;       // the lane's chunk within the region of K or of V^T
+      if (!is_v[r]) {
+        // chunk pg of K's region: part pg / 32 of the key that row pg % 16 of product pg % 32 / 16 takes
+        const int part = pg / 32, kp = pg % 32, cl = kp % 16;
+        const int key = 8 * (cl / 4) + 4 * (kp / 16) + cl % 4;
+        lane_second[r] = key >= 16;
+        lane_off[r] = (key % 16) * D + part * 8;
+      } else {
+        const int p = pg % (32 * DCH);                // the chunk within its half's region
+        const int d = p / 2, sub = (p % 2) ^ ((d >> 3) & 1);
+        lane_second[r] = pg >= 32 * DCH;
+        lane_off[r] = d * page_size + sub * 8;
+      }
     }
   }
   // Tiles are fetched in order, so the page of the tile's first key is tracked by addition
@@ -742,8 +771,16 @@ void attention_prefill_shared_kernel(
 #pragma unroll
     for (int r = 0; r < UCH; ++r) {
       // the same for every lane of the wave: a key's row of K is D long, a key's column of V^T one element
-      const unsigned off = second_half[r] ? ob : oa;
-      const bf16_t* base = (is_v[r] ? v_head : k_head) + (second_half[r] ? at_b : at_a) + (is_v[r] ? off : off * D);
+      const bf16_t* base;
+      if constexpr (!ODD) {
+        const unsigned off = second_half[r] ? ob : oa;
+        base = (is_v[r] ? v_head : k_head) + (second_half[r] ? at_b : at_a) + (is_v[r] ? off : off * D);
+      } else {  // both halves' places on the scalar unit, the lane takes its own
+        const bf16_t* head_base = is_v[r] ? v_head : k_head;
+        const bf16_t* base_a = head_base + at_a + (is_v[r] ? oa : oa * D);
+        const bf16_t* base_b = head_base + at_b + (is_v[r] ? ob : ob * D);
+        base = lane_second[r] ? base_b : base_a;
+      }
       __builtin_amdgcn_global_load_lds(
           (const __attribute__((address_space(1))) void*)(base + lane_off[r]),
           (__attribute__((address_space(3))) void*)&lds[buf][block_at[r]], 16, 0, 0);
@@ -763,12 +800,19 @@ void attention_prefill_shared_kernel(
   // probabilities of the eight consecutive keys 8g..8g+7, whose values (dim row 16c+col) lie in
   // LDS as one chunk of 16 bytes.
   int k_at[2][DK];
+  int k_tail_at[2];   // ODD: the lane's four dims of the last sixteen
   const int key_row = 8 * (col / 4) + col % 4;  // of the first product; the second's: four rows on
 #pragma unroll
-  for (int b = 0; b < 2; ++b)
+  for (int b = 0; b < 2; ++b) {
 #pragma unroll
-    for (int c = 0; c < DK; ++c)
-      k_at[b][c] = (key_row + 4 * b) * D + ((c * 4 + grp) ^ k_swizzle<R>(key_row + 4 * b)) * 8;
+    for (int c = 0; c < DK; ++c) {
+      if constexpr (!ODD)
+        k_at[b][c] = (key_row + 4 * b) * D + ((c * 4 + grp) ^ k_swizzle<R>(key_row + 4 * b)) * 8;
+      else
+        k_at[b][c] = ((c * 4 + grp) * 32 + b * 16 + col) * 8;
+    }
+    k_tail_at[b] = ((4 * DK + (grp >> 1)) * 32 + b * 16 + col) * 8 + (grp & 1) * 4;
+  }
   const int v_at = (grp >> 1) * VH_ELEMS + col * 16 + ((grp & 1) ^ (col >> 3)) * 8;
   // the tiles that the wave sees, [see_from, see_until], and among them those that need no mask,
   // [plain_until, plain_from] (tile starts; an empty range where there is no such tile)
@@ -795,6 +839,11 @@ void attention_prefill_shared_kernel(
         kf0[c] = *reinterpret_cast<const bf16x8*>(ks + k_at[0][c]);
         kf1[c] = *reinterpret_cast<const bf16x8*>(ks + k_at[1][c]);
       }
+      short4v kt0 = short4v{0, 0, 0, 0}, kt1 = short4v{0, 0, 0, 0};
+      if constexpr (ODD) {
+        kt0 = *reinterpret_cast<const short4v*>(ks + k_tail_at[0]);
+        kt1 = *reinterpret_cast<const short4v*>(ks + k_tail_at[1]);
+      }
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
         vf[c] = *reinterpret_cast<const bf16x8*>(vs + c * 256 + v_at);
@@ -813,6 +862,13 @@ void attention_prefill_shared_kernel(
           sa[j] = mfma32(kf0[c], qreg[j][c], sa[j]);
           sb[j] = mfma32(kf1[c], qreg[j][c], sb[j]);
         }
+      if constexpr (ODD) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          sa[j] = mfma16(kt0, qtail[j], sa[j]);
+          sb[j] = mfma16(kt1, qtail[j], sb[j]);
+        }
+      }
       float sv[2][8];
 #pragma unroll
       for (int j = 0; j < 2; ++j)
@@ -1020,9 +1076,9 @@ extern "C" int dli_attention_mfma_supports(int head_dim, int page_size) {
 }
 
 // Query heads that one workgroup of the shared-tile kernel takes (4, 2 or 1), or 0 if the shape
-// has to take the plain kernel (head_dim not a multiple of 32).
+// has to take the plain kernel (heads of 16).
 static int shared_heads_per_wg(int head_dim, int group) {
-  if (head_dim % 32 != 0) return 0;
+  if (head_dim % 16 != 0 || head_dim < 32) return 0;
   return group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
 }
 
@@ -1193,7 +1249,7 @@ extern "C" int dli_attention_prefill_max_cuts() { return PREFILL_MAX_CUTS; }
 // tile_cut (or null: every tile whole): per entry of the tile list -1, or run | runs << 4 |
 // place << 8 for one of the 2 to dli_attention_prefill_max_cuts() runs of a tile whose keys that
 // many workgroups share, `place` numbering the cut tiles from 0 to cut_tiles - 1; all runs of a
-// tile must be listed. Only without a window and for head sizes that are multiples of 32.
+// tile must be listed. Only without a window and for heads of 32 and more.
 // cut_room: the most runs of any tile; cut_buf: cut_tiles * cut_room *
 // dli_attention_prefill_cut_floats() values; cut_count: one counter per cut tile and workgroup of
 // a tile (cut_tiles * q_heads is enough), zero before the first launch; every launch leaves them
@@ -1227,7 +1283,7 @@ extern "C" int dli_attention_prefill_bf16(const void* q, int64_t q_stride, const
         kv_heads, page_size, scale * LOG2E, window, hw, tile_cut, cut_room, cut_buf, cut_count);  \
     break;
     switch (head_dim / 16) {
-      SHARED_CASE(2) SHARED_CASE(4) SHARED_CASE(6) SHARED_CASE(8)
+      SHARED_CASE(2) SHARED_CASE(3) SHARED_CASE(4) SHARED_CASE(5) SHARED_CASE(6) SHARED_CASE(7) SHARED_CASE(8)
       default: return DLI_ERR_ARGUMENT;
     }
 #undef SHARED_CASE

@@ -169,11 +169,11 @@ def prefill_tiles(ctx: Any, head_dim: int, q_heads: int, kv_heads: int, first_en
     """The tile list of the step's portions for :func:`ops.attention_prefill` (made once per step
     and shape; the buffers of the cut tiles serve every layer of that shape in turn)."""
     rows = ops.attention_prefill_tile_rows(head_dim, q_heads, kv_heads)
-    # a workgroup takes a tile for 4 * 32 / rows query heads where it shares tiles (head sizes that
-    # are multiples of 32), else for one
-    per_tile = q_heads * rows // 128 if head_dim % 32 == 0 else q_heads
     units = ops.compute_units(device)
     cut_floats = ops.attention_prefill_cut_floats(head_dim, q_heads, kv_heads)
+    # a workgroup takes a tile for 4 * 32 / rows query heads where the kernel's waves share key
+    # tiles (heads of 32 and more: the kernel that can also cut a tile's keys), else for one
+    per_tile = q_heads * rows // 128 if cut_floats > 0 else q_heads
     may_cut = window == 0 and cut_floats > 0
 
     def make() -> PrefillTiles:

@@ -340,7 +340,8 @@ def test_attention_prefill_mfma(ops, qh, kvh, d, bs, window):
     assert err < tol(torch.bfloat16), err
 
 
-@pytest.mark.parametrize("qh,kvh,d", [(16, 16, 64), (8, 4, 32), (12, 4, 128), (16, 4, 64), (9, 3, 64), (8, 2, 96)])
+@pytest.mark.parametrize("qh,kvh,d", [(16, 16, 64), (8, 4, 32), (12, 4, 128), (16, 4, 64), (9, 3, 64), (8, 2, 96),
+                                      (8, 2, 80), (6, 3, 48), (7, 1, 112), (10, 2, 80)])
 def test_attention_prefill_of_a_launch_of_one_and_a_half_workgroups_a_unit(ops, qh, kvh, d):
     """A launch in which compute units work on two tiles of different lengths at a time (and, with
     many heads, in which the order of the workgroups differs from the grid's), listed as the engine
