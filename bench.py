@@ -304,6 +304,9 @@ def main() -> int:
     ap.add_argument("--shape", default="Llama-3.2-1B", choices=sorted(SHAPES),
                     help="layer sizes (the default is the configuration that the headline number is quoted on)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has")
+    ap.add_argument("--size", action="append", default=[], metavar="KEY=INT",
+                    help="another value for a size of the shape's config.json, e.g. --size head_dim=80 "
+                         "--size hidden_size=2560 (measurements at other sizes; the line's model name says so)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--decode-steps", type=int, default=8,
@@ -332,6 +335,13 @@ def main() -> int:
     import torch
 
     raw = dict(SHAPES[args.shape])
+    for item in args.size:
+        key, _, value = item.partition("=")
+        if key not in raw or not isinstance(raw[key], int) or isinstance(raw[key], bool):
+            ap.error(f"--size {item}: {key!r} is no integer size of the shape's configuration")
+        raw[key] = int(value)
+    if args.size:
+        args.shape += " with " + ", ".join(args.size)
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
