@@ -18,6 +18,7 @@ The reference replays CUDA graphs of batched decode in fixed buckets the same wa
 from __future__ import annotations
 
 import gc
+import weakref
 
 from dataclasses import dataclass
 from typing import Optional, Sequence
@@ -37,6 +38,8 @@ from .table_rows import TableRows
 # than STAND_IN_ROWS times its rows.
 RECORD_AFTER_STEPS = 64
 STAND_IN_ROWS = 4
+
+_RECORDERS: "weakref.WeakSet[DecodeGraphs]" = weakref.WeakSet()  # every recorder that has not been collected yet
 
 
 def _bucket(n: int) -> int:
@@ -75,6 +78,7 @@ class DecodeGraphs:
         self.n_groups = step_fn.manager.num_groups
         self.captured: dict[tuple, _Captured] = {}
         self._asked: dict[tuple, int] = {}   # decode steps that a shape that is not recorded has been asked for
+        _RECORDERS.add(self)
         self.replays = 0
         self.enabled = self._supported()
 
@@ -173,9 +177,13 @@ class DecodeGraphs:
         # No cyclic garbage collection while the stream is capturing: a dead cycle that holds
         # device memory or an older graph (an engine that was dropped) would be destroyed in the
         # middle of the capture, and freeing those is not allowed there (the process aborts).
-        # Such cycles wait for the first collection after the capture (collecting them here, before
-        # it, took 30 ms beside a loaded model: three times what the recording itself takes).
+        # Where the process has had other recorders than this one, such cycles are collected here,
+        # before the capture, with the device idle (an older graph is then never taken apart while
+        # a newer one runs). A process with one engine skips this: the collection takes 30 ms
+        # beside a loaded model, three times what the recording itself takes.
         collecting = gc.isenabled()
+        if len(_RECORDERS) > 1:
+            gc.collect()
         gc.disable()
         try:
             with torch.cuda.graph(graph):
