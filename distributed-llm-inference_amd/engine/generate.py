@@ -42,19 +42,20 @@ def pages_for_requests(lengths: Sequence[int], block_size: int, max_num_seqs: in
     return max(1, min(wanted, most)) if each else 1
 
 
-GRAPHS_PAY_FROM = 64  # decode steps of a call from which recording its decode graphs pays
+GRAPHS_PAY_FROM = 128  # decode steps of a call from which recording its decode graphs pays
 
 
 def graphs_pay(max_tokens: Sequence[int], max_num_seqs: int) -> bool:
     """Whether a call that builds its own engine should record decode graphs: the graphs of a
-    call are recorded during it (a handful of them, some 10 ms each at the 1B sizes: the shapes
-    that a batch's tail asks for a few times are served by a recorded shape of more rows) and
-    save up to a millisecond a decode step afterwards, so they pay from a few dozen steps on
-    (64 requests, prompts of 128 to 2,048 tokens, seconds without and with them: 32 tokens each
-    0.31 and 0.33, 64 tokens 0.40 and 0.41, 128 tokens 0.59 and 0.53, 256 tokens 0.97 and 0.82,
-    1,024 tokens 3.43 and 2.49; 8 requests: 32 tokens 0.088 and 0.084, 128 tokens 0.27 and 0.19,
-    1,024 tokens 2.02 and 1.05). The steps are estimated as the longest generation times the
-    rounds that the requests need at ``max_num_seqs`` a time."""
+    call are recorded during it (a handful of them, some 10 ms each at the 1B sizes, and 30 ms
+    once for collecting the engine of an earlier call: the shapes that a batch's tail asks for a
+    few times are served by a recorded shape of more rows) and save up to a millisecond a decode
+    step afterwards, so they pay from about a hundred steps on (calls in a row in one process, 64
+    requests, prompts of 128 to 2,048 tokens, seconds without and with them: 64 tokens each 0.41
+    and 0.48, 128 tokens 0.60 and 0.58, 256 tokens 0.99 and 0.85, 1,024 tokens 3.41 and 2.52; 8
+    requests: 64 tokens 0.152 and 0.163, 128 tokens 0.28 and 0.22, 1,024 tokens 2.03 and 1.09).
+    The steps are estimated as the longest generation times the rounds that the requests need at
+    ``max_num_seqs`` a time."""
     if not max_tokens:
         return False
     rounds = -(-len(max_tokens) // max(1, max_num_seqs))

@@ -71,10 +71,10 @@ def test_a_call_records_graphs_where_it_decodes_long_enough():
     from dli_amd.engine.generate import GRAPHS_PAY_FROM, graphs_pay
 
     assert not graphs_pay([], 64)
-    assert not graphs_pay([16, 32], 256)                       # 32 decode steps
+    assert not graphs_pay([16, 64], 256)                       # 64 decode steps
     assert graphs_pay([16, GRAPHS_PAY_FROM], 256)
-    assert graphs_pay([32] * 600, 256)                         # three rounds of 32 steps
-    assert not graphs_pay([32] * 256, 256) and graphs_pay([32] * 257, 256)
+    assert graphs_pay([64] * 600, 256)                         # three rounds of 64 steps
+    assert not graphs_pay([64] * 256, 256) and graphs_pay([64] * 257, 256)
 
 
 def test_which_tiles_of_a_short_launch_have_their_keys_cut():
