@@ -146,3 +146,31 @@ def test_the_tile_list_of_a_step_lists_every_tile_once_or_all_of_its_runs():
         assert max(r[0][1] for r in runs.values()) == room
         assert sorted(r[0][2] for r in runs.values()) == list(range(n_cut))
         assert len(ent) * per_tile <= 3 * units
+
+
+def test_which_recorded_shape_stands_in_for_one_that_is_not_recorded():
+    """Fewest rows first, then the same plans, then the narrowest table; never fewer rows than
+    requests, more than four times the shape's own rows, a narrower table, another number of
+    steps or another kind of output."""
+    from dli_amd.engine import decode_graph
+    from dli_amd.engine.decode_graph import DecodeGraphs
+
+    graphs = DecodeGraphs.__new__(DecodeGraphs)   # the choice reads the recorded shapes only
+    plans_a, plans_b = (2, 2), (4, 4)
+
+    def choice(key, requests, recorded):
+        graphs.captured = {k: f"graph of {k}" for k in recorded}
+        got = graphs._stand_in(key, requests)
+        return None if got is None else got[0]
+
+    want = (4, plans_a, 64, True, 1)
+    assert choice(want, 3, []) is None
+    assert choice(want, 3, [(8, plans_b, 64, True, 1), (16, plans_a, 64, True, 1)]) == (8, plans_b, 64, True, 1)
+    assert choice(want, 3, [(8, plans_b, 64, True, 1), (8, plans_a, 128, True, 1)]) == (8, plans_a, 128, True, 1)
+    assert choice(want, 3, [(8, plans_a, 256, True, 1), (8, plans_a, 128, True, 1)]) == (8, plans_a, 128, True, 1)
+    assert choice(want, 3, [(4, plans_b, 128, True, 1)]) == (4, plans_b, 128, True, 1)   # its own rows, other plans
+    assert choice(want, 3, [(2, plans_a, 64, True, 1)]) is None                          # too few rows
+    assert choice(want, 3, [(8, plans_a, 32, True, 1)]) is None                          # too narrow a table
+    assert choice(want, 3, [(8, plans_a, 64, True, 2), (8, plans_a, 64, False, 1)]) is None
+    assert choice(want, 3, [(4 * decode_graph.STAND_IN_ROWS, plans_a, 64, True, 1)]) is not None
+    assert choice(want, 3, [(4 * decode_graph.STAND_IN_ROWS + 16, plans_a, 64, True, 1)]) is None
