@@ -64,7 +64,7 @@ class HostBatch:
     state_slots: np.ndarray       # int32 [entries]
     logit_rows: np.ndarray        # int32 [k], in the caller's order of entries and wants
     slots: list                   # per group: int64 [tokens]
-    tables: list                  # per group: one int64 array of pages per entry
+    tables: list                  # per group: int64 [entries, widest table], a row of pages per entry, padded with zeros
 
     @property
     def num_tokens(self) -> int:

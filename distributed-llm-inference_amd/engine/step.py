@@ -67,18 +67,21 @@ class StepFunction:
     def lay_out(self, entries: Sequence[StepEntry]) -> HostBatch:
         """Check the entries against the cache manager and lay the batch out in host arrays."""
         mgr, ps = self.manager, self.manager.page_size
+        count = len(entries)
         seen = set()
+        lengths = []
         for e in entries:
             if e.seq_id in seen:
                 raise StepError(f"request {e.seq_id!r} appears twice in one step")
             seen.add(e.seq_id)
             n = len(e.tokens)
+            lengths.append(n)
             if n == 0:
                 raise StepError(f"request {e.seq_id!r} brings no tokens")
-            if e.start != mgr.num_computed_tokens(e.seq_id):
+            computed = mgr.num_computed_tokens(e.seq_id)
+            if e.start != computed:
                 raise StepError(
-                    f"request {e.seq_id!r}: portion starts at {e.start} but "
-                    f"{mgr.num_computed_tokens(e.seq_id)} tokens are computed")
+                    f"request {e.seq_id!r}: portion starts at {e.start} but {computed} tokens are computed")
             if e.start + n > mgr.num_tokens(e.seq_id):
                 raise StepError(f"request {e.seq_id!r}: no cache slots reserved up to {e.start + n}")
             for wnt in e.want:
@@ -86,57 +89,64 @@ class StepFunction:
                     raise StepError(f"request {e.seq_id!r}: wanted place {wnt} outside its {n} tokens")
 
         # single-token entries first, then portions; each kind in the given order
-        order = [i for i, e in enumerate(entries) if len(e.tokens) == 1] + \
-                [i for i, e in enumerate(entries) if len(e.tokens) != 1]
-        num_decode = sum(1 for e in entries if len(e.tokens) == 1)
-        q_start = np.zeros(len(entries) + 1, np.int32)
-        first_row = {}
-        for k, i in enumerate(order):
-            first_row[i] = int(q_start[k])
-            q_start[k + 1] = q_start[k] + len(entries[i].tokens)
+        order = [i for i in range(count) if lengths[i] == 1] + [i for i in range(count) if lengths[i] != 1]
+        num_decode = sum(1 for n in lengths if n == 1)
+        ordered = [entries[i] for i in order]
+        q_start = np.zeros(count + 1, np.int32)
+        np.cumsum([lengths[i] for i in order], out=q_start[1:])
+        first_row = dict(zip(order, q_start[:-1].tolist()))
         total = int(q_start[-1])
+        starts = np.asarray([e.start for e in ordered], np.int64)
+        kv_len = (starts + np.asarray([lengths[i] for i in order], np.int64)).astype(np.int32)
+        state_slots = np.asarray([mgr.state_slot(e.seq_id) for e in ordered], np.int32)
         token_ids = np.empty(total, np.int64)
         positions = np.empty(total, np.int32)
-        kv_len = np.empty(len(entries), np.int32)
-        state_slots = np.empty(len(entries), np.int32)
-        n_groups = mgr.num_groups
-        slots = [np.empty(total, np.int64) for _ in range(n_groups)]
-        tables: list[list[np.ndarray]] = [[] for _ in range(n_groups)]
-        for k, i in enumerate(order):
-            e = entries[i]
-            r0, n = int(q_start[k]), len(e.tokens)
-            token_ids[r0:r0 + n] = e.tokens
-            pos = np.arange(e.start, e.start + n, dtype=np.int64)
-            positions[r0:r0 + n] = pos
-            kv_len[k] = e.start + n
-            state_slots[k] = mgr.state_slot(e.seq_id)
-            for g in range(n_groups):
-                table = np.asarray(mgr.table_ref(e.seq_id, g), dtype=np.int64)
-                if table.size * ps < e.start + n:
-                    raise StepError(f"request {e.seq_id!r}: block table shorter than its keys")
-                # a page that the window has passed gives a negative slot, refused below
-                slots[g][r0:r0 + n] = table[pos // ps] * ps + pos % ps
-                tables[g].append(table)
+        # the single tokens at once, the portions one by one
+        token_ids[:num_decode] = [e.tokens[0] for e in ordered[:num_decode]]
+        positions[:num_decode] = starts[:num_decode]
+        for k in range(num_decode, count):
+            e, r0, r1 = ordered[k], int(q_start[k]), int(q_start[k + 1])
+            token_ids[r0:r1] = e.tokens
+            positions[r0:r1] = np.arange(e.start, e.start + r1 - r0)
         if total and (int(token_ids.min()) < 0 or int(token_ids.max()) >= self.vocab_size):
             bad = int(token_ids[(token_ids < 0) | (token_ids >= self.vocab_size)][0])
             raise StepError(f"token id {bad} outside the vocabulary")
         logit_rows = np.asarray(
             [first_row[i] + int(w) for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
-        limit = self.store.num_pages
+
+        n_groups, limit = mgr.num_groups, self.store.num_pages
+        pos64 = positions.astype(np.int64)
+        row_entry = np.repeat(np.arange(count), np.diff(q_start)) if total else np.zeros(0, np.int64)
+        slots: list[np.ndarray] = []
+        tables: list[np.ndarray] = []
         for g in range(n_groups):
-            if total and (int(slots[g].min()) < 0 or int(slots[g].max()) >= limit * ps):
-                raise StepError("a cache slot lies outside the pool, or in a page that the window has passed")
-            pages = np.concatenate(tables[g]) if tables[g] else np.zeros(0, np.int64)
-            if pages.size and (int(pages.min()) < RELEASED or int(pages.max()) >= limit):
+            # the block tables of the group as the rows of one array, padded with zeros
+            lists = [mgr.table_ref(e.seq_id, g) for e in ordered]
+            width = max(map(len, lists), default=1) or 1
+            rows = np.zeros((max(count, 1), width), np.int64)
+            held = np.zeros(max(count, 1), np.int64)
+            for k, t in enumerate(lists):
+                rows[k, :len(t)] = t
+                held[k] = len(t)
+            short = np.flatnonzero(held[:count] * ps < kv_len)
+            if short.size:
+                raise StepError(f"request {ordered[int(short[0])].seq_id!r}: block table shorter than its keys")
+            if rows.size and (int(rows.min()) < RELEASED or int(rows.max()) >= limit):
                 raise StepError("a block table names a page outside the pool")
-        return HostBatch(order=order, seq_ids=[entries[i].seq_id for i in order], num_decode=num_decode,
+            # a page that the window has passed gives a negative slot, refused here
+            where = rows[row_entry, pos64 // ps] * ps + pos64 % ps
+            if total and (int(where.min()) < 0 or int(where.max()) >= limit * ps):
+                raise StepError("a cache slot lies outside the pool, or in a page that the window has passed")
+            rows[rows == RELEASED] = 0  # pages that the window has passed: never read
+            slots.append(where)
+            tables.append(rows)
+        return HostBatch(order=order, seq_ids=[e.seq_id for e in ordered], num_decode=num_decode,
                          token_ids=token_ids, positions=positions, q_start=q_start, kv_len=kv_len,
                          state_slots=state_slots, logit_rows=logit_rows, slots=slots, tables=tables)
 
     def upload_context(self, batch: HostBatch) -> StepContext:
         """The device-side context of a laid-out step (one copy from pinned memory)."""
-        n_groups, total, entries = self.manager.num_groups, batch.num_tokens, batch.order
-        tables, slots = batch.tables, batch.slots
+        n_groups, total = self.manager.num_groups, batch.num_tokens
         dev = self.rt.device
         # every integer array of the step goes to the device in one copy from pinned memory
         pending: list[np.ndarray] = []
@@ -145,21 +155,15 @@ class StepFunction:
             pending.append(np.ascontiguousarray(a, dtype=np.int32))
             return len(pending) - 1
 
-        group_arrays: list[tuple[int, int, int]] = []
-        for g in range(n_groups):
-            width = max((len(t) for t in tables[g]), default=1) or 1
-            host = np.zeros((max(len(entries), 1), width), np.int64)
-            for k, t in enumerate(tables[g]):
-                host[k, :t.size] = t
-            host[host == RELEASED] = 0  # pages that the window has passed: never read
-            group_arrays.append((to_dev(slots[g]), to_dev(host), width))
+        group_arrays = [(to_dev(batch.slots[g]), to_dev(batch.tables[g]), batch.tables[g].shape[1])
+                        for g in range(n_groups)]
         named = {name: to_dev(a) for name, a in (
             ("token_ids", batch.token_ids), ("positions", batch.positions), ("q_start", batch.q_start),
             ("kv_len", batch.kv_len), ("state_slots", batch.state_slots), ("logit_rows", batch.logit_rows))}
         views = upload(pending, dev)
         groups = [GroupView(views[s_], views[t_], width) for s_, t_, width in group_arrays]
         return StepContext(
-            device=dev, page_size=self.manager.page_size, num_tokens=total, num_entries=len(entries),
+            device=dev, page_size=self.manager.page_size, num_tokens=total, num_entries=len(batch.order),
             num_decode=batch.num_decode, groups=groups, q_start_host=batch.q_start, kv_len_host=batch.kv_len,
             state_slots_host=batch.state_slots, seq_ids=batch.seq_ids, **{name: views[i] for name, i in named.items()})
 
