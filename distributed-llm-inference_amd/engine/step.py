@@ -250,9 +250,9 @@ class StepFunction:
                     raise StepError(f"request {e.seq_id!r}: no cache room reserved for {steps} tokens")
         rounds = self.graphs.run(entries, sampling, steps=steps)
         for i, e in enumerate(entries):
-            for j in range(steps - 1):
-                if mgr.append_slots(e.seq_id, [rounds[j][i]]):
-                    raise StepError("a page reserved ahead was shared")
+            # all tokens but the last in one call: the pages were reserved, none of them is shared
+            if mgr.append_slots(e.seq_id, [rounds[j][i] for j in range(steps - 1)]):
+                raise StepError("a page reserved ahead was shared")
             mgr.mark_computed(e.seq_id, e.start + steps)
         self.steps_run += steps
         return rounds
